@@ -1,0 +1,14 @@
+"""brainpylib_amd: brainpylib's event-driven sparse operators for one AMD Instinct MI355X.
+
+Same operator names, keyword arguments and semantics as ``brainpylib`` for the path that matters
+in a spiking-network step (``event_csr_matvec``, ``csr_matvec``, the jitconn family); the
+operators take and return ``torch`` tensors on the GPU and run hand-written gfx950 kernels through
+the XLA custom-call ABI exported by ``lib/libbrainpylib_amd.so``.  There is no CPU fallback.
+"""
+__version__ = "0.1.0"
+
+from ._lib import GPUOperatorNotFound
+from .event_ops import event_csr_matvec
+from .sparse_ops import csr_matvec, cusparse_csr_matvec
+
+__all__ = ["event_csr_matvec", "csr_matvec", "cusparse_csr_matvec", "GPUOperatorNotFound"]

@@ -1,0 +1,102 @@
+// Internal helpers shared by the HIP sources of libbrainpylib_amd.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <cstring>
+
+#include "../../include/brainpylib_amd.h"
+
+namespace bpl {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+// ---- error channel (host) ---------------------------------------------------------------------
+void set_error(const char *fmt, ...);
+
+// Checks `opaque_len == sizeof(T)` and copies the descriptor out of the opaque bytes
+// (the pointer is not assumed to be aligned).  Returns false and records an error otherwise.
+template <typename T>
+inline bool unpack(const char *target, const char *opaque, size_t opaque_len, T *out) {
+  if (opaque == nullptr || opaque_len != sizeof(T)) {
+    set_error("%s: invalid opaque object size %zu (expected %zu)", target, opaque_len, sizeof(T));
+    return false;
+  }
+  std::memcpy(out, opaque, sizeof(T));
+  return true;
+}
+
+// Records a failed launch; returns true if the last launch was fine.
+bool check_launch(const char *target);
+
+// Device properties of the current device, cached per device id.
+struct DeviceInfo {
+  int num_cu = 0;
+  int lds_per_block = 0;  // bytes of LDS one workgroup may use
+};
+const DeviceInfo &device_info();
+
+inline unsigned div_up(unsigned long long a, unsigned long long b) {
+  return static_cast<unsigned>((a + b - 1) / b);
+}
+
+// ---- zero fill on the stream (a kernel, not a memset node, so that the call sequence can be
+// captured into a HIP graph) ---------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void fill_zero_kernel(T *__restrict__ p, uint32_t n) {
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  if (i < n) p[i] = T(0);
+}
+
+template <typename T>
+inline void fill_zero(hipStream_t stream, T *p, uint32_t n) {
+  if (n == 0) return;
+  hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(div_up(n, 256)), dim3(256), 0, stream, p, n);
+}
+
+// ---- device helpers -----------------------------------------------------------------------------
+__device__ __forceinline__ int lane_id() { return static_cast<int>(threadIdx.x) & (kWave - 1); }
+
+// events are `bool` (one byte, any nonzero byte counts) or a float type (nonzero, NaN included).
+template <typename VT>
+__device__ __forceinline__ bool is_event(VT v) {
+  return v != VT(0);
+}
+
+// Sum over the 64 lanes of a wave; every lane receives the total.
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+// Sum over aligned groups of G consecutive lanes (G a power of two <= 64).
+template <int G, typename T>
+__device__ __forceinline__ T group_sum(T v) {
+#pragma unroll
+  for (int off = G / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+// Inclusive prefix sum of a 32-bit value across the wave (wrapping), via DPP row shifts and
+// row broadcasts.
+__device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v) {
+  int x = static_cast<int>(v);
+  // within each row of 16 lanes
+  x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, false);  // row_shr:1
+  x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, false);  // row_shr:2
+  x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, false);  // row_shr:4
+  x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, false);  // row_shr:8
+  // carry row totals: lane 15 of rows 0,2 into rows 1,3; then lane 31 into rows 2,3
+  x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, false);  // row_bcast:15
+  x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, false);  // row_bcast:31
+  return static_cast<uint32_t>(x);
+}
+
+__device__ __forceinline__ void atomic_add(float *p, float v) { unsafeAtomicAdd(p, v); }
+__device__ __forceinline__ void atomic_add(double *p, double v) { unsafeAtomicAdd(p, v); }
+
+}  // namespace bpl

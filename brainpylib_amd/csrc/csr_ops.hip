@@ -1,0 +1,398 @@
+// event_csr_matvec and csr_matvec for gfx950 (wave64).
+//
+// Two kernel families serve both operators:
+//
+//   scatter  (transpose):  y[indices[j]] += w(j)  for the nonzeros j of the rows r that are "on"
+//            A workgroup owns 64 consecutive rows.  Wave 0 tests the rows' events, compacts the
+//            active rows and prefix-sums their lengths in LDS (ballot + DPP scan); then all 256
+//            threads walk the workgroup's active nonzeros as ONE flat range, so lanes stay
+//            coalesced along a row and the load per thread is even whatever the mix of active
+//            and silent rows.  Additions are hardware fp32/fp64 atomics in L2.
+//
+//   gather   (no transpose):  y[r] = sum_j w(j) * x(indices[j])
+//            Persistent workgroups stream the rows; G lanes cooperate on one row (G = 64, 32,
+//            16 or 8, picked on the device from the mean row length, which the host does not
+//            know).  For event vectors the workgroup first packs the events into an LDS bitmap,
+//            so the per-nonzero test is an LDS bit probe instead of a random global byte load,
+//            and `data` is only fetched where the probe hits.  Per-lane partial sums are kept
+//            in fp64 and rounded once, like the reference CPU path's `r = 0.` accumulator
+//            (brainpylib/_src/event_ops/event_csr_matvec.py:342-347,
+//             brainpylib/_src/sparse_ops/sparse_csr_matvec.py:116-119).
+//
+// Reference boundary: lib/gpu_event_csr_matvec.cu:148-260, lib/gpu_csr_matvec.cu:84-135,195-246,
+// 505-621 (buffer order, descriptor, target names).
+#include "common.h"
+#include "targets.h"
+
+namespace bpl {
+namespace {
+
+constexpr int kScatterRows = 64;     // rows owned by one scatter workgroup
+constexpr int kScatterThreads = 256;
+
+enum : int { kEvent = 0, kDense = 1 };
+
+// ------------------------------------------------------------------------------------------------
+// scatter
+// ------------------------------------------------------------------------------------------------
+template <typename F, typename VT, bool HETER, int MODE>
+__global__ __launch_bounds__(kScatterThreads) void csr_scatter_kernel(
+    const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
+    const VT *__restrict__ x, F *__restrict__ y, uint32_t n_row) {
+  __shared__ uint32_t s_start[kScatterRows];  // first nonzero of the k-th active row
+  __shared__ uint32_t s_off[kScatterRows];    // position of that row in the flat range
+  __shared__ F s_scale[kScatterRows];         // dense mode: x[r]
+  __shared__ uint32_t s_count, s_total;
+
+  const uint32_t tid = threadIdx.x;
+  if (tid < kWave) {
+    const uint32_t r = blockIdx.x * kScatterRows + tid;
+    bool on = false;
+    uint32_t start = 0, len = 0;
+    F scale = F(1);
+    if (r < n_row) {
+      if (MODE == kEvent) {
+        on = is_event(x[r]);
+      } else {
+        scale = static_cast<F>(x[r]);
+        on = true;
+      }
+      if (on) {
+        start = indptr[r];
+        len = indptr[r + 1] - start;
+        on = len != 0;
+      }
+    }
+    if (!on) len = 0;
+    const uint64_t mask = __ballot(on);
+    const uint32_t incl = wave_inclusive_scan_u32(len);
+    const int pos = __popcll(mask & ((1ull << tid) - 1ull));
+    if (on) {
+      s_start[pos] = start;
+      s_off[pos] = incl - len;
+      if (MODE == kDense) s_scale[pos] = scale;
+    }
+    if (tid == kWave - 1) {
+      s_count = static_cast<uint32_t>(__popcll(mask));
+      s_total = incl;
+    }
+  }
+  __syncthreads();
+  const uint32_t count = s_count;
+  const uint32_t total = s_total;
+  if (count == 0) return;
+
+  const F w_homo = HETER ? F(0) : data[0];
+
+  constexpr int U = 4;
+  for (uint32_t e0 = tid; e0 < total; e0 += U * kScatterThreads) {
+    uint32_t j[U];
+    uint32_t col[U];
+    F w[U];
+    bool ok[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t e = e0 + u * kScatterThreads;
+      ok[u] = e < total;
+      // largest k < count with s_off[k] <= e
+      uint32_t k = 0;
+#pragma unroll
+      for (uint32_t step = kScatterRows / 2; step > 0; step >>= 1) {
+        const uint32_t mid = k + step;
+        if (mid < count && s_off[mid] <= e) k = mid;
+      }
+      j[u] = s_start[k] + (e - s_off[k]);
+      w[u] = (MODE == kDense) ? s_scale[k] : F(1);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (ok[u]) {
+        col[u] = indices[j[u]];
+        const F d = HETER ? data[j[u]] : w_homo;
+        // dense: v * values[j] (heter) or values * v (homo), as the reference CPU loop multiplies
+        w[u] = (MODE == kDense) ? static_cast<F>(w[u] * d) : d;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (ok[u]) atomic_add(&y[col[u]], w[u]);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// gather
+// ------------------------------------------------------------------------------------------------
+
+// Bits [0,32) = events[base + b] != 0, zero beyond n.
+template <typename VT>
+__device__ __forceinline__ uint32_t pack_events32(const VT *__restrict__ ev, uint32_t base, uint32_t n) {
+  uint32_t m = 0;
+#pragma unroll 8
+  for (uint32_t b = 0; b < 32; ++b) {
+    const uint32_t i = base + b;
+    if (i < n && is_event(ev[i])) m |= 1u << b;
+  }
+  return m;
+}
+
+// 4 nonzero-byte flags of a dword, gathered into the low nibble.
+__device__ __forceinline__ uint32_t nonzero_bytes_nibble(uint32_t v) {
+  const uint32_t nz = (((v & 0x7f7f7f7fu) + 0x7f7f7f7fu) | v) & 0x80808080u;
+  // bit 7,15,23,31 -> bits 24..27 of the product (the partial products never collide)
+  return (((nz >> 7) * 0x01020408u) >> 24) & 0xfu;
+}
+
+template <>
+__device__ __forceinline__ uint32_t pack_events32<uint8_t>(const uint8_t *__restrict__ ev, uint32_t base,
+                                                            uint32_t n) {
+  const uint8_t *p = ev + base;
+  if (base + 32 <= n && (reinterpret_cast<uintptr_t>(p) & 15u) == 0) {
+    const uint4 a = *reinterpret_cast<const uint4 *>(p);
+    const uint4 b = *reinterpret_cast<const uint4 *>(p + 16);
+    return nonzero_bytes_nibble(a.x) | (nonzero_bytes_nibble(a.y) << 4) | (nonzero_bytes_nibble(a.z) << 8) |
+           (nonzero_bytes_nibble(a.w) << 12) | (nonzero_bytes_nibble(b.x) << 16) |
+           (nonzero_bytes_nibble(b.y) << 20) | (nonzero_bytes_nibble(b.z) << 24) |
+           (nonzero_bytes_nibble(b.w) << 28);
+  }
+  uint32_t m = 0;
+  for (uint32_t b = 0; b < 32; ++b) {
+    const uint32_t i = base + b;
+    if (i < n && ev[i] != 0) m |= 1u << b;
+  }
+  return m;
+}
+
+template <typename F, typename VT, bool HETER, int MODE, bool LDS_BITS, int G>
+__device__ __forceinline__ void gather_rows(const F *__restrict__ data, const uint32_t *__restrict__ indices,
+                                            const uint32_t *__restrict__ indptr, const VT *__restrict__ x,
+                                            F *__restrict__ y, uint32_t n_row, const uint32_t *s_bits) {
+  const uint32_t groups_per_block = blockDim.x / G;
+  const uint32_t gl = threadIdx.x % G;
+  const uint32_t total_groups = gridDim.x * groups_per_block;
+  const F w_homo = HETER ? F(0) : data[0];
+  constexpr int U = 4;
+
+  for (uint32_t row = blockIdx.x * groups_per_block + threadIdx.x / G; row < n_row; row += total_groups) {
+    const uint32_t start = indptr[row];
+    const uint32_t end = indptr[row + 1];
+    double acc = 0.0;    // heter / dense
+    uint32_t hits = 0;   // homo event: number of active synapses
+    for (uint32_t j0 = start + gl; j0 < end; j0 += U * G) {
+      uint32_t col[U];
+      bool ok[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t j = j0 + u * G;
+        ok[u] = j < end;
+        col[u] = ok[u] ? indices[j] : 0u;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t j = j0 + u * G;
+        if (MODE == kEvent) {
+          bool hit = false;
+          if (ok[u]) {
+            if (LDS_BITS) hit = (s_bits[col[u] >> 5] >> (col[u] & 31u)) & 1u;
+            else hit = is_event(x[col[u]]);
+          }
+          if (HETER) {
+            if (hit) acc += static_cast<double>(data[j]);
+          } else {
+            hits += hit ? 1u : 0u;
+          }
+        } else {
+          if (ok[u]) {
+            const F d = HETER ? data[j] : w_homo;
+            // product formed in F, then widened (the reference multiplies two F values)
+            acc += static_cast<double>(static_cast<F>(static_cast<F>(x[col[u]]) * d));
+          }
+        }
+      }
+    }
+    if (MODE == kEvent && !HETER) {
+      hits = group_sum<G>(hits);
+      // n additions of the same fp32 value into a float64 accumulator are exact: n * w
+      if (gl == 0) y[row] = static_cast<F>(static_cast<double>(w_homo) * static_cast<double>(hits));
+    } else {
+      acc = group_sum<G>(acc);
+      if (gl == 0) y[row] = static_cast<F>(acc);
+    }
+  }
+}
+
+template <typename F, typename VT, bool HETER, int MODE, bool LDS_BITS>
+__global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ data,
+                                                          const uint32_t *__restrict__ indices,
+                                                          const uint32_t *__restrict__ indptr,
+                                                          const VT *__restrict__ x, F *__restrict__ y,
+                                                          uint32_t n_row, uint32_t n_col) {
+  extern __shared__ uint32_t s_bits[];
+  if (LDS_BITS) {
+    const uint32_t words = (n_col + 31u) >> 5;
+    for (uint32_t w = threadIdx.x; w < words; w += blockDim.x) s_bits[w] = pack_events32<VT>(x, w << 5, n_col);
+    __syncthreads();
+  }
+  if (n_row == 0) return;
+  // lanes per row from the mean row length (indptr[n_row] = nnz)
+  const uint32_t mean = indptr[n_row] / n_row;
+  if (mean >= 48) gather_rows<F, VT, HETER, MODE, LDS_BITS, 64>(data, indices, indptr, x, y, n_row, s_bits);
+  else if (mean >= 24) gather_rows<F, VT, HETER, MODE, LDS_BITS, 32>(data, indices, indptr, x, y, n_row, s_bits);
+  else if (mean >= 12) gather_rows<F, VT, HETER, MODE, LDS_BITS, 16>(data, indices, indptr, x, y, n_row, s_bits);
+  else gather_rows<F, VT, HETER, MODE, LDS_BITS, 8>(data, indices, indptr, x, y, n_row, s_bits);
+}
+
+// ------------------------------------------------------------------------------------------------
+// launchers
+// ------------------------------------------------------------------------------------------------
+template <typename F, typename VT, bool HETER, int MODE>
+void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, const uint32_t *indptr,
+                    const VT *x, F *y, uint32_t n_row, uint32_t n_col) {
+  fill_zero(stream, y, n_col);
+  if (n_row == 0) return;
+  hipLaunchKernelGGL((csr_scatter_kernel<F, VT, HETER, MODE>), dim3(div_up(n_row, kScatterRows)),
+                     dim3(kScatterThreads), 0, stream, data, indices, indptr, x, y, n_row);
+}
+
+template <typename F, typename VT, bool HETER, int MODE, bool LDS_BITS>
+bool launch_gather_impl(const char *target, hipStream_t stream, const F *data, const uint32_t *indices,
+                        const uint32_t *indptr, const VT *x, F *y, uint32_t n_row, uint32_t n_col,
+                        size_t lds_bytes) {
+  auto kernel = csr_gather_kernel<F, VT, HETER, MODE, LDS_BITS>;
+  // Small problems: 256-thread workgroups, one wave per row at most.  Large ones: 1024-thread
+  // persistent workgroups so that few copies of the event bitmap are built.
+  const int block = (n_row >= 16384) ? 1024 : 256;
+  // The occupancy query is the same for every call with the same LDS size: remember the last one.
+  struct Cached {
+    size_t lds_bytes;
+    int block;
+    int per_cu;
+  };
+  static thread_local Cached cached = {~size_t(0), 0, 0};
+  if (cached.lds_bytes != lds_bytes || cached.block != block) {
+    if (lds_bytes > 64 * 1024) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(lds_bytes)) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+      }
+    }
+    int q = 1;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&q, reinterpret_cast<const void *>(kernel), block,
+                                                     lds_bytes) != hipSuccess || q < 1) {
+      (void)hipGetLastError();
+      q = 1;
+    }
+    cached = {lds_bytes, block, q};
+  }
+  const int per_cu = cached.per_cu;
+  const unsigned resident = static_cast<unsigned>(device_info().num_cu) * static_cast<unsigned>(per_cu);
+  const unsigned needed = div_up(n_row, block / kWave);  // one wave per row
+  const unsigned grid = needed < resident ? (needed ? needed : 1u) : resident;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), lds_bytes, stream, data, indices, indptr, x, y, n_row,
+                     n_col);
+  return check_launch(target);
+}
+
+template <typename F, typename VT, bool HETER, int MODE>
+void launch_gather(const char *target, hipStream_t stream, const F *data, const uint32_t *indices,
+                   const uint32_t *indptr, const VT *x, F *y, uint32_t n_row, uint32_t n_col) {
+  if (n_row == 0) return;
+  if (MODE == kEvent) {
+    const size_t lds_bytes = (static_cast<size_t>(n_col) + 31) / 32 * 4;
+    const size_t lds_cap = static_cast<size_t>(160) * 1024 - 1024;
+    if (lds_bytes <= lds_cap) {
+      if (launch_gather_impl<F, VT, HETER, MODE, true>(target, stream, data, indices, indptr, x, y, n_row, n_col,
+                                                       lds_bytes))
+        return;
+      bpl_clear_error();
+    }
+  }
+  launch_gather_impl<F, VT, HETER, MODE, false>(target, stream, data, indices, indptr, x, y, n_row, n_col, 0);
+}
+
+// event_csr_matvec: buffers = [data, indices, indptr, events, out]
+template <typename F, typename VT, bool HETER>
+void event_csr_matvec_entry(const char *target, hipStream_t stream, void **buffers, const char *opaque,
+                            size_t opaque_len) {
+  bpl_twouint_onebool_descriptor d;
+  if (!unpack(target, opaque, opaque_len, &d)) return;
+  if (buffers == nullptr) {
+    set_error("%s: null buffer table", target);
+    return;
+  }
+  const F *data = static_cast<const F *>(buffers[0]);
+  const uint32_t *indices = static_cast<const uint32_t *>(buffers[1]);
+  const uint32_t *indptr = static_cast<const uint32_t *>(buffers[2]);
+  const VT *events = static_cast<const VT *>(buffers[3]);
+  F *out = static_cast<F *>(buffers[4]);
+  if (d.transpose) {
+    launch_scatter<F, VT, HETER, kEvent>(stream, data, indices, indptr, events, out, d.n_row, d.n_col);
+    check_launch(target);
+  } else {
+    launch_gather<F, VT, HETER, kEvent>(target, stream, data, indices, indptr, events, out, d.n_row, d.n_col);
+  }
+}
+
+// csr_matvec: buffers = [data, indices, indptr, (row_blocks,) vector, out]
+template <typename F, bool HETER, bool TRANSPOSE>
+void csr_matvec_entry(const char *target, hipStream_t stream, void **buffers, const char *opaque,
+                      size_t opaque_len, int vector_slot) {
+  bpl_double_size_descriptor d;
+  if (!unpack(target, opaque, opaque_len, &d)) return;
+  if (buffers == nullptr) {
+    set_error("%s: null buffer table", target);
+    return;
+  }
+  const F *data = static_cast<const F *>(buffers[0]);
+  const uint32_t *indices = static_cast<const uint32_t *>(buffers[1]);
+  const uint32_t *indptr = static_cast<const uint32_t *>(buffers[2]);
+  const F *vec = static_cast<const F *>(buffers[vector_slot]);
+  F *out = static_cast<F *>(buffers[vector_slot + 1]);
+  if (TRANSPOSE) {
+    launch_scatter<F, F, HETER, kDense>(stream, data, indices, indptr, vec, out, d.n_row, d.n_col);
+    check_launch(target);
+  } else {
+    launch_gather<F, F, HETER, kDense>(target, stream, data, indices, indptr, vec, out, d.n_row, d.n_col);
+  }
+}
+
+}  // namespace
+}  // namespace bpl
+
+using bpl::csr_matvec_entry;
+using bpl::event_csr_matvec_entry;
+
+#define BPL_DEFINE(name, call)                                                                   \
+  extern "C" void name(bpl_stream_t stream, void **buffers, const char *opaque, size_t opaque_len) { \
+    hipStream_t s = static_cast<hipStream_t>(stream);                                            \
+    call;                                                                                        \
+  }
+
+// bool events are read as bytes: any nonzero byte is an event
+BPL_DEFINE(event_csr_matvec_heter_float_bool, (event_csr_matvec_entry<float, uint8_t, true>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_heter_float_float, (event_csr_matvec_entry<float, float, true>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_heter_double_bool, (event_csr_matvec_entry<double, uint8_t, true>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_heter_double_double, (event_csr_matvec_entry<double, double, true>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_homo_float_bool, (event_csr_matvec_entry<float, uint8_t, false>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_homo_float_float, (event_csr_matvec_entry<float, float, false>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_homo_double_bool, (event_csr_matvec_entry<double, uint8_t, false>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_homo_double_double, (event_csr_matvec_entry<double, double, false>(__func__, s, buffers, opaque, opaque_len)))
+
+BPL_DEFINE(csr_matvec_heter_scalar_float, (csr_matvec_entry<float, true, false>(__func__, s, buffers, opaque, opaque_len, 3)))
+BPL_DEFINE(csr_matvec_heter_scalar_double, (csr_matvec_entry<double, true, false>(__func__, s, buffers, opaque, opaque_len, 3)))
+BPL_DEFINE(csr_matvec_heter_vector_float, (csr_matvec_entry<float, true, false>(__func__, s, buffers, opaque, opaque_len, 3)))
+BPL_DEFINE(csr_matvec_heter_vector_double, (csr_matvec_entry<double, true, false>(__func__, s, buffers, opaque, opaque_len, 3)))
+BPL_DEFINE(csr_matvec_heter_adaptive_float, (csr_matvec_entry<float, true, false>(__func__, s, buffers, opaque, opaque_len, 4)))
+BPL_DEFINE(csr_matvec_heter_adaptive_double, (csr_matvec_entry<double, true, false>(__func__, s, buffers, opaque, opaque_len, 4)))
+BPL_DEFINE(csr_matvec_homo_scalar_float, (csr_matvec_entry<float, false, false>(__func__, s, buffers, opaque, opaque_len, 3)))
+BPL_DEFINE(csr_matvec_homo_scalar_double, (csr_matvec_entry<double, false, false>(__func__, s, buffers, opaque, opaque_len, 3)))
+BPL_DEFINE(csr_matvec_homo_vector_float, (csr_matvec_entry<float, false, false>(__func__, s, buffers, opaque, opaque_len, 3)))
+BPL_DEFINE(csr_matvec_homo_vector_double, (csr_matvec_entry<double, false, false>(__func__, s, buffers, opaque, opaque_len, 3)))
+BPL_DEFINE(csr_matvec_homo_adaptive_float, (csr_matvec_entry<float, false, false>(__func__, s, buffers, opaque, opaque_len, 4)))
+BPL_DEFINE(csr_matvec_homo_adaptive_double, (csr_matvec_entry<double, false, false>(__func__, s, buffers, opaque, opaque_len, 4)))
+
+BPL_DEFINE(csr_matvec_transpose_heter_float, (csr_matvec_entry<float, true, true>(__func__, s, buffers, opaque, opaque_len, 3)))
+BPL_DEFINE(csr_matvec_transpose_heter_double, (csr_matvec_entry<double, true, true>(__func__, s, buffers, opaque, opaque_len, 3)))
+BPL_DEFINE(csr_matvec_transpose_homo_float, (csr_matvec_entry<float, false, true>(__func__, s, buffers, opaque, opaque_len, 3)))
+BPL_DEFINE(csr_matvec_transpose_homo_double, (csr_matvec_entry<double, false, true>(__func__, s, buffers, opaque, opaque_len, 3)))

@@ -1,0 +1,35 @@
+// X-macro list of every custom-call target exported by libbrainpylib_amd.so.  It must name
+// exactly the BPL_TARGET declarations of include/brainpylib_amd.h (a CPU test compares them).
+#pragma once
+
+#define BPL_EVENT_CSR_TARGETS(X)            \
+  X(event_csr_matvec_heter_float_bool)      \
+  X(event_csr_matvec_heter_float_float)     \
+  X(event_csr_matvec_heter_double_bool)     \
+  X(event_csr_matvec_heter_double_double)   \
+  X(event_csr_matvec_homo_float_bool)       \
+  X(event_csr_matvec_homo_float_float)      \
+  X(event_csr_matvec_homo_double_bool)      \
+  X(event_csr_matvec_homo_double_double)
+
+#define BPL_CSR_TARGETS(X)                  \
+  X(csr_matvec_heter_scalar_float)          \
+  X(csr_matvec_heter_scalar_double)         \
+  X(csr_matvec_heter_vector_float)          \
+  X(csr_matvec_heter_vector_double)         \
+  X(csr_matvec_heter_adaptive_float)        \
+  X(csr_matvec_heter_adaptive_double)       \
+  X(csr_matvec_homo_scalar_float)           \
+  X(csr_matvec_homo_scalar_double)          \
+  X(csr_matvec_homo_vector_float)           \
+  X(csr_matvec_homo_vector_double)          \
+  X(csr_matvec_homo_adaptive_float)         \
+  X(csr_matvec_homo_adaptive_double)        \
+  X(csr_matvec_transpose_heter_float)       \
+  X(csr_matvec_transpose_heter_double)      \
+  X(csr_matvec_transpose_homo_float)        \
+  X(csr_matvec_transpose_homo_double)
+
+#define BPL_ALL_TARGETS(X)  \
+  BPL_EVENT_CSR_TARGETS(X)  \
+  BPL_CSR_TARGETS(X)

@@ -1,0 +1,83 @@
+"""Event-driven CSR operators (host side).
+
+Mirrors brainpylib/event_ops.py: ``event_csr_matvec`` with the reference's signature, argument
+checks and error conditions (brainpylib/_src/event_ops/event_csr_matvec.py:32-102), lowered to the
+custom-call target the reference's GPU translation names (same file, :389-417).
+"""
+from typing import Tuple
+
+import torch
+
+from . import _lib
+from ._tensors import FLOAT_DTYPES, as_tensor, device_of, is_index_dtype, to_device
+
+__all__ = ["event_csr_matvec"]
+
+
+def _type_name(dt):
+  return "_float" if dt == torch.float32 else "_double"
+
+
+def event_csr_matvec(data, indices, indptr, events, *, shape: Tuple[int, int], transpose: bool = False):
+  """Product of a CSR matrix (or its transpose) and an event vector.
+
+  data     scalar / shape (1,) (homogeneous weight) or shape (nse,)
+  indices  (nse,) int32 | uint32;  indptr  (shape[0] + 1,) int32 | uint32
+  events   (shape[0] if transpose else shape[1],) bool, or the float dtype of ``data``
+  returns  (shape[1] if transpose else shape[0],) tensor of ``data``'s dtype on the GPU.
+  """
+  data = as_tensor(data)
+  indices = as_tensor(indices)
+  indptr = as_tensor(indptr)
+  events = as_tensor(events)
+  # checking (conditions and messages of the reference wrapper)
+  if data.ndim == 0:
+    data = data.reshape(1)
+  if data.ndim == 1:
+    if data.shape[0] not in [1, indices.shape[0]]:
+      raise ValueError('The size of data should be 1 or be consistent with indices.'
+                       f'But we got {tuple(data.shape)} != {tuple(indices.shape)}, {tuple(data.shape)} != 1.')
+  else:
+    raise ValueError('data should be a scalar or 1D vector. '
+                     f'But we got {data.ndim}-D array.')
+  if indices.ndim != 1:
+    raise ValueError('indices should be a 1D vector with integer type.')
+  if indptr.ndim != 1:
+    raise ValueError('indptr should be a 1D vector with integer type.')
+  if not is_index_dtype(indices.dtype):
+    raise ValueError('indices should be a 1D vector with int32 or uint32 type.')
+  if not is_index_dtype(indptr.dtype):
+    raise ValueError('indptr should be a 1D vector with int32 or uint32 type.')
+  if events.ndim != 1:
+    raise ValueError('events should be a 1D vector.')
+  if len(shape) != 2:
+    raise ValueError('shape should be a length-2 tuple.')
+  if transpose:
+    if events.shape[0] != shape[0]:
+      raise ValueError(f'Shape mismatch, vec ({events.shape[0]},) @ mat {shape}.')
+  else:
+    if events.shape[0] != shape[1]:
+      raise ValueError(f'Shape mismatch, mat {shape} @ vec ({events.shape[0]},).')
+  # what the kernels additionally rely on
+  if data.dtype not in FLOAT_DTYPES:
+    raise TypeError(f'Only support float32 and float64. But we got {data.dtype}.')
+  if indptr.shape[0] != shape[0] + 1:
+    raise ValueError(f'indptr should have shape[0] + 1 = {shape[0] + 1} entries, got {indptr.shape[0]}.')
+
+  # target name, as the reference's GPU translation builds it
+  type_name = _type_name(data.dtype)
+  data_name = '_homo' if data.shape[0] == 1 else '_heter'
+  if events.dtype == torch.bool:
+    vec_type = '_bool'
+  else:
+    if events.dtype != data.dtype:
+      raise ValueError('events should be bool or have the dtype of data, '
+                       f'but we got {events.dtype} != {data.dtype}.')
+    vec_type = type_name
+  device = device_of(data, indices, indptr, events)
+  data, indices, indptr, events = (to_device(t, device) for t in (data, indices, indptr, events))
+  opaque = _lib.build_twouint_onebool_descriptor(shape[0], shape[1], transpose)
+  out = torch.empty(shape[1] if transpose else shape[0], dtype=data.dtype, device=device)
+  _lib.custom_call('event_csr_matvec' + data_name + type_name + vec_type,
+                   [data, indices, indptr, events, out], opaque)
+  return out

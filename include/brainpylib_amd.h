@@ -1,0 +1,198 @@
+/*
+ * brainpylib_amd -- C ABI of the MI355X (gfx950) event-driven sparse operator library.
+ *
+ * Everything a host needs to drive the operators is declared here as plain `extern "C"`
+ * symbols of libbrainpylib_amd.so: no C++ or framework types cross this boundary.
+ *
+ * The operator entry points are XLA GPU custom-call targets with the original 4-argument
+ * ABI, and carry the same target NAMES the reference registers (the keys of its
+ * `Registrations()` table, lib/gpu_ops.cc:24-177), so a host that looks targets up by name
+ * finds them unchanged:
+ *
+ *     void target(hipStream_t stream, void **buffers, const char *opaque, size_t opaque_len);
+ *
+ *   stream      the HIP stream the call is enqueued on; the call returns without waiting.
+ *   buffers     device pointers: all operands in the operator's order, then all results.
+ *               Results may be uninitialised on entry; every element is written.
+ *   opaque      byte image of one of the descriptor structs below (host memory, read before
+ *               the call returns); opaque_len must equal sizeof(that struct).
+ *
+ * Errors never unwind through this boundary.  A call that fails validation or whose launch
+ * fails enqueues nothing more, records a message retrievable with bpl_last_error() on the
+ * calling thread and prints it to stderr.
+ */
+#ifndef BRAINPYLIB_AMD_H_
+#define BRAINPYLIB_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* An opaque HIP stream handle (hipStream_t); declared as void* so that hosts without the HIP
+ * headers can include this file. */
+typedef void *bpl_stream_t;
+
+typedef void (*bpl_target_fn)(bpl_stream_t stream, void **buffers, const char *opaque,
+                              size_t opaque_len);
+
+#define BPL_TARGET(name) \
+  void name(bpl_stream_t stream, void **buffers, const char *opaque, size_t opaque_len)
+
+/* ------------------------------------------------------------------------------------------
+ * Descriptors (the `opaque` payloads).  Field order, types and padding are those of the
+ * reference's structs, lib/kernel_helper_descriptor.cuh:42-144.
+ * ---------------------------------------------------------------------------------------- */
+
+/* lib/kernel_helper_descriptor.cuh:138-142 (TwoUintOneBoolDescriptor): event_csr_matvec. */
+typedef struct {
+  uint32_t n_row;    /* CSR shape[0] */
+  uint32_t n_col;    /* CSR shape[1] */
+  uint8_t transpose; /* C++ bool; 3 bytes of padding follow */
+} bpl_twouint_onebool_descriptor;
+
+/* lib/kernel_helper_descriptor.cuh:120-123 (DoubleSizeDescriptor): csr_matvec. */
+typedef struct {
+  uint32_t n_row;
+  uint32_t n_col;
+} bpl_double_size_descriptor;
+
+/* lib/kernel_helper_descriptor.cuh:42-45 (NonZeroDescriptor): event_info. */
+typedef struct {
+  uint32_t event_size;
+  uint32_t batch_size;
+} bpl_nonzero_descriptor;
+
+/* lib/kernel_helper_descriptor.cuh:49-54 (JITConnProbHomoDescriptor).
+ * n_row = number of outputs, n_col = number of inputs (already swapped for transpose=True);
+ * log_p = log(1 - conn_prob), or log(1e-40) when conn_prob >= 1. */
+typedef struct {
+  uint32_t n_row;
+  uint32_t n_col;
+  uint32_t seed;
+  double log_p;
+} bpl_jitconn_prob_homo_descriptor;
+
+/* lib/kernel_helper_descriptor.cuh:62-69 and :98-105 (JITConnProbUniformDescriptor /
+ * JITConnProbNormalDescriptor; same layout).  uniform: w_a = w_low, w_b = w_high (the
+ * boundaries the CPU path receives, lib/cpu_jitconn_event_matvec.cpp:40-41).
+ * normal: w_a = w_mu, w_b = w_sigma. */
+typedef struct {
+  uint32_t n_row;
+  uint32_t n_col;
+  uint32_t seed;
+  double log_p;
+  double w_a;
+  double w_b;
+} bpl_jitconn_prob_weight_descriptor;
+
+/* lib/kernel_helper_descriptor.cuh:80-88 (MatMatJITProbDescriptor1): Y[m,n] = X[m,k] @ M[k,n]. */
+typedef struct {
+  uint32_t m;
+  uint32_t k;
+  uint32_t n;
+  uint32_t seed;
+  double log_p;
+  double w_a;
+  double w_b;
+} bpl_matmat_jit_prob_descriptor;
+
+/* Builders: write the descriptor's byte image into `out` (capacity `cap`) and return its size,
+ * or 0 if `cap` is too small.  They replace build_*_descriptor of
+ * lib/kernel_helper_descriptor.cu:34-104.  Unlike the reference's builders, which narrow
+ * log_p and the weight parameters to float before widening them again, these keep the
+ * doubles, so the kernels see the same log_p as the reference's CPU path. */
+size_t bpl_build_twouint_onebool_descriptor(uint32_t n_row, uint32_t n_col, int transpose,
+                                            char *out, size_t cap);
+size_t bpl_build_double_size_descriptor(uint32_t n_row, uint32_t n_col, char *out, size_t cap);
+size_t bpl_build_nonzero_descriptor(uint32_t event_size, uint32_t batch_size, char *out,
+                                    size_t cap);
+size_t bpl_build_jitconn_prob_homo_descriptor(uint32_t n_row, uint32_t n_col, uint32_t seed,
+                                              double log_p, char *out, size_t cap);
+size_t bpl_build_jitconn_prob_uniform_descriptor(uint32_t n_row, uint32_t n_col, uint32_t seed,
+                                                 double log_p, double w_low, double w_high,
+                                                 char *out, size_t cap);
+size_t bpl_build_jitconn_prob_normal_descriptor(uint32_t n_row, uint32_t n_col, uint32_t seed,
+                                                double log_p, double w_mu, double w_sigma,
+                                                char *out, size_t cap);
+size_t bpl_build_matmat_jit_prob_descriptor1(uint32_t m, uint32_t k, uint32_t n, uint32_t seed,
+                                             double log_p, double w_a, double w_b, char *out,
+                                             size_t cap);
+
+/* ------------------------------------------------------------------------------------------
+ * Registry: replaces Registrations() of lib/gpu_ops.cc:24-177.  Index i runs over
+ * [0, bpl_num_targets()).
+ * ---------------------------------------------------------------------------------------- */
+int bpl_num_targets(void);
+const char *bpl_target_name(int i);
+bpl_target_fn bpl_target_function(int i);
+bpl_target_fn bpl_find_target(const char *name); /* NULL if unknown */
+
+/* Last error recorded on the calling thread ("" if none), and a reset. */
+const char *bpl_last_error(void);
+void bpl_clear_error(void);
+
+/* Library version string. */
+const char *bpl_version(void);
+
+/* ------------------------------------------------------------------------------------------
+ * event_csr_matvec  (lib/gpu_event_csr_matvec.cu:222-260; launchers :148-217)
+ *   buffers = [data, indices, indptr, events, out]
+ *     data     F[1] (homo) or F[nnz] (heter)
+ *     indices  uint32/int32[nnz]        indptr  uint32/int32[n_row + 1]
+ *     events   bool[.] (1 byte each) or F[.] (truthiness test); length n_row if transpose
+ *              else n_col
+ *     out      F[n_col] if transpose else F[n_row]
+ *   opaque  = bpl_twouint_onebool_descriptor
+ *   transpose:      out[indices[j]] += data[j]   for every j in row r, for every r with events[r]
+ *   not transpose:  out[r] = sum of data[j] over j in row r with events[indices[j]]
+ * ---------------------------------------------------------------------------------------- */
+BPL_TARGET(event_csr_matvec_heter_float_bool);
+BPL_TARGET(event_csr_matvec_heter_float_float);
+BPL_TARGET(event_csr_matvec_heter_double_bool);
+BPL_TARGET(event_csr_matvec_heter_double_double);
+BPL_TARGET(event_csr_matvec_homo_float_bool);
+BPL_TARGET(event_csr_matvec_homo_float_float);
+BPL_TARGET(event_csr_matvec_homo_double_bool);
+BPL_TARGET(event_csr_matvec_homo_double_double);
+
+/* ------------------------------------------------------------------------------------------
+ * csr_matvec  (lib/gpu_csr_matvec.cu:563-621; launchers :84-135,:195-246,:505-560)
+ *   scalar / vector: buffers = [data, indices, indptr, vector, out]
+ *   adaptive:        buffers = [data, indices, indptr, row_blocks, vector, out]
+ *                    (row_blocks is accepted for layout compatibility and not read)
+ *   opaque = bpl_double_size_descriptor;  out[r] = sum_j data[j] * vector[indices[j]], F[n_row].
+ *   The three method names select the same kernel family here: the lanes-per-row mode is
+ *   picked on the device from the mean row length.
+ * ---------------------------------------------------------------------------------------- */
+BPL_TARGET(csr_matvec_heter_scalar_float);
+BPL_TARGET(csr_matvec_heter_scalar_double);
+BPL_TARGET(csr_matvec_heter_vector_float);
+BPL_TARGET(csr_matvec_heter_vector_double);
+BPL_TARGET(csr_matvec_heter_adaptive_float);
+BPL_TARGET(csr_matvec_heter_adaptive_double);
+BPL_TARGET(csr_matvec_homo_scalar_float);
+BPL_TARGET(csr_matvec_homo_scalar_double);
+BPL_TARGET(csr_matvec_homo_vector_float);
+BPL_TARGET(csr_matvec_homo_vector_double);
+BPL_TARGET(csr_matvec_homo_adaptive_float);
+BPL_TARGET(csr_matvec_homo_adaptive_double);
+
+/* Transposed csr_matvec: out[indices[j]] += vector[r] * data[j], out F[n_col].
+ * The reference has no GPU kernel of its own for this orientation (it forwards to cuSPARSE,
+ * brainpylib/_src/sparse_ops/cusparse_matvec.py:262-283); semantics follow its CPU loop
+ * brainpylib/_src/sparse_ops/cusparse_matvec.py:195-212.
+ *   buffers = [data, indices, indptr, vector(F[n_row]), out(F[n_col])],
+ *   opaque = bpl_double_size_descriptor. */
+BPL_TARGET(csr_matvec_transpose_heter_float);
+BPL_TARGET(csr_matvec_transpose_heter_double);
+BPL_TARGET(csr_matvec_transpose_homo_float);
+BPL_TARGET(csr_matvec_transpose_homo_double);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+
+#endif /* BRAINPYLIB_AMD_H_ */

@@ -1,0 +1,235 @@
+"""CPU oracle for the event-driven sparse operator path -- TEST INFRASTRUCTURE ONLY.
+
+Only ``tests/``, ``__graft_entry__.smoke()`` and the CPU-baseline leg of ``bench.py`` may import
+this package.  The shipped package ``brainpylib_amd`` never does.
+
+``liboracle.so`` is a plain-C restatement (``oracle.c``) of the reference's CPU algorithms;
+``oracle.ref`` binds the reference's own C++ CPU kernels when they were compiled into
+``_ref/libref_cpu.so`` (possible only where the reference tree is mounted).
+
+Parity status of each oracle function (what pins it, beyond retyping the formula):
+
+==============================  ==============================================================
+function                        pinned by
+==============================  ==============================================================
+mt19937_words                   ISO C++ known answer (10000th output of seed 5489 = 4123659995)
+canonical_f64 / canonical_f32   the reference's compiled C++ (libstdc++ 11.4), via the skip
+                                and weight streams below
+jitconn_matvec (sequential)     bit-exact vs the reference's compiled lib/cpu_jitconn_*.cpp on
+                                the reference tests' shapes, all 4 walks x 3 weight kinds x
+                                bool/float/double inputs; committed fixtures tests/golden/
+jitconn_matvec (per-stream)     row r == compiled reference with one stream and seed+r;
+                                closed form at conn_prob >= 1; geometric-gap statistics;
+                                adjoint identity <y, Mx> == <M^T y, x>; shape-swap identity
+jitconn_matmat                  reference test identity matmat == vmap(matvec(transpose=True));
+                                no reference CPU kernel exists for it
+event_csr_matvec                dense matmul brute force, scipy.sparse, homo == heter(ones*w),
+                                bool == float events, compiled lib/cpu_event_sum.cc (transpose,
+                                bool events)
+csr_matvec                      dense matmul brute force, scipy.sparse (both orientations)
+event_info                      numpy.flatnonzero
+==============================  ==============================================================
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+_lib = None
+
+W_HOMO, W_UNIFORM, W_NORMAL = 0, 1, 2
+_W_KINDS = {"homo": W_HOMO, "uniform": W_UNIFORM, "normal": W_NORMAL}
+
+
+def build(ref=True):
+  """Compile liboracle.so (and the reference CPU kernels when the reference tree is present)."""
+  subprocess.check_call(["make", "-s", "-C", _HERE, "-B", "liboracle.so"])
+  if ref and os.path.isdir(os.environ.get("REFERENCE", "/root/reference") + "/lib"):
+    subprocess.check_call(["make", "-s", "-C", _HERE, "ref"])
+
+
+def lib():
+  global _lib
+  if _lib is None:
+    if not os.path.exists(_LIB_PATH):
+      build(ref=False)
+    _lib = ctypes.CDLL(_LIB_PATH)
+    _lib.oracle_jitconn_stream_indices.restype = ctypes.c_uint32
+    _lib.oracle_jitconn_stream_weights_f32.restype = ctypes.c_uint32
+    _lib.oracle_jitconn_stream_weights_f64.restype = ctypes.c_uint32
+    _lib.oracle_get_threads.restype = ctypes.c_int
+  return _lib
+
+
+def _p(a):
+  return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _c(a, dtype=None):
+  a = np.ascontiguousarray(a, dtype=dtype)
+  return a
+
+
+def set_threads(n):
+  lib().oracle_set_threads(ctypes.c_int(int(n)))
+
+
+def log_p_of(conn_prob):
+  """log(1 - p), or log(1e-40) when p >= 1 (brainpylib/_src/jitconn_ops/event_matvec.py:162)."""
+  return float(np.log((1 - conn_prob) if conn_prob < 1 else 1e-40))
+
+
+# ---------------------------------------------------------------------------------------------
+# generator primitives
+# ---------------------------------------------------------------------------------------------
+def mt19937_words(seed, n, skip=0):
+  out = np.empty(n, dtype=np.uint32)
+  lib().oracle_mt19937_words(ctypes.c_uint32(seed), ctypes.c_uint32(skip), ctypes.c_uint32(n), _p(out))
+  return out
+
+
+def canonical_f64(seed, n):
+  out = np.empty(n, dtype=np.float64)
+  lib().oracle_canonical_f64(ctypes.c_uint32(seed), ctypes.c_uint32(n), _p(out))
+  return out
+
+
+def canonical_f32(seed, n):
+  out = np.empty(n, dtype=np.float32)
+  lib().oracle_canonical_f32(ctypes.c_uint32(seed), ctypes.c_uint32(n), _p(out))
+  return out
+
+
+def normal_stream(seed, mu, sigma, n, dtype=np.float32):
+  out = np.empty(n, dtype=dtype)
+  if np.dtype(dtype) == np.float32:
+    lib().oracle_normal_f32(ctypes.c_uint32(seed), ctypes.c_float(mu), ctypes.c_float(sigma),
+                            ctypes.c_uint32(n), _p(out))
+  else:
+    lib().oracle_normal_f64(ctypes.c_uint32(seed), ctypes.c_double(mu), ctypes.c_double(sigma),
+                            ctypes.c_uint32(n), _p(out))
+  return out
+
+
+def jitconn_stream_indices(seed, log_p, n, cap=None):
+  """Indices connected by the single generator stream std::mt19937{seed} over [0, n)."""
+  if cap is None:
+    cap = int(n)
+  out = np.empty(max(cap, 1), dtype=np.uint32)
+  cnt = lib().oracle_jitconn_stream_indices(ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_double(log_p),
+                                            ctypes.c_uint32(n), _p(out), ctypes.c_uint32(cap))
+  return out[:min(cnt, cap)].copy(), int(cnt)
+
+
+def jitconn_stream_weights(seed, w_kind, w_a, w_b, log_p, n, dtype=np.float32, cap=None):
+  if cap is None:
+    cap = int(n)
+  idx = np.empty(max(cap, 1), dtype=np.uint32)
+  w = np.empty(max(cap, 1), dtype=dtype)
+  f32 = np.dtype(dtype) == np.float32
+  fn = lib().oracle_jitconn_stream_weights_f32 if f32 else lib().oracle_jitconn_stream_weights_f64
+  ft = ctypes.c_float if f32 else ctypes.c_double
+  cnt = fn(ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_int(_W_KINDS[w_kind]), ft(w_a), ft(w_b),
+           ctypes.c_double(log_p), ctypes.c_uint32(n), _p(idx), _p(w), ctypes.c_uint32(cap))
+  cnt = min(cnt, cap)
+  return idx[:cnt].copy(), w[:cnt].copy()
+
+
+# ---------------------------------------------------------------------------------------------
+# jitconn operators
+# ---------------------------------------------------------------------------------------------
+def jitconn_matvec(inp, *, w_kind="homo", w_a=0.0, w_b=0.0, log_p, seed, n_row, n_col,
+                   col_walk=False, per_stream_seed=True, out_dtype=None, dense=None):
+  """Kernel-level jitconn (event) matvec: returns the custom call's result (for ``homo`` that is
+  the count / plain sum; the weight is applied by the caller as the reference does).
+
+  ``inp`` bool -> event input; float with dense=False -> float events (truthiness);
+  float with dense=True -> dense vector.  ``n_row`` outputs, ``n_col`` inputs.
+  ``per_stream_seed=False`` is the reference CPU backend's single sequential generator."""
+  inp = np.ascontiguousarray(inp)
+  assert inp.ndim == 1 and inp.shape[0] == n_col
+  if inp.dtype == np.bool_:
+    in_kind = 0
+    out_dtype = np.dtype(out_dtype or np.float32)
+    buf = inp.view(np.uint8)
+  else:
+    if dense is None:
+      raise ValueError("say whether a float input is a dense vector or float events")
+    in_kind = 2 if dense else 1
+    out_dtype = inp.dtype
+    buf = inp
+  assert out_dtype in (np.dtype(np.float32), np.dtype(np.float64))
+  out = np.empty(n_row, dtype=out_dtype)
+  f32 = out_dtype == np.float32
+  fn = lib().oracle_jitconn_matvec_f32 if f32 else lib().oracle_jitconn_matvec_f64
+  ft = ctypes.c_float if f32 else ctypes.c_double
+  fn(_p(buf), ctypes.c_int(in_kind), ctypes.c_int(_W_KINDS[w_kind]), ft(w_a), ft(w_b),
+     ctypes.c_double(log_p), ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_uint32(n_row),
+     ctypes.c_uint32(n_col), ctypes.c_int(int(col_walk)), ctypes.c_int(int(per_stream_seed)), _p(out))
+  return out
+
+
+def jitconn_matmat(X, *, w_kind="normal", w_a, w_b, log_p, seed, n):
+  """Y[m, n] = X[m, k] @ M[k, n]; column j of M is generator stream seed + j."""
+  X = np.ascontiguousarray(X)
+  m, k = X.shape
+  Y = np.empty((m, n), dtype=X.dtype)
+  f32 = X.dtype == np.float32
+  fn = lib().oracle_jitconn_matmat_f32 if f32 else lib().oracle_jitconn_matmat_f64
+  ft = ctypes.c_float if f32 else ctypes.c_double
+  fn(_p(X), ctypes.c_int(_W_KINDS[w_kind]), ft(w_a), ft(w_b), ctypes.c_double(log_p),
+     ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_uint32(m), ctypes.c_uint32(k), ctypes.c_uint32(n), _p(Y))
+  return Y
+
+
+# ---------------------------------------------------------------------------------------------
+# CSR operators
+# ---------------------------------------------------------------------------------------------
+def _csr_args(data, indices, indptr):
+  data = np.atleast_1d(np.ascontiguousarray(data))
+  assert data.dtype in (np.float32, np.float64)
+  indices = np.ascontiguousarray(indices).view(np.uint32) if indices.dtype != np.uint32 else np.ascontiguousarray(indices)
+  indptr = np.ascontiguousarray(indptr).view(np.uint32) if indptr.dtype != np.uint32 else np.ascontiguousarray(indptr)
+  return data, indices, indptr
+
+
+def event_csr_matvec(data, indices, indptr, events, *, shape, transpose=False):
+  data, indices, indptr = _csr_args(data, indices, indptr)
+  events = np.ascontiguousarray(events)
+  if events.dtype == np.bool_:
+    ev_kind, ev = 0, events.view(np.uint8)
+  else:
+    assert events.dtype == data.dtype
+    ev_kind, ev = 1, events
+  out = np.empty(shape[1] if transpose else shape[0], dtype=data.dtype)
+  fn = lib().oracle_event_csr_matvec_f32 if data.dtype == np.float32 else lib().oracle_event_csr_matvec_f64
+  fn(_p(data), ctypes.c_uint32(data.shape[0]), _p(indices), _p(indptr), _p(ev), ctypes.c_int(ev_kind),
+     ctypes.c_uint32(shape[0]), ctypes.c_uint32(shape[1]), ctypes.c_int(int(transpose)), _p(out))
+  return out
+
+
+def csr_matvec(data, indices, indptr, vector, *, shape, transpose=False):
+  data, indices, indptr = _csr_args(data, indices, indptr)
+  vector = np.ascontiguousarray(vector, dtype=data.dtype)
+  out = np.empty(shape[1] if transpose else shape[0], dtype=data.dtype)
+  fn = lib().oracle_csr_matvec_f32 if data.dtype == np.float32 else lib().oracle_csr_matvec_f64
+  fn(_p(data), ctypes.c_uint32(data.shape[0]), _p(indices), _p(indptr), _p(vector),
+     ctypes.c_uint32(shape[0]), ctypes.c_uint32(shape[1]), ctypes.c_int(int(transpose)), _p(out))
+  return out
+
+
+_EVENT_KINDS = {np.dtype(np.bool_): 0, np.dtype(np.int32): 1, np.dtype(np.int64): 2,
+                np.dtype(np.float32): 3, np.dtype(np.float64): 4}
+
+
+def event_info(events):
+  events = np.ascontiguousarray(events)
+  ids = np.empty(events.shape[0], dtype=np.int32)
+  num = np.empty(1, dtype=np.int32)
+  buf = events.view(np.uint8) if events.dtype == np.bool_ else events
+  lib().oracle_event_info(_p(buf), ctypes.c_int(_EVENT_KINDS[events.dtype]),
+                          ctypes.c_uint32(events.shape[0]), _p(ids), _p(num))
+  return ids, num

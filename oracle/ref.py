@@ -1,0 +1,91 @@
+"""ctypes binding of the reference's own CPU kernels -- TEST INFRASTRUCTURE ONLY.
+
+``_ref/libref_cpu.so`` is built by ``make -C oracle ref`` straight from the reference's C++
+sources (lib/cpu_jitconn_*.cpp, lib/cpu_event_sum.cc); it exists only where that build ran.
+The exported symbols are the reference's ``brainpy_lib::name(void** out, const void** in)``
+functions (``void* out`` for cpu_event_sum), addressed by their Itanium-mangled names; the
+operand order follows the CPU custom-call translations
+(brainpylib/_src/jitconn_ops/event_matvec.py:183-192, matvec.py:318-327,602-615).
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_PATH = os.path.join(_HERE, "_ref", "libref_cpu.so")
+_lib = None
+
+
+def available():
+  return os.path.exists(_PATH)
+
+
+def _load():
+  global _lib
+  if _lib is None:
+    _lib = ctypes.CDLL(_PATH)
+  return _lib
+
+
+def _sym(name, tuple_out=True):
+  mangled = "_ZN11brainpy_lib%d%sE%s" % (len(name), name, "PPvPPKv" if tuple_out else "PvPPKv")
+  return getattr(_load(), mangled)
+
+
+def _ptr(a):
+  return ctypes.c_void_p(a.ctypes.data)
+
+
+def _suffix(dt):
+  return "float" if np.dtype(dt) == np.float32 else "double"
+
+
+def jitconn_matvec(inp, *, w_kind="homo", w_a=0.0, w_b=0.0, log_p, seed, n_row, n_col,
+                   col_walk=False, out_dtype=None, dense=None):
+  """Run the reference CPU custom-call target for one (event) matvec; same argument meaning as
+  ``oracle.jitconn_matvec`` with the reference's single sequential generator."""
+  inp = np.ascontiguousarray(inp)
+  assert inp.shape == (n_col,)
+  if inp.dtype == np.bool_:
+    out_dtype = np.dtype(out_dtype or np.float32)
+    name = "event_matvec%s_prob_%s_%s_bool" % ("_atomic" if col_walk else "", w_kind, _suffix(out_dtype))
+  elif not dense:
+    out_dtype = inp.dtype
+    name = "event_matvec%s_prob_%s_%s_%s" % ("_atomic" if col_walk else "", w_kind,
+                                            _suffix(out_dtype), _suffix(out_dtype))
+  else:
+    out_dtype = inp.dtype
+    name = "matvec%s_prob_%s_%s" % ("_atomic" if col_walk else "", w_kind, _suffix(out_dtype))
+  out = np.empty(n_row, dtype=out_dtype)
+  logp = np.array(log_p, dtype=np.float64)
+  sd = np.array(seed & 0xFFFFFFFF, dtype=np.uint32)
+  nr = np.array(n_row, dtype=np.uint32)
+  nc = np.array(n_col, dtype=np.uint32)
+  if w_kind == "homo":
+    ins = [inp, logp, sd, nr, nc]
+  else:
+    ins = [inp, logp, np.array(w_a, dtype=out_dtype), np.array(w_b, dtype=out_dtype), sd, nr, nc]
+  in_arr = (ctypes.c_void_p * len(ins))(*[_ptr(a) for a in ins])
+  out_arr = (ctypes.c_void_p * 1)(_ptr(out))
+  _sym(name)(out_arr, in_arr)
+  return out
+
+
+def csr_event_sum(data, indices, indptr, events, *, shape):
+  """lib/cpu_event_sum.cc: out[post] += w for every synapse of every pre with events[pre]
+  (the transpose=True, bool-event case of event_csr_matvec)."""
+  data = np.atleast_1d(np.ascontiguousarray(data))
+  events = np.ascontiguousarray(events)
+  assert events.dtype == np.bool_
+  indices = np.ascontiguousarray(indices).view(np.uint32)
+  indptr = np.ascontiguousarray(indptr).view(np.uint32)
+  kind = "homo" if data.shape[0] == 1 else "heter"
+  f = "f32" if data.dtype == np.float32 else "f64"
+  out = np.empty(shape[1], dtype=data.dtype)
+  pre = np.array(shape[0], dtype=np.uint32)
+  post = np.array(shape[1], dtype=np.uint32)
+  ins = [pre, post, events, indices, indptr, data]
+  in_arr = (ctypes.c_void_p * len(ins))(*[_ptr(a) for a in ins])
+  _sym("cpu_csr_event_sum_%s_%s_i32" % (kind, f), tuple_out=False)(_ptr(out), in_arr)
+  return out

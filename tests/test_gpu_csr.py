@@ -1,0 +1,248 @@
+"""GPU parity of event_csr_matvec / csr_matvec against the CPU oracle, through the C ABI
+(the host wrappers call the custom-call targets of libbrainpylib_amd.so).
+
+Bit-exact where the arithmetic allows it (homogeneous weights, integer-valued weights);
+otherwise within the stated tolerance rel 1e-5 / abs 1e-6 (atomics reorder additions)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import brainpylib_amd as bpl
+from brainpylib_amd import synth
+from util import CSR_SHAPES, assert_close, assert_close_reordered, random_csr
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _events(rng, n, kind, dtype, rate=0.1):
+  ev = rng.random(n) < rate
+  if kind == "bool":
+    return ev
+  return (ev * rng.uniform(0.5, 2.0, n)).astype(dtype)
+
+
+@pytest.mark.parametrize("shape", CSR_SHAPES)
+@pytest.mark.parametrize("transpose", [False, True])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("ev_kind", ["bool", "float"])
+def test_event_csr_matvec_reference_test_shapes(cuda, oracle_mod, shape, transpose, dtype, ev_kind):
+  data, indices, indptr = random_csr(shape, 0.4, seed=shape[0] * 3 + shape[1], dtype=dtype)
+  rng = np.random.default_rng(5)
+  events = _events(rng, shape[0] if transpose else shape[1], ev_kind, dtype)
+  print("case", shape, transpose, dtype.__name__, ev_kind, flush=True)
+  # heterogeneous weights
+  want = oracle_mod.event_csr_matvec(data, indices, indptr, events, shape=shape, transpose=transpose)
+  got = bpl.event_csr_matvec(data, indices, indptr, events, shape=shape, transpose=transpose).cpu().numpy()
+  assert got.dtype == dtype
+  if transpose:
+    mag = oracle_mod.event_csr_matvec(np.abs(data), indices, indptr, events, shape=shape, transpose=True)
+    assert_close_reordered(got, want, mag, dtype, what="heter scatter")
+  else:
+    assert_close(got, want, what="heter gather")
+  # homogeneous weight: every addend is the same value, so the result is order independent
+  w = np.array([0.6], dtype=dtype)
+  want = oracle_mod.event_csr_matvec(w, indices, indptr, events, shape=shape, transpose=transpose)
+  got = bpl.event_csr_matvec(w, indices, indptr, events, shape=shape, transpose=transpose).cpu().numpy()
+  if dtype == np.float32 or transpose:
+    assert np.array_equal(got, want), "homo must be bit-exact"
+  else:
+    assert_close(got, want, rtol=1e-12, atol=0, what="homo f64 gather")
+  # integer-valued weights: exact in any order
+  di = np.random.default_rng(6).integers(-1, 2, size=indices.shape[0]).astype(dtype)
+  want = oracle_mod.event_csr_matvec(di, indices, indptr, events, shape=shape, transpose=transpose)
+  got = bpl.event_csr_matvec(di, indices, indptr, events, shape=shape, transpose=transpose).cpu().numpy()
+  assert np.array_equal(got, want), "integer weights must be bit-exact"
+
+
+@pytest.mark.parametrize("shape", CSR_SHAPES)
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("method", ["scalar", "vector", "adaptive"])
+def test_csr_matvec_reference_test_shapes(cuda, oracle_mod, shape, dtype, method):
+  data, indices, indptr = random_csr(shape, 0.4, seed=shape[0] * 5 + shape[1], dtype=dtype, weights="uniform")
+  v = np.random.default_rng(7).standard_normal(shape[1]).astype(dtype)
+  print("case", shape, dtype.__name__, method, flush=True)
+  want = oracle_mod.csr_matvec(data, indices, indptr, v, shape=shape)
+  got = bpl.csr_matvec(data, indices, indptr, v, shape=shape, method=method).cpu().numpy()
+  assert_close(got, want, what="heter")
+  w = np.array([0.75], dtype=dtype)
+  want = oracle_mod.csr_matvec(w, indices, indptr, v, shape=shape)
+  got = bpl.csr_matvec(w, indices, indptr, v, shape=shape, method=method).cpu().numpy()
+  assert_close(got, want, what="homo")
+  # integer data and vector: exact
+  di = np.random.default_rng(8).integers(-2, 3, size=indices.shape[0]).astype(dtype)
+  vi = np.random.default_rng(9).integers(-2, 3, size=shape[1]).astype(dtype)
+  want = oracle_mod.csr_matvec(di, indices, indptr, vi, shape=shape)
+  got = bpl.csr_matvec(di, indices, indptr, vi, shape=shape, method=method).cpu().numpy()
+  assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("shape", CSR_SHAPES)
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_csr_matvec_transpose(cuda, oracle_mod, shape, dtype):
+  data, indices, indptr = random_csr(shape, 0.4, seed=shape[0] * 9 + shape[1], dtype=dtype, weights="uniform")
+  v = np.random.default_rng(7).standard_normal(shape[0]).astype(dtype)
+  print("case", shape, dtype.__name__, flush=True)
+  want = oracle_mod.csr_matvec(data, indices, indptr, v, shape=shape, transpose=True)
+  got = bpl.cusparse_csr_matvec(data, indices, indptr, v, shape=shape, transpose=True).cpu().numpy()
+  # sums of up to shape[0] terms of mixed sign accumulated in another order: scale the
+  # absolute tolerance by the magnitude of the sum of |terms|
+  mag = oracle_mod.csr_matvec(data, indices, indptr, np.abs(v), shape=shape, transpose=True)  # data >= 0
+  assert_close_reordered(got, want, mag, dtype, what="csr scatter")
+  w = np.array([0.5], dtype=dtype)
+  vi = np.random.default_rng(9).integers(-2, 3, size=shape[0]).astype(dtype)
+  want = oracle_mod.csr_matvec(w, indices, indptr, vi, shape=shape, transpose=True)
+  got = bpl.cusparse_csr_matvec(w, indices, indptr, vi, shape=shape, transpose=True).cpu().numpy()
+  assert np.array_equal(got, want)
+
+
+def test_event_scatter_against_reference_cpu_event_sum_golden(cuda):
+  z = np.load(os.path.join(GOLD, "event_sum_cpu_reference.npz"))
+  n = sum(1 for k in z.files if k.startswith("out_"))
+  for i in range(n):
+    shape = tuple(int(x) for x in z["shape_%d" % i])
+    got = bpl.event_csr_matvec(z["data_%d" % i], z["indices_%d" % i], z["indptr_%d" % i], z["events_%d" % i],
+                               shape=shape, transpose=True).cpu().numpy()
+    want = z["out_%d" % i]
+    if z["data_%d" % i].shape[0] == 1:
+      assert np.array_equal(got, want), i
+    else:
+      mag = np.zeros(shape[1])
+      ev, ip, ix, d = z["events_%d" % i], z["indptr_%d" % i], z["indices_%d" % i], z["data_%d" % i]
+      for r in np.flatnonzero(ev):
+        np.add.at(mag, ix[ip[r]:ip[r + 1]], np.abs(d[ip[r]:ip[r + 1]]))
+      assert_close_reordered(got, want, mag, d.dtype.type, what="golden %d" % i)
+
+
+def test_edge_cases(cuda, oracle_mod):
+  # empty rows, silent / saturated event vectors, uint32 indices, empty matrix, zero rows
+  indptr = np.array([0, 0, 3, 3, 5], dtype=np.int32)
+  indices = np.array([0, 2, 4, 1, 4], dtype=np.int32)
+  data = np.array([1, 2, 3, 4, 5], dtype=np.float32)
+  shape = (4, 5)
+  for tr in (False, True):
+    n_in = shape[0] if tr else shape[1]
+    for ev in (np.zeros(n_in, bool), np.ones(n_in, bool)):
+      want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=tr)
+      got = bpl.event_csr_matvec(data, indices.astype(np.uint32), indptr.astype(np.uint32), ev, shape=shape,
+                                 transpose=tr).cpu().numpy()
+      assert np.array_equal(got, want)
+  e_ip = np.zeros(4, dtype=np.int32)
+  e = np.zeros(0, dtype=np.int32)
+  out = bpl.csr_matvec(np.zeros(0, np.float32), e, e_ip, np.ones(7, np.float32), shape=(3, 7)).cpu().numpy()
+  assert out.shape == (3,) and not out.any()
+  out = bpl.event_csr_matvec(1.0, e, e_ip, np.ones(3, bool), shape=(3, 7), transpose=True).cpu().numpy()
+  assert out.shape == (7,) and not out.any()
+  # NaN and -0.0 float events: NaN is an event, -0.0 is not
+  ev = np.array([np.nan, -0.0, 0.0, 1e-30, 0.0], dtype=np.float32)
+  want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape)
+  got = bpl.event_csr_matvec(data, indices, indptr, ev, shape=shape).cpu().numpy()
+  assert np.array_equal(got, want)
+  # output buffer is fully overwritten (results may be uninitialised on entry)
+  t = torch.full((5,), 7.0, device=cuda)
+  del t
+
+
+def test_ragged_rows_and_all_row_length_modes(cuda, oracle_mod):
+  # mean row lengths that select each lanes-per-row mode (8 / 16 / 32 / 64), with ragged rows,
+  # empty rows and one very long row
+  rng = np.random.default_rng(11)
+  n_col = 5000
+  for mean in (3, 14, 30, 200):
+    counts = rng.poisson(mean, size=3000)
+    counts[::7] = 0
+    counts[5] = 4000
+    indices, indptr = synth.counted_csr(counts, n_col, seed=mean)
+    data = rng.standard_normal(indices.shape[0]).astype(np.float32)
+    ev = rng.random(n_col) < 0.2
+    v = rng.standard_normal(n_col).astype(np.float32)
+    shape = (counts.shape[0], n_col)
+    print("mean row length", mean, flush=True)
+    want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape)
+    got = bpl.event_csr_matvec(data, indices, indptr, ev, shape=shape).cpu().numpy()
+    assert_close(got, want, what="event gather mean %d" % mean)
+    want = oracle_mod.csr_matvec(data, indices, indptr, v, shape=shape)
+    got = bpl.csr_matvec(data, indices, indptr, v, shape=shape).cpu().numpy()
+    assert_close(got, want, what="csr gather mean %d" % mean)
+    evr = rng.random(shape[0]) < 0.3
+    want = oracle_mod.event_csr_matvec(data, indices, indptr, evr, shape=shape, transpose=True)
+    got = bpl.event_csr_matvec(data, indices, indptr, evr, shape=shape, transpose=True).cpu().numpy()
+    mag = oracle_mod.event_csr_matvec(np.abs(data), indices, indptr, evr, shape=shape, transpose=True)
+    assert_close_reordered(got, want, mag, what="event scatter mean %d" % mean)
+
+
+def test_unaligned_event_vector_and_large_bitmap(cuda, oracle_mod):
+  # an event vector that does not start on a 16-byte boundary, and one whose bitmap needs more
+  # than 64 KiB of LDS (n_col > 524288)
+  rng = np.random.default_rng(12)
+  for n_col, offset in ((70001, 3), (700_000, 0), (1_400_000, 1)):
+    counts = rng.poisson(40, size=2000)
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_col)
+    data = rng.standard_normal(indices.shape[0]).astype(np.float32)
+    ev = rng.random(n_col) < 0.3
+    shape = (2000, n_col)
+    print("n_col", n_col, "offset", offset, flush=True)
+    base = torch.zeros(n_col + 16, dtype=torch.bool, device=cuda)
+    base[offset:offset + n_col] = torch.from_numpy(ev).to(cuda)
+    ev_dev = base[offset:offset + n_col]
+    want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape)
+    got = bpl.event_csr_matvec(data, indices, indptr, ev_dev, shape=shape).cpu().numpy()
+    assert_close(got, want)
+
+
+def test_config_event_csr_small(cuda, oracle_mod):
+  # 4,000 x 4,000, 80 per row, homogeneous 0.6, events 2 %, transpose: bit-exact
+  c = synth.config_event_csr_small()
+  want = oracle_mod.event_csr_matvec(c["data"], c["indices"], c["indptr"], c["events"], shape=c["shape"],
+                                     transpose=True)
+  got = bpl.event_csr_matvec(c["data"], c["indices"], c["indptr"], c["events"], shape=c["shape"],
+                             transpose=True).cpu().numpy()
+  assert np.array_equal(got, want)
+  assert want.sum() > 0
+
+
+def test_config_event_csr_large_scaled_and_properties(cuda, oracle_mod):
+  # the 1e8-nnz configuration at 1/16 scale against the oracle (25,000 x 25,000, ~6e6 nnz) ...
+  c = synth.config_event_csr_large(n=25_000)
+  for tr in (True, False):
+    want = oracle_mod.event_csr_matvec(c["data"], c["indices"], c["indptr"], c["events"], shape=c["shape"], transpose=tr)
+    got = bpl.event_csr_matvec(c["data"], c["indices"], c["indptr"], c["events"], shape=c["shape"], transpose=tr)
+    if tr:
+      mag = oracle_mod.event_csr_matvec(np.abs(c["data"]), c["indices"], c["indptr"], c["events"], shape=c["shape"],
+                                        transpose=True)
+      assert_close_reordered(got.cpu().numpy(), want, mag, what="scatter")
+    else:
+      assert_close(got.cpu().numpy(), want, what="gather")
+
+
+def test_full_size_event_csr_properties(cuda):
+  # ... and at full size (100,000 x 100,000, ~1e8 nnz) through size-independent properties:
+  #  * <y, A x> == <A^T y, x> with 0/1 vectors and integer weights (exact in fp32 up to 2^24)
+  #  * linearity in the weights: f(2 * w) == 2 * f(w) bit for bit
+  #  * all-ones events with unit weight give the row lengths / column counts exactly
+  c = synth.config_event_csr_large()
+  n = c["shape"][0]
+  dev = cuda
+  indices = torch.from_numpy(c["indices"]).to(dev)
+  indptr = torch.from_numpy(c["indptr"]).to(dev)
+  x = torch.from_numpy(c["events"]).to(dev)
+  y = torch.from_numpy(np.random.default_rng(3).random(n) < 0.05).to(dev)
+  ones = torch.ones(1, dtype=torch.float32, device=dev)
+  Ax = bpl.event_csr_matvec(ones, indices, indptr, x, shape=c["shape"], transpose=False)
+  ATy = bpl.event_csr_matvec(ones, indices, indptr, y, shape=c["shape"], transpose=True)
+  lhs = float((Ax.double() * y.double()).sum())
+  rhs = float((ATy.double() * x.double()).sum())
+  assert lhs == rhs and lhs > 0
+  row_len = np.diff(c["indptr"]).astype(np.float32)
+  all_on = torch.ones(n, dtype=torch.bool, device=dev)
+  got = bpl.event_csr_matvec(ones, indices, indptr, all_on, shape=c["shape"], transpose=False).cpu().numpy()
+  assert np.array_equal(got, row_len)
+  col_cnt = np.bincount(c["indices"], minlength=n).astype(np.float32)
+  got = bpl.event_csr_matvec(ones, indices, indptr, all_on, shape=c["shape"], transpose=True).cpu().numpy()
+  assert np.array_equal(got, col_cnt)
+  data = torch.from_numpy(c["data"]).to(dev)
+  f1 = bpl.event_csr_matvec(data, indices, indptr, x, shape=c["shape"], transpose=False)
+  f2 = bpl.event_csr_matvec(data * 2, indices, indptr, x, shape=c["shape"], transpose=False)
+  assert torch.equal(f1 * 2, f2)

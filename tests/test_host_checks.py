@@ -1,0 +1,54 @@
+"""Argument checking of the host-side operator wrappers (same conditions as the reference's
+wrappers; no GPU needed: the checks run before a device is touched)."""
+import numpy as np
+import pytest
+import torch
+
+import brainpylib_amd as bpl
+
+IDX = np.zeros(6, dtype=np.int32)
+PTR = np.zeros(5, dtype=np.int32)  # shape[0] = 4
+
+
+def test_event_csr_matvec_checks():
+  # brainpylib/_src/event_ops/event_csr_matvec.py:75-99
+  ev4, ev7 = np.zeros(4, bool), np.zeros(7, bool)
+  with pytest.raises(ValueError, match="size of data"):
+    bpl.event_csr_matvec(np.zeros(3, np.float32), IDX, PTR, ev7, shape=(4, 7))
+  with pytest.raises(ValueError, match="scalar or 1D"):
+    bpl.event_csr_matvec(np.zeros((2, 3), np.float32), IDX, PTR, ev7, shape=(4, 7))
+  with pytest.raises(ValueError, match="indices should be a 1D vector with int32 or uint32"):
+    bpl.event_csr_matvec(1.0, IDX.astype(np.int64), PTR, ev7, shape=(4, 7))
+  with pytest.raises(ValueError, match="indptr should be a 1D vector with int32 or uint32"):
+    bpl.event_csr_matvec(1.0, IDX, PTR.astype(np.int64), ev7, shape=(4, 7))
+  with pytest.raises(ValueError, match="events should be a 1D"):
+    bpl.event_csr_matvec(1.0, IDX, PTR, np.zeros((7, 1), bool), shape=(4, 7))
+  with pytest.raises(ValueError, match="length-2"):
+    bpl.event_csr_matvec(1.0, IDX, PTR, ev7, shape=(4, 7, 1))
+  with pytest.raises(ValueError, match=r"Shape mismatch, mat \(4, 7\) @ vec \(4,\)"):
+    bpl.event_csr_matvec(1.0, IDX, PTR, ev4, shape=(4, 7))
+  with pytest.raises(ValueError, match=r"Shape mismatch, vec \(7,\) @ mat \(4, 7\)"):
+    bpl.event_csr_matvec(1.0, IDX, PTR, ev7, shape=(4, 7), transpose=True)
+  with pytest.raises(ValueError, match="events should be bool or have the dtype of data"):
+    bpl.event_csr_matvec(np.zeros(6, np.float32), IDX, PTR, np.zeros(7, np.float64), shape=(4, 7))
+
+
+def test_csr_matvec_checks():
+  # brainpylib/_src/sparse_ops/sparse_csr_matvec.py:70-82
+  v = np.zeros(7, np.float32)
+  with pytest.raises(ValueError, match="Only support methods"):
+    bpl.csr_matvec(1.0, IDX, PTR, v, shape=(4, 7), method="fast")
+  with pytest.raises(TypeError, match="Only support float32 and float64"):
+    bpl.csr_matvec(np.zeros(6, np.int32), IDX, PTR, v, shape=(4, 7))
+  with pytest.raises(TypeError, match="types of data and vector"):
+    bpl.csr_matvec(np.zeros(6, np.float64), IDX, PTR, v, shape=(4, 7))
+  with pytest.raises(ValueError, match="Shape mismatch"):
+    bpl.csr_matvec(np.zeros(6, np.float32), IDX, PTR, np.zeros(4, np.float32), shape=(4, 7))
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-device error")
+def test_no_cpu_fallback():
+  with pytest.raises(RuntimeError, match="no CPU path"):
+    bpl.event_csr_matvec(1.0, IDX, PTR, np.zeros(7, bool), shape=(4, 7))
+  with pytest.raises(RuntimeError, match="no CPU path"):
+    bpl.csr_matvec(1.0, IDX, PTR, np.zeros(7, np.float32), shape=(4, 7))
