@@ -1,0 +1,256 @@
+"""Benchmark of the event-driven sparse operator path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-extra] [--skip-cpu]
+
+A step is one event_csr_matvec call over the 100,000 x 100,000, ~1e8-nnz heterogeneous-weight
+matrix with 5 % of the event vector active, in the row-gather orientation (transpose=False),
+which streams all 1e8 column indices: that is the kernel the HBM roofline applies to.  Inputs
+are resident in HBM before the timed region.  The JSON line also carries, under "extra", the
+scatter orientation (transpose=True) of the same matrix, the 4,000-neuron configuration, and
+csr_matvec at ~1e8 nnz.
+
+Prints ONE JSON line on stdout; progress goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+  sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+
+
+def log(*a):
+  print(*a, file=sys.stderr, flush=True)
+
+
+def time_calls(fn, steps, warmup):
+  """Per-call GPU durations (HIP events on the stream the kernels are enqueued on) and the
+  wall time of the K back-to-back calls."""
+  import torch
+  for _ in range(warmup):
+    fn()
+  torch.cuda.synchronize()
+  starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+  ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+  t0 = time.perf_counter()
+  for i in range(steps):
+    starts[i].record()
+    fn()
+    ends[i].record()
+  torch.cuda.synchronize()
+  wall = time.perf_counter() - t0
+  dur_ms = np.array([s.elapsed_time(e) for s, e in zip(starts, ends)])
+  return dur_ms, wall
+
+
+def stats(dur_ms):
+  return dict(mean_us=float(dur_ms.mean() * 1e3), median_us=float(np.median(dur_ms) * 1e3),
+              p95_us=float(np.percentile(dur_ms, 95) * 1e3), min_us=float(dur_ms.min() * 1e3))
+
+
+def check(got, want, what, mag=None):
+  got = np.asarray(got, dtype=np.float64)
+  want = np.asarray(want, dtype=np.float64)
+  bound = 1e-6 + 1e-5 * np.abs(want)
+  if mag is not None:  # sums accumulated in another order (atomics): reordering bound
+    bound = bound + 4 * np.finfo(np.float32).eps * np.asarray(mag, dtype=np.float64)
+  err = np.abs(got - want)
+  bad = int((err > bound).sum())
+  log("parity %-34s max abs err %.3e  violations %d / %d" % (what, float(err.max(initial=0)), bad, got.size))
+  if bad:
+    raise SystemExit("parity gate failed for " + what)
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=200)
+  ap.add_argument("--warmup", type=int, default=20)
+  ap.add_argument("--skip-extra", action="store_true", help="only the headline workload")
+  ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU baseline")
+  args = ap.parse_args()
+  if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+    raise SystemExit("bench.py: this build runs on ONE GPU (the operators are single-device, like the "
+                     "reference's); --gpus %d is not supported." % args.gpus)
+
+  import torch
+  import brainpylib_amd as bpl
+  from brainpylib_amd import synth
+  import oracle  # checker and CPU baseline only
+
+  assert torch.cuda.is_available(), "bench.py needs a HIP device"
+  dev = torch.device("cuda:0")
+  torch.cuda.set_device(dev)
+  cores = len(os.sched_getaffinity(0))
+
+  # ---------------------------------------------------------------------------------------------
+  # headline workload: event_csr_matvec, 100,000 x 100,000, ~1e8 nnz, heterogeneous weights
+  # ---------------------------------------------------------------------------------------------
+  t0 = time.time()
+  c = synth.config_event_csr_large()
+  n_row, n_col = c["shape"]
+  nnz = int(c["indices"].shape[0])
+  log("generated event_csr_matvec workload: nnz %d in %.1f s" % (nnz, time.time() - t0))
+  data = torch.from_numpy(c["data"]).to(dev)
+  indices = torch.from_numpy(c["indices"]).to(dev)
+  indptr = torch.from_numpy(c["indptr"]).to(dev)
+  events = torch.from_numpy(c["events"]).to(dev)
+
+  # parity gate at full size (the oracle's single-thread loops take well under a second each)
+  want_g = oracle.event_csr_matvec(c["data"], c["indices"], c["indptr"], c["events"], shape=c["shape"])
+  got_g = bpl.event_csr_matvec(data, indices, indptr, events, shape=c["shape"]).cpu().numpy()
+  check(got_g, want_g, "event_csr_matvec gather 1e8 nnz")
+  want_s = oracle.event_csr_matvec(c["data"], c["indices"], c["indptr"], c["events"], shape=c["shape"], transpose=True)
+  mag_s = oracle.event_csr_matvec(np.abs(c["data"]), c["indices"], c["indptr"], c["events"], shape=c["shape"],
+                                  transpose=True)
+  got_s = bpl.event_csr_matvec(data, indices, indptr, events, shape=c["shape"], transpose=True).cpu().numpy()
+  check(got_s, want_s, "event_csr_matvec scatter 1e8 nnz", mag_s)
+
+  hits = int(c["events"][c["indices"]].sum())                 # synapses whose pre-neuron fired (gather view)
+  active = int(c["events"].sum())
+  delivered = int(np.diff(c["indptr"].astype(np.int64))[c["events"]].sum())  # scatter view
+
+  def gather():
+    return bpl.event_csr_matvec(data, indices, indptr, events, shape=c["shape"], transpose=False)
+
+  dur, wall = time_calls(gather, args.steps, args.warmup)
+  ms_per_step = wall / args.steps * 1e3
+  kernel_ms = float(dur.mean())
+  # algorithmic bytes of one gather call: indptr + all indices + the data elements that are
+  # hit + the event vector + the output
+  bytes_gather = 4 * (n_row + 1) + 4 * nnz + 4 * hits + n_col * 1 + 4 * n_row
+  achieved = bytes_gather / (kernel_ms * 1e-3) / 1e9
+  value = nnz / (ms_per_step * 1e-3) / 1e9
+  log("gather: %.1f us/call (events) %.1f us/step (wall)  %.1f GSOP/s  %.0f GB/s algorithmic" % (
+    kernel_ms * 1e3, ms_per_step * 1e3, value, achieved))
+
+  extra = {"gather_call_us": stats(dur), "nnz": nnz, "hits": hits, "active_rows": active}
+
+  # ---------------------------------------------------------------------------------------------
+  # CPU baseline: the oracle's restatement of the reference's CPU loop for this exact call
+  # (heterogeneous gather: single-threaded in the reference), bounded to ~10-20 s
+  # ---------------------------------------------------------------------------------------------
+  cpu_baseline = None
+  if not args.skip_cpu:
+    oracle.set_threads(1)
+    n_cpu, t_cpu = 0, 0.0
+    while t_cpu < 10.0 and n_cpu < 50:
+      t1 = time.perf_counter()
+      oracle.event_csr_matvec(c["data"], c["indices"], c["indptr"], c["events"], shape=c["shape"])
+      t_cpu += time.perf_counter() - t1
+      n_cpu += 1
+    cpu_baseline = {"value": nnz / (t_cpu / n_cpu) / 1e9, "unit": "GSOP/s", "cores": 1, "kind": "port",
+                    "sample": "%d full calls of the same workload (%.2f s each), C restatement of "
+                              "event_csr_matvec.py:334-347 compiled with gcc -O2" % (n_cpu, t_cpu / n_cpu)}
+    log("cpu baseline: %.3f s/call -> %.2f GSOP/s on 1 of %d cores" % (t_cpu / n_cpu, cpu_baseline["value"], cores))
+
+  if not args.skip_extra:
+    # scatter orientation of the same matrix
+    def scatter():
+      return bpl.event_csr_matvec(data, indices, indptr, events, shape=c["shape"], transpose=True)
+    dur_s, wall_s = time_calls(scatter, args.steps, args.warmup)
+    bytes_scatter = n_row * 1 + 8 * active + delivered * 8 + 4 * n_col
+    extra["scatter_1e8"] = dict(stats(dur_s), delivered_synapses=delivered,
+                                gsop_per_s=delivered / (dur_s.mean() * 1e-3) / 1e9,
+                                algorithmic_gb_per_s=bytes_scatter / (dur_s.mean() * 1e-3) / 1e9,
+                                wall_us_per_call=wall_s / args.steps * 1e6)
+    if not args.skip_cpu:
+      t1 = time.perf_counter()
+      for _ in range(20):
+        oracle.event_csr_matvec(c["data"], c["indices"], c["indptr"], c["events"], shape=c["shape"], transpose=True)
+      t_cpu = (time.perf_counter() - t1) / 20
+      extra["scatter_1e8"]["cpu_port_1core_us"] = t_cpu * 1e6
+    log("scatter 1e8: %s" % extra["scatter_1e8"])
+
+    # homogeneous weight, gather: only the index stream is read
+    w = torch.tensor([0.6], dtype=torch.float32, device=dev)
+    dur_h, _ = time_calls(lambda: bpl.event_csr_matvec(w, indices, indptr, events, shape=c["shape"]), args.steps,
+                          args.warmup)
+    bytes_h = 4 * (n_row + 1) + 4 * nnz + n_col + 4 * n_row
+    extra["gather_homo_1e8"] = dict(stats(dur_h), gsop_per_s=nnz / (dur_h.mean() * 1e-3) / 1e9,
+                                    algorithmic_gb_per_s=bytes_h / (dur_h.mean() * 1e-3) / 1e9)
+    log("gather homo 1e8: %s" % extra["gather_homo_1e8"])
+    del data, indices, indptr, events
+
+    # 4,000 x 4,000, 80 per row, homogeneous 0.6, 2 % events, scatter (the reference's own CPU-sized case)
+    s = synth.config_event_csr_small()
+    sd = {k: torch.from_numpy(v).to(dev) for k, v in s.items() if isinstance(v, np.ndarray)}
+    got = bpl.event_csr_matvec(sd["data"], sd["indices"], sd["indptr"], sd["events"], shape=s["shape"], transpose=True)
+    want = oracle.event_csr_matvec(s["data"], s["indices"], s["indptr"], s["events"], shape=s["shape"], transpose=True)
+    if not np.array_equal(got.cpu().numpy(), want):
+      raise SystemExit("parity gate failed for the 4,000-neuron configuration")
+    dur_c1, wall_c1 = time_calls(lambda: bpl.event_csr_matvec(sd["data"], sd["indices"], sd["indptr"], sd["events"],
+                                                              shape=s["shape"], transpose=True), args.steps, args.warmup)
+    deliv = int(np.diff(s["indptr"])[s["events"]].sum())
+    extra["scatter_4000"] = dict(stats(dur_c1), delivered_synapses=deliv, wall_us_per_call=wall_c1 / args.steps * 1e6)
+    if not args.skip_cpu:
+      t1 = time.perf_counter()
+      for _ in range(2000):
+        oracle.event_csr_matvec(s["data"], s["indices"], s["indptr"], s["events"], shape=s["shape"], transpose=True)
+      extra["scatter_4000"]["cpu_port_1core_us"] = (time.perf_counter() - t1) / 2000 * 1e6
+    log("scatter 4000: %s" % extra["scatter_4000"])
+
+    # csr_matvec, 1,000,000 x 1,000,000, ~1e8 nnz
+    t0 = time.time()
+    m = synth.config_csr_matvec()
+    log("generated csr_matvec workload in %.1f s" % (time.time() - t0))
+    md = {k: torch.from_numpy(v).to(dev) for k, v in m.items() if isinstance(v, np.ndarray)}
+    nnz3 = int(m["indices"].shape[0])
+    oracle.set_threads(cores)
+    t1 = time.perf_counter()
+    want = oracle.csr_matvec(m["data"], m["indices"], m["indptr"], m["vector"], shape=m["shape"])
+    t_cpu3 = time.perf_counter() - t1
+    got = bpl.csr_matvec(md["data"], md["indices"], md["indptr"], md["vector"], shape=m["shape"]).cpu().numpy()
+    check(got, want, "csr_matvec 1e8 nnz")
+    dur3, _ = time_calls(lambda: bpl.csr_matvec(md["data"], md["indices"], md["indptr"], md["vector"], shape=m["shape"]),
+                         max(20, args.steps // 4), 5)
+    bytes3 = 4 * (m["shape"][0] + 1) + 8 * nnz3 + 4 * m["shape"][1] + 4 * m["shape"][0]
+    extra["csr_matvec_1e8"] = dict(stats(dur3), nnz=nnz3, gsop_per_s=nnz3 / (dur3.mean() * 1e-3) / 1e9,
+                                   algorithmic_gb_per_s=bytes3 / (dur3.mean() * 1e-3) / 1e9,
+                                   cpu_port_allcores_ms=t_cpu3 * 1e3, cpu_cores=cores)
+    log("csr_matvec 1e8: %s" % extra["csr_matvec_1e8"])
+    want = oracle.csr_matvec(m["data"], m["indices"], m["indptr"], m["vector"], shape=m["shape"], transpose=True)
+    mag = oracle.csr_matvec(m["data"], m["indices"], m["indptr"], np.abs(m["vector"]), shape=m["shape"], transpose=True)
+    got = bpl.cusparse_csr_matvec(md["data"], md["indices"], md["indptr"], md["vector"], shape=m["shape"],
+                                  transpose=True).cpu().numpy()
+    check(got, want, "csr_matvec transposed 1e8 nnz", mag)
+    dur3t, _ = time_calls(lambda: bpl.cusparse_csr_matvec(md["data"], md["indices"], md["indptr"], md["vector"],
+                                                          shape=m["shape"], transpose=True), max(20, args.steps // 4), 5)
+    extra["csr_matvec_transposed_1e8"] = dict(stats(dur3t), gsop_per_s=nnz3 / (dur3t.mean() * 1e-3) / 1e9,
+                                              algorithmic_gb_per_s=bytes3 / (dur3t.mean() * 1e-3) / 1e9)
+    log("csr_matvec transposed 1e8: %s" % extra["csr_matvec_transposed_1e8"])
+
+  result = {
+    "metric": "GSOP/s + % HBM roofline, event_csr_matvec 1e8 nnz; jitconn GSOP/s at p=0.001",
+    "value": value,
+    "unit": "GSOP/s (CSR nonzeros scanned per second, event_csr_matvec transpose=False)",
+    "n_gpus": 1,
+    "steps": args.steps,
+    "warmup": args.warmup,
+    "ms_per_step": ms_per_step,
+    "higher_is_better": True,
+    "scaling": "weak",
+    "vs_baseline": None,
+    "dtype": "f32",
+    "data": "synthetic",
+    "config": {"workload": "event_csr_matvec heterogeneous 100000x100000, nnz~Binomial(1e5,0.01)/row (%d nnz), "
+                           "weights N(0,0.1^2), events Bernoulli(0.05), transpose=False, seed 1" % nnz},
+    "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                 "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                 "kernel": "csr_gather_kernel<float,bool,heter,event,lds-bitmap>",
+                 "algorithmic_bytes_per_launch": bytes_gather, "kernel_us": kernel_ms * 1e3},
+    "cpu_baseline": cpu_baseline,
+    "extra": extra,
+  }
+  print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+  main()
