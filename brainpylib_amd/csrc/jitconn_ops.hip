@@ -1,0 +1,335 @@
+// Just-in-time-connectivity operators for gfx950: the matrix is never stored, its rows are
+// regenerated in registers on every call from per-stream std::mt19937 generators (mt_wave.h)
+// with geometric skip sampling, exactly the loop of the reference's CPU kernels
+//   first = ceil(log(U)/log_p);  while (i < n) { [w = weight draw;] use(i, w); i += ceil(log(U)/log_p); }
+// (lib/cpu_jitconn_event_matvec.cpp:20-31, lib/cpu_jitconn_matvec.cpp:20-29 and their *_atomic
+// twins).  Stream `o` is std::mt19937{seed + o}.
+//
+// One wave64 owns one stream.  Each lane draws one synapse of the next batch (its skip and its
+// weight), a DPP prefix sum over the skips places the 64 synapses, a ballot finds where the row
+// ends.  The only memory traffic is the input vector (events are packed into an LDS bitmap when
+// it fits) and the output.
+//
+//   row walk  ("outdim_parallel"):  stream per output element, inputs gathered, one store.
+//   column walk ("atomic"):         stream per input element, silent inputs are skipped
+//                                   entirely (compacted per workgroup), outputs by atomics.
+//
+// Reference boundary: lib/gpu_jitconn_event_matvec.cu:111-135,432-522,
+// lib/gpu_jitconn_event_matvec_atomic.cu:61-85, lib/gpu_jitconn_matvec.cu:115-138,
+// lib/gpu_jitconn_matvec_atomic.cu:53-77 (buffers = [input, out]; descriptors; target names).
+#include <cmath>
+
+#include "common.h"
+#include "mt_wave.h"
+#include "targets.h"
+
+namespace bpl {
+namespace {
+
+enum : int { kHomo = 0, kUniform = 1, kNormal = 2 };
+enum : int { kInEvent = 0, kInDense = 1 };
+
+// weight draws ----------------------------------------------------------------------------------
+// std::uniform_real_distribution<T>{a,b}: canonical * (b - a) + a, no contraction
+__device__ __forceinline__ float uniform_weight(const uint32_t *w, float a, float b) {
+  return __fadd_rn(__fmul_rn(canonical_f32(w[0]), __fsub_rn(b, a)), a);
+}
+__device__ __forceinline__ double uniform_weight(const uint32_t *w, double a, double b) {
+  return __dadd_rn(__dmul_rn(canonical_f64(w[0], w[1]), __dsub_rn(b, a)), a);
+}
+
+template <typename T1>
+struct WeightWords {
+  static constexpr int value = sizeof(T1) == 4 ? 1 : 2;  // mt19937 words per uniform weight
+};
+
+// Walks stream std::mt19937{stream_seed} over [0, n): calls f(index, weight, valid) once per
+// batch with the whole wave converged; `valid` marks the lanes that hold a synapse of the row.
+template <typename T1, int W, typename F>
+__device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t stream_seed, uint32_t n, double log_p,
+                                            T1 wa, T1 wb, F &&f) {
+  mt_seed(st, stream_seed, lane);
+  uint32_t pos = 0;
+  // With every skip >= 1 a row ends within n/64 + 1 batches; the cap only guards against a
+  // generator state that yields zero skips forever (log_p is validated on the host).
+  const uint32_t max_batches = n / 16u + 1024u;
+  if (W == kHomo) {
+    // stream: K K K ...   synapse s sits at K_0 + ... + K_s
+    uint32_t carry = 0;
+    for (uint32_t b = 0; b < max_batches; ++b) {
+      uint32_t w[2] = {1u, 1u};
+      mt_generate<2>(st, pos, lane, kWave, w);
+      const uint32_t skip = skip_from_words(w[0], w[1], log_p);
+      const uint32_t idx = carry + wave_inclusive_scan_u32(skip);
+      const uint64_t done = __ballot(idx >= n);
+      const int nvalid = done ? (__ffsll(static_cast<unsigned long long>(done)) - 1) : kWave;
+      f(idx, T1(1), lane < nvalid);
+      if (done) break;
+      carry = __builtin_amdgcn_readlane(idx, kWave - 1);
+    }
+  } else if (W == kUniform) {
+    // stream: K  (w K) (w K) ...   synapse s sits at K_0 + ... + K_s, its weight precedes K_{s+1}
+    constexpr int WW = WeightWords<T1>::value;
+    constexpr int K = WW + 2;
+    constexpr int NL = (K == 3) ? 64 : 32;  // K * NL <= 227
+    uint32_t w0[2] = {1u, 1u};
+    mt_generate<2>(st, pos, lane, 1, w0);
+    uint32_t carry = __builtin_amdgcn_readfirstlane(skip_from_words(w0[0], w0[1], log_p));
+    for (uint32_t b = 0; b < max_batches; ++b) {
+      uint32_t w[K];
+#pragma unroll
+      for (int i = 0; i < K; ++i) w[i] = 1u;
+      mt_generate<K>(st, pos, lane, NL, w);
+      const T1 weight = uniform_weight(w, wa, wb);
+      uint32_t skip = skip_from_words(w[WW], w[WW + 1], log_p);
+      if (lane >= NL) skip = 0;
+      const uint32_t incl = wave_inclusive_scan_u32(skip);
+      const uint32_t idx = carry + incl - skip;
+      const uint64_t done = __ballot(lane < NL && idx >= n);
+      const int nvalid = done ? (__ffsll(static_cast<unsigned long long>(done)) - 1) : NL;
+      f(idx, weight, lane < nvalid);
+      if (done) break;
+      carry += __builtin_amdgcn_readlane(incl, kWave - 1);
+    }
+  }
+}
+
+// ---- event probes -------------------------------------------------------------------------------
+template <typename VT>
+__device__ __forceinline__ uint32_t pack32(const VT *__restrict__ ev, uint32_t base, uint32_t n) {
+  uint32_t m = 0;
+#pragma unroll 8
+  for (uint32_t b = 0; b < 32; ++b) {
+    const uint32_t i = base + b;
+    if (i < n && is_event(ev[i])) m |= 1u << b;
+  }
+  return m;
+}
+
+// ---- row walk -------------------------------------------------------------------------------------
+template <typename T1, typename VT, int IN, int W, bool LDS_BITS>
+__global__ __launch_bounds__(1024) void jitconn_rowwalk_kernel(const VT *__restrict__ in, T1 *__restrict__ out,
+                                                               uint32_t n_out, uint32_t n_in, uint32_t seed,
+                                                               double log_p, T1 wa, T1 wb) {
+  extern __shared__ uint32_t smem[];
+  const int lane = lane_id();
+  const uint32_t wave = threadIdx.x / kWave;
+  const uint32_t nwaves = blockDim.x / kWave;
+  uint32_t *st = smem + wave * kMtStateWords;
+  const uint32_t *bits = smem + nwaves * kMtStateWords;
+  if (LDS_BITS) {
+    uint32_t *wbits = smem + nwaves * kMtStateWords;
+    const uint32_t words = (n_in + 31u) >> 5;
+    for (uint32_t i = threadIdx.x; i < words; i += blockDim.x) wbits[i] = pack32<VT>(in, i << 5, n_in);
+    __syncthreads();
+  }
+  for (uint32_t o = blockIdx.x * nwaves + wave; o < n_out; o += gridDim.x * nwaves) {
+    double acc = 0.0;
+    uint32_t cnt = 0;
+    walk_stream<T1, W>(st, lane, seed + o, n_in, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
+      if (IN == kInDense) {
+        if (valid) {
+          const T1 v = static_cast<T1>(in[idx]);
+          acc += static_cast<double>(W == kHomo ? v : static_cast<T1>(w * v));
+        }
+      } else {
+        bool hit = false;
+        if (valid) {
+          if (LDS_BITS) hit = (bits[idx >> 5] >> (idx & 31u)) & 1u;
+          else hit = is_event(in[idx]);
+        }
+        if (W == kHomo) cnt += static_cast<uint32_t>(__popcll(__ballot(hit)));
+        else if (hit) acc += static_cast<double>(w);
+      }
+    });
+    if (IN == kInEvent && W == kHomo) {
+      if (lane == 0) out[o] = static_cast<T1>(cnt);
+    } else {
+      acc = wave_sum(acc);
+      if (lane == 0) out[o] = static_cast<T1>(acc);
+    }
+  }
+}
+
+// ---- column walk ------------------------------------------------------------------------------------
+constexpr int kColThreads = 256;
+
+template <typename T1, typename VT, int IN, int W>
+__global__ __launch_bounds__(kColThreads) void jitconn_colwalk_kernel(const VT *__restrict__ in,
+                                                                      T1 *__restrict__ out, uint32_t n_out,
+                                                                      uint32_t n_in, uint32_t seed, double log_p,
+                                                                      T1 wa, T1 wb) {
+  constexpr int kWaves = kColThreads / kWave;
+  __shared__ uint32_t s_state[kWaves * kMtStateWords];
+  __shared__ uint32_t s_col[kColThreads];
+  __shared__ T1 s_val[kColThreads];
+  __shared__ uint32_t s_wave_cnt[kWaves];
+
+  const int lane = lane_id();
+  const uint32_t wave = threadIdx.x / kWave;
+  const uint32_t c = blockIdx.x * kColThreads + threadIdx.x;
+  T1 v = T1(0);
+  bool on = false;
+  if (c < n_in) {
+    const VT x = in[c];
+    on = is_event(x);
+    v = static_cast<T1>(x);
+  }
+  const uint64_t mask = __ballot(on);
+  if (lane == 0) s_wave_cnt[wave] = static_cast<uint32_t>(__popcll(mask));
+  __syncthreads();
+  uint32_t base = 0, count = 0;
+#pragma unroll
+  for (uint32_t i = 0; i < kWaves; ++i) {
+    if (i < wave) base += s_wave_cnt[i];
+    count += s_wave_cnt[i];
+  }
+  if (on) {
+    const uint32_t k = base + static_cast<uint32_t>(__popcll(mask & ((1ull << lane) - 1ull)));
+    s_col[k] = c;
+    s_val[k] = v;
+  }
+  __syncthreads();
+
+  uint32_t *st = s_state + wave * kMtStateWords;
+  for (uint32_t k = wave; k < count; k += kWaves) {
+    const uint32_t col = s_col[k];
+    const T1 val = s_val[k];
+    walk_stream<T1, W>(st, lane, seed + col, n_out, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
+      if (valid) {
+        T1 add;
+        if (IN == kInDense) add = (W == kHomo) ? val : static_cast<T1>(w * val);
+        else add = w;  // homo: w == 1
+        atomic_add(&out[idx], add);
+      }
+    });
+  }
+}
+
+// ---- launchers ----------------------------------------------------------------------------------------
+bool valid_log_p(const char *target, double log_p) {
+  if (!(log_p < 0.0) || std::isinf(log_p)) {
+    set_error("%s: log_p must be finite and negative (conn_prob in (0, 1]), got %g", target, log_p);
+    return false;
+  }
+  return true;
+}
+
+template <typename T1, typename VT, int IN, int W, bool LDS_BITS>
+void launch_rowwalk_impl(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, uint32_t n_in, uint32_t seed,
+                         double log_p, T1 wa, T1 wb, int nwaves, size_t lds_bytes) {
+  auto kernel = jitconn_rowwalk_kernel<T1, VT, IN, W, LDS_BITS>;
+  const int block = nwaves * kWave;
+  struct Cached {
+    size_t lds_bytes;
+    int block;
+    int per_cu;
+  };
+  static thread_local Cached cached = {~size_t(0), 0, 0};
+  if (cached.lds_bytes != lds_bytes || cached.block != block) {
+    if (lds_bytes > 64 * 1024)
+      (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(lds_bytes));
+    int q = 1;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&q, reinterpret_cast<const void *>(kernel), block, lds_bytes) !=
+            hipSuccess || q < 1) {
+      (void)hipGetLastError();
+      q = 1;
+    }
+    cached = {lds_bytes, block, q};
+  }
+  const unsigned resident = static_cast<unsigned>(device_info().num_cu) * static_cast<unsigned>(cached.per_cu);
+  const unsigned needed = div_up(n_out, nwaves);
+  const unsigned grid = needed < resident ? needed : resident;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), lds_bytes, stream, in, out, n_out, n_in, seed, log_p, wa, wb);
+}
+
+template <typename T1, typename VT, int IN, int W>
+void launch_rowwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, uint32_t n_in, uint32_t seed,
+                    double log_p, T1 wa, T1 wb) {
+  if (n_out == 0) return;
+  const size_t state_bytes = kMtStateWords * 4;
+  const size_t cap = static_cast<size_t>(160) * 1024 - 512;
+  if (IN == kInEvent) {
+    const size_t bitmap = (static_cast<size_t>(n_in) + 31) / 32 * 4;
+    // as many waves per workgroup as fit beside the bitmap (at most 16)
+    for (int nwaves = 16; nwaves >= 8; nwaves -= 4) {
+      const size_t lds = bitmap + nwaves * state_bytes;
+      if (lds <= cap) {
+        // small bitmaps: 8-wave workgroups, several per CU
+        const int nw = (bitmap <= 16 * 1024) ? 8 : nwaves;
+        launch_rowwalk_impl<T1, VT, IN, W, true>(stream, in, out, n_out, n_in, seed, log_p, wa, wb, nw,
+                                                 bitmap + nw * state_bytes);
+        return;
+      }
+    }
+  }
+  launch_rowwalk_impl<T1, VT, IN, W, false>(stream, in, out, n_out, n_in, seed, log_p, wa, wb, 8, 8 * state_bytes);
+}
+
+template <typename T1, typename VT, int IN, int W>
+void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, uint32_t n_in, uint32_t seed,
+                    double log_p, T1 wa, T1 wb) {
+  fill_zero(stream, out, n_out);
+  if (n_in == 0 || n_out == 0) return;
+  hipLaunchKernelGGL((jitconn_colwalk_kernel<T1, VT, IN, W>), dim3(div_up(n_in, kColThreads)), dim3(kColThreads), 0,
+                     stream, in, out, n_out, n_in, seed, log_p, wa, wb);
+}
+
+// buffers = [input, out]
+template <typename T1, typename VT, int IN, int W, bool COLWALK>
+void jitconn_entry(const char *target, hipStream_t stream, void **buffers, const char *opaque, size_t opaque_len) {
+  uint32_t n_row, n_col, seed;
+  double log_p, a = 0, b = 0;
+  if (W == kHomo) {
+    bpl_jitconn_prob_homo_descriptor d;
+    if (!unpack(target, opaque, opaque_len, &d)) return;
+    n_row = d.n_row, n_col = d.n_col, seed = d.seed, log_p = d.log_p;
+  } else {
+    bpl_jitconn_prob_weight_descriptor d;
+    if (!unpack(target, opaque, opaque_len, &d)) return;
+    n_row = d.n_row, n_col = d.n_col, seed = d.seed, log_p = d.log_p, a = d.w_a, b = d.w_b;
+  }
+  if (!valid_log_p(target, log_p)) return;
+  if (buffers == nullptr) {
+    set_error("%s: null buffer table", target);
+    return;
+  }
+  const VT *in = static_cast<const VT *>(buffers[0]);
+  T1 *out = static_cast<T1 *>(buffers[1]);
+  if (COLWALK) launch_colwalk<T1, VT, IN, W>(stream, in, out, n_row, n_col, seed, log_p, static_cast<T1>(a), static_cast<T1>(b));
+  else launch_rowwalk<T1, VT, IN, W>(stream, in, out, n_row, n_col, seed, log_p, static_cast<T1>(a), static_cast<T1>(b));
+  check_launch(target);
+}
+
+}  // namespace
+}  // namespace bpl
+
+using namespace bpl;
+
+#define BPL_DEFINE(name, ...)                                                                      \
+  extern "C" void name(bpl_stream_t stream, void **buffers, const char *opaque, size_t opaque_len) { \
+    jitconn_entry<__VA_ARGS__>(__func__, static_cast<hipStream_t>(stream), buffers, opaque, opaque_len); \
+  }
+
+// event input: <result type, event type, kInEvent, weight kind, column walk>
+#define BPL_EVENT_FAMILY(wname, W)                                                                           \
+  BPL_DEFINE(gpu_event_matvec_prob_##wname##_v2_float_bool, float, uint8_t, kInEvent, W, false)               \
+  BPL_DEFINE(gpu_event_matvec_prob_##wname##_v2_float_float, float, float, kInEvent, W, false)                \
+  BPL_DEFINE(gpu_event_matvec_prob_##wname##_v2_double_bool, double, uint8_t, kInEvent, W, false)             \
+  BPL_DEFINE(gpu_event_matvec_prob_##wname##_v2_double_double, double, double, kInEvent, W, false)            \
+  BPL_DEFINE(gpu_event_matvec_atomic_prob_##wname##_v2_float_bool, float, uint8_t, kInEvent, W, true)         \
+  BPL_DEFINE(gpu_event_matvec_atomic_prob_##wname##_v2_float_float, float, float, kInEvent, W, true)          \
+  BPL_DEFINE(gpu_event_matvec_atomic_prob_##wname##_v2_double_bool, double, uint8_t, kInEvent, W, true)       \
+  BPL_DEFINE(gpu_event_matvec_atomic_prob_##wname##_v2_double_double, double, double, kInEvent, W, true)
+
+#define BPL_DENSE_FAMILY(wname, W)                                                           \
+  BPL_DEFINE(gpu_matvec_prob_##wname##_v2_float, float, float, kInDense, W, false)            \
+  BPL_DEFINE(gpu_matvec_prob_##wname##_v2_double, double, double, kInDense, W, false)         \
+  BPL_DEFINE(gpu_matvec_atomic_prob_##wname##_v2_float, float, float, kInDense, W, true)      \
+  BPL_DEFINE(gpu_matvec_atomic_prob_##wname##_v2_double, double, double, kInDense, W, true)
+
+BPL_EVENT_FAMILY(homo, kHomo)
+BPL_EVENT_FAMILY(uniform, kUniform)
+BPL_DENSE_FAMILY(homo, kHomo)
+BPL_DENSE_FAMILY(uniform, kUniform)

@@ -1,0 +1,113 @@
+// A std::mt19937 stream generated cooperatively by one wave64, state in LDS.
+//
+// The jitconn operators draw one generator stream per output row (or per input column):
+// stream i is std::mt19937{seed + i}, the generator of the reference's CPU backend
+// (lib/cpu_jitconn_event_matvec.cpp:20-21), restarted per stream the way the reference's GPU
+// backend restarts its generator per row (lib/gpu_jitconn_event_matvec.cu:94-96).  A row is
+// then exactly what the reference CPU code produces for a one-row matrix seeded `seed + i`.
+//
+// MT19937 produces word t from words t-624, t-623 and t-227, so up to 227 consecutive words can
+// be produced at once from the previous 624: each lane computes K consecutive words
+// (64*K <= 227) of the next batch and the 624-word state is a circular buffer in LDS.
+// Seeding is a serial 623-step recurrence; it runs on the scalar unit (the seed is wave
+// uniform) and the values are packed 64 at a time into a vector register with v_writelane.
+#pragma once
+
+#include "common.h"
+
+namespace bpl {
+
+constexpr int kMtN = 624;
+constexpr int kMtM = 397;
+constexpr int kMtStateWords = 640;  // LDS words reserved per wave
+
+__device__ __forceinline__ void mt_seed(uint32_t *st, uint32_t seed, int lane) {
+  uint32_t x = __builtin_amdgcn_readfirstlane(seed);
+#pragma unroll 1
+  for (int base = 0; base < kMtStateWords; base += kWave) {
+    uint32_t v = 0;
+#pragma unroll
+    for (int i = 0; i < kWave; ++i) {
+      // lane i of v <- x  (x lives in a scalar register)
+      asm volatile("v_writelane_b32 %0, %1, %2" : "+v"(v) : "s"(x), "n"(i));
+      x = 1812433253u * (x ^ (x >> 30)) + static_cast<uint32_t>(base + i + 1);
+    }
+    if (base + lane < kMtN) st[base + lane] = v;
+  }
+}
+
+__device__ __forceinline__ uint32_t mt_twist(uint32_t a, uint32_t b, uint32_t c) {
+  const uint32_t y = (a & 0x80000000u) | (b & 0x7fffffffu);
+  return c ^ (y >> 1) ^ ((y & 1u) ? 0x9908b0dfu : 0u);
+}
+
+__device__ __forceinline__ uint32_t mt_temper(uint32_t y) {
+  y ^= y >> 11;
+  y ^= (y << 7) & 0x9d2c5680u;
+  y ^= (y << 15) & 0xefc60000u;
+  y ^= y >> 18;
+  return y;
+}
+
+// Produces the next K * nlanes words of the stream; lane l < nlanes receives words
+// K*l .. K*l + K-1 of them (tempered) in w[].  `pos` is the state slot of the first new word
+// (wave uniform, < 624) and is advanced.  Requires K * nlanes <= 227.
+template <int K>
+__device__ __forceinline__ void mt_generate(uint32_t *st, uint32_t &pos, int lane, int nlanes, uint32_t (&w)[K]) {
+  static_assert(K >= 1 && K <= 4, "words per lane");
+  if (lane < nlanes) {
+    uint32_t s = pos + static_cast<uint32_t>(K * lane);
+    if (s >= kMtN) s -= kMtN;
+    uint32_t near_[K + 1], far_[K], slot[K];
+#pragma unroll
+    for (int i = 0; i <= K; ++i) {
+      uint32_t a = s + i;
+      if (a >= kMtN) a -= kMtN;
+      if (i < K) slot[i] = a;
+      near_[i] = st[a];
+    }
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+      uint32_t a = s + i + kMtM;
+      if (a >= kMtN) a -= kMtN;
+      far_[i] = st[a];
+    }
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+      const uint32_t n = mt_twist(near_[i], near_[i + 1], far_[i]);
+      st[slot[i]] = n;
+      w[i] = mt_temper(n);
+    }
+  }
+  pos += static_cast<uint32_t>(K * nlanes);
+  if (pos >= kMtN) pos -= kMtN;
+}
+
+// libstdc++ generate_canonical<double,53>(mt19937): low word first, the 64-bit sum rounded once
+// to double, scaled by 2^-64, clamped below 1.
+__device__ __forceinline__ double canonical_f64(uint32_t lo, uint32_t hi) {
+  const double s = __dadd_rn(static_cast<double>(lo), __dmul_rn(static_cast<double>(hi), 4294967296.0));
+  const double r = s * 0x1p-64;  // exact scaling
+  return r >= 1.0 ? 0x1.fffffffffffffp-1 : r;  // nextafter(1, 0)
+}
+
+// libstdc++ generate_canonical<float,24>(mt19937): one word rounded to float, scaled by 2^-32.
+__device__ __forceinline__ float canonical_f32(uint32_t word) {
+  const float r = static_cast<float>(word) * 0x1p-32f;
+  return r >= 1.0f ? 0x1.fffffep-1f : r;  // nextafterf(1, 0)
+}
+
+// (unsigned int) of a double as x86-64 compiles it: truncate to int64, keep the low 32 bits;
+// out of range and NaN give 0.
+__device__ __forceinline__ uint32_t f64_to_u32_x86(double x) {
+  if (!(x > -9223372036854775808.0 && x < 9223372036854775808.0)) return 0u;
+  return static_cast<uint32_t>(static_cast<uint64_t>(static_cast<long long>(x)));
+}
+
+// One geometric skip: (unsigned) ceil(log(U) / log_p)  (lib/cpu_jitconn_event_matvec.cpp:24).
+__device__ __forceinline__ uint32_t skip_from_words(uint32_t lo, uint32_t hi, double log_p) {
+  const double u = canonical_f64(lo, hi);
+  return f64_to_u32_x86(ceil(log(u) / log_p));
+}
+
+}  // namespace bpl

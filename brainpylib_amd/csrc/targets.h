@@ -30,6 +30,33 @@
   X(csr_matvec_transpose_homo_float)        \
   X(csr_matvec_transpose_homo_double)
 
+#define BPL_JITCONN_TARGETS(X) \
+  X(gpu_event_matvec_prob_homo_v2_float_bool) \
+  X(gpu_event_matvec_prob_homo_v2_float_float) \
+  X(gpu_event_matvec_prob_homo_v2_double_bool) \
+  X(gpu_event_matvec_prob_homo_v2_double_double) \
+  X(gpu_event_matvec_atomic_prob_homo_v2_float_bool) \
+  X(gpu_event_matvec_atomic_prob_homo_v2_float_float) \
+  X(gpu_event_matvec_atomic_prob_homo_v2_double_bool) \
+  X(gpu_event_matvec_atomic_prob_homo_v2_double_double) \
+  X(gpu_matvec_prob_homo_v2_float) \
+  X(gpu_matvec_prob_homo_v2_double) \
+  X(gpu_matvec_atomic_prob_homo_v2_float) \
+  X(gpu_matvec_atomic_prob_homo_v2_double) \
+  X(gpu_event_matvec_prob_uniform_v2_float_bool) \
+  X(gpu_event_matvec_prob_uniform_v2_float_float) \
+  X(gpu_event_matvec_prob_uniform_v2_double_bool) \
+  X(gpu_event_matvec_prob_uniform_v2_double_double) \
+  X(gpu_event_matvec_atomic_prob_uniform_v2_float_bool) \
+  X(gpu_event_matvec_atomic_prob_uniform_v2_float_float) \
+  X(gpu_event_matvec_atomic_prob_uniform_v2_double_bool) \
+  X(gpu_event_matvec_atomic_prob_uniform_v2_double_double) \
+  X(gpu_matvec_prob_uniform_v2_float) \
+  X(gpu_matvec_prob_uniform_v2_double) \
+  X(gpu_matvec_atomic_prob_uniform_v2_float) \
+  X(gpu_matvec_atomic_prob_uniform_v2_double)
+
 #define BPL_ALL_TARGETS(X)  \
   BPL_EVENT_CSR_TARGETS(X)  \
-  BPL_CSR_TARGETS(X)
+  BPL_CSR_TARGETS(X)        \
+  BPL_JITCONN_TARGETS(X)

@@ -1,0 +1,143 @@
+"""Just-in-time-connectivity operators (host side).
+
+Mirrors brainpylib/jitconn_ops.py: same function names, keyword arguments, defaults and checks as
+brainpylib/_src/jitconn_ops/event_matvec.py:36-147 and matvec.py:29-284, lowered to the
+custom-call targets their GPU translations name (event_matvec.py:201-239, matvec.py:338-368).
+
+The matrix ``M`` of shape ``shape`` is never stored: ``transpose`` only swaps the roles of the two
+dimensions before the kernel, ``outdim_parallel`` selects one generator stream per output element
+(True) or per input element with atomic accumulation (False).  Flipping BOTH flags gives the
+exact transpose of the same matrix (the reference's transpose rule, event_matvec.py:263-273).
+"""
+from typing import Optional, Tuple
+
+import numpy as np
+import torch
+
+from . import _lib
+from ._tensors import FLOAT_DTYPES, as_tensor, device_of, to_device
+
+__all__ = [
+  'event_matvec_prob_conn_homo_weight', 'event_matvec_prob_conn_uniform_weight',
+  'matvec_prob_conn_homo_weight', 'matvec_prob_conn_uniform_weight',
+]
+
+
+def _log_p(conn_prob):
+  # event_matvec.py:217
+  return float(np.log((1 - conn_prob) if conn_prob < 1 else 1e-40))
+
+
+def _check_vector(vec, shape, transpose, what):
+  if vec.ndim != 1:
+    raise ValueError(f'{what} should be a 1D vector.')
+  if len(shape) != 2:
+    raise ValueError('shape should be a length-2 tuple.')
+  if transpose:
+    if vec.shape[0] != shape[0]:
+      raise ValueError(f'Shape mismatch, vec ({vec.shape[0]},) @ mat {shape}.')
+  else:
+    if vec.shape[0] != shape[1]:
+      raise ValueError(f'Shape mismatch, mat {shape} @ vec ({vec.shape[0]},).')
+
+
+def _seed(seed):
+  if seed is None:
+    seed = int(np.random.randint(0, int(1e8)))
+  return int(seed)
+
+
+def _type_name(dt):
+  return '_float' if dt == torch.float32 else '_double'
+
+
+def _run(fn_prefix, w_kind, inp, out_dtype, suffix, *, conn_prob, shape, seed, transpose, outdim_parallel, w_a=0.0,
+         w_b=0.0):
+  n_row, n_col = (shape[1], shape[0]) if transpose else (shape[0], shape[1])
+  if not (conn_prob > 0):
+    raise ValueError(f'conn_prob should be in (0, 1], got {conn_prob}.')
+  device = device_of(inp)
+  inp = to_device(inp, device)
+  log_p = _log_p(conn_prob)
+  if w_kind == 'homo':
+    opaque = _lib.build_jitconn_prob_homo_descriptor(n_row, n_col, seed, log_p)
+  elif w_kind == 'uniform':
+    opaque = _lib.build_jitconn_prob_uniform_descriptor(n_row, n_col, seed, log_p, w_a, w_b)
+  else:
+    opaque = _lib.build_jitconn_prob_normal_descriptor(n_row, n_col, seed, log_p, w_a, w_b)
+  name = fn_prefix + ('' if outdim_parallel else '_atomic') + '_prob_' + w_kind + '_v2' + suffix
+  out = torch.empty(n_row, dtype=out_dtype, device=device)
+  _lib.custom_call(name, [inp, out], opaque)
+  return out
+
+
+def _event_types(events):
+  # event_matvec.py:206-214: bool events give the default float type, float events their own
+  if events.dtype == torch.bool:
+    return torch.float32, '_float_bool'
+  if events.dtype not in FLOAT_DTYPES:
+    raise TypeError(f'events should be bool, float32 or float64, got {events.dtype}.')
+  t = _type_name(events.dtype)
+  return events.dtype, t + t
+
+
+def event_matvec_prob_conn_homo_weight(events, weight, *, conn_prob: float, shape: Tuple[int, int],
+                                       seed: Optional[int] = None, transpose: bool = False,
+                                       outdim_parallel: bool = True):
+  """``y = M @ events`` with ``M`` drawn just in time: each entry is ``weight`` with probability
+  ``conn_prob``.  The kernel counts the active synapses per output; the product with ``weight``
+  is applied afterwards, as in the reference."""
+  events = as_tensor(events)
+  _check_vector(events, shape, transpose, 'events')
+  out_dtype, suffix = _event_types(events)
+  r = _run('gpu_event_matvec', 'homo', events, out_dtype, suffix, conn_prob=conn_prob, shape=shape, seed=_seed(seed),
+           transpose=transpose, outdim_parallel=outdim_parallel)
+  weight = as_tensor(weight).to(device=r.device, dtype=r.dtype)
+  return r * weight
+
+
+def event_matvec_prob_conn_uniform_weight(events, *, w_low: float, w_high: float, conn_prob: float,
+                                          shape: Tuple[int, int], seed: Optional[int] = None,
+                                          transpose: bool = False, outdim_parallel: bool = True):
+  """``y = M @ events`` with each connection's weight drawn uniformly from [w_low, w_high)."""
+  events = as_tensor(events)
+  assert w_high > w_low
+  _check_vector(events, shape, transpose, 'events')
+  out_dtype, suffix = _event_types(events)
+  return _run('gpu_event_matvec', 'uniform', events, out_dtype, suffix, conn_prob=conn_prob, shape=shape,
+              seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, w_a=w_low, w_b=w_high)
+
+
+def _dense(vector):
+  vector = as_tensor(vector)
+  if vector.dtype not in FLOAT_DTYPES:
+    raise TypeError(f'vector should be float32 or float64, got {vector.dtype}.')
+  return vector
+
+
+def matvec_prob_conn_homo_weight(vector, weight, *, conn_prob: float, shape: Tuple[int, int],
+                                 seed: Optional[int] = None, transpose: bool = False, outdim_parallel: bool = True,
+                                 version: str = 'v2'):
+  """``y = M @ vector`` with ``M`` drawn just in time with the scalar ``weight`` at each connection."""
+  vector = _dense(vector)
+  _check_vector(vector, shape, transpose, 'vector')
+  assert version in ['v1', 'v2']
+  if version != 'v2':
+    raise _lib.GPUOperatorNotFound('matvec_prob_homo version v1 (superseded Bernoulli-per-entry kernel)')
+  r = _run('gpu_matvec', 'homo', vector, vector.dtype, _type_name(vector.dtype), conn_prob=conn_prob, shape=shape,
+           seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel)
+  weight = as_tensor(weight).to(device=r.device, dtype=r.dtype)
+  return r * weight
+
+
+def matvec_prob_conn_uniform_weight(vector, *, w_low: float, w_high: float, conn_prob: float, shape: Tuple[int, int],
+                                    seed: Optional[int] = None, transpose: bool = False,
+                                    outdim_parallel: bool = True, version: str = 'v2'):
+  """``y = M @ vector`` with each connection's weight drawn uniformly from [w_low, w_high)."""
+  vector = _dense(vector)
+  assert w_high > w_low
+  _check_vector(vector, shape, transpose, 'vector')
+  if version != 'v2':
+    raise _lib.GPUOperatorNotFound('matvec_prob_uniform version v1 (superseded Bernoulli-per-entry kernel)')
+  return _run('gpu_matvec', 'uniform', vector, vector.dtype, _type_name(vector.dtype), conn_prob=conn_prob, shape=shape,
+              seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, w_a=w_low, w_b=w_high)

@@ -191,6 +191,54 @@ BPL_TARGET(csr_matvec_transpose_heter_double);
 BPL_TARGET(csr_matvec_transpose_homo_float);
 BPL_TARGET(csr_matvec_transpose_homo_double);
 
+/* ------------------------------------------------------------------------------------------
+ * jitconn (event) matvec, version 2 kernels: y = M @ x with M regenerated on the fly.
+ *   (lib/gpu_jitconn_event_matvec.cu:432-522, lib/gpu_jitconn_event_matvec_atomic.cu,
+ *    lib/gpu_jitconn_matvec.cu:400-490, lib/gpu_jitconn_matvec_atomic.cu; names
+ *    lib/gpu_ops.cc:107-158)
+ *   buffers = [input, out]
+ *     input  event targets: bool[n_col] (1 byte each) or F[n_col] (truthiness test)
+ *            dense targets: F[n_col]
+ *     out    F[n_row]
+ *   opaque = bpl_jitconn_prob_homo_descriptor (homo) or bpl_jitconn_prob_weight_descriptor
+ *            (uniform: w_a = low, w_b = high; normal: w_a = mean, w_b = stddev)
+ *   Generator contract: stream i is std::mt19937{seed + i} with the libstdc++ distributions, walked
+ *   exactly like the reference CPU kernels (lib/cpu_jitconn_event_matvec.cpp:20-31): output row i
+ *   of a non-atomic target (input column i of an *_atomic_* target) equals what the reference CPU
+ *   target computes for a matrix with that single stream and seed `seed + i`.  The reference's
+ *   own backends disagree with each other on the matrix (one sequential mt19937 on CPU, cuRAND
+ *   XORWOW per row on GPU); this library follows the CPU generator with the GPU's per-stream
+ *   seeding.
+ *   homo targets return counts (event input) or plain sums (dense input); the caller multiplies
+ *   by the weight, as the reference does (brainpylib/_src/jitconn_ops/event_matvec.py:67-68).
+ *   non-atomic ("outdim_parallel"): one stream per output row.  *_atomic_*: one stream per input
+ *   column, accumulated with atomics.
+ * ---------------------------------------------------------------------------------------- */
+BPL_TARGET(gpu_event_matvec_prob_homo_v2_float_bool);
+BPL_TARGET(gpu_event_matvec_prob_homo_v2_float_float);
+BPL_TARGET(gpu_event_matvec_prob_homo_v2_double_bool);
+BPL_TARGET(gpu_event_matvec_prob_homo_v2_double_double);
+BPL_TARGET(gpu_event_matvec_atomic_prob_homo_v2_float_bool);
+BPL_TARGET(gpu_event_matvec_atomic_prob_homo_v2_float_float);
+BPL_TARGET(gpu_event_matvec_atomic_prob_homo_v2_double_bool);
+BPL_TARGET(gpu_event_matvec_atomic_prob_homo_v2_double_double);
+BPL_TARGET(gpu_matvec_prob_homo_v2_float);
+BPL_TARGET(gpu_matvec_prob_homo_v2_double);
+BPL_TARGET(gpu_matvec_atomic_prob_homo_v2_float);
+BPL_TARGET(gpu_matvec_atomic_prob_homo_v2_double);
+BPL_TARGET(gpu_event_matvec_prob_uniform_v2_float_bool);
+BPL_TARGET(gpu_event_matvec_prob_uniform_v2_float_float);
+BPL_TARGET(gpu_event_matvec_prob_uniform_v2_double_bool);
+BPL_TARGET(gpu_event_matvec_prob_uniform_v2_double_double);
+BPL_TARGET(gpu_event_matvec_atomic_prob_uniform_v2_float_bool);
+BPL_TARGET(gpu_event_matvec_atomic_prob_uniform_v2_float_float);
+BPL_TARGET(gpu_event_matvec_atomic_prob_uniform_v2_double_bool);
+BPL_TARGET(gpu_event_matvec_atomic_prob_uniform_v2_double_double);
+BPL_TARGET(gpu_matvec_prob_uniform_v2_float);
+BPL_TARGET(gpu_matvec_prob_uniform_v2_double);
+BPL_TARGET(gpu_matvec_atomic_prob_uniform_v2_float);
+BPL_TARGET(gpu_matvec_atomic_prob_uniform_v2_double);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

@@ -1,0 +1,232 @@
+"""GPU parity of the jitconn operators through the C ABI.
+
+Generator contract: stream i is std::mt19937{seed + i}; output row i of a row-walk target
+(input column i of an *_atomic_* target) is what the reference's CPU kernel computes for that
+single stream.  Checked against (a) golden vectors produced by the reference's compiled CPU
+kernels one stream at a time, (b) the per-stream oracle, (c) exact integer probes that pin the
+generated index sets, (d) full-size properties."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import brainpylib_amd as bpl
+from brainpylib_amd import _lib, synth
+from util import JIT_SHAPES, assert_close, assert_close_reordered
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+KINDS_BUILT = ("homo", "uniform")
+
+
+def kernel_call(inp, *, w_kind, w_a=0.0, w_b=0.0, log_p, seed, n_row, n_col, col_walk, dense, out_dtype=None,
+                device="cuda:0"):
+  """Calls the custom-call target directly (homo returns counts / plain sums)."""
+  t = torch.from_numpy(np.ascontiguousarray(inp)).to(device)
+  if t.dtype == torch.bool:
+    odt = torch.float32 if out_dtype in (None, np.float32, "float32") else torch.float64
+    suffix = ("_float" if odt == torch.float32 else "_double") + "_bool"
+    prefix = "gpu_event_matvec"
+  else:
+    odt = t.dtype
+    tn = "_float" if odt == torch.float32 else "_double"
+    prefix, suffix = ("gpu_matvec", tn) if dense else ("gpu_event_matvec", tn + tn)
+  if w_kind == "homo":
+    opaque = _lib.build_jitconn_prob_homo_descriptor(n_row, n_col, seed, log_p)
+  elif w_kind == "uniform":
+    opaque = _lib.build_jitconn_prob_uniform_descriptor(n_row, n_col, seed, log_p, w_a, w_b)
+  else:
+    opaque = _lib.build_jitconn_prob_normal_descriptor(n_row, n_col, seed, log_p, w_a, w_b)
+  out = torch.full((n_row,), 123.0, dtype=odt, device=device)  # poisoned: every element must be written
+  name = prefix + ("_atomic" if col_walk else "") + "_prob_" + w_kind + "_v2" + suffix
+  _lib.custom_call(name, [t, out], opaque)
+  return out.cpu().numpy()
+
+
+def _golden_cases():
+  z = np.load(os.path.join(GOLD, "jitconn_cpu_reference.npz"))
+  zs = np.load(os.path.join(GOLD, "jitconn_cpu_reference_streams.npz"))
+  n = sum(1 for k in z.files if k.startswith("meta_"))
+  for i in range(n):
+    yield i, z["in_%d" % i], json.loads(str(z["meta_%d" % i])), zs["out_%d" % i]
+
+
+def _abs_bound(oracle, inp, meta):
+  """sum of |addends| per output, for the reordering tolerance"""
+  wmax = 1.0 if meta["w_kind"] == "homo" else max(abs(meta["w_a"]), abs(meta["w_b"]))
+  mag_in = np.abs(inp.astype(np.float64)) if meta["dense"] else (inp != 0).astype(np.float64)
+  s = oracle.jitconn_matvec(mag_in, log_p=oracle.log_p_of(meta["conn_prob"]), seed=meta["seed"], n_row=meta["n_row"],
+                            n_col=meta["n_col"], col_walk=meta["col_walk"], dense=True, per_stream_seed=True)
+  return wmax * s
+
+
+def test_reference_golden_streams(cuda, oracle_mod):
+  n = 0
+  for i, inp, meta, want in _golden_cases():
+    if meta["w_kind"] not in KINDS_BUILT:
+      continue
+    got = kernel_call(inp, w_kind=meta["w_kind"], w_a=meta["w_a"], w_b=meta["w_b"],
+                      log_p=oracle_mod.log_p_of(meta["conn_prob"]), seed=meta["seed"], n_row=meta["n_row"],
+                      n_col=meta["n_col"], col_walk=meta["col_walk"], dense=meta["dense"], out_dtype=meta["out_dtype"])
+    if meta["w_kind"] == "homo" and not meta["dense"]:
+      assert np.array_equal(got.astype(np.float64), want.astype(np.float64)), (i, meta)  # counts: exact
+    else:
+      dt = np.float32 if got.dtype == np.float32 else np.float64
+      assert_close_reordered(got, want, _abs_bound(oracle_mod, inp, meta), dt, what=str(meta))
+    n += 1
+  assert n == 300
+
+
+@pytest.mark.parametrize("shape", JIT_SHAPES + [(64, 64), (3, 70000)])
+@pytest.mark.parametrize("p", [0.01, 0.1, 0.5])
+def test_index_sets_bit_exact_via_integer_probes(cuda, oracle_mod, shape, p):
+  # dense float64 vectors 1, c and c^2 give count, sum and sum of squares of every row's index set,
+  # all exact integers below 2^53: equal to the oracle's bit for bit
+  n_row, n_col = shape
+  lp = oracle_mod.log_p_of(p)
+  c = np.arange(n_col, dtype=np.float64)
+  print("case", shape, p, flush=True)
+  for col_walk in (False, True):
+    for vec in (np.ones(n_col), c, c * c):
+      want = oracle_mod.jitconn_matvec(vec, log_p=lp, seed=1234, n_row=n_row, n_col=n_col, col_walk=col_walk,
+                                       dense=True, per_stream_seed=True)
+      got = kernel_call(vec, w_kind="homo", log_p=lp, seed=1234, n_row=n_row, n_col=n_col, col_walk=col_walk,
+                        dense=True)
+      assert np.array_equal(got, want), (shape, p, col_walk)
+
+
+def test_full_matrix_recovered_by_one_hot_events(cuda, oracle_mod):
+  # every entry of a 100 x 200 implicit matrix, both walks, against the per-stream oracle's index lists
+  n_row, n_col, seed = 100, 200, 77
+  lp = oracle_mod.log_p_of(0.1)
+  M = np.zeros((n_row, n_col))
+  for r in range(n_row):
+    idx, _ = oracle_mod.jitconn_stream_indices(seed + r, lp, n_col)
+    M[r, idx] = 1
+  got = np.zeros((n_row, n_col))
+  for c in range(n_col):
+    ev = np.zeros(n_col, dtype=bool)
+    ev[c] = True
+    got[:, c] = kernel_call(ev, w_kind="homo", log_p=lp, seed=seed, n_row=n_row, n_col=n_col, col_walk=False,
+                            dense=False)
+  assert np.array_equal(got, M)
+  # column walk of the swapped shape generates the transpose of the same matrix
+  gotT = np.zeros((n_col, n_row))
+  for r in range(n_row):
+    ev = np.zeros(n_row, dtype=bool)
+    ev[r] = True
+    gotT[:, r] = kernel_call(ev, w_kind="homo", log_p=lp, seed=seed, n_row=n_col, n_col=n_row, col_walk=True,
+                             dense=False)
+  assert np.array_equal(gotT, M.T)
+  assert M[:, 0].sum() == 0  # index 0 is never connected
+
+
+def test_closed_form_and_edges(cuda, oracle_mod):
+  lp = oracle_mod.log_p_of(1.0)  # every skip is 1: indices 1..n-1
+  v = np.arange(1, 301, dtype=np.float64)
+  out = kernel_call(v, w_kind="homo", log_p=lp, seed=3, n_row=70, n_col=300, col_walk=False, dense=True)
+  assert np.array_equal(out, np.full(70, v[1:].sum()))
+  out = kernel_call(v[:70].copy(), w_kind="homo", log_p=lp, seed=3, n_row=300, n_col=70, col_walk=True, dense=True)
+  want = np.full(300, v[:70].sum())
+  want[0] = 0
+  assert np.array_equal(out, want)
+  # seed + stream wraps modulo 2^32
+  ev = np.random.default_rng(0).random(500) < 0.5
+  lp = oracle_mod.log_p_of(0.05)
+  want = oracle_mod.jitconn_matvec(ev, log_p=lp, seed=2 ** 32 - 3, n_row=10, n_col=500, per_stream_seed=True)
+  got = kernel_call(ev, w_kind="homo", log_p=lp, seed=2 ** 32 - 3, n_row=10, n_col=500, col_walk=False, dense=False)
+  assert np.array_equal(got, want)
+  # silent input, single element, and an invalid log_p that must be refused, not looped on
+  got = kernel_call(np.zeros(500, bool), w_kind="homo", log_p=lp, seed=1, n_row=10, n_col=500, col_walk=True, dense=False)
+  assert not got.any()
+  got = kernel_call(np.ones(1, bool), w_kind="homo", log_p=lp, seed=1, n_row=5, n_col=1, col_walk=False, dense=False)
+  assert not got.any()
+  with pytest.raises(RuntimeError, match="log_p must be finite and negative"):
+    kernel_call(ev, w_kind="homo", log_p=0.0, seed=1, n_row=10, n_col=500, col_walk=False, dense=False)
+
+
+@pytest.mark.parametrize("shape", JIT_SHAPES)
+@pytest.mark.parametrize("outdim_parallel", [True, False])
+def test_wrapper_determinism_and_shape_swap(cuda, shape, outdim_parallel):
+  # brainpylib/_src/jitconn_ops/tests/test_event_matvec.py:63-87
+  rng = np.random.default_rng(1)
+  for transpose in (False, True):
+    ev = rng.random(shape[0] if transpose else shape[1]) < 0.1
+    kw = dict(conn_prob=0.1, seed=1234, outdim_parallel=outdim_parallel)
+    r1 = bpl.event_matvec_prob_conn_homo_weight(ev, 1.5, shape=shape, transpose=transpose, **kw)
+    r2 = bpl.event_matvec_prob_conn_homo_weight(ev, 1.5, shape=shape, transpose=transpose, **kw)
+    r3 = bpl.event_matvec_prob_conn_homo_weight(ev, 1.5, shape=shape[::-1], transpose=not transpose, **kw)
+    assert torch.equal(r1, r2) and torch.equal(r1, r3)
+    assert r1.shape[0] == (shape[1] if transpose else shape[0]) and r1.dtype == torch.float32
+    u1 = bpl.event_matvec_prob_conn_uniform_weight(ev, w_low=-1.0, w_high=1.0, shape=shape, transpose=transpose, **kw)
+    u3 = bpl.event_matvec_prob_conn_uniform_weight(ev, w_low=-1.0, w_high=1.0, shape=shape[::-1],
+                                                   transpose=not transpose, **kw)
+    assert torch.allclose(u1, u3, rtol=1e-5, atol=1e-6)
+    fv = rng.standard_normal(ev.shape[0]).astype(np.float32)
+    m1 = bpl.matvec_prob_conn_homo_weight(fv, 0.5, shape=shape, transpose=transpose, **kw)
+    m3 = bpl.matvec_prob_conn_homo_weight(fv, 0.5, shape=shape[::-1], transpose=not transpose, **kw)
+    assert torch.allclose(m1, m3, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("w_kind,a,b", [("homo", 0.0, 0.0), ("uniform", -1.0, 1.0)])
+def test_row_walk_and_column_walk_are_adjoint(cuda, oracle_mod, w_kind, a, b):
+  # flipping transpose AND outdim_parallel gives M^T of the same M: <y, M x> == <M^T y, x>
+  n_out, n_in = 300, 500
+  rng = np.random.default_rng(5)
+  x = rng.integers(-3, 4, n_in).astype(np.float64)
+  y = rng.integers(-3, 4, n_out).astype(np.float64)
+  lp = oracle_mod.log_p_of(0.2)
+  Mx = kernel_call(x, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=11, n_row=n_out, n_col=n_in, col_walk=False, dense=True)
+  MTy = kernel_call(y, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=11, n_row=n_in, n_col=n_out, col_walk=True, dense=True)
+  assert abs(y @ Mx - MTy @ x) <= 1e-9 * max(1.0, abs(y @ Mx))
+
+
+def test_uniform_weights_against_oracle_streams(cuda, oracle_mod):
+  # one-hot dense input in float64 isolates single weights: they must equal the oracle's draws
+  n_row, n_col, seed = 6, 400, 9
+  lp = oracle_mod.log_p_of(0.05)
+  for dt in (np.float32, np.float64):
+    for r in range(n_row):
+      idx, w = oracle_mod.jitconn_stream_weights(seed + r, "uniform", 0.25, 1.75, lp, n_col, dtype=dt)
+      for k in (0, len(idx) // 2, len(idx) - 1):
+        e = np.zeros(n_col, dtype=dt)
+        e[idx[k]] = 1
+        got = kernel_call(e, w_kind="uniform", w_a=0.25, w_b=1.75, log_p=lp, seed=seed, n_row=n_row, n_col=n_col,
+                          col_walk=False, dense=True)
+        assert got[r] == w[k], (dt, r, k)
+
+
+def test_config_jitconn_event_full_size(cuda, oracle_mod):
+  # 1e6 x 1e6, conn_prob 0.001 (~1e9 implicit synapses), events 1 %, seed 42: all four flag
+  # combinations.  Row walks: 300 sampled rows against single-stream oracle calls.  Column walks:
+  # the whole output against the oracle run over the ~1e4 active columns only.  Plus the adjoint
+  # identity between the two walks on exact integer data.
+  c = synth.config_jitconn_event()
+  n = c["shape"][0]
+  ev = c["events"]
+  lp = oracle_mod.log_p_of(c["conn_prob"])
+  seed = c["seed"]
+  got_row = kernel_call(ev, w_kind="homo", log_p=lp, seed=seed, n_row=n, n_col=n, col_walk=False, dense=False)
+  rows = np.random.default_rng(0).choice(n, 300, replace=False)
+  for r in rows:
+    idx, cnt = oracle_mod.jitconn_stream_indices(seed + int(r), lp, n)
+    assert cnt == idx.shape[0]
+    assert got_row[r] == ev[idx].sum(), r
+  got_col = kernel_call(ev, w_kind="homo", log_p=lp, seed=seed, n_row=n, n_col=n, col_walk=True, dense=False)
+  want_col = np.zeros(n)
+  for col in np.flatnonzero(ev):
+    idx, _ = oracle_mod.jitconn_stream_indices(seed + int(col), lp, n)
+    np.add.at(want_col, idx, 1.0)
+  assert np.array_equal(got_col.astype(np.float64), want_col)
+  # the public wrappers: weight applied afterwards, transpose only swaps the (square) shape
+  w = bpl.event_matvec_prob_conn_homo_weight(ev, c["weight"], conn_prob=c["conn_prob"], shape=c["shape"], seed=seed)
+  assert np.array_equal(w.cpu().numpy(), got_row * np.float32(0.1))
+  wt = bpl.event_matvec_prob_conn_homo_weight(ev, c["weight"], conn_prob=c["conn_prob"], shape=c["shape"], seed=seed,
+                                              transpose=True, outdim_parallel=False)
+  assert np.array_equal(wt.cpu().numpy(), got_col * np.float32(0.1))
+  # adjoint: <y, M x> == <M^T y, x>, counts are exact in fp32 below 2^24
+  y = np.random.default_rng(1).random(n) < 0.01
+  MTy = kernel_call(y, w_kind="homo", log_p=lp, seed=seed, n_row=n, n_col=n, col_walk=True, dense=False)
+  assert float(got_row.astype(np.float64) @ y) == float(MTy.astype(np.float64) @ ev)
