@@ -38,6 +38,14 @@ struct DeviceInfo {
 };
 const DeviceInfo &device_info();
 
+// Scratch device memory for operators that need a staging buffer (the custom-call ABI provides
+// none): one allocation per (device, stream), grown on demand and kept until the process ends.
+// Work enqueued on one stream is ordered, so calls on the same stream can share the buffer;
+// calls on different streams get different buffers.  Returns nullptr (and records an error) if
+// the allocation fails.  Not usable while the stream is being captured into a graph the first
+// time a size is requested (hipMalloc is not capturable).
+void *stream_workspace(hipStream_t stream, size_t bytes);
+
 inline unsigned div_up(unsigned long long a, unsigned long long b) {
   return static_cast<unsigned>((a + b - 1) / b);
 }

@@ -1,0 +1,178 @@
+// jitconn matmat for gfx950:  Y[m,n] = X[m,k] @ M[k,n],  M regenerated on the fly.
+//
+// Column j of M is generator stream std::mt19937{seed + j} walked over the k inputs, the same
+// stream the matvec operators use for output j with transpose=True, so that
+// matmat(X)[i,:] == matvec(X[i,:], transpose=True) -- the identity the reference's tests assert
+// (brainpylib/_src/jitconn_ops/tests/matmat_testcase.py:133-138).
+//
+// The reference kernel (lib/gpu_jitconn_matmat.cu:236-276) gives each thread a few rows of X for
+// one column and reads X[row*k + id] with unrelated ids in neighbouring threads.  Here one
+// wave64 owns a column: X is first transposed into a scratch buffer XT[k][m] (rows padded to a
+// multiple of 64), then for every synapse (id, w) of the column the wave reads the contiguous
+// row XT[id][0..m) and each lane accumulates its own output rows, in stream order, with the same
+// multiply-then-add the CPU path performs.
+//
+// Reference boundary: lib/gpu_jitconn_matmat.cu:279-317,364-455 (buffers = [X, Y], descriptor
+// MatMatJITProbDescriptor1, target names lib/gpu_ops.cc:161-174).
+#include "common.h"
+#include "jitconn_stream.h"
+#include "targets.h"
+
+namespace bpl {
+namespace {
+
+constexpr int kTile = 32;
+
+// XT[c][r] = X[r][c] for r < m (rows of XT have m_pad entries, the padding is zeroed)
+template <typename T>
+__global__ __launch_bounds__(kTile * 8) void transpose_pad_kernel(const T *__restrict__ X, T *__restrict__ XT,
+                                                                  uint32_t m, uint32_t k, uint32_t m_pad) {
+  __shared__ T tile[kTile][kTile + 1];
+  const uint32_t c0 = blockIdx.x * kTile, r0 = blockIdx.y * kTile;
+  const uint32_t tx = threadIdx.x % kTile, ty = threadIdx.x / kTile;  // 32 x 8
+  for (uint32_t i = ty; i < kTile; i += 8) {
+    const uint32_t r = r0 + i, c = c0 + tx;
+    tile[i][tx] = (r < m && c < k) ? X[static_cast<size_t>(r) * k + c] : T(0);
+  }
+  __syncthreads();
+  for (uint32_t i = ty; i < kTile; i += 8) {
+    const uint32_t c = c0 + i, r = r0 + tx;
+    if (c < k && r < m_pad) XT[static_cast<size_t>(c) * m_pad + r] = tile[tx][i];
+  }
+}
+
+__device__ __forceinline__ float read_lane(float v, int l) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+__device__ __forceinline__ double read_lane(double v, int l) {
+  const long long b = __builtin_bit_cast(long long, v);
+  const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(b), l));
+  const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(b >> 32), l));
+  return __builtin_bit_cast(double, (static_cast<long long>(hi) << 32) | lo);
+}
+
+__device__ __forceinline__ float mul_rn(float a, float b) { return __fmul_rn(a, b); }
+__device__ __forceinline__ double mul_rn(double a, double b) { return __dmul_rn(a, b); }
+__device__ __forceinline__ float add_rn(float a, float b) { return __fadd_rn(a, b); }
+__device__ __forceinline__ double add_rn(double a, double b) { return __dadd_rn(a, b); }
+
+// MT = 64-row tiles of Y one wave accumulates (m_pad / 64 per pass of blockIdx.y)
+template <typename T1, int W, int MT>
+__global__ __launch_bounds__(256) void jitconn_matmat_kernel(const T1 *__restrict__ XT, T1 *__restrict__ Y,
+                                                             uint32_t m, uint32_t k, uint32_t n, uint32_t m_pad,
+                                                             uint32_t seed, double log_p, T1 wa, T1 wb) {
+  constexpr int kWaves = 4;
+  constexpr int kWords = StreamLds<T1, W>::words;
+  __shared__ __attribute__((aligned(8))) uint32_t s_state[kWaves * kWords];
+  const int lane = lane_id();
+  const uint32_t wave = threadIdx.x / kWave;
+  uint32_t *st = s_state + wave * kWords;
+  const uint32_t row_base = blockIdx.y * (MT * kWave);  // first row of Y of this pass
+
+  for (uint32_t j = blockIdx.x * kWaves + wave; j < n; j += gridDim.x * kWaves) {
+    T1 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = T1(0);
+    walk_stream<T1, W>(st, lane, seed + j, k, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
+      uint64_t mask = __ballot(valid);
+      constexpr int U = 4;
+      while (mask) {
+        uint32_t id[U];
+        T1 ws[U];
+        T1 x[U][MT];
+        int got = 0;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (mask) {
+            const int s = __ffsll(static_cast<unsigned long long>(mask)) - 1;
+            mask &= mask - 1;
+            ++got;
+            id[u] = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(idx), s));
+            ws[u] = read_lane(w, s);
+          } else {  // pad the group (loaded but not accumulated)
+            id[u] = 0u;
+            ws[u] = T1(0);
+          }
+        }
+        const int group = got;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const T1 *row = XT + static_cast<size_t>(id[u]) * m_pad + row_base + lane;
+#pragma unroll
+          for (int t = 0; t < MT; ++t) x[u][t] = row[t * kWave];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (u < group) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) acc[t] = add_rn(acc[t], mul_rn(ws[u], x[u][t]));
+          }
+        }
+      }
+    });
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const uint32_t r = row_base + t * kWave + lane;
+      if (r < m) Y[static_cast<size_t>(r) * n + j] = acc[t];
+    }
+  }
+}
+
+template <typename T1, int W>
+void matmat_entry(const char *target, hipStream_t stream, void **buffers, const char *opaque, size_t opaque_len) {
+  bpl_matmat_jit_prob_descriptor d;
+  if (!unpack(target, opaque, opaque_len, &d)) return;
+  if (!(d.log_p < 0.0) || std::isinf(d.log_p)) {
+    set_error("%s: log_p must be finite and negative (conn_prob in (0, 1]), got %g", target, d.log_p);
+    return;
+  }
+  if (buffers == nullptr) {
+    set_error("%s: null buffer table", target);
+    return;
+  }
+  const T1 *X = static_cast<const T1 *>(buffers[0]);
+  T1 *Y = static_cast<T1 *>(buffers[1]);
+  const uint32_t m = d.m, k = d.k, n = d.n;
+  if (m == 0 || n == 0) return;
+  // rows of XT are padded to what one pass of the kernel reads: 64, 128 or a multiple of 256
+  uint32_t m_pad = (m + kWave - 1) / kWave * kWave;
+  if (m_pad > 2 * kWave) m_pad = (m + 4 * kWave - 1) / (4 * kWave) * (4 * kWave);
+  if (k == 0) {
+    fill_zero(stream, Y, m * n);  // m * n fits 32 bits whenever Y is addressable by the kernels below
+    check_launch(target);
+    return;
+  }
+  T1 *XT = static_cast<T1 *>(stream_workspace(stream, static_cast<size_t>(k) * m_pad * sizeof(T1)));
+  if (XT == nullptr) return;
+  hipLaunchKernelGGL(transpose_pad_kernel<T1>, dim3(div_up(k, kTile), div_up(m_pad, kTile)), dim3(kTile * 8), 0,
+                     stream, X, XT, m, k, m_pad);
+  const T1 wa = static_cast<T1>(d.w_a), wb = static_cast<T1>(d.w_b);
+  const uint32_t tiles = m_pad / kWave;
+  const unsigned grid_x = div_up(n, 4);
+  if (tiles == 1) {
+    hipLaunchKernelGGL((jitconn_matmat_kernel<T1, W, 1>), dim3(grid_x, 1), dim3(256), 0, stream, XT, Y, m, k, n, m_pad,
+                       d.seed, d.log_p, wa, wb);
+  } else if (tiles == 2) {
+    hipLaunchKernelGGL((jitconn_matmat_kernel<T1, W, 2>), dim3(grid_x, 1), dim3(256), 0, stream, XT, Y, m, k, n, m_pad,
+                       d.seed, d.log_p, wa, wb);
+  } else {
+    hipLaunchKernelGGL((jitconn_matmat_kernel<T1, W, 4>), dim3(grid_x, div_up(tiles, 4)), dim3(256), 0, stream, XT, Y,
+                       m, k, n, m_pad, d.seed, d.log_p, wa, wb);
+  }
+  check_launch(target);
+}
+
+}  // namespace
+}  // namespace bpl
+
+using namespace bpl;
+
+#define BPL_DEFINE(name, T1, W)                                                                    \
+  extern "C" void name(bpl_stream_t stream, void **buffers, const char *opaque, size_t opaque_len) { \
+    matmat_entry<T1, W>(__func__, static_cast<hipStream_t>(stream), buffers, opaque, opaque_len);   \
+  }
+
+BPL_DEFINE(gpu_matmat_prob_prob_normal_float_v1, float, kNormal)
+BPL_DEFINE(gpu_matmat_prob_prob_normal_double_v1, double, kNormal)
+BPL_DEFINE(gpu_matmat_prob_prob_uniform_float_v1, float, kUniform)
+BPL_DEFINE(gpu_matmat_prob_prob_uniform_double_v1, double, kUniform)

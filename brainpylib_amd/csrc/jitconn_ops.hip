@@ -20,79 +20,11 @@
 #include <cmath>
 
 #include "common.h"
-#include "mt_wave.h"
+#include "jitconn_stream.h"
 #include "targets.h"
 
 namespace bpl {
 namespace {
-
-enum : int { kHomo = 0, kUniform = 1, kNormal = 2 };
-enum : int { kInEvent = 0, kInDense = 1 };
-
-// weight draws ----------------------------------------------------------------------------------
-// std::uniform_real_distribution<T>{a,b}: canonical * (b - a) + a, no contraction
-__device__ __forceinline__ float uniform_weight(const uint32_t *w, float a, float b) {
-  return __fadd_rn(__fmul_rn(canonical_f32(w[0]), __fsub_rn(b, a)), a);
-}
-__device__ __forceinline__ double uniform_weight(const uint32_t *w, double a, double b) {
-  return __dadd_rn(__dmul_rn(canonical_f64(w[0], w[1]), __dsub_rn(b, a)), a);
-}
-
-template <typename T1>
-struct WeightWords {
-  static constexpr int value = sizeof(T1) == 4 ? 1 : 2;  // mt19937 words per uniform weight
-};
-
-// Walks stream std::mt19937{stream_seed} over [0, n): calls f(index, weight, valid) once per
-// batch with the whole wave converged; `valid` marks the lanes that hold a synapse of the row.
-template <typename T1, int W, typename F>
-__device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t stream_seed, uint32_t n, double log_p,
-                                            T1 wa, T1 wb, F &&f) {
-  mt_seed(st, stream_seed, lane);
-  uint32_t pos = 0;
-  // With every skip >= 1 a row ends within n/64 + 1 batches; the cap only guards against a
-  // generator state that yields zero skips forever (log_p is validated on the host).
-  const uint32_t max_batches = n / 16u + 1024u;
-  if (W == kHomo) {
-    // stream: K K K ...   synapse s sits at K_0 + ... + K_s
-    uint32_t carry = 0;
-    for (uint32_t b = 0; b < max_batches; ++b) {
-      uint32_t w[2] = {1u, 1u};
-      mt_generate<2>(st, pos, lane, kWave, w);
-      const uint32_t skip = skip_from_words(w[0], w[1], log_p);
-      const uint32_t idx = carry + wave_inclusive_scan_u32(skip);
-      const uint64_t done = __ballot(idx >= n);
-      const int nvalid = done ? (__ffsll(static_cast<unsigned long long>(done)) - 1) : kWave;
-      f(idx, T1(1), lane < nvalid);
-      if (done) break;
-      carry = __builtin_amdgcn_readlane(idx, kWave - 1);
-    }
-  } else if (W == kUniform) {
-    // stream: K  (w K) (w K) ...   synapse s sits at K_0 + ... + K_s, its weight precedes K_{s+1}
-    constexpr int WW = WeightWords<T1>::value;
-    constexpr int K = WW + 2;
-    constexpr int NL = (K == 3) ? 64 : 32;  // K * NL <= 227
-    uint32_t w0[2] = {1u, 1u};
-    mt_generate<2>(st, pos, lane, 1, w0);
-    uint32_t carry = __builtin_amdgcn_readfirstlane(skip_from_words(w0[0], w0[1], log_p));
-    for (uint32_t b = 0; b < max_batches; ++b) {
-      uint32_t w[K];
-#pragma unroll
-      for (int i = 0; i < K; ++i) w[i] = 1u;
-      mt_generate<K>(st, pos, lane, NL, w);
-      const T1 weight = uniform_weight(w, wa, wb);
-      uint32_t skip = skip_from_words(w[WW], w[WW + 1], log_p);
-      if (lane >= NL) skip = 0;
-      const uint32_t incl = wave_inclusive_scan_u32(skip);
-      const uint32_t idx = carry + incl - skip;
-      const uint64_t done = __ballot(lane < NL && idx >= n);
-      const int nvalid = done ? (__ffsll(static_cast<unsigned long long>(done)) - 1) : NL;
-      f(idx, weight, lane < nvalid);
-      if (done) break;
-      carry += __builtin_amdgcn_readlane(incl, kWave - 1);
-    }
-  }
-}
 
 // ---- event probes -------------------------------------------------------------------------------
 template <typename VT>
@@ -111,14 +43,15 @@ template <typename T1, typename VT, int IN, int W, bool LDS_BITS>
 __global__ __launch_bounds__(1024) void jitconn_rowwalk_kernel(const VT *__restrict__ in, T1 *__restrict__ out,
                                                                uint32_t n_out, uint32_t n_in, uint32_t seed,
                                                                double log_p, T1 wa, T1 wb) {
-  extern __shared__ uint32_t smem[];
+  extern __shared__ __attribute__((aligned(8))) uint32_t smem[];
   const int lane = lane_id();
   const uint32_t wave = threadIdx.x / kWave;
   const uint32_t nwaves = blockDim.x / kWave;
-  uint32_t *st = smem + wave * kMtStateWords;
-  const uint32_t *bits = smem + nwaves * kMtStateWords;
+  constexpr int kWords = StreamLds<T1, W>::words;
+  uint32_t *st = smem + wave * kWords;
+  const uint32_t *bits = smem + nwaves * kWords;
   if (LDS_BITS) {
-    uint32_t *wbits = smem + nwaves * kMtStateWords;
+    uint32_t *wbits = smem + nwaves * kWords;
     const uint32_t words = (n_in + 31u) >> 5;
     for (uint32_t i = threadIdx.x; i < words; i += blockDim.x) wbits[i] = pack32<VT>(in, i << 5, n_in);
     __syncthreads();
@@ -160,7 +93,8 @@ __global__ __launch_bounds__(kColThreads) void jitconn_colwalk_kernel(const VT *
                                                                       uint32_t n_in, uint32_t seed, double log_p,
                                                                       T1 wa, T1 wb) {
   constexpr int kWaves = kColThreads / kWave;
-  __shared__ uint32_t s_state[kWaves * kMtStateWords];
+  constexpr int kWords = StreamLds<T1, W>::words;
+  __shared__ __attribute__((aligned(8))) uint32_t s_state[kWaves * kWords];
   __shared__ uint32_t s_col[kColThreads];
   __shared__ T1 s_val[kColThreads];
   __shared__ uint32_t s_wave_cnt[kWaves];
@@ -191,7 +125,7 @@ __global__ __launch_bounds__(kColThreads) void jitconn_colwalk_kernel(const VT *
   }
   __syncthreads();
 
-  uint32_t *st = s_state + wave * kMtStateWords;
+  uint32_t *st = s_state + wave * kWords;
   for (uint32_t k = wave; k < count; k += kWaves) {
     const uint32_t col = s_col[k];
     const T1 val = s_val[k];
@@ -248,7 +182,7 @@ template <typename T1, typename VT, int IN, int W>
 void launch_rowwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, uint32_t n_in, uint32_t seed,
                     double log_p, T1 wa, T1 wb) {
   if (n_out == 0) return;
-  const size_t state_bytes = kMtStateWords * 4;
+  const size_t state_bytes = StreamLds<T1, W>::words * 4;
   const size_t cap = static_cast<size_t>(160) * 1024 - 512;
   if (IN == kInEvent) {
     const size_t bitmap = (static_cast<size_t>(n_in) + 31) / 32 * 4;
@@ -333,3 +267,5 @@ BPL_EVENT_FAMILY(homo, kHomo)
 BPL_EVENT_FAMILY(uniform, kUniform)
 BPL_DENSE_FAMILY(homo, kHomo)
 BPL_DENSE_FAMILY(uniform, kUniform)
+BPL_EVENT_FAMILY(normal, kNormal)
+BPL_DENSE_FAMILY(normal, kNormal)

@@ -1,0 +1,227 @@
+// Generator-stream walker shared by the jitconn kernels: one wave64 walks one std::mt19937
+// stream (mt_wave.h) and hands the synapses it finds, 64 lanes at a time, to a callback.
+#pragma once
+
+#include <cmath>
+
+#include "common.h"
+#include "mt_wave.h"
+
+namespace bpl {
+
+enum : int { kHomo = 0, kUniform = 1, kNormal = 2 };
+enum : int { kInEvent = 0, kInDense = 1 };
+
+// weight draws ----------------------------------------------------------------------------------
+// std::uniform_real_distribution<T>{a,b}: canonical * (b - a) + a, no contraction
+__device__ __forceinline__ float uniform_weight(const uint32_t *w, float a, float b) {
+  return __fadd_rn(__fmul_rn(canonical_f32(w[0]), __fsub_rn(b, a)), a);
+}
+__device__ __forceinline__ double uniform_weight(const uint32_t *w, double a, double b) {
+  return __dadd_rn(__dmul_rn(canonical_f64(w[0], w[1]), __dsub_rn(b, a)), a);
+}
+
+template <typename T1>
+struct WeightWords {
+  static constexpr int value = sizeof(T1) == 4 ? 1 : 2;  // mt19937 words per uniform weight
+};
+
+// LDS words one wave needs: the generator state, plus (double-precision normal weights only) a
+// 128-word staging buffer for the batch and 64 (index, weight) slots for the serial parser.
+template <typename T1, int W>
+struct StreamLds {
+  static constexpr bool serial = (W == kNormal && sizeof(T1) == 8);
+  static constexpr int words = serial ? (kMtStateWords + 128 + 64 + 128) : kMtStateWords;
+};
+
+// std::normal_distribution<float> (libstdc++, Marsaglia polar): candidate pair from two words
+struct PolarF32 {
+  float x, y, r2;
+  bool ok;
+};
+__device__ __forceinline__ PolarF32 polar_attempt(uint32_t w0, uint32_t w1) {
+  PolarF32 a;
+  a.x = __fsub_rn(__fmul_rn(2.0f, canonical_f32(w0)), 1.0f);
+  a.y = __fsub_rn(__fmul_rn(2.0f, canonical_f32(w1)), 1.0f);
+  a.r2 = __fadd_rn(__fmul_rn(a.x, a.x), __fmul_rn(a.y, a.y));
+  a.ok = !(a.r2 > 1.0f || a.r2 == 0.0f);
+  return a;
+}
+
+// Walks stream std::mt19937{stream_seed} over [0, n): calls f(index, weight, valid) once per
+// batch with the whole wave converged; `valid` marks the lanes that hold a synapse of the row.
+template <typename T1, int W, typename F>
+__device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t stream_seed, uint32_t n, double log_p,
+                                            T1 wa, T1 wb, F &&f) {
+  mt_seed(st, stream_seed, lane);
+  uint32_t pos = 0;
+  // With every skip >= 1 a row ends within n/64 + 1 batches; the cap only guards against a
+  // generator state that yields zero skips forever (log_p is validated on the host).
+  const uint32_t max_batches = n / 16u + 1024u;
+  if constexpr (W == kHomo) {
+    // stream: K K K ...   synapse s sits at K_0 + ... + K_s
+    uint32_t carry = 0;
+    for (uint32_t b = 0; b < max_batches; ++b) {
+      uint32_t w[2] = {1u, 1u};
+      mt_generate<2>(st, pos, lane, kWave, w);
+      const uint32_t skip = skip_from_words(w[0], w[1], log_p);
+      const uint32_t idx = carry + wave_inclusive_scan_u32(skip);
+      const uint64_t done = __ballot(idx >= n);
+      const int nvalid = done ? (__ffsll(static_cast<unsigned long long>(done)) - 1) : kWave;
+      f(idx, T1(1), lane < nvalid);
+      if (done) break;
+      carry = __builtin_amdgcn_readlane(idx, kWave - 1);
+    }
+  } else if constexpr (W == kUniform) {
+    // stream: K  (w K) (w K) ...   synapse s sits at K_0 + ... + K_s, its weight precedes K_{s+1}
+    constexpr int WW = WeightWords<T1>::value;
+    constexpr int K = WW + 2;
+    constexpr int NL = (K == 3) ? 64 : 32;  // K * NL <= 227
+    uint32_t w0[2] = {1u, 1u};
+    mt_generate<2>(st, pos, lane, 1, w0);
+    uint32_t carry = __builtin_amdgcn_readfirstlane(skip_from_words(w0[0], w0[1], log_p));
+    for (uint32_t b = 0; b < max_batches; ++b) {
+      uint32_t w[K];
+#pragma unroll
+      for (int i = 0; i < K; ++i) w[i] = 1u;
+      mt_generate<K>(st, pos, lane, NL, w);
+      const T1 weight = uniform_weight(w, wa, wb);
+      uint32_t skip = skip_from_words(w[WW], w[WW + 1], log_p);
+      if (lane >= NL) skip = 0;
+      const uint32_t incl = wave_inclusive_scan_u32(skip);
+      const uint32_t idx = carry + incl - skip;
+      const uint64_t done = __ballot(lane < NL && idx >= n);
+      const int nvalid = done ? (__ffsll(static_cast<unsigned long long>(done)) - 1) : NL;
+      f(idx, weight, lane < nvalid);
+      if (done) break;
+      carry += __builtin_amdgcn_readlane(incl, kWave - 1);
+    }
+  } else if constexpr (W == kNormal && sizeof(T1) == 4) {
+    // stream in 2-word units: K  (A..A K) (K) (A..A K) (K) ...   A = polar attempt (x word, y word),
+    // the last A of a group is the accepted one; the first K after it belongs to the synapse
+    // that receives y*mult, the second K to the synapse that receives the cached x*mult.
+    // Every lane evaluates its unit both ways; a scalar automaton over the accept mask
+    // assigns the roles.
+    uint32_t w0[2] = {1u, 1u};
+    mt_generate<2>(st, pos, lane, 1, w0);
+    uint32_t carry = __builtin_amdgcn_readfirstlane(skip_from_words(w0[0], w0[1], log_p));
+    int state = 0;  // 0: attempt expected, 1: first skip after an accept, 2: second skip
+    float prev_x62 = 0.f, prev_x63 = 0.f, prev_y63 = 0.f;
+    for (uint32_t b = 0; b < max_batches; ++b) {
+      uint32_t w[2] = {1u, 1u};
+      mt_generate<2>(st, pos, lane, kWave, w);
+      const PolarF32 a = polar_attempt(w[0], w[1]);
+      const uint64_t okm = __ballot(a.ok);
+      uint64_t k1 = 0, k2 = 0;
+      for (int p = 0; p < kWave;) {
+        if (state == 0) {
+          const uint64_t m = okm >> p;
+          if (m == 0) break;  // only rejected attempts remain in this batch
+          p += __ffsll(static_cast<unsigned long long>(m));
+          state = 1;
+        } else if (state == 1) {
+          k1 |= 1ull << p;
+          ++p;
+          state = 2;
+        } else {
+          k2 |= 1ull << p;
+          ++p;
+          state = 0;
+        }
+      }
+      const bool is_k1 = (k1 >> lane) & 1ull;
+      const bool is_k2 = (k2 >> lane) & 1ull;
+      const bool is_k = is_k1 || is_k2;
+      float xw = 0.f, yw = 0.f;
+      if (a.ok) {
+        const float mult = __fsqrt_rn(__fdiv_rn(__fmul_rn(-2.0f, logf(a.r2)), a.r2));
+        xw = __fmul_rn(a.x, mult);
+        yw = __fmul_rn(a.y, mult);
+      }
+      float y_m1 = __shfl_up(yw, 1, kWave);
+      float x_m2 = __shfl_up(xw, 2, kWave);
+      if (lane == 0) y_m1 = prev_y63, x_m2 = prev_x62;
+      if (lane == 1) x_m2 = prev_x63;
+      const float raw = is_k1 ? y_m1 : x_m2;
+      const T1 weight = static_cast<T1>(__fadd_rn(__fmul_rn(raw, static_cast<float>(wb)), static_cast<float>(wa)));
+      const uint32_t skip = is_k ? skip_from_words(w[0], w[1], log_p) : 0u;
+      const uint32_t incl = wave_inclusive_scan_u32(skip);
+      const uint32_t idx = carry + incl - skip;
+      const uint64_t done = __ballot(is_k && idx >= n);
+      const int first = done ? (__ffsll(static_cast<unsigned long long>(done)) - 1) : kWave;
+      f(idx, weight, is_k && lane < first);
+      if (done) break;
+      carry += __builtin_amdgcn_readlane(incl, kWave - 1);
+      prev_x62 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, xw), 62));
+      prev_x63 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, xw), 63));
+      prev_y63 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, yw), 63));
+    }
+  } else {
+    // std::normal_distribution<double>: every draw is one canonical double (2 words).  The wave
+    // generates 64 doubles at a time; lane 0 replays the reference loop over them and leaves the
+    // synapses it finds in LDS slots, which the whole wave then consumes.
+    uint32_t *buf = st + kMtStateWords;                                   // 128 words
+    uint32_t *slot_idx = buf + 128;                                       // 64 indices
+    double *slot_w = reinterpret_cast<double *>(slot_idx + 64);           // 64 weights (8-byte aligned)
+    int state = 0;  // 0: first skip, 1: x expected, 2: y expected, 3: skip expected
+    uint32_t col = 0;
+    double x = 0.0, saved = 0.0;
+    bool has_saved = false;
+    for (uint32_t b = 0; b < max_batches; ++b) {
+      uint32_t w[2] = {1u, 1u};
+      mt_generate<2>(st, pos, lane, kWave, w);
+      buf[2 * lane] = w[0];
+      buf[2 * lane + 1] = w[1];
+      int count = 0, finished = 0;
+      if (lane == 0) {
+        for (int i = 0; i < kWave && !finished; ++i) {
+          const double u = canonical_f64(buf[2 * i], buf[2 * i + 1]);
+          bool emit = false;
+          double wdraw = 0.0;
+          if (state == 0 || state == 3) {
+            const uint32_t skip = f64_to_u32_x86(ceil(log(u) / log_p));
+            col = (state == 0) ? skip : col + skip;
+            if (col >= n) {
+              finished = 1;
+            } else if (has_saved) {  // the next weight costs no draw
+              has_saved = false;
+              wdraw = saved;
+              emit = true;
+              state = 3;
+            } else {
+              state = 1;
+            }
+          } else if (state == 1) {
+            x = __dsub_rn(__dmul_rn(2.0, u), 1.0);
+            state = 2;
+          } else {
+            const double y = __dsub_rn(__dmul_rn(2.0, u), 1.0);
+            const double r2 = __dadd_rn(__dmul_rn(x, x), __dmul_rn(y, y));
+            if (r2 > 1.0 || r2 == 0.0) {
+              state = 1;
+            } else {
+              const double mult = sqrt(-2 * log(r2) / r2);
+              saved = __dmul_rn(x, mult);
+              has_saved = true;
+              wdraw = __dmul_rn(y, mult);
+              emit = true;
+              state = 3;
+            }
+          }
+          if (emit) {
+            slot_idx[count] = col;
+            slot_w[count] = __dadd_rn(__dmul_rn(wdraw, static_cast<double>(wb)), static_cast<double>(wa));
+            ++count;
+          }
+        }
+      }
+      count = __builtin_amdgcn_readfirstlane(count);
+      finished = __builtin_amdgcn_readfirstlane(finished);
+      const bool valid = lane < count;
+      f(valid ? slot_idx[lane] : 0u, valid ? static_cast<T1>(slot_w[lane]) : T1(0), valid);
+      if (finished) break;
+    }
+  }
+}
+
+}  // namespace bpl

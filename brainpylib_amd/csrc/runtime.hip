@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <mutex>
 #include <string>
+#include <vector>
 
 #include "common.h"
 #include "targets.h"
@@ -56,6 +57,45 @@ const DeviceInfo &device_info() {
     known[dev] = true;
   }
   return infos[dev];
+}
+
+void *stream_workspace(hipStream_t stream, size_t bytes) {
+  struct Entry {
+    int dev;
+    hipStream_t stream;
+    void *ptr;
+    size_t bytes;
+  };
+  static std::vector<Entry> entries;
+  static std::mutex mu;
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  std::lock_guard<std::mutex> lock(mu);
+  Entry *e = nullptr;
+  for (auto &x : entries)
+    if (x.dev == dev && x.stream == stream) e = &x;
+  if (e == nullptr) {
+    entries.push_back(Entry{dev, stream, nullptr, 0});
+    e = &entries.back();
+  }
+  if (e->bytes < bytes) {
+    // the old buffer may still be read by work already enqueued on this stream
+    if (e->ptr != nullptr) {
+      (void)hipStreamSynchronize(stream);
+      (void)hipFree(e->ptr);
+      e->ptr = nullptr;
+      e->bytes = 0;
+    }
+    const size_t want = bytes + bytes / 4;
+    if (hipMalloc(&e->ptr, want) != hipSuccess) {
+      (void)hipGetLastError();
+      e->ptr = nullptr;
+      set_error("workspace allocation of %zu bytes failed", want);
+      return nullptr;
+    }
+    e->bytes = want;
+  }
+  return e->ptr;
 }
 
 }  // namespace bpl

@@ -54,9 +54,28 @@
   X(gpu_matvec_prob_uniform_v2_float) \
   X(gpu_matvec_prob_uniform_v2_double) \
   X(gpu_matvec_atomic_prob_uniform_v2_float) \
-  X(gpu_matvec_atomic_prob_uniform_v2_double)
+  X(gpu_matvec_atomic_prob_uniform_v2_double) \
+  X(gpu_event_matvec_prob_normal_v2_float_bool) \
+  X(gpu_event_matvec_prob_normal_v2_float_float) \
+  X(gpu_event_matvec_prob_normal_v2_double_bool) \
+  X(gpu_event_matvec_prob_normal_v2_double_double) \
+  X(gpu_event_matvec_atomic_prob_normal_v2_float_bool) \
+  X(gpu_event_matvec_atomic_prob_normal_v2_float_float) \
+  X(gpu_event_matvec_atomic_prob_normal_v2_double_bool) \
+  X(gpu_event_matvec_atomic_prob_normal_v2_double_double) \
+  X(gpu_matvec_prob_normal_v2_float) \
+  X(gpu_matvec_prob_normal_v2_double) \
+  X(gpu_matvec_atomic_prob_normal_v2_float) \
+  X(gpu_matvec_atomic_prob_normal_v2_double)
+
+#define BPL_MATMAT_TARGETS(X) \
+  X(gpu_matmat_prob_prob_normal_float_v1) \
+  X(gpu_matmat_prob_prob_normal_double_v1) \
+  X(gpu_matmat_prob_prob_uniform_float_v1) \
+  X(gpu_matmat_prob_prob_uniform_double_v1)
 
 #define BPL_ALL_TARGETS(X)  \
   BPL_EVENT_CSR_TARGETS(X)  \
   BPL_CSR_TARGETS(X)        \
-  BPL_JITCONN_TARGETS(X)
+  BPL_JITCONN_TARGETS(X)    \
+  BPL_MATMAT_TARGETS(X)

@@ -19,7 +19,9 @@ from ._tensors import FLOAT_DTYPES, as_tensor, device_of, to_device
 
 __all__ = [
   'event_matvec_prob_conn_homo_weight', 'event_matvec_prob_conn_uniform_weight',
-  'matvec_prob_conn_homo_weight', 'matvec_prob_conn_uniform_weight',
+  'event_matvec_prob_conn_normal_weight',
+  'matvec_prob_conn_homo_weight', 'matvec_prob_conn_uniform_weight', 'matvec_prob_conn_normal_weight',
+  'matmat_prob_conn_uniform_weight', 'matmat_prob_conn_normal_weight',
 ]
 
 
@@ -108,6 +110,17 @@ def event_matvec_prob_conn_uniform_weight(events, *, w_low: float, w_high: float
               seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, w_a=w_low, w_b=w_high)
 
 
+def event_matvec_prob_conn_normal_weight(events, *, w_mu: float, w_sigma: float, conn_prob: float,
+                                         shape: Tuple[int, int], seed: Optional[int] = None,
+                                         transpose: bool = False, outdim_parallel: bool = True):
+  """``y = M @ events`` with each connection's weight drawn from N(w_mu, w_sigma^2)."""
+  events = as_tensor(events)
+  _check_vector(events, shape, transpose, 'events')
+  out_dtype, suffix = _event_types(events)
+  return _run('gpu_event_matvec', 'normal', events, out_dtype, suffix, conn_prob=conn_prob, shape=shape,
+              seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, w_a=w_mu, w_b=w_sigma)
+
+
 def _dense(vector):
   vector = as_tensor(vector)
   if vector.dtype not in FLOAT_DTYPES:
@@ -141,3 +154,58 @@ def matvec_prob_conn_uniform_weight(vector, *, w_low: float, w_high: float, conn
     raise _lib.GPUOperatorNotFound('matvec_prob_uniform version v1 (superseded Bernoulli-per-entry kernel)')
   return _run('gpu_matvec', 'uniform', vector, vector.dtype, _type_name(vector.dtype), conn_prob=conn_prob, shape=shape,
               seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, w_a=w_low, w_b=w_high)
+
+
+def matvec_prob_conn_normal_weight(vector, *, w_mu: float, w_sigma: float, conn_prob: float, shape: Tuple[int, int],
+                                   seed: Optional[int] = None, transpose: bool = False,
+                                   outdim_parallel: bool = True, version: str = 'v2'):
+  """``y = M @ vector`` with each connection's weight drawn from N(w_mu, w_sigma^2)."""
+  vector = _dense(vector)
+  _check_vector(vector, shape, transpose, 'vector')
+  if version != 'v2':
+    raise _lib.GPUOperatorNotFound('matvec_prob_normal version v1 (superseded Bernoulli-per-entry kernel)')
+  return _run('gpu_matvec', 'normal', vector, vector.dtype, _type_name(vector.dtype), conn_prob=conn_prob, shape=shape,
+              seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, w_a=w_mu, w_b=w_sigma)
+
+
+def _matmat(w_kind, matrix, w_a, w_b, conn_prob, shape, seed, version):
+  # checks of brainpylib/_src/jitconn_ops/matmat.py:226-235
+  matrix = as_tensor(matrix)
+  if matrix.ndim != 2:
+    raise ValueError('vector should be a 2D matrix.')
+  if len(shape) != 2:
+    raise ValueError('shape should be a length-2 tuple.')
+  if matrix.shape[1] != shape[0]:
+    raise ValueError(f'Shape mismatch, X {tuple(matrix.shape)} @ M ({shape},).')
+  if seed is None:
+    raise ValueError('Seed cannot be none.')
+  if matrix.dtype not in FLOAT_DTYPES:
+    raise TypeError(f'matrix should be float32 or float64, got {matrix.dtype}.')
+  if version != 'v1':
+    raise _lib.GPUOperatorNotFound(f'matmat_prob_{w_kind} version {version}: only v1 generates the matrix the '
+                                   'matvec operators generate')
+  if not (conn_prob > 0):
+    raise ValueError(f'conn_prob should be in (0, 1], got {conn_prob}.')
+  device = device_of(matrix)
+  matrix = to_device(matrix, device)
+  m, k = matrix.shape
+  n = shape[1]
+  opaque = _lib.build_matmat_jit_prob_descriptor1(m, k, n, int(seed), _log_p(conn_prob), w_a, w_b)
+  out = torch.empty((m, n), dtype=matrix.dtype, device=device)
+  _lib.custom_call('gpu_matmat_prob_prob_' + w_kind + _type_name(matrix.dtype) + '_v1', [matrix, out], opaque)
+  return out
+
+
+def matmat_prob_conn_uniform_weight(matrix, *, w_low: float, w_high: float, conn_prob: float, shape: Tuple[int, int],
+                                    seed: Optional[int] = None, version: str = 'v1'):
+  """``Y = X @ M`` with ``M`` of shape ``shape`` drawn just in time, weights uniform in [w_low, w_high)."""
+  assert w_high > w_low
+  return _matmat('uniform', matrix, w_low, w_high, conn_prob, shape, seed, version)
+
+
+def matmat_prob_conn_normal_weight(matrix, *, w_mu: float, w_sigma: float, conn_prob: float, shape: Tuple[int, int],
+                                   seed: Optional[int] = None, version: str = 'v1'):
+  """``Y = X @ M`` with ``M`` of shape ``shape`` drawn just in time, weights N(w_mu, w_sigma^2).
+
+  ``Y[i, :]`` equals ``matvec_prob_conn_normal_weight(X[i, :], shape=shape, transpose=True)``."""
+  return _matmat('normal', matrix, w_mu, w_sigma, conn_prob, shape, seed, version)

@@ -238,6 +238,34 @@ BPL_TARGET(gpu_matvec_prob_uniform_v2_float);
 BPL_TARGET(gpu_matvec_prob_uniform_v2_double);
 BPL_TARGET(gpu_matvec_atomic_prob_uniform_v2_float);
 BPL_TARGET(gpu_matvec_atomic_prob_uniform_v2_double);
+BPL_TARGET(gpu_event_matvec_prob_normal_v2_float_bool);
+BPL_TARGET(gpu_event_matvec_prob_normal_v2_float_float);
+BPL_TARGET(gpu_event_matvec_prob_normal_v2_double_bool);
+BPL_TARGET(gpu_event_matvec_prob_normal_v2_double_double);
+BPL_TARGET(gpu_event_matvec_atomic_prob_normal_v2_float_bool);
+BPL_TARGET(gpu_event_matvec_atomic_prob_normal_v2_float_float);
+BPL_TARGET(gpu_event_matvec_atomic_prob_normal_v2_double_bool);
+BPL_TARGET(gpu_event_matvec_atomic_prob_normal_v2_double_double);
+BPL_TARGET(gpu_matvec_prob_normal_v2_float);
+BPL_TARGET(gpu_matvec_prob_normal_v2_double);
+BPL_TARGET(gpu_matvec_atomic_prob_normal_v2_float);
+BPL_TARGET(gpu_matvec_atomic_prob_normal_v2_double);
+
+/* ------------------------------------------------------------------------------------------
+ * jitconn matmat: Y[m,n] = X[m,k] @ M[k,n], row-major X and Y, M regenerated on the fly
+ *   (lib/gpu_jitconn_matmat.cu:279-317,364-455; names lib/gpu_ops.cc:161-174)
+ *   buffers = [X (F[m*k]), Y (F[m*n])],  opaque = bpl_matmat_jit_prob_descriptor
+ *   (normal: w_a = mean, w_b = stddev; uniform: w_a = low, w_b = high).
+ *   Column j of M is generator stream seed + j over the k inputs, i.e. row i of Y equals the
+ *   matvec target's result for X[i,:] with n_row = n, n_col = k (the reference tests' identity
+ *   matmat == vmap(matvec(transpose=True)), brainpylib/_src/jitconn_ops/tests/matmat_testcase.py:133-138).
+ *   The reference's experimental _v2/_v3 normal kernels generate a different matrix from _v1
+ *   and from matvec and are not provided.
+ * ---------------------------------------------------------------------------------------- */
+BPL_TARGET(gpu_matmat_prob_prob_normal_float_v1);
+BPL_TARGET(gpu_matmat_prob_prob_normal_double_v1);
+BPL_TARGET(gpu_matmat_prob_prob_uniform_float_v1);
+BPL_TARGET(gpu_matmat_prob_prob_uniform_double_v1);
 
 #ifdef __cplusplus
 } /* extern "C" */

@@ -18,7 +18,7 @@ from util import JIT_SHAPES, assert_close, assert_close_reordered
 
 pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(__file__), "golden")
-KINDS_BUILT = ("homo", "uniform")
+KINDS_BUILT = ("homo", "uniform", "normal")
 
 
 def kernel_call(inp, *, w_kind, w_a=0.0, w_b=0.0, log_p, seed, n_row, n_col, col_walk, dense, out_dtype=None,
@@ -53,13 +53,21 @@ def _golden_cases():
     yield i, z["in_%d" % i], json.loads(str(z["meta_%d" % i])), zs["out_%d" % i]
 
 
-def _abs_bound(oracle, inp, meta):
-  """sum of |addends| per output, for the reordering tolerance"""
-  wmax = 1.0 if meta["w_kind"] == "homo" else max(abs(meta["w_a"]), abs(meta["w_b"]))
+def _abs_bound(oracle, inp, meta, dtype):
+  """sum of |addends| per output element, for the reordering tolerance: rebuilt from the
+  oracle's per-stream (index, weight) lists"""
   mag_in = np.abs(inp.astype(np.float64)) if meta["dense"] else (inp != 0).astype(np.float64)
-  s = oracle.jitconn_matvec(mag_in, log_p=oracle.log_p_of(meta["conn_prob"]), seed=meta["seed"], n_row=meta["n_row"],
-                            n_col=meta["n_col"], col_walk=meta["col_walk"], dense=True, per_stream_seed=True)
-  return wmax * s
+  lp = oracle.log_p_of(meta["conn_prob"])
+  n_outer, n_inner = (meta["n_col"], meta["n_row"]) if meta["col_walk"] else (meta["n_row"], meta["n_col"])
+  bound = np.zeros(meta["n_row"])
+  for s_ in range(n_outer):
+    idx, w = oracle.jitconn_stream_weights(meta["seed"] + s_, meta["w_kind"], meta["w_a"], meta["w_b"], lp, n_inner,
+                                           dtype=dtype)
+    if meta["col_walk"]:
+      np.add.at(bound, idx, np.abs(w.astype(np.float64)) * mag_in[s_])
+    else:
+      bound[s_] = (np.abs(w.astype(np.float64)) * mag_in[idx]).sum()
+  return bound
 
 
 def test_reference_golden_streams(cuda, oracle_mod):
@@ -74,9 +82,9 @@ def test_reference_golden_streams(cuda, oracle_mod):
       assert np.array_equal(got.astype(np.float64), want.astype(np.float64)), (i, meta)  # counts: exact
     else:
       dt = np.float32 if got.dtype == np.float32 else np.float64
-      assert_close_reordered(got, want, _abs_bound(oracle_mod, inp, meta), dt, what=str(meta))
+      assert_close_reordered(got, want, _abs_bound(oracle_mod, inp, meta, dt), dt, what=str(meta))
     n += 1
-  assert n == 300
+  assert n == 450
 
 
 @pytest.mark.parametrize("shape", JIT_SHAPES + [(64, 64), (3, 70000)])
@@ -170,7 +178,7 @@ def test_wrapper_determinism_and_shape_swap(cuda, shape, outdim_parallel):
     assert torch.allclose(m1, m3, rtol=1e-5, atol=1e-5)
 
 
-@pytest.mark.parametrize("w_kind,a,b", [("homo", 0.0, 0.0), ("uniform", -1.0, 1.0)])
+@pytest.mark.parametrize("w_kind,a,b", [("homo", 0.0, 0.0), ("uniform", -1.0, 1.0), ("normal", 0.5, 2.0)])
 def test_row_walk_and_column_walk_are_adjoint(cuda, oracle_mod, w_kind, a, b):
   # flipping transpose AND outdim_parallel gives M^T of the same M: <y, M x> == <M^T y, x>
   n_out, n_in = 300, 500
@@ -183,19 +191,45 @@ def test_row_walk_and_column_walk_are_adjoint(cuda, oracle_mod, w_kind, a, b):
   assert abs(y @ Mx - MTy @ x) <= 1e-9 * max(1.0, abs(y @ Mx))
 
 
-def test_uniform_weights_against_oracle_streams(cuda, oracle_mod):
-  # one-hot dense input in float64 isolates single weights: they must equal the oracle's draws
-  n_row, n_col, seed = 6, 400, 9
+@pytest.mark.parametrize("w_kind,a,b", [("uniform", 0.25, 1.75), ("normal", 0.5, 2.0)])
+def test_single_weights_against_oracle_streams(cuda, oracle_mod, w_kind, a, b):
+  # one-hot dense inputs isolate single weights of a stream.  Uniform weights must equal the
+  # oracle's draws bit for bit; normal weights go through logf/sqrtf (libm on the host, the
+  # device's own on the GPU) and may differ in the last place.
+  n_row, n_col, seed = 4, 3000, 9
   lp = oracle_mod.log_p_of(0.05)
   for dt in (np.float32, np.float64):
     for r in range(n_row):
-      idx, w = oracle_mod.jitconn_stream_weights(seed + r, "uniform", 0.25, 1.75, lp, n_col, dtype=dt)
-      for k in (0, len(idx) // 2, len(idx) - 1):
+      idx, w = oracle_mod.jitconn_stream_weights(seed + r, w_kind, a, b, lp, n_col, dtype=dt)
+      assert len(idx) > 100
+      # all weights of the row at once: W[k] lands in output k of a column walk over one-hot ... use
+      # the row walk with a one-hot per probe for a handful of positions spread over several batches
+      for k in (0, 1, 2, 63, 64, 65, len(idx) // 2, len(idx) - 2, len(idx) - 1):
         e = np.zeros(n_col, dtype=dt)
         e[idx[k]] = 1
-        got = kernel_call(e, w_kind="uniform", w_a=0.25, w_b=1.75, log_p=lp, seed=seed, n_row=n_row, n_col=n_col,
+        got = kernel_call(e, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=seed, n_row=n_row, n_col=n_col,
                           col_walk=False, dense=True)
-        assert got[r] == w[k], (dt, r, k)
+        if w_kind == "uniform":
+          assert got[r] == w[k], (dt, r, k)
+        else:
+          assert abs(got[r] - w[k]) <= 4 * np.finfo(dt).eps * max(1.0, abs(w[k])), (dt, r, k, got[r], w[k])
+
+
+def test_normal_weights_whole_rows(cuda, oracle_mod):
+  # dense float64 probes c and c^2 weighted by the normal draws: compares every (index, weight)
+  # pairing of long rows (many parser batches, both skip roles, batch-boundary carries)
+  n_row, n_col, seed = 64, 20000, 5
+  lp = oracle_mod.log_p_of(0.1)
+  c = np.arange(n_col, dtype=np.float64) / n_col
+  for dt in (np.float32, np.float64):
+    for vec in (np.ones(n_col, dtype=dt), c.astype(dt), (c * c).astype(dt)):
+      want = oracle_mod.jitconn_matvec(vec, w_kind="normal", w_a=0.1, w_b=1.0, log_p=lp, seed=seed, n_row=n_row,
+                                       n_col=n_col, dense=True, per_stream_seed=True)
+      got = kernel_call(vec, w_kind="normal", w_a=0.1, w_b=1.0, log_p=lp, seed=seed, n_row=n_row, n_col=n_col,
+                        col_walk=False, dense=True)
+      meta = dict(dense=True, conn_prob=0.1, col_walk=False, n_row=n_row, n_col=n_col, seed=seed, w_kind="normal",
+                  w_a=0.1, w_b=1.0)
+      assert_close_reordered(got, want, _abs_bound(oracle_mod, vec, meta, dt), dt, what="normal rows")
 
 
 def test_config_jitconn_event_full_size(cuda, oracle_mod):
@@ -230,3 +264,49 @@ def test_config_jitconn_event_full_size(cuda, oracle_mod):
   y = np.random.default_rng(1).random(n) < 0.01
   MTy = kernel_call(y, w_kind="homo", log_p=lp, seed=seed, n_row=n, n_col=n, col_walk=True, dense=False)
   assert float(got_row.astype(np.float64) @ y) == float(MTy.astype(np.float64) @ ev)
+
+
+@pytest.mark.parametrize("m", [1, 5, 8, 15, 33, 64, 70, 130, 300])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_matmat_against_oracle_and_vmapped_matvec(cuda, oracle_mod, m, dtype):
+  # m values of the reference test (matmat_testcase.py:39-44) plus tile boundaries of the kernel
+  k, n, seed, p = 230, 150, 7, 0.2
+  X = np.random.default_rng(m).standard_normal((m, k)).astype(dtype)
+  lp = oracle_mod.log_p_of(p)
+  print("case", m, dtype.__name__, flush=True)
+  # uniform weights: same operations in the same order as the CPU loop -> bit-exact
+  want = oracle_mod.jitconn_matmat(X, w_kind="uniform", w_a=-0.5, w_b=1.5, log_p=lp, seed=seed, n=n)
+  got = bpl.matmat_prob_conn_uniform_weight(X, w_low=-0.5, w_high=1.5, conn_prob=p, shape=(k, n), seed=seed).cpu().numpy()
+  assert got.shape == (m, n) and np.array_equal(got, want)
+  # normal weights: logf/sqrtf of the device vs libm may differ in the last place
+  want = oracle_mod.jitconn_matmat(X, w_kind="normal", w_a=0.0, w_b=0.01, log_p=lp, seed=seed, n=n)
+  got_t = bpl.matmat_prob_conn_normal_weight(X, w_mu=0.0, w_sigma=0.01, conn_prob=p, shape=(k, n), seed=seed)
+  got = got_t.cpu().numpy()
+  mag = oracle_mod.jitconn_matmat(np.abs(X), w_kind="uniform", w_a=0.05, w_b=0.0500001, log_p=lp, seed=seed, n=n)
+  assert_close_reordered(got, want, mag, dtype, what="matmat normal")
+  # the reference tests' identity: matmat(X) == vmap(matvec(transpose=True))(X)
+  for i in range(0, m, max(1, m // 4)):
+    yi = bpl.matvec_prob_conn_normal_weight(X[i], w_mu=0.0, w_sigma=0.01, conn_prob=p, shape=(k, n), seed=seed,
+                                            transpose=True)
+    assert torch.allclose(got_t[i], yi, rtol=1e-5, atol=1e-6)
+
+
+def test_config_jitconn_matmat_full_size(cuda, oracle_mod):
+  # 10,000 x 10,000 implicit matrix, conn_prob 0.1, N(0, 0.01^2) from seed 7, times B[10000, 128]:
+  # out = (B^T @ M)^T in the reference's orientation (X = B^T, m = 128).
+  c = synth.config_jitconn_matmat()
+  X = np.ascontiguousarray(c["B"].T)
+  oracle_mod.set_threads(min(16, len(os.sched_getaffinity(0))))
+  lp = oracle_mod.log_p_of(c["conn_prob"])
+  # the oracle on 16 of the 128 rows of X (each regenerates all 10,000 streams: ~1e7 draws per row)
+  rows = np.arange(0, 128, 8)
+  want = oracle_mod.jitconn_matmat(X[rows], w_kind="normal", w_a=c["w_mu"], w_b=c["w_sigma"], log_p=lp, seed=c["seed"],
+                                   n=c["shape"][1])
+  oracle_mod.set_threads(1)
+  got = bpl.matmat_prob_conn_normal_weight(X, w_mu=c["w_mu"], w_sigma=c["w_sigma"], conn_prob=c["conn_prob"],
+                                           shape=c["shape"], seed=c["seed"]).cpu().numpy()
+  assert got.shape == (128, 10000)
+  # |addends| bound: sum_i |w| |x_i| <= about 0.05 * sum of |x| over the ~1000 connected inputs
+  err = np.abs(got[rows].astype(np.float64) - want)
+  bound = 1e-6 + 1e-5 * np.abs(want) + 4 * np.finfo(np.float32).eps * 0.05 * 1000
+  assert (err <= bound).all(), float(err.max())
