@@ -75,6 +75,9 @@ def main():
   ap.add_argument("--warmup", type=int, default=20)
   ap.add_argument("--skip-extra", action="store_true", help="only the headline workload")
   ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU baseline")
+  ap.add_argument("--pmc", action="store_true",
+                  help="counter-collection mode for rocprofv3 --pmc: three plain copies of 400 MB (the "
+                       "calibration kernel) and three calls of the headline kernel, nothing else")
   args = ap.parse_args()
   if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
     raise SystemExit("bench.py: this build runs on ONE GPU (the operators are single-device, like the "
@@ -112,6 +115,19 @@ def main():
                                   transpose=True)
   got_s = bpl.event_csr_matvec(data, indices, indptr, events, shape=c["shape"], transpose=True).cpu().numpy()
   check(got_s, want_s, "event_csr_matvec scatter 1e8 nnz", mag_s)
+
+  if args.pmc:
+    src = torch.empty(100_000_000, dtype=torch.float32, device=dev).normal_()
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for _ in range(3):
+      dst.copy_(src)  # reads 400,000,000 bytes and writes 400,000,000 bytes
+    torch.cuda.synchronize()
+    for _ in range(3):
+      bpl.event_csr_matvec(data, indices, indptr, events, shape=c["shape"])
+    torch.cuda.synchronize()
+    log("pmc mode done")
+    return
 
   hits = int(c["events"][c["indices"]].sum())                 # synapses whose pre-neuron fired (gather view)
   active = int(c["events"].sum())
@@ -226,6 +242,65 @@ def main():
     extra["csr_matvec_transposed_1e8"] = dict(stats(dur3t), gsop_per_s=nnz3 / (dur3t.mean() * 1e-3) / 1e9,
                                               algorithmic_gb_per_s=bytes3 / (dur3t.mean() * 1e-3) / 1e9)
     log("csr_matvec transposed 1e8: %s" % extra["csr_matvec_transposed_1e8"])
+
+  if not args.skip_extra:
+    del md
+    torch.cuda.empty_cache()
+    # jitconn event matvec: 1e6 x 1e6 implicit matrix, conn_prob 0.001, events 1 %, seed 42
+    j = synth.config_jitconn_event()
+    n = j["shape"][0]
+    ev = torch.from_numpy(j["events"]).to(dev)
+    # number of implicit synapses the generator produces (exact): sum of a homo matvec over ones
+    ones = torch.ones(n, dtype=torch.float64, device=dev)
+    generated = int(bpl.matvec_prob_conn_homo_weight(ones, 1.0, conn_prob=j["conn_prob"], shape=j["shape"],
+                                                     seed=j["seed"]).sum().item())
+    lp = oracle.log_p_of(j["conn_prob"])
+    out_row = bpl.event_matvec_prob_conn_homo_weight(ev, j["weight"], conn_prob=j["conn_prob"], shape=j["shape"],
+                                                     seed=j["seed"]).cpu().numpy()
+    for r in np.random.default_rng(0).choice(n, 64, replace=False):
+      idx, _ = oracle.jitconn_stream_indices(j["seed"] + int(r), lp, n)
+      if out_row[r] != np.float32(j["events"][idx].sum()) * np.float32(0.1):
+        raise SystemExit("parity gate failed for jitconn event matvec row %d" % r)
+    jit = {"generated_synapses": generated}
+    for transpose in (False, True):
+      for odp in (True, False):
+        fn = lambda: bpl.event_matvec_prob_conn_homo_weight(ev, j["weight"], conn_prob=j["conn_prob"], shape=j["shape"],
+                                                            seed=j["seed"], transpose=transpose, outdim_parallel=odp)
+        d, _ = time_calls(fn, max(10, args.steps // 10), 3)
+        key = "transpose=%s,outdim_parallel=%s" % (transpose, odp)
+        jit[key] = dict(stats(d), implicit_gsyn_per_s=generated / (d.mean() * 1e-3) / 1e9)
+    if not args.skip_cpu:
+      # reference CPU algorithm (one sequential mt19937) on the first 4,000 rows of the same matrix
+      rows = 4000
+      t1 = time.perf_counter()
+      oracle.jitconn_matvec(j["events"], log_p=lp, seed=j["seed"], n_row=rows, n_col=n, per_stream_seed=False)
+      t_cpu = time.perf_counter() - t1
+      jit["cpu_port_1core"] = {"implicit_gsyn_per_s": generated * (rows / n) / t_cpu / 1e9,
+                               "sample": "first %d of %d rows, %.2f s" % (rows, n, t_cpu)}
+    extra["jitconn_event_matvec_1e9"] = jit
+    log("jitconn event matvec: %s" % jit)
+
+    # jitconn matmat: 10,000 x 10,000, conn_prob 0.1, N(0, 0.01^2), times B[10000, 128]
+    mm = synth.config_jitconn_matmat()
+    X = torch.from_numpy(np.ascontiguousarray(mm["B"].T)).to(dev)
+    fn = lambda: bpl.matmat_prob_conn_normal_weight(X, w_mu=mm["w_mu"], w_sigma=mm["w_sigma"], conn_prob=mm["conn_prob"],
+                                                    shape=mm["shape"], seed=mm["seed"])
+    got = fn().cpu().numpy()
+    lp = oracle.log_p_of(mm["conn_prob"])
+    t1 = time.perf_counter()
+    want = oracle.jitconn_matmat(mm["B"].T[:2].copy(), w_kind="normal", w_a=mm["w_mu"], w_b=mm["w_sigma"], log_p=lp,
+                                 seed=mm["seed"], n=mm["shape"][1])
+    t_cpu = time.perf_counter() - t1
+    check(got[:2], want, "jitconn matmat rows 0-1", np.full_like(want, 0.05 * 1000, dtype=np.float64))
+    gen_mm = int(bpl.matvec_prob_conn_homo_weight(torch.ones(mm["shape"][0], dtype=torch.float64, device=dev), 1.0,
+                                                  conn_prob=mm["conn_prob"], shape=mm["shape"], seed=mm["seed"],
+                                                  transpose=True).sum().item())
+    d, _ = time_calls(fn, max(10, args.steps // 10), 3)
+    extra["jitconn_matmat_1e4x128"] = dict(stats(d), generated_synapses=gen_mm,
+                                           gfma_per_s=gen_mm * 128 / (d.mean() * 1e-3) / 1e9,
+                                           cpu_port_1core_s_per_call=t_cpu * 64,
+                                           cpu_sample="2 of 128 rows of X, %.2f s" % t_cpu)
+    log("jitconn matmat: %s" % extra["jitconn_matmat_1e4x128"])
 
   result = {
     "metric": "GSOP/s + % HBM roofline, event_csr_matvec 1e8 nnz; jitconn GSOP/s at p=0.001",

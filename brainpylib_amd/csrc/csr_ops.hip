@@ -163,7 +163,12 @@ __device__ __forceinline__ uint32_t pack_events32<uint8_t>(const uint8_t *__rest
   return m;
 }
 
-template <typename F, typename VT, bool HETER, int MODE, bool LDS_BITS, int G>
+// G lanes walk the rows assigned to their group as ONE sequence of steps of U*G nonzeros: the
+// column indices of the next step (which may belong to the group's next row) are requested
+// before the loads that depend on the current step's indices are consumed, so a row change
+// does not drain the pipeline.  Loads are unconditional (out-of-row lanes re-read a valid
+// element and are masked out of the sum); only the `data` fetch of an event hit is predicated.
+template <typename F, typename VT, bool HETER, int MODE, bool LDS_BITS, int G, int U>
 __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const uint32_t *__restrict__ indices,
                                             const uint32_t *__restrict__ indptr, const VT *__restrict__ x,
                                             F *__restrict__ y, uint32_t n_row, const uint32_t *s_bits) {
@@ -171,52 +176,156 @@ __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const ui
   const uint32_t gl = threadIdx.x % G;
   const uint32_t total_groups = gridDim.x * groups_per_block;
   const F w_homo = HETER ? F(0) : data[0];
-  constexpr int U = 4;
 
-  for (uint32_t row = blockIdx.x * groups_per_block + threadIdx.x / G; row < n_row; row += total_groups) {
-    const uint32_t start = indptr[row];
-    const uint32_t end = indptr[row + 1];
-    double acc = 0.0;    // heter / dense
-    uint32_t hits = 0;   // homo event: number of active synapses
-    for (uint32_t j0 = start + gl; j0 < end; j0 += U * G) {
-      uint32_t col[U];
-      bool ok[U];
+  uint32_t row = blockIdx.x * groups_per_block + threadIdx.x / G;
+  if (row >= n_row) return;
+  uint32_t base = indptr[row], end = indptr[row + 1];        // current step: [base, base + U*G) of this row
+  uint32_t nrow_start = 0, nrow_end = 0;                      // bounds of the group's next row
+  if (row + total_groups < n_row) nrow_start = indptr[row + total_groups], nrow_end = indptr[row + total_groups + 1];
+
+  auto load_cols = [&](uint32_t b, uint32_t e, uint32_t (&c)[U]) {
+    const uint32_t safe = e ? e - 1 : 0u;  // any valid element (the matrix has at least one)
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const uint32_t j = j0 + u * G;
-        ok[u] = j < end;
-        col[u] = ok[u] ? indices[j] : 0u;
+    for (int u = 0; u < U; ++u) {
+      const uint32_t j = b + u * G + gl;
+      c[u] = indices[j < e ? j : safe];
+    }
+  };
+
+  uint32_t col[U];
+  load_cols(base, end, col);
+  double acc = 0.0;   // heter / dense
+  uint32_t hits = 0;  // homo event: number of active synapses
+  while (true) {
+    // where the next step is
+    const bool last_of_row = base + U * G >= end;
+    const uint32_t next_row = last_of_row ? row + total_groups : row;
+    const uint32_t next_base = last_of_row ? nrow_start : base + U * G;
+    const uint32_t next_end = last_of_row ? nrow_end : end;
+    const bool more = next_row < n_row;
+
+    // loads that depend on this step's indices
+    F val[U];
+    bool use[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t j = base + u * G + gl;
+      const bool ok = j < end;
+      if (MODE == kEvent) {
+        bool hit;
+        if (LDS_BITS) hit = (s_bits[col[u] >> 5] >> (col[u] & 31u)) & 1u;
+        else hit = is_event(x[col[u]]);
+        hit = hit && ok;
+        use[u] = hit;
+        val[u] = F(0);
+        if (HETER && hit) val[u] = data[j];
+      } else {
+        use[u] = ok;
+        const F d = HETER ? data[ok ? j : (end ? end - 1 : 0u)] : w_homo;
+        // product formed in F, then widened (the reference multiplies two F values)
+        val[u] = static_cast<F>(static_cast<F>(x[col[u]]) * d);
       }
+    }
+    // indices of the next step, and the row bounds one row further ahead
+    uint32_t coln[U];
+    if (more) {
+      load_cols(next_base, next_end, coln);
+      if (last_of_row && next_row + total_groups < n_row)
+        nrow_start = indptr[next_row + total_groups], nrow_end = indptr[next_row + total_groups + 1];
+    }
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const uint32_t j = j0 + u * G;
-        if (MODE == kEvent) {
-          bool hit = false;
-          if (ok[u]) {
-            if (LDS_BITS) hit = (s_bits[col[u] >> 5] >> (col[u] & 31u)) & 1u;
-            else hit = is_event(x[col[u]]);
-          }
-          if (HETER) {
-            if (hit) acc += static_cast<double>(data[j]);
-          } else {
-            hits += hit ? 1u : 0u;
-          }
+    for (int u = 0; u < U; ++u) {
+      if (MODE == kEvent && !HETER) hits += use[u] ? 1u : 0u;
+      else acc += use[u] ? static_cast<double>(val[u]) : 0.0;
+    }
+    if (last_of_row) {
+      if (MODE == kEvent && !HETER) {
+        hits = group_sum<G>(hits);
+        // n additions of the same fp32 value into a float64 accumulator are exact: n * w
+        if (gl == 0) y[row] = static_cast<F>(static_cast<double>(w_homo) * static_cast<double>(hits));
+        hits = 0;
+      } else {
+        acc = group_sum<G>(acc);
+        if (gl == 0) y[row] = static_cast<F>(acc);
+        acc = 0.0;
+      }
+    }
+    if (!more) break;
+    row = next_row, base = next_base, end = next_end;
+#pragma unroll
+    for (int u = 0; u < U; ++u) col[u] = coln[u];
+  }
+}
+
+// Long rows: one wave per row.  Row bounds and base pointers are wave uniform (scalar
+// registers), lanes address their elements as base + small offset, full steps of U*64 nonzeros
+// run without guards and only the last step of a row is predicated.
+template <typename F, typename VT, bool HETER, int MODE, bool LDS_BITS, int U>
+__device__ __forceinline__ void gather_rows_wave(const F *__restrict__ data, const uint32_t *__restrict__ indices,
+                                                 const uint32_t *__restrict__ indptr, const VT *__restrict__ x,
+                                                 F *__restrict__ y, uint32_t n_row, const uint32_t *s_bits) {
+  const uint32_t lane = static_cast<uint32_t>(lane_id());
+  const uint32_t waves_per_block = blockDim.x / kWave;
+  const uint32_t total_waves = gridDim.x * waves_per_block;
+  const F w_homo = HETER ? F(0) : data[0];
+
+  auto step = [&](const uint32_t *ip, const F *dp, uint32_t b, uint32_t len, bool guard, double &acc, uint32_t &hits) {
+    uint32_t col[U];
+    bool ok[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t off = b + u * kWave + lane;
+      ok[u] = !guard || off < len;
+      col[u] = ok[u] ? ip[off] : 0u;
+    }
+    F val[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t off = b + u * kWave + lane;
+      if (MODE == kEvent) {
+        bool hit;
+        if (LDS_BITS) hit = (s_bits[col[u] >> 5] >> (col[u] & 31u)) & 1u;
+        else hit = ok[u] && is_event(x[col[u]]);
+        hit = hit && ok[u];
+        if (HETER) {
+          val[u] = F(0);
+          if (hit) val[u] = dp[off];
         } else {
-          if (ok[u]) {
-            const F d = HETER ? data[j] : w_homo;
-            // product formed in F, then widened (the reference multiplies two F values)
-            acc += static_cast<double>(static_cast<F>(static_cast<F>(x[col[u]]) * d));
-          }
+          hits += hit ? 1u : 0u;
+        }
+      } else {
+        val[u] = F(0);
+        if (ok[u]) {
+          const F d = HETER ? dp[off] : w_homo;
+          // product formed in F, then widened (the reference multiplies two F values)
+          val[u] = static_cast<F>(static_cast<F>(x[col[u]]) * d);
         }
       }
     }
+    if (!(MODE == kEvent && !HETER)) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) acc += static_cast<double>(val[u]);
+    }
+  };
+
+  for (uint32_t row = blockIdx.x * waves_per_block + threadIdx.x / kWave; row < n_row; row += total_waves) {
+    const uint32_t urow = __builtin_amdgcn_readfirstlane(row);
+    const uint32_t start = indptr[urow];
+    const uint32_t len = indptr[urow + 1] - start;
+    const uint32_t *ip = indices + start;
+    const F *dp = data + (HETER ? start : 0u);
+    double acc = 0.0;
+    uint32_t hits = 0;
+    uint32_t b = 0;
+    for (; b + U * kWave <= len; b += U * kWave) step(ip, dp, b, len, false, acc, hits);
+    if (b < len) step(ip, dp, b, len, true, acc, hits);
     if (MODE == kEvent && !HETER) {
-      hits = group_sum<G>(hits);
+      hits = wave_sum(hits);
       // n additions of the same fp32 value into a float64 accumulator are exact: n * w
-      if (gl == 0) y[row] = static_cast<F>(static_cast<double>(w_homo) * static_cast<double>(hits));
+      if (lane == 0) y[urow] = static_cast<F>(static_cast<double>(w_homo) * static_cast<double>(hits));
     } else {
-      acc = group_sum<G>(acc);
-      if (gl == 0) y[row] = static_cast<F>(acc);
+      acc = wave_sum(acc);
+      if (lane == 0) y[urow] = static_cast<F>(acc);
     }
   }
 }
@@ -234,12 +343,18 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
     __syncthreads();
   }
   if (n_row == 0) return;
-  // lanes per row from the mean row length (indptr[n_row] = nnz)
-  const uint32_t mean = indptr[n_row] / n_row;
-  if (mean >= 48) gather_rows<F, VT, HETER, MODE, LDS_BITS, 64>(data, indices, indptr, x, y, n_row, s_bits);
-  else if (mean >= 24) gather_rows<F, VT, HETER, MODE, LDS_BITS, 32>(data, indices, indptr, x, y, n_row, s_bits);
-  else if (mean >= 12) gather_rows<F, VT, HETER, MODE, LDS_BITS, 16>(data, indices, indptr, x, y, n_row, s_bits);
-  else gather_rows<F, VT, HETER, MODE, LDS_BITS, 8>(data, indices, indptr, x, y, n_row, s_bits);
+  const uint32_t nnz = indptr[n_row];
+  if (nnz == 0) {  // nothing to gather (and no valid element to point masked lanes at)
+    for (uint32_t r = blockIdx.x * blockDim.x + threadIdx.x; r < n_row; r += gridDim.x * blockDim.x) y[r] = F(0);
+    return;
+  }
+  // lanes per row from the mean row length
+  const uint32_t mean = nnz / n_row;
+  if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, LDS_BITS, 8>(data, indices, indptr, x, y, n_row, s_bits);
+  else if (mean >= 48) gather_rows_wave<F, VT, HETER, MODE, LDS_BITS, 2>(data, indices, indptr, x, y, n_row, s_bits);
+  else if (mean >= 24) gather_rows<F, VT, HETER, MODE, LDS_BITS, 32, 2>(data, indices, indptr, x, y, n_row, s_bits);
+  else if (mean >= 12) gather_rows<F, VT, HETER, MODE, LDS_BITS, 16, 2>(data, indices, indptr, x, y, n_row, s_bits);
+  else gather_rows<F, VT, HETER, MODE, LDS_BITS, 8, 2>(data, indices, indptr, x, y, n_row, s_bits);
 }
 
 // ------------------------------------------------------------------------------------------------
