@@ -200,8 +200,7 @@ def main():
     sd = {k: torch.from_numpy(v).to(dev) for k, v in s.items() if isinstance(v, np.ndarray)}
     got = bpl.event_csr_matvec(sd["data"], sd["indices"], sd["indptr"], sd["events"], shape=s["shape"], transpose=True)
     want = oracle.event_csr_matvec(s["data"], s["indices"], s["indptr"], s["events"], shape=s["shape"], transpose=True)
-    if not np.array_equal(got.cpu().numpy(), want):
-      raise SystemExit("parity gate failed for the 4,000-neuron configuration")
+    check(got.cpu().numpy(), want, "event_csr_matvec scatter 4,000")
     dur_c1, wall_c1 = time_calls(lambda: bpl.event_csr_matvec(sd["data"], sd["indices"], sd["indptr"], sd["events"],
                                                               shape=s["shape"], transpose=True), args.steps, args.warmup)
     deliv = int(np.diff(s["indptr"])[s["events"]].sum())

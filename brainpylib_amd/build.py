@@ -24,7 +24,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = [
   "--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
   "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-  "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
+  "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-Wno-pass-failed",
 ]
 
 

@@ -121,6 +121,144 @@ __global__ __launch_bounds__(kScatterThreads) void csr_scatter_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
+// scatter, output window in LDS
+// ------------------------------------------------------------------------------------------------
+// Random global atomics retire at about one cache-line request per lane; the same additions made
+// in LDS and written out once, lane-contiguous, need a small fraction of the requests.  When
+// the output vector can be cut into a few windows that fit in LDS, workgroup (g, b) owns row
+// group g and output window b: it compacts the group's active rows, streams their column
+// indices (every window's workgroup reads them; they come from L2 / Infinity Cache after the
+// first), fetches `data` only for the nonzeros that fall into its window, accumulates them with
+// LDS atomics and finally adds the window's nonzero entries to y with contiguous atomics.
+constexpr int kWinThreads = 1024;
+constexpr int kWinMaxRows = 2048;  // rows per workgroup = capacity of the active-row list
+
+template <typename F, typename VT, bool HETER, int MODE>
+__global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
+    const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
+    const VT *__restrict__ x, F *__restrict__ y, uint32_t n_row, uint32_t n_col, uint32_t rows_per_wg,
+    uint32_t win, uint32_t n_win, F *__restrict__ partial) {
+  extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
+  F *window = reinterpret_cast<F *>(smem_raw);
+  F *s_scale = window + win;  // dense mode: x[r] per active row
+  uint32_t *s_start = reinterpret_cast<uint32_t *>(s_scale + (MODE == kDense ? kWinMaxRows : 0));
+  uint32_t *s_len = s_start + kWinMaxRows;
+  __shared__ uint32_t s_count, s_next;
+
+  const uint32_t tid = threadIdx.x;
+  const uint32_t lane = tid % kWave, wave = tid / kWave;
+  constexpr uint32_t kWaves = kWinThreads / kWave;
+  const uint32_t b = blockIdx.x % n_win, g = blockIdx.x / n_win;
+  const uint32_t c0 = b * win;
+  const uint32_t width = (c0 + win <= n_col) ? win : n_col - c0;
+
+  for (uint32_t i = tid; i < width; i += kWinThreads) window[i] = F(0);
+  if (tid == 0) s_count = 0, s_next = kWaves;
+  __syncthreads();
+
+  // active rows of the group (order does not matter)
+  for (uint32_t t0 = 0; t0 < rows_per_wg; t0 += kWinThreads) {
+    const uint32_t r = g * rows_per_wg + t0 + tid;
+    bool on = false;
+    uint32_t start = 0, len = 0;
+    F scale = F(1);
+    if (t0 + tid < rows_per_wg && r < n_row) {
+      if (MODE == kEvent) {
+        on = is_event(x[r]);
+      } else {
+        scale = static_cast<F>(x[r]);
+        on = scale != F(0);  // a zero input adds nothing
+      }
+      if (on) {
+        start = indptr[r];
+        len = indptr[r + 1] - start;
+        on = len != 0;
+      }
+    }
+    const uint64_t mask = __ballot(on);
+    uint32_t base = 0;
+    if (lane == 0 && mask) base = atomicAdd(&s_count, static_cast<uint32_t>(__popcll(mask)));
+    base = __builtin_amdgcn_readfirstlane(base);
+    if (on) {
+      const uint32_t k = base + static_cast<uint32_t>(__popcll(mask & ((1ull << lane) - 1ull)));
+      s_start[k] = start;
+      s_len[k] = len;
+      if (MODE == kDense) s_scale[k] = scale;
+    }
+  }
+  __syncthreads();
+  const uint32_t count = s_count;
+  const F w_homo = HETER ? F(0) : data[0];
+
+  // waves take active rows from a shared counter; full steps of U*64 nonzeros run unguarded
+  constexpr int U = 8;
+  auto step = [&](const uint32_t *ip, const F *dp, uint32_t b0, uint32_t len, F scale, bool guard) {
+    uint32_t rel[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t j = b0 + u * kWave + lane;
+      rel[u] = 0xffffffffu;  // outside every window
+      if (!guard || j < len) rel[u] = ip[j] - c0;
+    }
+    F w[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {  // all data loads of the step first, then the LDS atomics
+      w[u] = w_homo;
+      if (HETER && rel[u] < width) w[u] = dp[b0 + u * kWave + lane];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (rel[u] < width) atomicAdd(&window[rel[u]], (MODE == kDense) ? static_cast<F>(scale * w[u]) : w[u]);
+    }
+  };
+  uint32_t k = wave;
+  while (k < count) {
+    const uint32_t start = s_start[k], len = s_len[k];
+    const F scale = (MODE == kDense) ? s_scale[k] : F(1);
+    const uint32_t *ip = indices + start;
+    const F *dp = data + (HETER ? start : 0u);
+    uint32_t b0 = 0;
+    for (; b0 + U * kWave <= len; b0 += U * kWave) step(ip, dp, b0, len, scale, false);
+    if (b0 < len) step(ip, dp, b0, len, scale, true);
+    uint32_t nk = 0;
+    if (lane == 0) nk = atomicAdd(&s_next, 1u);
+    k = __builtin_amdgcn_readfirstlane(nk);
+  }
+  __syncthreads();
+
+  if (partial != nullptr) {
+    // plain contiguous stores of the whole window into this row group's slice; a second
+    // kernel sums the slices
+    F *dst = partial + static_cast<size_t>(g) * n_col + c0;
+    for (uint32_t i = tid; i < width; i += kWinThreads) dst[i] = window[i];
+  } else {
+    for (uint32_t i = tid; i < width; i += kWinThreads) {
+      const F v = window[i];
+      if (v != F(0)) atomic_add(&y[c0 + i], v);
+    }
+  }
+}
+
+// y[c] = sum over row groups of partial[g][c]
+template <typename F>
+__global__ __launch_bounds__(256) void sum_partials_kernel(const F *__restrict__ partial, F *__restrict__ y,
+                                                           uint32_t n_col, uint32_t groups) {
+  const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+  if (c >= n_col) return;
+  F acc = F(0);
+  uint32_t g = 0;
+  for (; g + 4 <= groups; g += 4) {
+    const F a0 = partial[static_cast<size_t>(g) * n_col + c];
+    const F a1 = partial[static_cast<size_t>(g + 1) * n_col + c];
+    const F a2 = partial[static_cast<size_t>(g + 2) * n_col + c];
+    const F a3 = partial[static_cast<size_t>(g + 3) * n_col + c];
+    acc += (a0 + a1) + (a2 + a3);
+  }
+  for (; g < groups; ++g) acc += partial[static_cast<size_t>(g) * n_col + c];
+  y[c] = acc;
+}
+
+// ------------------------------------------------------------------------------------------------
 // gather
 // ------------------------------------------------------------------------------------------------
 
@@ -128,7 +266,6 @@ __global__ __launch_bounds__(kScatterThreads) void csr_scatter_kernel(
 template <typename VT>
 __device__ __forceinline__ uint32_t pack_events32(const VT *__restrict__ ev, uint32_t base, uint32_t n) {
   uint32_t m = 0;
-#pragma unroll 8
   for (uint32_t b = 0; b < 32; ++b) {
     const uint32_t i = base + b;
     if (i < n && is_event(ev[i])) m |= 1u << b;
@@ -363,8 +500,53 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
 template <typename F, typename VT, bool HETER, int MODE>
 void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, const uint32_t *indptr,
                     const VT *x, F *y, uint32_t n_row, uint32_t n_col) {
+  if (n_col == 0) return;
+  if (n_row == 0) {
+    fill_zero(stream, y, n_col);
+    return;
+  }
+  // Output windows in LDS when at most 4 of them cover the output vector.
+  const size_t list_bytes = kWinMaxRows * (8 + (MODE == kDense ? sizeof(F) : 0));
+  const uint32_t win_cap = static_cast<uint32_t>((static_cast<size_t>(128) * 1024) / sizeof(F));
+  const uint32_t n_win = div_up(n_col, win_cap);
+  if (n_win <= 4) {
+    const uint32_t win = div_up(n_col, n_win);
+    // one workgroup per CU in total, between 64 and kWinMaxRows rows each
+    const unsigned want_groups = static_cast<unsigned>(device_info().num_cu) / n_win;
+    uint32_t rows_per_wg = div_up(n_row, want_groups ? want_groups : 1u);
+    if (rows_per_wg < 64) rows_per_wg = 64;
+    if (rows_per_wg > kWinMaxRows) rows_per_wg = kWinMaxRows;
+    const unsigned groups = div_up(n_row, rows_per_wg);
+    const size_t lds = static_cast<size_t>(win) * sizeof(F) + list_bytes;
+    auto kernel = csr_scatter_window_kernel<F, VT, HETER, MODE>;
+    static thread_local size_t attr_set_for = 0;
+    if (lds > 64 * 1024 && attr_set_for < lds) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(lds)) == hipSuccess)
+        attr_set_for = lds;
+      else
+        (void)hipGetLastError();
+    }
+    if (lds <= 64 * 1024 || attr_set_for >= lds) {
+      // Per-row-group partial outputs in scratch memory, summed by a second kernel (no global
+      // atomics, no zero fill), as long as they stay small; else atomics into the zeroed y.
+      const size_t partial_bytes = static_cast<size_t>(groups) * n_col * sizeof(F);
+      F *partial = nullptr;
+      if (groups > 1 && partial_bytes <= (static_cast<size_t>(64) << 20))
+        partial = static_cast<F *>(stream_workspace(stream, partial_bytes));
+      if (partial == nullptr) {
+        bpl_clear_error();
+        fill_zero(stream, y, n_col);
+      }
+      hipLaunchKernelGGL(kernel, dim3(groups * n_win), dim3(kWinThreads), lds, stream, data, indices, indptr, x, y,
+                         n_row, n_col, rows_per_wg, win, n_win, partial);
+      if (partial != nullptr)
+        hipLaunchKernelGGL(sum_partials_kernel<F>, dim3(div_up(n_col, 256)), dim3(256), 0, stream, partial, y, n_col,
+                           groups);
+      return;
+    }
+  }
   fill_zero(stream, y, n_col);
-  if (n_row == 0) return;
   hipLaunchKernelGGL((csr_scatter_kernel<F, VT, HETER, MODE>), dim3(div_up(n_row, kScatterRows)),
                      dim3(kScatterThreads), 0, stream, data, indices, indptr, x, y, n_row);
 }

@@ -30,7 +30,6 @@ namespace {
 template <typename VT>
 __device__ __forceinline__ uint32_t pack32(const VT *__restrict__ ev, uint32_t base, uint32_t n) {
   uint32_t m = 0;
-#pragma unroll 8
   for (uint32_t b = 0; b < 32; ++b) {
     const uint32_t i = base + b;
     if (i < n && is_event(ev[i])) m |= 1u << b;
