@@ -118,10 +118,10 @@ def build_jitconn_prob_homo_descriptor(n_row, n_col, seed, prob):
                 ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_double(prob))
 
 
-def build_jitconn_prob_uniform_descriptor(n_row, n_col, seed, prob, w_low, w_high):
+def build_jitconn_prob_uniform_descriptor(n_row, n_col, seed, prob, w_min, w_range):
   return _build("bpl_build_jitconn_prob_uniform_descriptor", ctypes.c_uint32(n_row), ctypes.c_uint32(n_col),
-                ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_double(prob), ctypes.c_double(w_low),
-                ctypes.c_double(w_high))
+                ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_double(prob), ctypes.c_double(w_min),
+                ctypes.c_double(w_range))
 
 
 def build_jitconn_prob_normal_descriptor(n_row, n_col, seed, prob, w_mu, w_sigma):

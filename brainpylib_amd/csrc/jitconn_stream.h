@@ -13,12 +13,14 @@ enum : int { kHomo = 0, kUniform = 1, kNormal = 2 };
 enum : int { kInEvent = 0, kInDense = 1 };
 
 // weight draws ----------------------------------------------------------------------------------
-// std::uniform_real_distribution<T>{a,b}: canonical * (b - a) + a, no contraction
-__device__ __forceinline__ float uniform_weight(const uint32_t *w, float a, float b) {
-  return __fadd_rn(__fmul_rn(canonical_f32(w[0]), __fsub_rn(b, a)), a);
+// std::uniform_real_distribution<T>{a,b} computes canonical * (b - a) + a; the descriptor carries
+// a and the range b - a (as the reference's GPU descriptors do, lib/gpu_jitconn_event_matvec.cu:
+// 221-222), so the range is formed by the caller.  No contraction.
+__device__ __forceinline__ float uniform_weight(const uint32_t *w, float a, float range) {
+  return __fadd_rn(__fmul_rn(canonical_f32(w[0]), range), a);
 }
-__device__ __forceinline__ double uniform_weight(const uint32_t *w, double a, double b) {
-  return __dadd_rn(__dmul_rn(canonical_f64(w[0], w[1]), __dsub_rn(b, a)), a);
+__device__ __forceinline__ double uniform_weight(const uint32_t *w, double a, double range) {
+  return __dadd_rn(__dmul_rn(canonical_f64(w[0], w[1]), range), a);
 }
 
 template <typename T1>

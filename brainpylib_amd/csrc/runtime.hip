@@ -168,8 +168,8 @@ static size_t build_weight(uint32_t n_row, uint32_t n_col, uint32_t seed, double
 }
 
 size_t bpl_build_jitconn_prob_uniform_descriptor(uint32_t n_row, uint32_t n_col, uint32_t seed, double log_p,
-                                                 double w_low, double w_high, char *out, size_t cap) {
-  return build_weight(n_row, n_col, seed, log_p, w_low, w_high, out, cap);
+                                                 double w_min, double w_range, char *out, size_t cap) {
+  return build_weight(n_row, n_col, seed, log_p, w_min, w_range, out, cap);
 }
 
 size_t bpl_build_jitconn_prob_normal_descriptor(uint32_t n_row, uint32_t n_col, uint32_t seed, double log_p,

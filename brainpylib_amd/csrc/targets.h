@@ -74,8 +74,16 @@
   X(gpu_matmat_prob_prob_uniform_float_v1) \
   X(gpu_matmat_prob_prob_uniform_double_v1)
 
+#define BPL_NONZERO_TARGETS(X) \
+  X(nonzero_bool) \
+  X(nonzero_int) \
+  X(nonzero_long) \
+  X(nonzero_float) \
+  X(nonzero_double)
+
 #define BPL_ALL_TARGETS(X)  \
   BPL_EVENT_CSR_TARGETS(X)  \
   BPL_CSR_TARGETS(X)        \
   BPL_JITCONN_TARGETS(X)    \
-  BPL_MATMAT_TARGETS(X)
+  BPL_MATMAT_TARGETS(X)     \
+  BPL_NONZERO_TARGETS(X)

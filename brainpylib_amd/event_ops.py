@@ -11,7 +11,7 @@ import torch
 from . import _lib
 from ._tensors import FLOAT_DTYPES, as_tensor, device_of, is_index_dtype, to_device
 
-__all__ = ["event_csr_matvec"]
+__all__ = ["event_csr_matvec", "event_info"]
 
 
 def _type_name(dt):
@@ -81,3 +81,30 @@ def event_csr_matvec(data, indices, indptr, events, *, shape: Tuple[int, int], t
   _lib.custom_call('event_csr_matvec' + data_name + type_name + vec_type,
                    [data, indices, indptr, events, out], opaque)
   return out
+
+
+_NONZERO_SUFFIX = {torch.bool: 'bool', torch.int32: 'int', torch.int64: 'long', torch.float32: 'float',
+                   torch.float64: 'double'}
+
+
+def event_info(events):
+  """Collects the event positions and their number (brainpylib/_src/event_ops/
+  event_info_collection.py:24-45).
+
+  events: 1-D vector (a leading batch dimension is accepted, as the reference's vmap rule
+  produces).  Returns ``(event_ids, event_num)``: int32 positions in increasing order padded with
+  -1 to the length of ``events``, and the count with shape (1,) (or (batch,))."""
+  events = as_tensor(events)
+  if events.ndim not in (1, 2):
+    raise TypeError('Only support 1D boolean vector.')
+  if events.dtype not in _NONZERO_SUFFIX:
+    raise ValueError(f'events should be bool, int32, int64, float32 or float64, got {events.dtype}.')
+  device = device_of(events)
+  events = to_device(events, device)
+  batch = 1 if events.ndim == 1 else events.shape[0]
+  size = events.shape[-1]
+  ids = torch.empty(events.shape, dtype=torch.int32, device=device)
+  num = torch.empty((batch,), dtype=torch.int32, device=device)
+  _lib.custom_call('nonzero_' + _NONZERO_SUFFIX[events.dtype], [events, ids, num],
+                   _lib.build_nonzero_descriptor(size, batch))
+  return ids, num

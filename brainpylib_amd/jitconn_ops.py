@@ -49,6 +49,14 @@ def _seed(seed):
   return int(seed)
 
 
+def _uniform_range(w_low, w_high, dtype):
+  """(w_min, w_range) of the uniform descriptor.  The range is formed in the result type, the
+  way std::uniform_real_distribution<T>{a, b} forms b - a on the reference's CPU path."""
+  np_dt = np.float32 if dtype == torch.float32 else np.float64
+  lo, hi = np_dt(w_low), np_dt(w_high)
+  return float(lo), float(np_dt(hi - lo))
+
+
 def _type_name(dt):
   return '_float' if dt == torch.float32 else '_double'
 
@@ -106,8 +114,9 @@ def event_matvec_prob_conn_uniform_weight(events, *, w_low: float, w_high: float
   assert w_high > w_low
   _check_vector(events, shape, transpose, 'events')
   out_dtype, suffix = _event_types(events)
+  w_min, w_range = _uniform_range(w_low, w_high, out_dtype)
   return _run('gpu_event_matvec', 'uniform', events, out_dtype, suffix, conn_prob=conn_prob, shape=shape,
-              seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, w_a=w_low, w_b=w_high)
+              seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, w_a=w_min, w_b=w_range)
 
 
 def event_matvec_prob_conn_normal_weight(events, *, w_mu: float, w_sigma: float, conn_prob: float,
@@ -152,8 +161,9 @@ def matvec_prob_conn_uniform_weight(vector, *, w_low: float, w_high: float, conn
   _check_vector(vector, shape, transpose, 'vector')
   if version != 'v2':
     raise _lib.GPUOperatorNotFound('matvec_prob_uniform version v1 (superseded Bernoulli-per-entry kernel)')
+  w_min, w_range = _uniform_range(w_low, w_high, vector.dtype)
   return _run('gpu_matvec', 'uniform', vector, vector.dtype, _type_name(vector.dtype), conn_prob=conn_prob, shape=shape,
-              seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, w_a=w_low, w_b=w_high)
+              seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, w_a=w_min, w_b=w_range)
 
 
 def matvec_prob_conn_normal_weight(vector, *, w_mu: float, w_sigma: float, conn_prob: float, shape: Tuple[int, int],
@@ -200,7 +210,9 @@ def matmat_prob_conn_uniform_weight(matrix, *, w_low: float, w_high: float, conn
                                     seed: Optional[int] = None, version: str = 'v1'):
   """``Y = X @ M`` with ``M`` of shape ``shape`` drawn just in time, weights uniform in [w_low, w_high)."""
   assert w_high > w_low
-  return _matmat('uniform', matrix, w_low, w_high, conn_prob, shape, seed, version)
+  dt = as_tensor(matrix).dtype
+  w_min, w_range = _uniform_range(w_low, w_high, dt if dt in FLOAT_DTYPES else torch.float32)
+  return _matmat('uniform', matrix, w_min, w_range, conn_prob, shape, seed, version)
 
 
 def matmat_prob_conn_normal_weight(matrix, *, w_mu: float, w_sigma: float, conn_prob: float, shape: Tuple[int, int],

@@ -76,9 +76,9 @@ typedef struct {
 } bpl_jitconn_prob_homo_descriptor;
 
 /* lib/kernel_helper_descriptor.cuh:62-69 and :98-105 (JITConnProbUniformDescriptor /
- * JITConnProbNormalDescriptor; same layout).  uniform: w_a = w_low, w_b = w_high (the
- * boundaries the CPU path receives, lib/cpu_jitconn_event_matvec.cpp:40-41).
- * normal: w_a = w_mu, w_b = w_sigma. */
+ * JITConnProbNormalDescriptor; same layout).  uniform: w_a = w_min, w_b = w_range = w_high - w_low,
+ * what the reference's GPU translation packs (brainpylib/_src/jitconn_ops/event_matvec.py:360-365);
+ * a weight is canonical * w_range + w_min in the result type.  normal: w_a = w_mu, w_b = w_sigma. */
 typedef struct {
   uint32_t n_row;
   uint32_t n_col;
@@ -112,7 +112,7 @@ size_t bpl_build_nonzero_descriptor(uint32_t event_size, uint32_t batch_size, ch
 size_t bpl_build_jitconn_prob_homo_descriptor(uint32_t n_row, uint32_t n_col, uint32_t seed,
                                               double log_p, char *out, size_t cap);
 size_t bpl_build_jitconn_prob_uniform_descriptor(uint32_t n_row, uint32_t n_col, uint32_t seed,
-                                                 double log_p, double w_low, double w_high,
+                                                 double log_p, double w_min, double w_range,
                                                  char *out, size_t cap);
 size_t bpl_build_jitconn_prob_normal_descriptor(uint32_t n_row, uint32_t n_col, uint32_t seed,
                                                 double log_p, double w_mu, double w_sigma,
@@ -201,7 +201,7 @@ BPL_TARGET(csr_matvec_transpose_homo_double);
  *            dense targets: F[n_col]
  *     out    F[n_row]
  *   opaque = bpl_jitconn_prob_homo_descriptor (homo) or bpl_jitconn_prob_weight_descriptor
- *            (uniform: w_a = low, w_b = high; normal: w_a = mean, w_b = stddev)
+ *            (uniform: w_a = low, w_b = high - low; normal: w_a = mean, w_b = stddev)
  *   Generator contract: stream i is std::mt19937{seed + i} with the libstdc++ distributions, walked
  *   exactly like the reference CPU kernels (lib/cpu_jitconn_event_matvec.cpp:20-31): output row i
  *   of a non-atomic target (input column i of an *_atomic_* target) equals what the reference CPU
@@ -255,7 +255,7 @@ BPL_TARGET(gpu_matvec_atomic_prob_normal_v2_double);
  * jitconn matmat: Y[m,n] = X[m,k] @ M[k,n], row-major X and Y, M regenerated on the fly
  *   (lib/gpu_jitconn_matmat.cu:279-317,364-455; names lib/gpu_ops.cc:161-174)
  *   buffers = [X (F[m*k]), Y (F[m*n])],  opaque = bpl_matmat_jit_prob_descriptor
- *   (normal: w_a = mean, w_b = stddev; uniform: w_a = low, w_b = high).
+ *   (normal: w_a = mean, w_b = stddev; uniform: w_a = low, w_b = high - low).
  *   Column j of M is generator stream seed + j over the k inputs, i.e. row i of Y equals the
  *   matvec target's result for X[i,:] with n_row = n, n_col = k (the reference tests' identity
  *   matmat == vmap(matvec(transpose=True)), brainpylib/_src/jitconn_ops/tests/matmat_testcase.py:133-138).
@@ -266,6 +266,21 @@ BPL_TARGET(gpu_matmat_prob_prob_normal_float_v1);
 BPL_TARGET(gpu_matmat_prob_prob_normal_double_v1);
 BPL_TARGET(gpu_matmat_prob_prob_uniform_float_v1);
 BPL_TARGET(gpu_matmat_prob_prob_uniform_double_v1);
+
+/* ------------------------------------------------------------------------------------------
+ * event_info ("nonzero"): ordered positions of the nonzero events and their number
+ *   (lib/gpu_event_info.cu:48-96; names lib/gpu_ops.cc:64-69)
+ *   buffers = [events T[batch_size][event_size], event_ids int32[batch_size][event_size],
+ *              event_num int32[batch_size]],  opaque = bpl_nonzero_descriptor
+ *   event_ids rows: increasing positions, then -1 (the order of the reference's CPU kernel,
+ *   brainpylib/_src/event_ops/event_info_collection.py:143-155; its GPU kernel leaves the order
+ *   unspecified).  T = bool(1 byte) / int32 / int64 / float / double.  batch_size <= 65535.
+ * ---------------------------------------------------------------------------------------- */
+BPL_TARGET(nonzero_bool);
+BPL_TARGET(nonzero_int);
+BPL_TARGET(nonzero_long);
+BPL_TARGET(nonzero_float);
+BPL_TARGET(nonzero_double);
 
 #ifdef __cplusplus
 } /* extern "C" */

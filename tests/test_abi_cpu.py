@@ -94,3 +94,38 @@ def test_bad_opaque_is_reported_not_thrown(name, capfd):
 def test_unknown_target_fails_loudly():
   with pytest.raises(_lib.GPUOperatorNotFound):
     _lib.target("gpu_no_such_op")
+
+
+def test_gpu_ops_module_matches_reference_interface():
+  # lib/gpu_ops.cc:179-198: registrations() -> {name: PyCapsule("xla._CUSTOM_CALL_TARGET")}, build_* -> bytes
+  from brainpylib_amd import gpu_ops
+  regs = gpu_ops.registrations()
+  assert sorted(regs) == sorted(_lib.target_names())
+  api = ctypes.pythonapi
+  api.PyCapsule_GetName.restype = ctypes.c_char_p
+  api.PyCapsule_GetName.argtypes = [ctypes.py_object]
+  api.PyCapsule_GetPointer.restype = ctypes.c_void_p
+  api.PyCapsule_GetPointer.argtypes = [ctypes.py_object, ctypes.c_char_p]
+  lib = _lib.lib()
+  for name, cap in regs.items():
+    assert api.PyCapsule_GetName(cap) == b"xla._CUSTOM_CALL_TARGET"
+    assert api.PyCapsule_GetPointer(cap, b"xla._CUSTOM_CALL_TARGET") == lib.bpl_find_target(name.encode())
+  assert gpu_ops.build_twouint_onebool_descriptor(3, 4, True) == struct.pack("<IIB3x", 3, 4, 1)
+  assert gpu_ops.build_double_size_descriptor(5, 6) == struct.pack("<II", 5, 6)
+  assert gpu_ops.build_nonzero_descriptor(7, 8) == struct.pack("<II", 7, 8)
+  assert gpu_ops.build_jitconn_prob_homo_descriptor(1, 2, 3, -0.25) == struct.pack("<III4xd", 1, 2, 3, -0.25)
+  assert gpu_ops.build_jitconn_prob_uniform_descriptor(1, 2, 3, -0.25, 0.5, 1.0) == struct.pack(
+    "<III4xddd", 1, 2, 3, -0.25, 0.5, 1.0)
+  assert gpu_ops.build_jitconn_prob_normal_descriptor(1, 2, 3, -0.25, 0.5, 1.5) == struct.pack(
+    "<III4xddd", 1, 2, 3, -0.25, 0.5, 1.5)
+  assert gpu_ops.build_matmat_jit_prob_descriptor1(1, 2, 3, 4, -0.25, 0.5, 1.5) == struct.pack(
+    "<IIIIddd", 1, 2, 3, 4, -0.25, 0.5, 1.5)
+
+
+def test_jax_registration_shim_needs_jax():
+  from brainpylib_amd import jax_register
+  try:
+    import jax  # noqa: F401
+  except ImportError:
+    with pytest.raises(ImportError):
+      jax_register.register()

@@ -1,0 +1,35 @@
+"""GPU parity of event_info (the nonzero_* targets) against the ordered CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import brainpylib_amd as bpl
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [np.bool_, np.int32, np.int64, np.float32, np.float64])
+@pytest.mark.parametrize("size", [1, 63, 64, 1000, 1024, 1025, 100_000, 1_500_000])
+def test_event_info_matches_oracle(cuda, oracle_mod, dtype, size):
+  rng = np.random.default_rng(size)
+  ev = ((rng.random(size) < 0.1) * rng.integers(1, 5, size)).astype(dtype)
+  want_ids, want_num = oracle_mod.event_info(ev)
+  ids, num = bpl.event_info(ev)
+  assert ids.dtype == torch.int32 and num.dtype == torch.int32 and num.shape == (1,)
+  assert np.array_equal(num.cpu().numpy(), want_num)
+  assert np.array_equal(ids.cpu().numpy(), want_ids)
+  # the reference's own check: event_num == sum(events != 0)
+  # (brainpylib/_src/event_ops/tests/test_event_info_collection.py:39-40)
+  assert int(num[0]) == int((ev != 0).sum())
+
+
+def test_event_info_edges_and_batch(cuda, oracle_mod):
+  for ev in (np.zeros(5000, bool), np.ones(5000, bool)):
+    ids, num = bpl.event_info(ev)
+    w_ids, w_num = oracle_mod.event_info(ev)
+    assert np.array_equal(ids.cpu().numpy(), w_ids) and np.array_equal(num.cpu().numpy(), w_num)
+  ev = np.random.default_rng(0).random((7, 3000)) < 0.2
+  ids, num = bpl.event_info(ev)
+  for b in range(7):
+    w_ids, w_num = oracle_mod.event_info(ev[b])
+    assert np.array_equal(ids[b].cpu().numpy(), w_ids) and int(num[b]) == int(w_num[0])

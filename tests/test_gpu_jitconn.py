@@ -36,7 +36,10 @@ def kernel_call(inp, *, w_kind, w_a=0.0, w_b=0.0, log_p, seed, n_row, n_col, col
   if w_kind == "homo":
     opaque = _lib.build_jitconn_prob_homo_descriptor(n_row, n_col, seed, log_p)
   elif w_kind == "uniform":
-    opaque = _lib.build_jitconn_prob_uniform_descriptor(n_row, n_col, seed, log_p, w_a, w_b)
+    # descriptor carries (w_min, w_range); the range is formed in the result type like the CPU path's b - a
+    np_dt = np.float32 if odt == torch.float32 else np.float64
+    opaque = _lib.build_jitconn_prob_uniform_descriptor(n_row, n_col, seed, log_p, float(np_dt(w_a)),
+                                                        float(np_dt(np_dt(w_b) - np_dt(w_a))))
   else:
     opaque = _lib.build_jitconn_prob_normal_descriptor(n_row, n_col, seed, log_p, w_a, w_b)
   out = torch.full((n_row,), 123.0, dtype=odt, device=device)  # poisoned: every element must be written
