@@ -75,9 +75,10 @@ def main():
   ap.add_argument("--warmup", type=int, default=20)
   ap.add_argument("--skip-extra", action="store_true", help="only the headline workload")
   ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU baseline")
-  ap.add_argument("--pmc", action="store_true",
-                  help="counter-collection mode for rocprofv3 --pmc: three plain copies of 400 MB (the "
-                       "calibration kernel) and three calls of the headline kernel, nothing else")
+  ap.add_argument("--pmc", choices=["gather", "jitconn"], default=None,
+                  help="counter-collection mode for rocprofv3 --pmc.  gather: three plain copies of 400 MB "
+                       "(the calibration kernel) and three calls of the headline kernel.  jitconn: three calls "
+                       "of jitconn event matvec (1e6 x 1e6, p=0.001) in both walks.  Nothing else runs.")
   args = ap.parse_args()
   if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
     raise SystemExit("bench.py: this build runs on ONE GPU (the operators are single-device, like the "
@@ -92,6 +93,17 @@ def main():
   dev = torch.device("cuda:0")
   torch.cuda.set_device(dev)
   cores = len(os.sched_getaffinity(0))
+
+  if args.pmc == "jitconn":
+    j = synth.config_jitconn_event()
+    ev = torch.from_numpy(j["events"]).to(dev)
+    for odp in (True, False):
+      for _ in range(3):
+        bpl.event_matvec_prob_conn_homo_weight(ev, j["weight"], conn_prob=j["conn_prob"], shape=j["shape"],
+                                               seed=j["seed"], outdim_parallel=odp)
+    torch.cuda.synchronize()
+    log("pmc mode done")
+    return
 
   # ---------------------------------------------------------------------------------------------
   # headline workload: event_csr_matvec, 100,000 x 100,000, ~1e8 nnz, heterogeneous weights
@@ -116,7 +128,7 @@ def main():
   got_s = bpl.event_csr_matvec(data, indices, indptr, events, shape=c["shape"], transpose=True).cpu().numpy()
   check(got_s, want_s, "event_csr_matvec scatter 1e8 nnz", mag_s)
 
-  if args.pmc:
+  if args.pmc == "gather":
     src = torch.empty(100_000_000, dtype=torch.float32, device=dev).normal_()
     dst = torch.empty_like(src)
     torch.cuda.synchronize()

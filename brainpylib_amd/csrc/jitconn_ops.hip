@@ -185,16 +185,18 @@ void launch_rowwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
   const size_t cap = static_cast<size_t>(160) * 1024 - 512;
   if (IN == kInEvent) {
     const size_t bitmap = (static_cast<size_t>(n_in) + 31) / 32 * 4;
-    // as many waves per workgroup as fit beside the bitmap (at most 16)
-    for (int nwaves = 16; nwaves >= 8; nwaves -= 4) {
-      const size_t lds = bitmap + nwaves * state_bytes;
-      if (lds <= cap) {
-        // small bitmaps: 8-wave workgroups, several per CU
-        const int nw = (bitmap <= 16 * 1024) ? 8 : nwaves;
-        launch_rowwalk_impl<T1, VT, IN, W, true>(stream, in, out, n_out, n_in, seed, log_p, wa, wb, nw,
-                                                 bitmap + nw * state_bytes);
-        return;
+    if (bitmap + 4 * state_bytes <= cap) {
+      // Small bitmaps: 8-wave workgroups, several per CU.  Large ones: one workgroup per CU with
+      // as many waves as fit beside the bitmap (each wave can issue one instruction every four
+      // cycles, so the number of resident waves bounds the VALU utilisation).
+      int nw = 8;
+      if (bitmap > 16 * 1024) {
+        nw = static_cast<int>((cap - bitmap) / state_bytes);
+        if (nw > 16) nw = 16;
       }
+      launch_rowwalk_impl<T1, VT, IN, W, true>(stream, in, out, n_out, n_in, seed, log_p, wa, wb, nw,
+                                               bitmap + nw * state_bytes);
+      return;
     }
   }
   launch_rowwalk_impl<T1, VT, IN, W, false>(stream, in, out, n_out, n_in, seed, log_p, wa, wb, 8, 8 * state_bytes);

@@ -53,8 +53,9 @@ __device__ __forceinline__ PolarF32 polar_attempt(uint32_t w0, uint32_t w1) {
 // Walks stream std::mt19937{stream_seed} over [0, n): calls f(index, weight, valid) once per
 // batch with the whole wave converged; `valid` marks the lanes that hold a synapse of the row.
 template <typename T1, int W, typename F>
-__device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t stream_seed, uint32_t n, double log_p,
+__device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t stream_seed, uint32_t n, double log_p_,
                                             T1 wa, T1 wb, F &&f) {
+  const SkipParams log_p = make_skip_params(log_p_);
   mt_seed(st, stream_seed, lane);
   uint32_t pos = 0;
   // With every skip >= 1 a row ends within n/64 + 1 batches; the cap only guards against a
@@ -146,7 +147,8 @@ __device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t str
       if (lane == 1) x_m2 = prev_x63;
       const float raw = is_k1 ? y_m1 : x_m2;
       const T1 weight = static_cast<T1>(__fadd_rn(__fmul_rn(raw, static_cast<float>(wb)), static_cast<float>(wa)));
-      const uint32_t skip = is_k ? skip_from_words(w[0], w[1], log_p) : 0u;
+      const uint32_t skip_any = skip_from_words(w[0], w[1], log_p);  // wave-converged call
+      const uint32_t skip = is_k ? skip_any : 0u;
       const uint32_t incl = wave_inclusive_scan_u32(skip);
       const uint32_t idx = carry + incl - skip;
       const uint64_t done = __ballot(is_k && idx >= n);
@@ -181,7 +183,7 @@ __device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t str
           bool emit = false;
           double wdraw = 0.0;
           if (state == 0 || state == 3) {
-            const uint32_t skip = f64_to_u32_x86(ceil(log(u) / log_p));
+            const uint32_t skip = f64_to_u32_x86(ceil(log(u) / log_p.log_p));
             col = (state == 0) ? skip : col + skip;
             if (col >= n) {
               finished = 1;

@@ -19,12 +19,12 @@ namespace bpl {
 
 constexpr int kMtN = 624;
 constexpr int kMtM = 397;
-constexpr int kMtStateWords = 640;  // LDS words reserved per wave
+constexpr int kMtStateWords = 624;  // LDS words reserved per wave
 
 __device__ __forceinline__ void mt_seed(uint32_t *st, uint32_t seed, int lane) {
   uint32_t x = __builtin_amdgcn_readfirstlane(seed);
 #pragma unroll 1
-  for (int base = 0; base < kMtStateWords; base += kWave) {
+  for (int base = 0; base < kMtN; base += kWave) {
     uint32_t v = 0;
 #pragma unroll
     for (int i = 0; i < kWave; ++i) {
@@ -100,14 +100,50 @@ __device__ __forceinline__ float canonical_f32(uint32_t word) {
 // (unsigned int) of a double as x86-64 compiles it: truncate to int64, keep the low 32 bits;
 // out of range and NaN give 0.
 __device__ __forceinline__ uint32_t f64_to_u32_x86(double x) {
+  if (x >= 0.0 && x < 4294967296.0) return static_cast<uint32_t>(x);  // the only case seen in practice
   if (!(x > -9223372036854775808.0 && x < 9223372036854775808.0)) return 0u;
   return static_cast<uint32_t>(static_cast<uint64_t>(static_cast<long long>(x)));
 }
 
-// One geometric skip: (unsigned) ceil(log(U) / log_p)  (lib/cpu_jitconn_event_matvec.cpp:24).
-__device__ __forceinline__ uint32_t skip_from_words(uint32_t lo, uint32_t hi, double log_p) {
+// Parameters of the skip computation, derived once per kernel from log_p.
+struct SkipParams {
+  double log_p;      // log(1 - p)
+  double inv_log2;   // ln(2) / log_p: skip = ceil(log2(U) * inv_log2)
+  double guard;      // half-width of the band around integers in which the fast path is not trusted
+};
+
+__device__ __forceinline__ SkipParams make_skip_params(double log_p) {
+  SkipParams sp;
+  sp.log_p = log_p;
+  sp.inv_log2 = 0.6931471805599453094 / log_p;
+  // The fast path takes log2 of the mantissa from the hardware fp32 log (documented to 1 ulp; 4e-7
+  // absolute on log2(U) is assumed here, which also covers rounding the mantissa to fp32), so the
+  // quotient is off by at most 4e-7 * |inv_log2| plus fp64 rounding.
+  sp.guard = 4e-7 * fabs(sp.inv_log2) + 1e-9;
+  return sp;
+}
+
+// One geometric skip: (unsigned) ceil(log(U) / log_p)  (lib/cpu_jitconn_event_matvec.cpp:24),
+// U = canonical double of two generator words.
+//
+// Exact path: fp64 log and IEEE division, as the CPU code.  Fast path: log2(U) = exponent +
+// v_log_f32(mantissa) and one multiply; its result is used only when it is further than
+// `guard` from an integer, i.e. when no rounding of the exact path could land on another
+// ceil().  If any lane of the wave is inside the band, the whole wave takes the exact path
+// (a wave-uniform branch); for conn_prob around 1e-3 that happens in a few per cent of the
+// batches, for very sparse matrices (guard >= 0.5) always.
+__device__ __forceinline__ uint32_t skip_from_words(uint32_t lo, uint32_t hi, const SkipParams &sp) {
   const double u = canonical_f64(lo, hi);
-  return f64_to_u32_x86(ceil(log(u) / log_p));
+  int e;
+  const double m = frexp(u, &e);  // u = m * 2^e, m in [0.5, 1)
+  const double l2 = static_cast<double>(e) + static_cast<double>(__log2f(static_cast<float>(m)));
+  const double q = l2 * sp.inv_log2;
+  const double c = ceil(q);
+  // distance of q to the nearest integer: c - q or q - (c - 1)
+  const double d = fmin(c - q, q - (c - 1.0));
+  const bool risky = !(d > sp.guard) || !(q < 4.0e9);
+  if (__ballot(risky) == 0) return static_cast<uint32_t>(c);
+  return f64_to_u32_x86(ceil(log(u) / sp.log_p));
 }
 
 }  // namespace bpl
