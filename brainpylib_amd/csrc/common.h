@@ -104,6 +104,44 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v) {
   return static_cast<uint32_t>(x);
 }
 
+// Bits [0,32) = events[base + b] != 0, zero beyond n.
+template <typename VT>
+__device__ __forceinline__ uint32_t pack_events32(const VT *__restrict__ ev, uint32_t base, uint32_t n) {
+  uint32_t m = 0;
+  for (uint32_t b = 0; b < 32; ++b) {
+    const uint32_t i = base + b;
+    if (i < n && is_event(ev[i])) m |= 1u << b;
+  }
+  return m;
+}
+
+// 4 nonzero-byte flags of a dword, gathered into the low nibble.
+__device__ __forceinline__ uint32_t nonzero_bytes_nibble(uint32_t v) {
+  const uint32_t nz = (((v & 0x7f7f7f7fu) + 0x7f7f7f7fu) | v) & 0x80808080u;
+  // bit 7,15,23,31 -> bits 24..27 of the product (the partial products never collide)
+  return (((nz >> 7) * 0x01020408u) >> 24) & 0xfu;
+}
+
+template <>
+__device__ __forceinline__ uint32_t pack_events32<uint8_t>(const uint8_t *__restrict__ ev, uint32_t base,
+                                                            uint32_t n) {
+  const uint8_t *p = ev + base;
+  if (base + 32 <= n && (reinterpret_cast<uintptr_t>(p) & 15u) == 0) {
+    const uint4 a = *reinterpret_cast<const uint4 *>(p);
+    const uint4 b = *reinterpret_cast<const uint4 *>(p + 16);
+    return nonzero_bytes_nibble(a.x) | (nonzero_bytes_nibble(a.y) << 4) | (nonzero_bytes_nibble(a.z) << 8) |
+           (nonzero_bytes_nibble(a.w) << 12) | (nonzero_bytes_nibble(b.x) << 16) |
+           (nonzero_bytes_nibble(b.y) << 20) | (nonzero_bytes_nibble(b.z) << 24) |
+           (nonzero_bytes_nibble(b.w) << 28);
+  }
+  uint32_t m = 0;
+  for (uint32_t b = 0; b < 32; ++b) {
+    const uint32_t i = base + b;
+    if (i < n && ev[i] != 0) m |= 1u << b;
+  }
+  return m;
+}
+
 __device__ __forceinline__ void atomic_add(float *p, float v) { unsafeAtomicAdd(p, v); }
 __device__ __forceinline__ void atomic_add(double *p, double v) { unsafeAtomicAdd(p, v); }
 

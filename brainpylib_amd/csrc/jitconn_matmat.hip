@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void jitconn_matmat_kernel(const T1 *__restric
     T1 acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = T1(0);
-    walk_stream<T1, W>(st, lane, seed + j, k, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
+    walk_stream<T1, W>(st, lane, seed + j, nullptr, k, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
       uint64_t mask = __ballot(valid);
       constexpr int U = 4;
       while (mask) {

@@ -26,22 +26,14 @@
 namespace bpl {
 namespace {
 
-// ---- event probes -------------------------------------------------------------------------------
-template <typename VT>
-__device__ __forceinline__ uint32_t pack32(const VT *__restrict__ ev, uint32_t base, uint32_t n) {
-  uint32_t m = 0;
-  for (uint32_t b = 0; b < 32; ++b) {
-    const uint32_t i = base + b;
-    if (i < n && is_event(ev[i])) m |= 1u << b;
-  }
-  return m;
-}
-
 // ---- row walk -------------------------------------------------------------------------------------
 template <typename T1, typename VT, int IN, int W, bool LDS_BITS>
 __global__ __launch_bounds__(1024) void jitconn_rowwalk_kernel(const VT *__restrict__ in, T1 *__restrict__ out,
                                                                uint32_t n_out, uint32_t n_in, uint32_t seed,
-                                                               double log_p, T1 wa, T1 wb) {
+                                                               double log_p, T1 wa, T1 wb, uint32_t first,
+                                                               const uint32_t *__restrict__ states) {
+  // Handles the n_out outputs first .. first + n_out - 1; `states` (optional) holds their
+  // generators' seeded states.
   extern __shared__ __attribute__((aligned(8))) uint32_t smem[];
   const int lane = lane_id();
   const uint32_t wave = threadIdx.x / kWave;
@@ -52,13 +44,15 @@ __global__ __launch_bounds__(1024) void jitconn_rowwalk_kernel(const VT *__restr
   if (LDS_BITS) {
     uint32_t *wbits = smem + nwaves * kWords;
     const uint32_t words = (n_in + 31u) >> 5;
-    for (uint32_t i = threadIdx.x; i < words; i += blockDim.x) wbits[i] = pack32<VT>(in, i << 5, n_in);
+    for (uint32_t i = threadIdx.x; i < words; i += blockDim.x) wbits[i] = pack_events32<VT>(in, i << 5, n_in);
     __syncthreads();
   }
-  for (uint32_t o = blockIdx.x * nwaves + wave; o < n_out; o += gridDim.x * nwaves) {
+  for (uint32_t i = blockIdx.x * nwaves + wave; i < n_out; i += gridDim.x * nwaves) {
+    const uint32_t o = first + i;
+    const uint32_t *pre = states ? states + static_cast<size_t>(i) * kMtN : nullptr;
     double acc = 0.0;
     uint32_t cnt = 0;
-    walk_stream<T1, W>(st, lane, seed + o, n_in, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
+    walk_stream<T1, W>(st, lane, seed + o, pre, n_in, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
       if (IN == kInDense) {
         if (valid) {
           const T1 v = static_cast<T1>(in[idx]);
@@ -128,7 +122,7 @@ __global__ __launch_bounds__(kColThreads) void jitconn_colwalk_kernel(const VT *
   for (uint32_t k = wave; k < count; k += kWaves) {
     const uint32_t col = s_col[k];
     const T1 val = s_val[k];
-    walk_stream<T1, W>(st, lane, seed + col, n_out, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
+    walk_stream<T1, W>(st, lane, seed + col, nullptr, n_out, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
       if (valid) {
         T1 add;
         if (IN == kInDense) add = (W == kHomo) ? val : static_cast<T1>(w * val);
@@ -138,6 +132,39 @@ __global__ __launch_bounds__(kColThreads) void jitconn_colwalk_kernel(const VT *
     });
   }
 }
+
+// ---- seeding ahead ------------------------------------------------------------------------------------
+constexpr int kSeedThreads = 128;
+
+__global__ __launch_bounds__(kSeedThreads) void mt_seed_streams_kernel(uint32_t seed, uint32_t first, uint32_t count,
+                                                                      uint32_t *__restrict__ states) {
+  __shared__ uint32_t s_tile[kSeedThreads / kWave][kWave][kWave + 1];
+  const uint32_t lane = static_cast<uint32_t>(lane_id()), wave = threadIdx.x / kWave;
+  const uint32_t base = (blockIdx.x * (kSeedThreads / kWave) + wave) * kWave;  // first stream of this wave
+  if (base >= count) return;
+  uint32_t (*tile)[kWave + 1] = s_tile[wave];
+  uint32_t x = seed + first + base + lane;  // lane l seeds stream base + l
+  for (uint32_t w0 = 0; w0 < kMtN; w0 += kWave) {
+    const uint32_t nw = (kMtN - w0 < kWave) ? kMtN - w0 : kWave;
+    for (uint32_t i = 0; i < nw; ++i) {
+      tile[i][lane] = x;  // word w0 + i of stream base + lane
+      x = 1812433253u * (x ^ (x >> 30)) + (w0 + i + 1);
+    }
+    // transposed: one contiguous run of words per stream
+    for (uint32_t r = 0; r < kWave && base + r < count; ++r)
+      if (lane < nw) states[static_cast<size_t>(base + r) * kMtN + w0 + lane] = tile[lane][r];
+  }
+}
+
+}  // namespace
+
+void launch_seed_streams(hipStream_t stream, uint32_t seed, uint32_t first, uint32_t count, uint32_t *states) {
+  if (count == 0) return;
+  hipLaunchKernelGGL(mt_seed_streams_kernel, dim3(div_up(count, kSeedThreads)), dim3(kSeedThreads), 0, stream, seed,
+                     first, count, states);
+}
+
+namespace {
 
 // ---- launchers ----------------------------------------------------------------------------------------
 bool valid_log_p(const char *target, double log_p) {
@@ -172,9 +199,21 @@ void launch_rowwalk_impl(hipStream_t stream, const VT *in, T1 *out, uint32_t n_o
     cached = {lds_bytes, block, q};
   }
   const unsigned resident = static_cast<unsigned>(device_info().num_cu) * static_cast<unsigned>(cached.per_cu);
-  const unsigned needed = div_up(n_out, nwaves);
-  const unsigned grid = needed < resident ? needed : resident;
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), lds_bytes, stream, in, out, n_out, n_in, seed, log_p, wa, wb);
+  // Large outputs: the generators are seeded ahead, a chunk of streams at a time, by a kernel that
+  // runs the recurrence on the vector unit; small ones seed in place.
+  uint32_t *states = nullptr;
+  if (n_out >= kSeedAheadMin)
+    states = static_cast<uint32_t *>(stream_workspace(stream, static_cast<size_t>(kSeedChunk) * kMtN * 4));
+  if (states == nullptr) bpl_clear_error();
+  const uint32_t chunk = states ? kSeedChunk : n_out;
+  for (uint32_t first = 0; first < n_out; first += chunk) {
+    const uint32_t count = (n_out - first < chunk) ? n_out - first : chunk;
+    if (states) launch_seed_streams(stream, seed, first, count, states);
+    const unsigned needed = div_up(count, nwaves);
+    const unsigned grid = needed < resident ? needed : resident;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), lds_bytes, stream, in, out, count, n_in, seed, log_p, wa, wb,
+                       first, static_cast<const uint32_t *>(states));
+  }
 }
 
 template <typename T1, typename VT, int IN, int W>

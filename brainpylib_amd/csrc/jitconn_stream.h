@@ -52,11 +52,15 @@ __device__ __forceinline__ PolarF32 polar_attempt(uint32_t w0, uint32_t w1) {
 
 // Walks stream std::mt19937{stream_seed} over [0, n): calls f(index, weight, valid) once per
 // batch with the whole wave converged; `valid` marks the lanes that hold a synapse of the row.
+//
+// `pre` points at the stream's 624 seeded state words when they were prepared by
+// launch_seed_streams(); with nullptr the wave seeds the generator itself on the scalar unit.
 template <typename T1, int W, typename F>
-__device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t stream_seed, uint32_t n, double log_p_,
-                                            T1 wa, T1 wb, F &&f) {
+__device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t stream_seed, const uint32_t *pre,
+                                            uint32_t n, double log_p_, T1 wa, T1 wb, F &&f) {
   const SkipParams log_p = make_skip_params(log_p_);
-  mt_seed(st, stream_seed, lane);
+  if (pre != nullptr) mt_load(st, pre, lane);
+  else mt_seed(st, stream_seed, lane);
   uint32_t pos = 0;
   // With every skip >= 1 a row ends within n/64 + 1 batches; the cap only guards against a
   // generator state that yields zero skips forever (log_p is validated on the host).
@@ -227,5 +231,17 @@ __device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t str
     }
   }
 }
+
+// Seeds `count` generators std::mt19937{seed + first + i} and stores their 624-word states at
+// states[i * 624].  One lane per stream: the 623-step recurrence of 64 streams advances in
+// lock step on the vector unit, and LDS transposes 64 x 64 tiles so that every state is written
+// with contiguous 256-byte stores.  The scalar unit (one per CU) can seed only one stream per
+// wave at a time and saturates when every row of a large matrix needs its own generator.
+void launch_seed_streams(hipStream_t stream, uint32_t seed, uint32_t first, uint32_t count, uint32_t *states);
+
+// Streams seeded per launch_seed_streams() call by the operators that use it, and the number
+// of streams from which they do.
+constexpr uint32_t kSeedChunk = 131072;
+constexpr uint32_t kSeedAheadMin = 8192;
 
 }  // namespace bpl

@@ -36,6 +36,13 @@ __device__ __forceinline__ void mt_seed(uint32_t *st, uint32_t seed, int lane) {
   }
 }
 
+// Copies a state seeded elsewhere (624 words at `src`) into the wave's LDS buffer.
+__device__ __forceinline__ void mt_load(uint32_t *st, const uint32_t *__restrict__ src, int lane) {
+#pragma unroll
+  for (int base = 0; base < kMtN; base += kWave)
+    if (base + lane < kMtN) st[base + lane] = src[base + lane];
+}
+
 __device__ __forceinline__ uint32_t mt_twist(uint32_t a, uint32_t b, uint32_t c) {
   const uint32_t y = (a & 0x80000000u) | (b & 0x7fffffffu);
   return c ^ (y >> 1) ^ ((y & 1u) ? 0x9908b0dfu : 0u);
