@@ -24,6 +24,7 @@ if ROOT not in sys.path:
   sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+GATHER_TRAFFIC_BYTES = 742.9e6  # measured HBM traffic of one launch of the headline kernel (see main())
 
 
 def log(*a):
@@ -328,8 +329,10 @@ def main():
     "data": "synthetic",
     "config": {"workload": "event_csr_matvec heterogeneous 100000x100000, nnz~Binomial(1e5,0.01)/row (%d nnz), "
                            "weights N(0,0.1^2), events Bernoulli(0.05), transpose=False, seed 1" % nnz},
+    # traffic: HBM bytes per launch of this kernel on this workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+    # scaled by a 400 MB copy (profiles/event_csr_gather_1e8_hbm_traffic_pmc.txt); it cannot be read in-process
     "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                 "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                 "frac": achieved / HBM_PEAK_GBS, "traffic": GATHER_TRAFFIC_BYTES if nnz == 100014049 else None,
                  "kernel": "csr_gather_kernel<float,bool,heter,event,lds-bitmap>",
                  "algorithmic_bytes_per_launch": bytes_gather, "kernel_us": kernel_ms * 1e3},
     "cpu_baseline": cpu_baseline,
