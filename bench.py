@@ -329,8 +329,9 @@ def main():
     "data": "synthetic",
     "config": {"workload": "event_csr_matvec heterogeneous 100000x100000, nnz~Binomial(1e5,0.01)/row (%d nnz), "
                            "weights N(0,0.1^2), events Bernoulli(0.05), transpose=False, seed 1" % nnz},
-    # traffic: HBM bytes per launch of this kernel on this workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-    # scaled by a 400 MB copy (profiles/event_csr_gather_1e8_hbm_traffic_pmc.txt); it cannot be read in-process
+    # traffic: HBM bytes per launch of this kernel on this workload, from two rocprofv3 --pmc runs (FETCH_SIZE,
+    # WRITE_SIZE; `--pmc gather` mode above) scaled by what a 400 MB copy reads on the same counters; counters
+    # cannot be read in-process, so the figure is a recorded constant for exactly this workload
     "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                  "frac": achieved / HBM_PEAK_GBS, "traffic": GATHER_TRAFFIC_BYTES if nnz == 100014049 else None,
                  "kernel": "csr_gather_kernel<float,bool,heter,event,lds-bitmap>",
