@@ -223,6 +223,41 @@ def main():
       for _ in range(2000):
         oracle.event_csr_matvec(s["data"], s["indices"], s["indptr"], s["events"], shape=s["shape"], transpose=True)
       extra["scatter_4000"]["cpu_port_1core_us"] = (time.perf_counter() - t1) / 2000 * 1e6
+    # the same call through the bare C ABI with pre-marshalled arguments (what a compiled host such as XLA
+    # pays per call; the figures above include this package's Python wrapper, ~15 us of argument checks)
+    import ctypes
+    from brainpylib_amd import _lib
+    fn_raw = _lib.target("event_csr_matvec_homo_float_bool")
+    out_raw = torch.empty(s["shape"][1], dtype=torch.float32, device=dev)
+    bufs = (ctypes.c_void_p * 5)(*[ctypes.c_void_p(t.data_ptr()) for t in
+                                   (sd["data"], sd["indices"], sd["indptr"], sd["events"], out_raw)])
+    opaque = _lib.build_twouint_onebool_descriptor(s["shape"][0], s["shape"][1], True)
+    stream_ptr = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    raw = lambda: fn_raw(stream_ptr, bufs, opaque, len(opaque))
+    # reference point: one trivial kernel launched the same way (the launch floor of this stack)
+    xs = torch.zeros(4000, device=dev)
+    dur_t, wall_t = time_calls(lambda: xs.add_(1.0), 1000, 50)
+    extra["scatter_4000"]["trivial_kernel_event_us"] = float(dur_t.mean() * 1e3)
+    extra["scatter_4000"]["trivial_kernel_wall_us"] = wall_t / 1000 * 1e6
+    dur_r, wall_r = time_calls(raw, 1000, 50)
+    check(out_raw.cpu().numpy(), want, "event_csr_matvec scatter 4,000 (bare ABI)")
+    extra["scatter_4000"]["bare_abi_wall_us_per_call"] = wall_r / 1000 * 1e6
+    extra["scatter_4000"]["bare_abi_event_us"] = stats(dur_r)
+    # the same call replayed from a HIP graph: what a simulation loop that captures its time step pays
+    gs = torch.cuda.Stream()
+    gs.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(gs):
+      bpl.event_csr_matvec(sd["data"], sd["indices"], sd["indptr"], sd["events"], shape=s["shape"], transpose=True)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=gs):
+      g_out = bpl.event_csr_matvec(sd["data"], sd["indices"], sd["indptr"], sd["events"], shape=s["shape"], transpose=True)
+    graph.replay()
+    torch.cuda.synchronize()
+    check(g_out.cpu().numpy(), want, "event_csr_matvec scatter 4,000 (graph)")
+    dur_g, wall_g = time_calls(graph.replay, args.steps, args.warmup)
+    extra["scatter_4000"]["graph_replay_us"] = stats(dur_g)
+    extra["scatter_4000"]["graph_replay_wall_us_per_call"] = wall_g / args.steps * 1e6
     log("scatter 4000: %s" % extra["scatter_4000"])
 
     # csr_matvec, 1,000,000 x 1,000,000, ~1e8 nnz
@@ -289,6 +324,13 @@ def main():
       t_cpu = time.perf_counter() - t1
       jit["cpu_port_1core"] = {"implicit_gsyn_per_s": generated * (rows / n) / t_cpu / 1e9,
                                "sample": "first %d of %d rows, %.2f s" % (rows, n, t_cpu)}
+    # dense-vector twin (jitconn matvec): same streams, float inputs gathered from L2
+    vec = torch.randn(n, dtype=torch.float32, device=dev)
+    for odp in (True, False):
+      fn = lambda: bpl.matvec_prob_conn_homo_weight(vec, j["weight"], conn_prob=j["conn_prob"], shape=j["shape"],
+                                                    seed=j["seed"], outdim_parallel=odp)
+      d, _ = time_calls(fn, max(5, args.steps // 20), 2)
+      jit["dense_matvec,outdim_parallel=%s" % odp] = dict(stats(d), implicit_gsyn_per_s=generated / (d.mean() * 1e-3) / 1e9)
     extra["jitconn_event_matvec_1e9"] = jit
     log("jitconn event matvec: %s" % jit)
 

@@ -8,6 +8,7 @@ only supplies device memory and the current HIP stream.
 There is no fallback: if the library is missing or a target is unknown, the call raises.
 """
 import ctypes
+import functools
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -100,36 +101,43 @@ def _build(fn_name, *args):
   return buf.raw[:n]
 
 
+@functools.lru_cache(maxsize=256)
 def build_twouint_onebool_descriptor(uint_x, uint_y, bool_x):
   return _build("bpl_build_twouint_onebool_descriptor", ctypes.c_uint32(uint_x), ctypes.c_uint32(uint_y),
                 ctypes.c_int(bool(bool_x)))
 
 
+@functools.lru_cache(maxsize=256)
 def build_double_size_descriptor(size_x, size_y):
   return _build("bpl_build_double_size_descriptor", ctypes.c_uint32(size_x), ctypes.c_uint32(size_y))
 
 
+@functools.lru_cache(maxsize=256)
 def build_nonzero_descriptor(event_size, batch_size):
   return _build("bpl_build_nonzero_descriptor", ctypes.c_uint32(event_size), ctypes.c_uint32(batch_size))
 
 
+@functools.lru_cache(maxsize=256)
 def build_jitconn_prob_homo_descriptor(n_row, n_col, seed, prob):
   return _build("bpl_build_jitconn_prob_homo_descriptor", ctypes.c_uint32(n_row), ctypes.c_uint32(n_col),
                 ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_double(prob))
 
 
+@functools.lru_cache(maxsize=256)
 def build_jitconn_prob_uniform_descriptor(n_row, n_col, seed, prob, w_min, w_range):
   return _build("bpl_build_jitconn_prob_uniform_descriptor", ctypes.c_uint32(n_row), ctypes.c_uint32(n_col),
                 ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_double(prob), ctypes.c_double(w_min),
                 ctypes.c_double(w_range))
 
 
+@functools.lru_cache(maxsize=256)
 def build_jitconn_prob_normal_descriptor(n_row, n_col, seed, prob, w_mu, w_sigma):
   return _build("bpl_build_jitconn_prob_normal_descriptor", ctypes.c_uint32(n_row), ctypes.c_uint32(n_col),
                 ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_double(prob), ctypes.c_double(w_mu),
                 ctypes.c_double(w_sigma))
 
 
+@functools.lru_cache(maxsize=256)
 def build_matmat_jit_prob_descriptor1(m, k, n, seed, log_p, w1, w2):
   return _build("bpl_build_matmat_jit_prob_descriptor1", ctypes.c_uint32(m), ctypes.c_uint32(k),
                 ctypes.c_uint32(n), ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_double(log_p),

@@ -46,6 +46,10 @@ const DeviceInfo &device_info();
 // time a size is requested (hipMalloc is not capturable).
 void *stream_workspace(hipStream_t stream, size_t bytes);
 
+// A few zero-initialised 32-bit counters per (device, stream) for kernels that elect a last
+// workgroup.  Every user leaves them at zero again.  nullptr if the allocation fails.
+uint32_t *stream_counters(hipStream_t stream);
+
 inline unsigned div_up(unsigned long long a, unsigned long long b) {
   return static_cast<unsigned>((a + b - 1) / b);
 }

@@ -98,6 +98,29 @@ void *stream_workspace(hipStream_t stream, size_t bytes) {
   return e->ptr;
 }
 
+uint32_t *stream_counters(hipStream_t stream) {
+  struct Entry {
+    int dev;
+    hipStream_t stream;
+    uint32_t *ptr;
+  };
+  static std::vector<Entry> entries;
+  static std::mutex mu;
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  std::lock_guard<std::mutex> lock(mu);
+  for (auto &x : entries)
+    if (x.dev == dev && x.stream == stream) return x.ptr;
+  uint32_t *p = nullptr;
+  constexpr size_t kBytes = 256;
+  if (hipMalloc(reinterpret_cast<void **>(&p), kBytes) != hipSuccess || hipMemset(p, 0, kBytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  entries.push_back(Entry{dev, stream, p});
+  return p;
+}
+
 }  // namespace bpl
 
 // ---- layout checks against the reference's structs (lib/kernel_helper_descriptor.cuh) ----------

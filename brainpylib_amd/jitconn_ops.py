@@ -57,6 +57,18 @@ def _uniform_range(w_low, w_high, dtype):
   return float(lo), float(np_dt(hi - lo))
 
 
+def _apply_weight(r, weight):
+  """r * weight with weight in r's dtype (event_matvec.py:67-68).  A Python / numpy scalar is
+  multiplied in as a scalar, which needs no host-to-device copy (and so can be graph captured)."""
+  if isinstance(weight, torch.Tensor):
+    return r * weight.to(device=r.device, dtype=r.dtype)
+  w = np.asarray(weight.value if hasattr(weight, 'value') else weight)
+  if w.ndim == 0:
+    np_dt = np.float32 if r.dtype == torch.float32 else np.float64
+    return r * float(np_dt(w))
+  return r * torch.from_numpy(np.ascontiguousarray(w)).to(device=r.device, dtype=r.dtype)
+
+
 def _type_name(dt):
   return '_float' if dt == torch.float32 else '_double'
 
@@ -102,8 +114,7 @@ def event_matvec_prob_conn_homo_weight(events, weight, *, conn_prob: float, shap
   out_dtype, suffix = _event_types(events)
   r = _run('gpu_event_matvec', 'homo', events, out_dtype, suffix, conn_prob=conn_prob, shape=shape, seed=_seed(seed),
            transpose=transpose, outdim_parallel=outdim_parallel)
-  weight = as_tensor(weight).to(device=r.device, dtype=r.dtype)
-  return r * weight
+  return _apply_weight(r, weight)
 
 
 def event_matvec_prob_conn_uniform_weight(events, *, w_low: float, w_high: float, conn_prob: float,
@@ -148,8 +159,7 @@ def matvec_prob_conn_homo_weight(vector, weight, *, conn_prob: float, shape: Tup
     raise _lib.GPUOperatorNotFound('matvec_prob_homo version v1 (superseded Bernoulli-per-entry kernel)')
   r = _run('gpu_matvec', 'homo', vector, vector.dtype, _type_name(vector.dtype), conn_prob=conn_prob, shape=shape,
            seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel)
-  weight = as_tensor(weight).to(device=r.device, dtype=r.dtype)
-  return r * weight
+  return _apply_weight(r, weight)
 
 
 def matvec_prob_conn_uniform_weight(vector, *, w_low: float, w_high: float, conn_prob: float, shape: Tuple[int, int],
