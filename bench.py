@@ -69,6 +69,46 @@ def check(got, want, what, mag=None):
     raise SystemExit("parity gate failed for " + what)
 
 
+def reference_shapes(bpl, synth, torch, dev):
+  """The reference's benchmark scripts time 100 jitted calls including dispatch on an unstated GPU; their
+  docstring figures (seconds per 100 calls) are quoted as ms per call.  Ours: mean HIP-event time per call."""
+  rows = []
+  # event_matvec_jitconn_performance.py:157-195: homogeneous weight 1.0, FixedProb(prob), events density = prob
+  ref_event = {(1000, 1000, 0.1): (0.957, 0.996, 1.294, 1.456), (10000, 10000, 0.1): (1.541, 1.557, 1.585, 1.890),
+               (10000, 10000, 0.2): (2.872, 2.905, 3.945, 2.663), (50000, 50000, 0.1): (1.485, 2.521, 6.014, 5.887),
+               (50000, 50000, 0.2): (4.123, 5.962, 10.801, 11.053)}
+  for (n0, n1, p), (csr_t, csr_n, jit_t, jit_n) in ref_event.items():
+    indices, indptr = synth.bernoulli_csr(n0, n1, p, seed=n0 + int(p * 100))
+    rng = np.random.default_rng(5)
+    d_idx, d_ptr = torch.from_numpy(indices).to(dev), torch.from_numpy(indptr).to(dev)
+    w = torch.ones(1, dtype=torch.float32, device=dev)
+    for transpose, ref_csr, ref_jit in ((True, csr_t, jit_t), (False, csr_n, jit_n)):
+      ev = torch.from_numpy(rng.random(n0 if transpose else n1) < p).to(dev)
+      d, _ = time_calls(lambda: bpl.event_csr_matvec(w, d_idx, d_ptr, ev, shape=(n0, n1), transpose=transpose), 100, 10)
+      dj, _ = time_calls(lambda: bpl.event_matvec_prob_conn_homo_weight(ev, 1.0, conn_prob=p, shape=(n0, n1), seed=1234,
+                                                                        transpose=transpose), 30, 3)
+      rows.append(dict(op="event_csr_matvec homo", shape=[n0, n1], prob=p, transpose=transpose,
+                       ours_ms=float(d.mean()), reference_docstring_ms=ref_csr))
+      rows.append(dict(op="jitconn event_matvec homo", shape=[n0, n1], prob=p, transpose=transpose,
+                       ours_ms=float(dj.mean()), reference_docstring_ms=ref_jit))
+      log(rows[-2]); log(rows[-1])
+    del d_idx, d_ptr
+  # csr_matvec_VS_cusparse_csr_matvec.py:76-111: heterogeneous weights, FixedProb(0.1), method='vector'
+  ref_csr = {(10000, 10000): 1.715, (100000, 10000): 3.428, (50000, 50000): 9.002, (100000, 50000): 16.211}
+  for (n0, n1), ref_ms in ref_csr.items():
+    indices, indptr = synth.bernoulli_csr(n0, n1, 0.1, seed=n0 + n1)
+    rng = np.random.default_rng(6)
+    d_idx, d_ptr = torch.from_numpy(indices).to(dev), torch.from_numpy(indptr).to(dev)
+    data = torch.from_numpy(rng.random(indices.shape[0], dtype=np.float32)).to(dev)
+    v = torch.from_numpy(rng.random(n1, dtype=np.float32)).to(dev)
+    d, _ = time_calls(lambda: bpl.csr_matvec(data, d_idx, d_ptr, v, shape=(n0, n1)), 50, 5)
+    rows.append(dict(op="csr_matvec heter", shape=[n0, n1], prob=0.1, nnz=int(indices.shape[0]),
+                     ours_ms=float(d.mean()), reference_docstring_ms=ref_ms))
+    log(rows[-1])
+    del d_idx, d_ptr, data
+  print(json.dumps({"reference_shapes": rows}), flush=True)
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -80,6 +120,10 @@ def main():
                   help="counter-collection mode for rocprofv3 --pmc.  gather: three plain copies of 400 MB "
                        "(the calibration kernel) and three calls of the headline kernel.  jitconn: three calls "
                        "of jitconn event matvec (1e6 x 1e6, p=0.001) in both walks.  Nothing else runs.")
+  ap.add_argument("--reference-shapes", action="store_true",
+                  help="instead of the headline run: the shapes of the reference's own benchmark scripts "
+                       "(event_matvec_jitconn_performance.py, csr_matvec_VS_cusparse_csr_matvec.py), with the "
+                       "per-call times pasted in their docstrings beside ours")
   args = ap.parse_args()
   if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
     raise SystemExit("bench.py: this build runs on ONE GPU (the operators are single-device, like the "
@@ -94,6 +138,10 @@ def main():
   dev = torch.device("cuda:0")
   torch.cuda.set_device(dev)
   cores = len(os.sched_getaffinity(0))
+
+  if args.reference_shapes:
+    reference_shapes(bpl, synth, torch, dev)
+    return
 
   if args.pmc == "jitconn":
     j = synth.config_jitconn_event()

@@ -28,6 +28,19 @@ namespace bpl {
 namespace {
 
 constexpr int kScatterRows = 64;     // rows owned by one scatter workgroup
+
+// The host does not know the number of nonzeros (it is indptr[n_row], in device memory), so where
+// the better kernel depends on the mean row length both candidates are launched and each one
+// returns at once unless the count lies in its range.
+struct NnzGate {
+  uint32_t lo, hi;  // run iff lo <= indptr[n_row] <= hi
+  __device__ __forceinline__ bool open(const uint32_t *__restrict__ indptr, uint32_t n_row) const {
+    if (lo == 0 && hi == 0xffffffffu) return true;
+    const uint32_t nnz = indptr[n_row];
+    return nnz >= lo && nnz <= hi;
+  }
+};
+constexpr NnzGate kAlways = {0u, 0xffffffffu};
 constexpr int kScatterThreads = 256;
 
 enum : int { kEvent = 0, kDense = 1 };
@@ -38,7 +51,8 @@ enum : int { kEvent = 0, kDense = 1 };
 template <typename F, typename VT, bool HETER, int MODE>
 __global__ __launch_bounds__(kScatterThreads) void csr_scatter_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
-    const VT *__restrict__ x, F *__restrict__ y, uint32_t n_row) {
+    const VT *__restrict__ x, F *__restrict__ y, uint32_t n_row, NnzGate gate) {
+  if (!gate.open(indptr, n_row)) return;
   __shared__ uint32_t s_start[kScatterRows];  // first nonzero of the k-th active row
   __shared__ uint32_t s_off[kScatterRows];    // position of that row in the flat range
   __shared__ F s_scale[kScatterRows];         // dense mode: x[r]
@@ -137,7 +151,8 @@ template <typename F, typename VT, bool HETER, int MODE>
 __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
     const VT *__restrict__ x, F *__restrict__ y, uint32_t n_row, uint32_t n_col, uint32_t rows_per_wg,
-    uint32_t win, uint32_t n_win, F *__restrict__ partial, uint32_t *__restrict__ done_counter) {
+    uint32_t win, uint32_t n_win, F *__restrict__ partial, uint32_t *__restrict__ done_counter, NnzGate gate) {
+  if (!gate.open(indptr, n_row)) return;
   extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
   F *window = reinterpret_cast<F *>(smem_raw);
   F *s_scale = window + win;  // dense mode: x[r] per active row
@@ -153,16 +168,22 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
   const uint32_t width = (c0 + win <= n_col) ? win : n_col - c0;
 
   for (uint32_t i = tid; i < width; i += kWinThreads) window[i] = F(0);
+  const F w_homo = HETER ? F(0) : data[0];
+
+  // The group's rows are taken kWinMaxRows at a time (the capacity of the active-row list).
+  for (uint32_t chunk0 = 0; chunk0 < rows_per_wg; chunk0 += kWinMaxRows) {
+  const uint32_t chunk_rows = (rows_per_wg - chunk0 < kWinMaxRows) ? rows_per_wg - chunk0 : kWinMaxRows;
+  if (static_cast<uint64_t>(g) * rows_per_wg + chunk0 >= n_row) break;  // uniform: no rows left
   if (tid == 0) s_count = 0, s_next = kWaves;
   __syncthreads();
 
-  // active rows of the group (order does not matter)
-  for (uint32_t t0 = 0; t0 < rows_per_wg; t0 += kWinThreads) {
-    const uint32_t r = g * rows_per_wg + t0 + tid;
+  // active rows of the chunk (order does not matter)
+  for (uint32_t t0 = 0; t0 < chunk_rows; t0 += kWinThreads) {
+    const uint32_t r = g * rows_per_wg + chunk0 + t0 + tid;
     bool on = false;
     uint32_t start = 0, len = 0;
     F scale = F(1);
-    if (t0 + tid < rows_per_wg && r < n_row) {
+    if (t0 + tid < chunk_rows && r < n_row) {
       if (MODE == kEvent) {
         on = is_event(x[r]);
       } else {
@@ -188,7 +209,6 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
   }
   __syncthreads();
   const uint32_t count = s_count;
-  const F w_homo = HETER ? F(0) : data[0];
 
   // waves take active rows from a shared counter; full steps of U*64 nonzeros run unguarded
   constexpr int U = 8;
@@ -224,7 +244,8 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     if (lane == 0) nk = atomicAdd(&s_next, 1u);
     k = __builtin_amdgcn_readfirstlane(nk);
   }
-  __syncthreads();
+  __syncthreads();  // the lists and counters are reused by the next chunk; the window is complete after the last
+  }
 
   if (partial != nullptr) {
     // plain contiguous stores of the whole window into this row group's slice; a second
@@ -271,7 +292,10 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
 // y[c] = sum over row groups of partial[g][c]
 template <typename F>
 __global__ __launch_bounds__(256) void sum_partials_kernel(const F *__restrict__ partial, F *__restrict__ y,
-                                                           uint32_t n_col, uint32_t groups) {
+                                                           uint32_t n_col, uint32_t groups,
+                                                           const uint32_t *__restrict__ indptr, uint32_t n_row,
+                                                           NnzGate gate) {
+  if (!gate.open(indptr, n_row)) return;
   const uint32_t c = blockIdx.x * 256u + threadIdx.x;
   if (c >= n_col) return;
   F acc = F(0);
@@ -496,55 +520,75 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
     fill_zero(stream, y, n_col);
     return;
   }
-  // Output windows in LDS when at most 4 of them cover the output vector.
+  // Output windows in LDS.  Every window's workgroup streams the column indices of the active
+  // rows again, which is still far cheaper than one random global atomic per nonzero (about
+  // 21 G/s) up to a few dozen windows when the activity is sparse (event input) and the rows are
+  // long.  With a dense input every row is active and only a handful of windows pay off.
   const size_t list_bytes = kWinMaxRows * (8 + (MODE == kDense ? sizeof(F) : 0));
   const uint32_t win_cap = static_cast<uint32_t>((static_cast<size_t>(128) * 1024) / sizeof(F));
   const uint32_t n_win = div_up(n_col, win_cap);
-  if (n_win <= 4) {
+  NnzGate direct_gate = kAlways;
+  if (n_win <= (MODE == kEvent ? 32u : 4u)) {
     const uint32_t win = div_up(n_col, n_win);
-    // one workgroup per CU in total, between 64 and kWinMaxRows rows each
+    // about one workgroup per CU in total, at least 64 rows each
     unsigned want_groups = static_cast<unsigned>(device_info().num_cu) / n_win;
+    if (want_groups == 0) want_groups = 1;
     // small outputs: at most 16 row groups, so that the last workgroup can sum their slices itself
     if (static_cast<size_t>(n_col) * 16 <= 131072 && n_row <= 16 * kWinMaxRows && want_groups > 16) want_groups = 16;
-    uint32_t rows_per_wg = div_up(n_row, want_groups ? want_groups : 1u);
+    uint32_t rows_per_wg = div_up(n_row, want_groups);
     if (rows_per_wg < 64) rows_per_wg = 64;
-    if (rows_per_wg > kWinMaxRows) rows_per_wg = kWinMaxRows;
     const unsigned groups = div_up(n_row, rows_per_wg);
+    // The window kernel hands whole rows to waves, one after the other: with more than a few
+    // windows it only beats the direct atomics when rows are long (64 nonzeros on average).
+    NnzGate window_gate = kAlways;
+    bool usable = true;
+    if (n_win > 4) {
+      const unsigned long long min_nnz = 64ull * n_row;
+      if (min_nnz > 0xffffffffull) {
+        usable = false;
+      } else {
+        window_gate = {static_cast<uint32_t>(min_nnz), 0xffffffffu};
+        direct_gate = {0u, static_cast<uint32_t>(min_nnz) - 1u};
+      }
+    }
     const size_t lds = static_cast<size_t>(win) * sizeof(F) + list_bytes;
     auto kernel = csr_scatter_window_kernel<F, VT, HETER, MODE>;
     static thread_local size_t attr_set_for = 0;
-    if (lds > 64 * 1024 && attr_set_for < lds) {
+    if (usable && lds > 64 * 1024 && attr_set_for < lds) {
       if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                               static_cast<int>(lds)) == hipSuccess)
         attr_set_for = lds;
       else
         (void)hipGetLastError();
     }
-    if (lds <= 64 * 1024 || attr_set_for >= lds) {
+    if (usable && (lds <= 64 * 1024 || attr_set_for >= lds)) {
       // Per-row-group partial outputs in scratch memory, summed by a second kernel (no global
       // atomics, no zero fill), as long as they stay small; else atomics into the zeroed y.
       const size_t partial_bytes = static_cast<size_t>(groups) * n_col * sizeof(F);
       F *partial = nullptr;
       if (groups > 1 && partial_bytes <= (static_cast<size_t>(64) << 20))
         partial = static_cast<F *>(stream_workspace(stream, partial_bytes));
-      if (partial == nullptr) {
-        bpl_clear_error();
-        fill_zero(stream, y, n_col);
-      }
+      const bool gated = n_win > 4;
+      if (partial == nullptr) bpl_clear_error();
+      if (partial == nullptr || gated) fill_zero(stream, y, n_col);
       // small slices: the last workgroup of the same launch sums them (one launch instead of two)
       uint32_t *done_counter = nullptr;
       if (partial != nullptr && static_cast<size_t>(groups) * n_col <= 131072) done_counter = stream_counters(stream);
       hipLaunchKernelGGL(kernel, dim3(groups * n_win), dim3(kWinThreads), lds, stream, data, indices, indptr, x, y,
-                         n_row, n_col, rows_per_wg, win, n_win, partial, done_counter);
+                         n_row, n_col, rows_per_wg, win, n_win, partial, done_counter, window_gate);
       if (partial != nullptr && done_counter == nullptr)
         hipLaunchKernelGGL(sum_partials_kernel<F>, dim3(div_up(n_col, 256)), dim3(256), 0, stream, partial, y, n_col,
-                           groups);
-      return;
+                           groups, indptr, n_row, window_gate);
+      if (!gated) return;
+    } else {
+      direct_gate = kAlways;
+      fill_zero(stream, y, n_col);
     }
+  } else {
+    fill_zero(stream, y, n_col);
   }
-  fill_zero(stream, y, n_col);
   hipLaunchKernelGGL((csr_scatter_kernel<F, VT, HETER, MODE>), dim3(div_up(n_row, kScatterRows)),
-                     dim3(kScatterThreads), 0, stream, data, indices, indptr, x, y, n_row);
+                     dim3(kScatterThreads), 0, stream, data, indices, indptr, x, y, n_row, direct_gate);
 }
 
 template <typename F, typename VT, bool HETER, int MODE, bool LDS_BITS>

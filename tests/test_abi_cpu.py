@@ -129,3 +129,16 @@ def test_jax_registration_shim_needs_jax():
   except ImportError:
     with pytest.raises(ImportError):
       jax_register.register()
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+  # no fallback: without the built library every operator raises
+  import numpy as np
+  import brainpylib_amd as bpl
+  monkeypatch.setattr(_lib, "_lib", None)
+  monkeypatch.setattr(_lib, "_targets", {})
+  monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libbrainpylib_amd.so")
+  with pytest.raises(_lib.GPUOperatorNotFound):
+    _lib.target("event_csr_matvec_homo_float_bool")
+  with pytest.raises(_lib.GPUOperatorNotFound):
+    _lib.build_double_size_descriptor(11, 12)

@@ -254,3 +254,27 @@ def test_full_size_event_csr_properties(cuda):
   f1 = bpl.event_csr_matvec(data, indices, indptr, x, shape=c["shape"], transpose=False)
   f2 = bpl.event_csr_matvec(data * 2, indices, indptr, x, shape=c["shape"], transpose=False)
   assert torch.equal(f1 * 2, f2)
+
+
+def test_scatter_many_windows_and_row_chunks(cuda, oracle_mod):
+  # transpose=True with (a) an output vector that needs several LDS windows and (b) row groups
+  # larger than the active-row list, so that a workgroup walks its rows in several chunks
+  rng = np.random.default_rng(21)
+  # (mean row length below/above 64 selects direct atomics/LDS windows when there are many windows)
+  for n_row, n_col, mean in ((5000, 700_000, 50), (600_000, 300, 3), (300_000, 200_000, 8),
+                             (20_000, 400_000, 100)):
+    counts = rng.poisson(mean, size=n_row)
+    indices, indptr = synth.counted_csr(np.minimum(counts, n_col), n_col, seed=n_row)
+    data = rng.standard_normal(indices.shape[0]).astype(np.float32)
+    shape = (n_row, n_col)
+    print("shape", shape, flush=True)
+    for rate in (0.02, 0.9):
+      ev = rng.random(n_row) < rate
+      want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True)
+      mag = oracle_mod.event_csr_matvec(np.abs(data), indices, indptr, ev, shape=shape, transpose=True)
+      got = bpl.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+      assert_close_reordered(got, want, mag, what="scatter %s rate %s" % (shape, rate))
+      ones = np.ones(1, dtype=np.float32)
+      want = oracle_mod.event_csr_matvec(ones, indices, indptr, ev, shape=shape, transpose=True)
+      got = bpl.event_csr_matvec(ones, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+      assert np.array_equal(got, want)  # integer counts are exact
