@@ -254,6 +254,21 @@ def main():
     extra["gather_homo_1e8"] = dict(stats(dur_h), gsop_per_s=nnz / (dur_h.mean() * 1e-3) / 1e9,
                                     algorithmic_gb_per_s=bytes_h / (dur_h.mean() * 1e-3) / 1e9)
     log("gather homo 1e8: %s" % extra["gather_homo_1e8"])
+
+    # vmap over event vectors (event_csr_matvec_batching): the same matrix against 8 and 32
+    # event vectors of the same rate; the index stream is read once per 8 vectors
+    rng_b = np.random.default_rng(99)
+    batched = {}
+    for nb in (8, 32):
+      evb = torch.from_numpy(rng_b.random((nb, n_col)) < 0.05).to(dev)
+      dur_b, _ = time_calls(lambda: bpl.event_csr_matvec_batching(
+        data[None], indices[None], indptr[None], evb, batch_size=nb, shape=c["shape"]), max(args.steps // 4, 5),
+        max(args.warmup // 4, 2))
+      batched["x%d" % nb] = dict(stats(dur_b), us_per_event_vector=float(dur_b.mean() * 1e3 / nb),
+                                 gsop_per_s=nb * nnz / (dur_b.mean() * 1e-3) / 1e9)
+      del evb
+    extra["gather_batched_1e8"] = batched
+    log("gather batched 1e8: %s" % batched)
     del data, indices, indptr, events
 
     # 4,000 x 4,000, 80 per row, homogeneous 0.6, 2 % events, scatter (the reference's own CPU-sized case)

@@ -108,6 +108,14 @@ def build_twouint_onebool_descriptor(uint_x, uint_y, bool_x):
 
 
 @functools.lru_cache(maxsize=256)
+def build_event_csr_batching_descriptor(n_row, n_col, batch_size, values_batch, indices_batch, indptr_batch,
+                                        events_batch, nnz, transpose):
+  u = ctypes.c_uint32
+  return _build("bpl_build_event_csr_batching_descriptor", u(n_row), u(n_col), u(batch_size), u(values_batch),
+                u(indices_batch), u(indptr_batch), u(events_batch), u(nnz), ctypes.c_int(bool(transpose)))
+
+
+@functools.lru_cache(maxsize=256)
 def build_double_size_descriptor(size_x, size_y):
   return _build("bpl_build_double_size_descriptor", ctypes.c_uint32(size_x), ctypes.c_uint32(size_y))
 

@@ -694,10 +694,283 @@ void csr_matvec_entry(const char *target, hipStream_t stream, void **buffers, co
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// Batched event gather: one matrix, several event vectors
+// (brainpylib/_src/event_ops/event_csr_matvec.py:152-193 is the CPU kernel of the batching
+// primitive; the reference has no GPU kernel for it, :227-229).
+// The column indices are streamed once per tile of kBatchTile event vectors: a byte per column
+// holds the tile's event flags, so one probe answers for eight vectors.
+// ------------------------------------------------------------------------------------------------
+constexpr int kBatchTile = 8;
+
+// mask[t * stride + c] bit b = events[((8 t + b) % events_batch) * n_col + c] != 0, for 8 t + b < batch
+template <typename VT>
+__global__ __launch_bounds__(256) void pack_event_masks_kernel(const VT *__restrict__ events,
+                                                               uint8_t *__restrict__ mask, uint32_t n_col,
+                                                               uint32_t stride, uint32_t batch,
+                                                               uint32_t events_batch) {
+  const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+  const uint32_t t = blockIdx.y;
+  if (c >= n_col) return;
+  uint32_t m = 0;
+#pragma unroll
+  for (uint32_t b = 0; b < kBatchTile; ++b) {
+    const uint32_t bi = t * kBatchTile + b;
+    if (bi < batch && is_event(events[static_cast<size_t>(bi % events_batch) * n_col + c])) m |= 1u << b;
+  }
+  mask[static_cast<size_t>(t) * stride + c] = static_cast<uint8_t>(m);
+}
+
+// Sums eight values per lane over aligned groups of G lanes (G = 8, 16, 32 or 64), halving the
+// number of live values at each of the first three exchange steps.  Lane gl of the group ends
+// up with the group total of value number k = (bit G/2 of gl)*4 + (bit G/4)*2 + (bit G/8);
+// the lanes whose low bits (below G/8) are zero are the ones meant to use it.
+template <int G, typename T>
+__device__ __forceinline__ T group_sum8(const T (&v)[8], uint32_t gl, uint32_t *k) {
+  constexpr int o1 = G / 2, o2 = G / 4, o3 = G / 8;
+  const bool h1 = gl & o1, h2 = gl & o2, h3 = gl & o3;
+  T a[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const T send = h1 ? v[i] : v[i + 4];
+    const T keep = h1 ? v[i + 4] : v[i];
+    a[i] = keep + __shfl_xor(send, o1, kWave);
+  }
+  T b[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const T send = h2 ? a[i] : a[i + 2];
+    const T keep = h2 ? a[i + 2] : a[i];
+    b[i] = keep + __shfl_xor(send, o2, kWave);
+  }
+  T c;
+  {
+    const T send = h3 ? b[0] : b[1];
+    const T keep = h3 ? b[1] : b[0];
+    c = keep + __shfl_xor(send, o3, kWave);
+  }
+#pragma unroll
+  for (int off = o3 / 2; off > 0; off >>= 1) c += __shfl_xor(c, off, kWave);
+  *k = (h1 ? 4u : 0u) | (h2 ? 2u : 0u) | (h3 ? 1u : 0u);
+  return c;
+}
+
+template <typename F, bool HETER, bool LDS_MASK, int G, int U>
+__device__ __forceinline__ void gather_rows_batched(const F *__restrict__ data,
+                                                    const uint32_t *__restrict__ indices,
+                                                    const uint32_t *__restrict__ indptr,
+                                                    const uint8_t *__restrict__ mask, F *__restrict__ y,
+                                                    uint32_t n_row, uint32_t batch, uint32_t tile) {
+  const uint32_t gl = threadIdx.x & (G - 1);
+  const uint32_t groups_per_block = blockDim.x / G;
+  const uint32_t total_groups = gridDim.x * groups_per_block;
+  const F w_homo = HETER ? F(0) : data[0];
+  for (uint32_t row = blockIdx.x * groups_per_block + threadIdx.x / G; row < n_row; row += total_groups) {
+    uint32_t start = indptr[row], end = indptr[row + 1];
+    if (G == kWave) {
+      start = __builtin_amdgcn_readfirstlane(start);
+      end = __builtin_amdgcn_readfirstlane(end);
+    }
+    double acc[kBatchTile];
+    uint32_t cnt[kBatchTile];
+#pragma unroll
+    for (int k = 0; k < kBatchTile; ++k) acc[k] = 0.0, cnt[k] = 0u;
+    // software pipeline: the column indices of the next step are requested before this step's
+    // probes and weights are waited for
+    uint32_t col[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t j = start + u * G + gl;
+      col[u] = j < end ? indices[j] : 0u;
+    }
+    for (uint32_t base = start; base < end; base += U * G) {
+      uint32_t coln[U];
+      const uint32_t nbase = base + U * G;
+      if (nbase < end) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t j = nbase + u * G + gl;
+          coln[u] = j < end ? indices[j] : 0u;
+        }
+      }
+      uint32_t m[U];
+      F val[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t j = base + u * G + gl;
+        m[u] = j < end ? static_cast<uint32_t>(mask[col[u]]) : 0u;
+      }
+      if (HETER) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t j = base + u * G + gl;
+          val[u] = F(0);
+          if (m[u] != 0u) val[u] = data[j];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (HETER) {
+          // v or +0.0 by bit k of the mask: sign-extend the bit into a word mask, AND both halves
+          const double v = static_cast<double>(val[u]);
+          const int lo = __double2loint(v), hi = __double2hiint(v);
+#pragma unroll
+          for (int k = 0; k < kBatchTile; ++k) {
+            const int t = __builtin_amdgcn_sbfe(static_cast<int>(m[u]), k, 1);
+            acc[k] += __hiloint2double(hi & t, lo & t);
+          }
+        } else {
+#pragma unroll
+          for (int k = 0; k < kBatchTile; ++k) cnt[k] += (m[u] >> k) & 1u;
+        }
+      }
+      if (nbase < end) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) col[u] = coln[u];
+      }
+    }
+    uint32_t k;
+    F result;
+    if (HETER) {
+      result = static_cast<F>(group_sum8<G>(acc, gl, &k));
+    } else {
+      // n additions of the same value into a float64 accumulator are exact: n * w
+      const uint32_t n = group_sum8<G>(cnt, gl, &k);
+      result = static_cast<F>(static_cast<double>(w_homo) * static_cast<double>(n));
+    }
+    const uint32_t bi = tile * kBatchTile + k;
+    if ((gl & (G / 8 - 1)) == 0 && bi < batch) y[static_cast<size_t>(bi) * n_row + row] = result;
+  }
+}
+
+// grid = (workgroups striding the rows, tiles of 8 event vectors)
+template <typename F, bool HETER, bool LDS_MASK>
+__global__ __launch_bounds__(1024) void csr_gather_batched_kernel(const F *__restrict__ data,
+                                                                  const uint32_t *__restrict__ indices,
+                                                                  const uint32_t *__restrict__ indptr,
+                                                                  const uint8_t *__restrict__ masks,
+                                                                  F *__restrict__ y, uint32_t n_row,
+                                                                  uint32_t mask_stride, uint32_t batch) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char s_mask[];
+  const uint32_t tile = blockIdx.y;
+  const uint8_t *mask = masks + static_cast<size_t>(tile) * mask_stride;
+  if (LDS_MASK) {
+    // rows of `masks` are padded to 16 bytes, so whole 16-byte pieces can be copied
+    const uint32_t vecs = mask_stride / 16u;
+    for (uint32_t i = threadIdx.x; i < vecs; i += blockDim.x)
+      reinterpret_cast<uint4 *>(s_mask)[i] = reinterpret_cast<const uint4 *>(mask)[i];
+    __syncthreads();
+  }
+  const uint8_t *probe = LDS_MASK ? reinterpret_cast<const uint8_t *>(s_mask) : mask;
+  const uint32_t nnz = indptr[n_row];
+  if (nnz == 0) {
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n_row; i += gridDim.x * blockDim.x)
+      for (uint32_t k = 0; k < kBatchTile; ++k)
+        if (tile * kBatchTile + k < batch) y[static_cast<size_t>(tile * kBatchTile + k) * n_row + i] = F(0);
+    return;
+  }
+  const uint32_t mean = nnz / n_row;
+  if (mean >= 32) gather_rows_batched<F, HETER, LDS_MASK, 64, 8>(data, indices, indptr, probe, y, n_row, batch, tile);
+  else gather_rows_batched<F, HETER, LDS_MASK, 8, 2>(data, indices, indptr, probe, y, n_row, batch, tile);
+}
+
+template <typename F, bool HETER, bool LDS_MASK>
+bool launch_gather_batched_impl(const char *target, hipStream_t stream, const F *data, const uint32_t *indices,
+                                const uint32_t *indptr, const uint8_t *masks, F *y, uint32_t n_row,
+                                uint32_t mask_stride, uint32_t batch, size_t lds_bytes) {
+  auto kernel = csr_gather_batched_kernel<F, HETER, LDS_MASK>;
+  const int block = (n_row >= 16384) ? 1024 : 256;
+  if (lds_bytes > 64 * 1024) {
+    static thread_local size_t attr_set_for = 0;
+    if (attr_set_for < lds_bytes) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(lds_bytes)) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+      }
+      attr_set_for = lds_bytes;
+    }
+  }
+  int per_cu = 1;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(kernel), block,
+                                                   lds_bytes) != hipSuccess || per_cu < 1) {
+    (void)hipGetLastError();
+    per_cu = 1;
+  }
+  const unsigned tiles = div_up(batch, kBatchTile);
+  const unsigned resident = static_cast<unsigned>(device_info().num_cu) * static_cast<unsigned>(per_cu);
+  const unsigned needed = div_up(n_row, block / kWave);
+  const unsigned gx = needed < resident ? (needed ? needed : 1u) : resident;
+  hipLaunchKernelGGL(kernel, dim3(gx, tiles), dim3(block), lds_bytes, stream, data, indices, indptr, masks, y, n_row,
+                     mask_stride, batch);
+  return check_launch(target);
+}
+
+// event_csr_matvec_batching: buffers = [values, indices, indptr, events, out], every operand
+// with a leading batch dimension that is indexed `bi % dim` as in the reference's CPU kernel.
+template <typename F, typename VT, bool HETER>
+void event_csr_batching_entry(const char *target, hipStream_t stream, void **buffers, const char *opaque,
+                              size_t opaque_len) {
+  bpl_event_csr_batching_descriptor d;
+  if (!unpack(target, opaque, opaque_len, &d)) return;
+  if (buffers == nullptr) {
+    set_error("%s: null buffer table", target);
+    return;
+  }
+  if (d.batch_size == 0) return;
+  if (d.values_batch == 0 || d.indices_batch == 0 || d.indptr_batch == 0 || d.events_batch == 0) {
+    set_error("%s: operand batch dimensions must be at least 1", target);
+    return;
+  }
+  const F *values = static_cast<const F *>(buffers[0]);
+  const uint32_t *indices = static_cast<const uint32_t *>(buffers[1]);
+  const uint32_t *indptr = static_cast<const uint32_t *>(buffers[2]);
+  const VT *events = static_cast<const VT *>(buffers[3]);
+  F *out = static_cast<F *>(buffers[4]);
+  const uint32_t n_in = d.transpose ? d.n_row : d.n_col;
+  const uint32_t n_out = d.transpose ? d.n_col : d.n_row;
+  if (n_out == 0) return;
+  const size_t value_stride = HETER ? d.nnz : 1u;
+  const bool shared_matrix = d.values_batch == 1 && d.indices_batch == 1 && d.indptr_batch == 1;
+  if (!d.transpose && shared_matrix && d.batch_size > 1 && d.n_col > 0) {
+    const unsigned tiles = div_up(d.batch_size, kBatchTile);
+    const uint32_t stride = div_up(d.n_col, 16) * 16u;  // the padding is never probed (columns < n_col)
+    uint8_t *masks = static_cast<uint8_t *>(stream_workspace(stream, static_cast<size_t>(tiles) * stride));
+    if (masks == nullptr) return;
+    hipLaunchKernelGGL(pack_event_masks_kernel<VT>, dim3(div_up(d.n_col, 256), tiles), dim3(256), 0, stream, events,
+                       masks, d.n_col, stride, d.batch_size, d.events_batch);
+    const size_t lds_bytes = stride;
+    const size_t lds_cap = static_cast<size_t>(160) * 1024 - 1024;
+    if (lds_bytes <= lds_cap &&
+        launch_gather_batched_impl<F, HETER, true>(target, stream, values, indices, indptr, masks, out, d.n_row,
+                                                   stride, d.batch_size, lds_bytes))
+      return;
+    bpl_clear_error();
+    launch_gather_batched_impl<F, HETER, false>(target, stream, values, indices, indptr, masks, out, d.n_row, stride,
+                                                d.batch_size, 0);
+    return;
+  }
+  for (uint32_t bi = 0; bi < d.batch_size; ++bi) {
+    const F *v = values + static_cast<size_t>(bi % d.values_batch) * value_stride;
+    const uint32_t *ix = indices + static_cast<size_t>(bi % d.indices_batch) * d.nnz;
+    const uint32_t *ip = indptr + static_cast<size_t>(bi % d.indptr_batch) * (static_cast<size_t>(d.n_row) + 1u);
+    const VT *ev = events + static_cast<size_t>(bi % d.events_batch) * n_in;
+    F *o = out + static_cast<size_t>(bi) * n_out;
+    if (d.transpose) {
+      launch_scatter<F, VT, HETER, kEvent>(stream, v, ix, ip, ev, o, d.n_row, d.n_col);
+      if (!check_launch(target)) return;
+    } else {
+      launch_gather<F, VT, HETER, kEvent>(target, stream, v, ix, ip, ev, o, d.n_row, d.n_col);
+    }
+  }
+}
+
 }  // namespace
 }  // namespace bpl
 
 using bpl::csr_matvec_entry;
+using bpl::event_csr_batching_entry;
 using bpl::event_csr_matvec_entry;
 
 #define BPL_DEFINE(name, call)                                                                   \
@@ -733,3 +1006,12 @@ BPL_DEFINE(csr_matvec_transpose_heter_float, (csr_matvec_entry<float, true, true
 BPL_DEFINE(csr_matvec_transpose_heter_double, (csr_matvec_entry<double, true, true>(__func__, s, buffers, opaque, opaque_len, 3)))
 BPL_DEFINE(csr_matvec_transpose_homo_float, (csr_matvec_entry<float, false, true>(__func__, s, buffers, opaque, opaque_len, 3)))
 BPL_DEFINE(csr_matvec_transpose_homo_double, (csr_matvec_entry<double, false, true>(__func__, s, buffers, opaque, opaque_len, 3)))
+
+BPL_DEFINE(event_csr_matvec_batching_heter_float_bool, (event_csr_batching_entry<float, uint8_t, true>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_batching_heter_float_float, (event_csr_batching_entry<float, float, true>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_batching_heter_double_bool, (event_csr_batching_entry<double, uint8_t, true>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_batching_heter_double_double, (event_csr_batching_entry<double, double, true>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_batching_homo_float_bool, (event_csr_batching_entry<float, uint8_t, false>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_batching_homo_float_float, (event_csr_batching_entry<float, float, false>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_batching_homo_double_bool, (event_csr_batching_entry<double, uint8_t, false>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_batching_homo_double_double, (event_csr_batching_entry<double, double, false>(__func__, s, buffers, opaque, opaque_len)))

@@ -36,6 +36,12 @@ py::dict Registrations() {
 PYBIND11_MODULE(gpu_ops, m) {
   m.doc() = "XLA custom-call targets and descriptor builders of brainpylib_amd (gfx950)";
   m.def("registrations", &Registrations);
+  m.def("build_event_csr_batching_descriptor",
+        [](uint32_t n_row, uint32_t n_col, uint32_t batch_size, uint32_t values_batch, uint32_t indices_batch,
+           uint32_t indptr_batch, uint32_t events_batch, uint32_t nnz, bool transpose) {
+          return BPL_PACK(bpl_build_event_csr_batching_descriptor, n_row, n_col, batch_size, values_batch,
+                          indices_batch, indptr_batch, events_batch, nnz, transpose ? 1 : 0);
+        });
   m.def("build_twouint_onebool_descriptor", [](uint32_t x, uint32_t y, bool b) {
     return BPL_PACK(bpl_build_twouint_onebool_descriptor, x, y, b ? 1 : 0);
   });

@@ -126,6 +126,7 @@ uint32_t *stream_counters(hipStream_t stream) {
 // ---- layout checks against the reference's structs (lib/kernel_helper_descriptor.cuh) ----------
 static_assert(sizeof(bpl_twouint_onebool_descriptor) == 12, "TwoUintOneBoolDescriptor is 12 bytes");
 static_assert(offsetof(bpl_twouint_onebool_descriptor, transpose) == 8, "bool at offset 8");
+static_assert(sizeof(bpl_event_csr_batching_descriptor) == 36, "batching descriptor is 36 bytes");
 static_assert(sizeof(bpl_double_size_descriptor) == 8, "DoubleSizeDescriptor is 8 bytes");
 static_assert(sizeof(bpl_nonzero_descriptor) == 8, "NonZeroDescriptor is 8 bytes");
 static_assert(sizeof(bpl_jitconn_prob_homo_descriptor) == 24, "JITConnProbHomoDescriptor is 24 bytes");
@@ -152,6 +153,24 @@ size_t bpl_build_twouint_onebool_descriptor(uint32_t n_row, uint32_t n_col, int 
   std::memset(&d, 0, sizeof(d));
   d.n_row = n_row;
   d.n_col = n_col;
+  d.transpose = transpose ? 1 : 0;
+  return pack(d, out, cap);
+}
+
+size_t bpl_build_event_csr_batching_descriptor(uint32_t n_row, uint32_t n_col, uint32_t batch_size,
+                                               uint32_t values_batch, uint32_t indices_batch,
+                                               uint32_t indptr_batch, uint32_t events_batch, uint32_t nnz,
+                                               int transpose, char *out, size_t cap) {
+  bpl_event_csr_batching_descriptor d;
+  std::memset(&d, 0, sizeof(d));
+  d.n_row = n_row;
+  d.n_col = n_col;
+  d.batch_size = batch_size;
+  d.values_batch = values_batch;
+  d.indices_batch = indices_batch;
+  d.indptr_batch = indptr_batch;
+  d.events_batch = events_batch;
+  d.nnz = nnz;
   d.transpose = transpose ? 1 : 0;
   return pack(d, out, cap);
 }

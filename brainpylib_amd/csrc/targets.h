@@ -81,8 +81,19 @@
   X(nonzero_float) \
   X(nonzero_double)
 
+#define BPL_EVENT_CSR_BATCHING_TARGETS(X)            \
+  X(event_csr_matvec_batching_heter_float_bool)      \
+  X(event_csr_matvec_batching_heter_float_float)     \
+  X(event_csr_matvec_batching_heter_double_bool)     \
+  X(event_csr_matvec_batching_heter_double_double)   \
+  X(event_csr_matvec_batching_homo_float_bool)       \
+  X(event_csr_matvec_batching_homo_float_float)      \
+  X(event_csr_matvec_batching_homo_double_bool)      \
+  X(event_csr_matvec_batching_homo_double_double)
+
 #define BPL_ALL_TARGETS(X)  \
   BPL_EVENT_CSR_TARGETS(X)  \
+  BPL_EVENT_CSR_BATCHING_TARGETS(X) \
   BPL_CSR_TARGETS(X)        \
   BPL_JITCONN_TARGETS(X)    \
   BPL_MATMAT_TARGETS(X)     \

@@ -11,7 +11,7 @@ import torch
 from . import _lib
 from ._tensors import FLOAT_DTYPES, as_tensor, device_of, is_index_dtype, to_device
 
-__all__ = ["event_csr_matvec", "event_info"]
+__all__ = ["event_csr_matvec", "event_csr_matvec_batching", "event_info"]
 
 
 def _type_name(dt):
@@ -80,6 +80,69 @@ def event_csr_matvec(data, indices, indptr, events, *, shape: Tuple[int, int], t
   out = torch.empty(shape[1] if transpose else shape[0], dtype=data.dtype, device=device)
   _lib.custom_call('event_csr_matvec' + data_name + type_name + vec_type,
                    [data, indices, indptr, events, out], opaque)
+  return out
+
+
+def event_csr_matvec_batching(values, indices, indptr, events, *, batch_size: int, shape: Tuple[int, int],
+                              transpose: bool = False):
+  """The primitive behind ``vmap(event_csr_matvec)``: every operand carries a leading batch
+  dimension and entry ``bi`` of the result uses row ``bi % dim`` of each operand
+  (brainpylib/_src/event_ops/event_csr_matvec.py:112-193; the batching rule passes a dimension
+  of 1 for operands that are not mapped).
+
+  values   (B_v, 1) homogeneous or (B_v, nse);  indices (B_i, nse);  indptr (B_p, shape[0] + 1)
+  events   (B_e, shape[0] if transpose else shape[1]) bool, or the float dtype of ``values``
+  returns  (batch_size, shape[1] if transpose else shape[0]) tensor of ``values``' dtype.
+
+  The reference has this operator on the CPU only.  Here one matrix shared by the whole batch
+  (B_v = B_i = B_p = 1) with ``transpose=False`` streams the column indices once per eight event
+  vectors; every other combination runs the single operator once per batch entry."""
+  values = as_tensor(values)
+  indices = as_tensor(indices)
+  indptr = as_tensor(indptr)
+  events = as_tensor(events)
+  for name, t in (("values", values), ("indices", indices), ("indptr", indptr), ("events", events)):
+    if t.ndim != 2:
+      raise ValueError(f'{name} should be a 2D array with a leading batch dimension, got {t.ndim}-D.')
+    if t.shape[0] < 1:
+      raise ValueError(f'{name} has an empty batch dimension.')
+  if len(shape) != 2:
+    raise ValueError('shape should be a length-2 tuple.')
+  if batch_size < 0:
+    raise ValueError('batch_size should not be negative.')
+  if values.dtype not in FLOAT_DTYPES:
+    raise TypeError(f'Only support float32 and float64. But we got {values.dtype}.')
+  if not is_index_dtype(indices.dtype) or not is_index_dtype(indptr.dtype):
+    raise ValueError('indices and indptr should have int32 or uint32 type.')
+  nse = indices.shape[1]
+  if values.shape[1] not in (1, nse):
+    raise ValueError('The size of data should be 1 or be consistent with indices.'
+                     f'But we got {tuple(values.shape)} != {tuple(indices.shape)}, {tuple(values.shape)} != 1.')
+  if indptr.shape[1] != shape[0] + 1:
+    raise ValueError(f'indptr should have shape[0] + 1 = {shape[0] + 1} entries, got {indptr.shape[1]}.')
+  n_in = shape[0] if transpose else shape[1]
+  if events.shape[1] != n_in:
+    if transpose:
+      raise ValueError(f'Shape mismatch, vec ({events.shape[1]},) @ mat {shape}.')
+    raise ValueError(f'Shape mismatch, mat {shape} @ vec ({events.shape[1]},).')
+  type_name = _type_name(values.dtype)
+  # (B, 1) values with a single nonzero are homogeneous, as in the reference (`values.shape[1] == 1`)
+  data_name = '_homo' if values.shape[1] == 1 else '_heter'
+  if events.dtype == torch.bool:
+    vec_type = '_bool'
+  else:
+    if events.dtype != values.dtype:
+      raise ValueError('events should be bool or have the dtype of data, '
+                       f'but we got {events.dtype} != {values.dtype}.')
+    vec_type = type_name
+  device = device_of(values, indices, indptr, events)
+  values, indices, indptr, events = (to_device(t, device).contiguous() for t in (values, indices, indptr, events))
+  opaque = _lib.build_event_csr_batching_descriptor(shape[0], shape[1], batch_size, values.shape[0],
+                                                    indices.shape[0], indptr.shape[0], events.shape[0], nse,
+                                                    transpose)
+  out = torch.empty((batch_size, shape[1] if transpose else shape[0]), dtype=values.dtype, device=device)
+  _lib.custom_call('event_csr_matvec_batching' + data_name + type_name + vec_type,
+                   [values, indices, indptr, events, out], opaque)
   return out
 
 

@@ -53,6 +53,22 @@ typedef struct {
   uint8_t transpose; /* C++ bool; 3 bytes of padding follow */
 } bpl_twouint_onebool_descriptor;
 
+/* Descriptor of the batched event_csr_matvec targets (no counterpart in the reference's GPU
+ * library: brainpylib/_src/event_ops/event_csr_matvec.py:227-229 leaves the GPU translation of
+ * `event_csr_matvec_batching_p` empty).  The fields are the static parameters and operand
+ * shapes that the reference's CPU kernel reads, :152-193. */
+typedef struct {
+  uint32_t n_row;         /* CSR shape[0] */
+  uint32_t n_col;         /* CSR shape[1] */
+  uint32_t batch_size;    /* rows of the result */
+  uint32_t values_batch;  /* leading dimension of every operand; entry bi uses row bi % dim */
+  uint32_t indices_batch;
+  uint32_t indptr_batch;
+  uint32_t events_batch;
+  uint32_t nnz;           /* second dimension of indices (and of values when heterogeneous) */
+  uint8_t transpose;      /* 3 bytes of padding follow */
+} bpl_event_csr_batching_descriptor;
+
 /* lib/kernel_helper_descriptor.cuh:120-123 (DoubleSizeDescriptor): csr_matvec. */
 typedef struct {
   uint32_t n_row;
@@ -104,6 +120,10 @@ typedef struct {
  * lib/kernel_helper_descriptor.cu:34-104.  Unlike the reference's builders, which narrow
  * log_p and the weight parameters to float before widening them again, these keep the
  * doubles, so the kernels see the same log_p as the reference's CPU path. */
+size_t bpl_build_event_csr_batching_descriptor(uint32_t n_row, uint32_t n_col, uint32_t batch_size,
+                                               uint32_t values_batch, uint32_t indices_batch,
+                                               uint32_t indptr_batch, uint32_t events_batch, uint32_t nnz,
+                                               int transpose, char *out, size_t cap);
 size_t bpl_build_twouint_onebool_descriptor(uint32_t n_row, uint32_t n_col, int transpose,
                                             char *out, size_t cap);
 size_t bpl_build_double_size_descriptor(uint32_t n_row, uint32_t n_col, char *out, size_t cap);
@@ -157,6 +177,30 @@ BPL_TARGET(event_csr_matvec_homo_float_bool);
 BPL_TARGET(event_csr_matvec_homo_float_float);
 BPL_TARGET(event_csr_matvec_homo_double_bool);
 BPL_TARGET(event_csr_matvec_homo_double_double);
+
+/* ------------------------------------------------------------------------------------------
+ * event_csr_matvec_batching  (the batching rule's primitive,
+ * brainpylib/_src/event_ops/event_csr_matvec.py:112-193, which the reference runs on the CPU
+ * only; these targets have no counterpart in lib/gpu_ops.cc)
+ *   buffers = [values, indices, indptr, events, out], row-major 2-D arrays:
+ *     values   F[values_batch][1] or F[values_batch][nnz]
+ *     indices  uint32/int32[indices_batch][nnz]   indptr  uint32/int32[indptr_batch][n_row + 1]
+ *     events   bool or F [events_batch][n_row if transpose else n_col]
+ *     out      F[batch_size][n_col if transpose else n_row]
+ *   opaque  = bpl_event_csr_batching_descriptor
+ *   out[bi] = event_csr_matvec(values[bi % values_batch], indices[bi % indices_batch],
+ *                              indptr[bi % indptr_batch], events[bi % events_batch])
+ *   With one shared matrix and transpose = 0 the column indices are streamed once per eight
+ *   event vectors.
+ * ---------------------------------------------------------------------------------------- */
+BPL_TARGET(event_csr_matvec_batching_heter_float_bool);
+BPL_TARGET(event_csr_matvec_batching_heter_float_float);
+BPL_TARGET(event_csr_matvec_batching_heter_double_bool);
+BPL_TARGET(event_csr_matvec_batching_heter_double_double);
+BPL_TARGET(event_csr_matvec_batching_homo_float_bool);
+BPL_TARGET(event_csr_matvec_batching_homo_float_float);
+BPL_TARGET(event_csr_matvec_batching_homo_double_bool);
+BPL_TARGET(event_csr_matvec_batching_homo_double_double);
 
 /* ------------------------------------------------------------------------------------------
  * csr_matvec  (lib/gpu_csr_matvec.cu:563-621; launchers :84-135,:195-246,:505-560)

@@ -211,6 +211,33 @@ def event_csr_matvec(data, indices, indptr, events, *, shape, transpose=False):
   return out
 
 
+def event_csr_matvec_batching(values, indices, indptr, events, *, batch_size, shape, transpose=False):
+  """2-D operands with a leading batch dimension; entry bi reads row bi % dim of each."""
+  values = np.ascontiguousarray(values)
+  assert values.ndim == 2 and values.dtype in (np.float32, np.float64)
+  indices = np.ascontiguousarray(indices).view(np.uint32) if indices.dtype == np.int32 else np.ascontiguousarray(
+    indices, dtype=np.uint32)
+  indptr = np.ascontiguousarray(indptr).view(np.uint32) if indptr.dtype == np.int32 else np.ascontiguousarray(
+    indptr, dtype=np.uint32)
+  events = np.ascontiguousarray(events)
+  assert indices.ndim == 2 and indptr.ndim == 2 and events.ndim == 2
+  assert indptr.shape[1] == shape[0] + 1 and values.shape[1] in (1, indices.shape[1])
+  assert events.shape[1] == (shape[0] if transpose else shape[1])
+  if events.dtype == np.bool_:
+    ev_kind, ev = 0, events.view(np.uint8)
+  else:
+    assert events.dtype == values.dtype
+    ev_kind, ev = 1, events
+  out = np.empty((batch_size, shape[1] if transpose else shape[0]), dtype=values.dtype)
+  fn = (lib().oracle_event_csr_matvec_batching_f32 if values.dtype == np.float32
+        else lib().oracle_event_csr_matvec_batching_f64)
+  u = ctypes.c_uint32
+  fn(_p(values), u(values.shape[0]), u(values.shape[1]), _p(indices), u(indices.shape[0]), u(indices.shape[1]),
+     _p(indptr), u(indptr.shape[0]), _p(ev), ctypes.c_int(ev_kind), u(events.shape[0]), u(batch_size),
+     u(shape[0]), u(shape[1]), ctypes.c_int(int(transpose)), _p(out))
+  return out
+
+
 def csr_matvec(data, indices, indptr, vector, *, shape, transpose=False):
   data, indices, indptr = _csr_args(data, indices, indptr)
   vector = np.ascontiguousarray(vector, dtype=data.dtype)

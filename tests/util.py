@@ -56,3 +56,18 @@ def assert_close_reordered(got, want, abs_sum, dtype=np.float32, what=""):
   bound = ATOL + RTOL * np.abs(want) + 4 * np.finfo(dtype).eps * np.asarray(abs_sum, dtype=np.float64)
   bad = err > bound
   assert not bad.any(), "%s: %d of %d elements off; max abs err %.3e" % (what, int(bad.sum()), bad.size, float(err.max()))
+
+
+def batched_csr(shape, mean, batch, seed, dtype=np.float32):
+  """`batch` different CSR matrices of one shape with the same number of nonzeros (the same row
+  counts in another order), as 2-D arrays: data (batch, nnz), indices (batch, nnz),
+  indptr (batch, shape[0] + 1)."""
+  rng = np.random.default_rng(seed)
+  counts = np.minimum(rng.poisson(mean, size=shape[0]), shape[1])
+  data, indices, indptr = [], [], []
+  for b in range(batch):
+    ix, ip = synth.counted_csr(rng.permutation(counts), shape[1], seed=seed * 31 + b)
+    indices.append(ix)
+    indptr.append(ip)
+    data.append(rng.standard_normal(ix.shape[0]).astype(dtype))
+  return np.stack(data), np.stack(indices), np.stack(indptr)
