@@ -8,7 +8,7 @@ from typing import Tuple
 
 import torch
 
-from . import _lib
+from . import _lib, sparse_ops
 from ._tensors import FLOAT_DTYPES, as_tensor, device_of, is_index_dtype, to_device
 
 __all__ = ["event_csr_matvec", "event_csr_matvec_batching", "event_info"]
@@ -64,23 +64,79 @@ def event_csr_matvec(data, indices, indptr, events, *, shape: Tuple[int, int], t
   if indptr.shape[0] != shape[0] + 1:
     raise ValueError(f'indptr should have shape[0] + 1 = {shape[0] + 1} entries, got {indptr.shape[0]}.')
 
-  # target name, as the reference's GPU translation builds it
-  type_name = _type_name(data.dtype)
-  data_name = '_homo' if data.shape[0] == 1 else '_heter'
-  if events.dtype == torch.bool:
-    vec_type = '_bool'
-  else:
-    if events.dtype != data.dtype:
-      raise ValueError('events should be bool or have the dtype of data, '
-                       f'but we got {events.dtype} != {data.dtype}.')
-    vec_type = type_name
+  if events.dtype != torch.bool and events.dtype != data.dtype:
+    raise ValueError('events should be bool or have the dtype of data, '
+                     f'but we got {events.dtype} != {data.dtype}.')
   device = device_of(data, indices, indptr, events)
   data, indices, indptr, events = (to_device(t, device) for t in (data, indices, indptr, events))
+  if sparse_ops._wants_grad(data, events):
+    return _EventCSRMatvec.apply(data, indices, indptr, events, tuple(shape), bool(transpose))
+  return _launch(data, indices, indptr, events, shape, transpose)
+
+
+def _launch(data, indices, indptr, events, shape, transpose):
+  """The custom call itself, on checked device tensors; the target name is built as the
+  reference's GPU translation builds it."""
+  type_name = _type_name(data.dtype)
+  data_name = '_homo' if data.shape[0] == 1 else '_heter'
+  vec_type = '_bool' if events.dtype == torch.bool else type_name
   opaque = _lib.build_twouint_onebool_descriptor(shape[0], shape[1], transpose)
-  out = torch.empty(shape[1] if transpose else shape[0], dtype=data.dtype, device=device)
+  out = torch.empty(shape[1] if transpose else shape[0], dtype=data.dtype, device=data.device)
   _lib.custom_call('event_csr_matvec' + data_name + type_name + vec_type,
                    [data, indices, indptr, events, out], opaque)
   return out
+
+
+class _EventCSRMatvec(torch.autograd.Function):
+  """Differentiation rules of event_csr_matvec
+  (brainpylib/_src/event_ops/event_csr_matvec.py:439-463).  Tangent of the weights: the same
+  operator on the tangent.  Tangent of float events: the dense CSR product with the tangent.
+  Cotangent of the weights: ``events[row] * ct[col]`` per nonzero when transposed, else
+  ``events[col] * ct[row]`` (summed for a homogeneous weight, as ``inner(ct, op(1))``).
+  Cotangent of float events: the dense product of the weights with ``ct`` along the other
+  orientation (the reference passes the operands of that product in another order, :449,
+  which only type-checks for a homogeneous weight; the product meant is computed here)."""
+
+  @staticmethod
+  def forward(data, indices, indptr, events, shape, transpose):
+    return _launch(data.detach(), indices, indptr, events.detach(), shape, transpose)
+
+  @staticmethod
+  def setup_context(ctx, inputs, output):
+    data, indices, indptr, events, ctx.shape, ctx.transpose = inputs
+    ctx.save_for_backward(data, indices, indptr, events)
+    ctx.save_for_forward(data, indices, indptr, events)
+    ctx.set_materialize_grads(False)
+
+  @staticmethod
+  def backward(ctx, ct):
+    data, indices, indptr, events = ctx.saved_tensors
+    g_data = g_events = None
+    if ct is not None:
+      ct = ct.contiguous()
+      if ctx.needs_input_grad[3]:
+        g_events = sparse_ops._launch(data.detach(), indices, indptr, ct, ctx.shape, not ctx.transpose)
+      if ctx.needs_input_grad[0]:
+        if data.shape[0] == 1:
+          ones = torch.ones(1, dtype=data.dtype, device=ct.device)
+          g_data = torch.inner(ct, _launch(ones, indices, indptr, events.detach(), ctx.shape, ctx.transpose)).reshape(1)
+        else:
+          row, col = sparse_ops.csr_to_coo(indices, indptr)
+          row, col = sparse_ops._int64(row), sparse_ops._int64(col)
+          ev = events.detach().to(data.dtype)
+          g_data = ev[row] * ct[col] if ctx.transpose else ev[col] * ct[row]
+    return g_data, None, None, g_events, None, None
+
+  @staticmethod
+  def jvp(ctx, d_data, d_indices, d_indptr, d_events, *_):
+    data, indices, indptr, events = ctx.saved_tensors
+    out = None
+    if d_data is not None:
+      out = _launch(d_data.contiguous(), indices, indptr, events, ctx.shape, ctx.transpose)
+    if d_events is not None:
+      t = sparse_ops._launch(data, indices, indptr, d_events.contiguous(), ctx.shape, ctx.transpose)
+      out = t if out is None else out + t
+    return out
 
 
 def event_csr_matvec_batching(values, indices, indptr, events, *, batch_size: int, shape: Tuple[int, int],

@@ -73,8 +73,8 @@ def _type_name(dt):
   return '_float' if dt == torch.float32 else '_double'
 
 
-def _run(fn_prefix, w_kind, inp, out_dtype, suffix, *, conn_prob, shape, seed, transpose, outdim_parallel, w_a=0.0,
-         w_b=0.0):
+def _launch(fn_prefix, w_kind, inp, out_dtype, suffix, *, conn_prob, shape, seed, transpose, outdim_parallel,
+            w_a=0.0, w_b=0.0):
   n_row, n_col = (shape[1], shape[0]) if transpose else (shape[0], shape[1])
   if not (conn_prob > 0):
     raise ValueError(f'conn_prob should be in (0, 1], got {conn_prob}.')
@@ -91,6 +91,45 @@ def _run(fn_prefix, w_kind, inp, out_dtype, suffix, *, conn_prob, shape, seed, t
   out = torch.empty(n_row, dtype=out_dtype, device=device)
   _lib.custom_call(name, [inp, out], opaque)
   return out
+
+
+class _JitconnMatvec(torch.autograd.Function):
+  """Differentiation rules of the jitconn matvec primitives with respect to the input vector
+  (brainpylib/_src/jitconn_ops/event_matvec.py:242-273, matvec.py:371-409): the tangent goes
+  through the dense-vector operator with the same matrix, the cotangent through the dense-vector
+  operator with ``transpose`` and ``outdim_parallel`` both flipped, which walks the same random
+  streams along the other axis and therefore is the exact transpose of the same matrix."""
+
+  @staticmethod
+  def forward(inp, fn_prefix, w_kind, out_dtype, suffix, kw):
+    return _launch(fn_prefix, w_kind, inp.detach(), out_dtype, suffix, **kw)
+
+  @staticmethod
+  def setup_context(ctx, inputs, output):
+    _, _, ctx.w_kind, ctx.out_dtype, _, ctx.kw = inputs
+    ctx.set_materialize_grads(False)
+
+  @staticmethod
+  def backward(ctx, ct):
+    if ct is None or not ctx.needs_input_grad[0]:
+      return None, None, None, None, None, None
+    kw = dict(ctx.kw, transpose=not ctx.kw['transpose'], outdim_parallel=not ctx.kw['outdim_parallel'])
+    g = _launch('gpu_matvec', ctx.w_kind, ct.contiguous(), ct.dtype, _type_name(ct.dtype), **kw)
+    return g, None, None, None, None, None
+
+  @staticmethod
+  def jvp(ctx, d_inp, *_):
+    if d_inp is None:
+      return None
+    d_inp = d_inp.to(ctx.out_dtype)
+    return _launch('gpu_matvec', ctx.w_kind, d_inp.contiguous(), ctx.out_dtype, _type_name(ctx.out_dtype), **ctx.kw)
+
+
+def _run(fn_prefix, w_kind, inp, out_dtype, suffix, **kw):
+  if inp.is_floating_point() and (inp.requires_grad or torch.autograd.forward_ad.unpack_dual(inp).tangent is not None):
+    # move first (differentiably), so that the gradient comes back on the caller's device
+    return _JitconnMatvec.apply(to_device(inp, device_of(inp)), fn_prefix, w_kind, out_dtype, suffix, kw)
+  return _launch(fn_prefix, w_kind, inp, out_dtype, suffix, **kw)
 
 
 def _event_types(events):
