@@ -116,6 +116,21 @@ def build_event_csr_batching_descriptor(n_row, n_col, batch_size, values_batch, 
 
 
 @functools.lru_cache(maxsize=256)
+def build_csr_event_sum_descriptor(pre_size, post_size):
+  return _build("bpl_build_csr_event_sum_descriptor", ctypes.c_uint32(pre_size), ctypes.c_uint32(post_size))
+
+
+@functools.lru_cache(maxsize=256)
+def build_coo_event_sum_descriptor(conn_size, post_size):
+  return _build("bpl_build_coo_event_sum_descriptor", ctypes.c_uint32(conn_size), ctypes.c_uint32(post_size))
+
+
+@functools.lru_cache(maxsize=256)
+def build_coo_atomic_sum_descriptor(conn_size, post_size):
+  return _build("bpl_build_coo_atomic_sum_descriptor", ctypes.c_uint32(conn_size), ctypes.c_uint32(post_size))
+
+
+@functools.lru_cache(maxsize=256)
 def build_double_size_descriptor(size_x, size_y):
   return _build("bpl_build_double_size_descriptor", ctypes.c_uint32(size_x), ctypes.c_uint32(size_y))
 

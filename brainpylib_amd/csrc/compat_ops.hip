@@ -1,0 +1,151 @@
+// The older operator family of the reference that its models still call through
+// brainpylib/_src/compat: csr_event_sum with 64-bit indices, coo_event_sum and coo_atomic_sum
+// (lib/gpu_event_sum.cu, lib/gpu_atomic_sum.cu).  Same target names, buffer order and 8-byte
+// descriptors.  These are thin kernels: one lane per connection (or one wave per active
+// row), global atomics into the zeroed result.  csr_event_sum with 32-bit indices is the
+// event_csr_matvec scatter and lives with it in csr_ops.hip.
+#include "common.h"
+
+namespace bpl {
+namespace {
+
+constexpr int kThreads = 256;
+
+// One wave per row: active rows add their nonzeros into the result.
+template <typename F, typename I, bool HETER>
+__global__ __launch_bounds__(kThreads) void csr_event_sum_kernel(const uint8_t *__restrict__ events,
+                                                                 const I *__restrict__ indices,
+                                                                 const I *__restrict__ indptr,
+                                                                 const F *__restrict__ values,
+                                                                 F *__restrict__ result, uint32_t pre_size) {
+  const uint32_t waves = gridDim.x * (kThreads / kWave);
+  const uint32_t lane = static_cast<uint32_t>(lane_id());
+  const F w_homo = HETER ? F(0) : values[0];
+  for (uint32_t r = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave; r < pre_size; r += waves) {
+    if (events[r] == 0) continue;
+    const uint64_t start = static_cast<uint64_t>(indptr[r]), end = static_cast<uint64_t>(indptr[r + 1]);
+    for (uint64_t j = start + lane; j < end; j += kWave)
+      atomic_add(result + static_cast<uint64_t>(indices[j]), HETER ? values[j] : w_homo);
+  }
+}
+
+// One lane per connection: result[post_ids[i]] += value if events[pre_ids[i]].
+template <typename F, typename I, bool HETER>
+__global__ __launch_bounds__(kThreads) void coo_event_sum_kernel(const uint8_t *__restrict__ events,
+                                                                 const I *__restrict__ pre_ids,
+                                                                 const I *__restrict__ post_ids,
+                                                                 const F *__restrict__ values,
+                                                                 F *__restrict__ result, uint32_t conn_size) {
+  const F w_homo = HETER ? F(0) : values[0];
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < conn_size; i += gridDim.x * kThreads) {
+    if (events[static_cast<uint64_t>(pre_ids[i])] != 0)
+      atomic_add(result + static_cast<uint64_t>(post_ids[i]), HETER ? values[i] : w_homo);
+  }
+}
+
+// One lane per connection: result[post_ids[i]] += values[pre_ids[i]] (heter) or values[0] (homo).
+template <typename F, typename I, bool HETER>
+__global__ __launch_bounds__(kThreads) void coo_atomic_sum_kernel(const F *__restrict__ values,
+                                                                  const I *__restrict__ post_ids,
+                                                                  const I *__restrict__ pre_ids,
+                                                                  F *__restrict__ result, uint32_t conn_size) {
+  const F w_homo = HETER ? F(0) : values[0];
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < conn_size; i += gridDim.x * kThreads)
+    atomic_add(result + static_cast<uint64_t>(post_ids[i]),
+               HETER ? values[static_cast<uint64_t>(pre_ids[i])] : w_homo);
+}
+
+inline unsigned grid_for(uint32_t items, uint32_t per_block) {
+  const unsigned want = div_up(items, per_block);
+  const unsigned cap = static_cast<unsigned>(device_info().num_cu) * 16u;
+  return want < cap ? (want ? want : 1u) : cap;
+}
+
+// gpu_csr_event_sum_*: buffers = [events, indices, indptr, values, result]
+template <typename F, typename I, bool HETER>
+void csr_event_sum_entry(const char *target, hipStream_t stream, void **buffers, const char *opaque, size_t len) {
+  bpl_csr_event_sum_descriptor d;
+  if (!unpack(target, opaque, len, &d)) return;
+  if (buffers == nullptr) {
+    set_error("%s: null buffer table", target);
+    return;
+  }
+  F *result = static_cast<F *>(buffers[4]);
+  fill_zero(stream, result, d.post_size);
+  if (d.pre_size == 0 || d.post_size == 0) return;
+  hipLaunchKernelGGL((csr_event_sum_kernel<F, I, HETER>), dim3(grid_for(d.pre_size, kThreads / kWave)), dim3(kThreads),
+                     0, stream, static_cast<const uint8_t *>(buffers[0]), static_cast<const I *>(buffers[1]),
+                     static_cast<const I *>(buffers[2]), static_cast<const F *>(buffers[3]), result, d.pre_size);
+  check_launch(target);
+}
+
+// gpu_coo_event_sum_*: buffers = [events, pre_ids, post_ids, values, result]
+template <typename F, typename I, bool HETER>
+void coo_event_sum_entry(const char *target, hipStream_t stream, void **buffers, const char *opaque, size_t len) {
+  bpl_coo_sum_descriptor d;
+  if (!unpack(target, opaque, len, &d)) return;
+  if (buffers == nullptr) {
+    set_error("%s: null buffer table", target);
+    return;
+  }
+  F *result = static_cast<F *>(buffers[4]);
+  fill_zero(stream, result, d.post_size);
+  if (d.conn_size == 0 || d.post_size == 0) return;
+  hipLaunchKernelGGL((coo_event_sum_kernel<F, I, HETER>), dim3(grid_for(d.conn_size, kThreads)), dim3(kThreads), 0,
+                     stream, static_cast<const uint8_t *>(buffers[0]), static_cast<const I *>(buffers[1]),
+                     static_cast<const I *>(buffers[2]), static_cast<const F *>(buffers[3]), result, d.conn_size);
+  check_launch(target);
+}
+
+// gpu_coo_atomic_sum_homo_*: buffers = [values, post_ids, result]
+// gpu_coo_atomic_sum_heter_*: buffers = [values, post_ids, pre_ids, result]
+template <typename F, typename I, bool HETER>
+void coo_atomic_sum_entry(const char *target, hipStream_t stream, void **buffers, const char *opaque, size_t len) {
+  bpl_coo_sum_descriptor d;
+  if (!unpack(target, opaque, len, &d)) return;
+  if (buffers == nullptr) {
+    set_error("%s: null buffer table", target);
+    return;
+  }
+  F *result = static_cast<F *>(buffers[HETER ? 3 : 2]);
+  fill_zero(stream, result, d.post_size);
+  if (d.conn_size == 0 || d.post_size == 0) return;
+  const I *post_ids = static_cast<const I *>(buffers[1]);
+  const I *pre_ids = HETER ? static_cast<const I *>(buffers[2]) : post_ids;
+  hipLaunchKernelGGL((coo_atomic_sum_kernel<F, I, HETER>), dim3(grid_for(d.conn_size, kThreads)), dim3(kThreads), 0,
+                     stream, static_cast<const F *>(buffers[0]), post_ids, pre_ids, result, d.conn_size);
+  check_launch(target);
+}
+
+}  // namespace
+}  // namespace bpl
+
+#define BPL_DEFINE(name, call)                                                                   \
+  extern "C" void name(bpl_stream_t stream, void **buffers, const char *opaque, size_t opaque_len) { \
+    hipStream_t s = static_cast<hipStream_t>(stream);                                            \
+    using namespace bpl;                                                                         \
+    call(__func__, s, buffers, opaque, opaque_len);                                              \
+  }
+
+BPL_DEFINE(gpu_csr_event_sum_homo_f32_i64, (csr_event_sum_entry<float, uint64_t, false>))
+BPL_DEFINE(gpu_csr_event_sum_homo_f64_i64, (csr_event_sum_entry<double, uint64_t, false>))
+BPL_DEFINE(gpu_csr_event_sum_heter_f32_i64, (csr_event_sum_entry<float, uint64_t, true>))
+BPL_DEFINE(gpu_csr_event_sum_heter_f64_i64, (csr_event_sum_entry<double, uint64_t, true>))
+
+BPL_DEFINE(gpu_coo_event_sum_homo_f32_i32, (coo_event_sum_entry<float, uint32_t, false>))
+BPL_DEFINE(gpu_coo_event_sum_homo_f32_i64, (coo_event_sum_entry<float, uint64_t, false>))
+BPL_DEFINE(gpu_coo_event_sum_homo_f64_i32, (coo_event_sum_entry<double, uint32_t, false>))
+BPL_DEFINE(gpu_coo_event_sum_homo_f64_i64, (coo_event_sum_entry<double, uint64_t, false>))
+BPL_DEFINE(gpu_coo_event_sum_heter_f32_i32, (coo_event_sum_entry<float, uint32_t, true>))
+BPL_DEFINE(gpu_coo_event_sum_heter_f32_i64, (coo_event_sum_entry<float, uint64_t, true>))
+BPL_DEFINE(gpu_coo_event_sum_heter_f64_i32, (coo_event_sum_entry<double, uint32_t, true>))
+BPL_DEFINE(gpu_coo_event_sum_heter_f64_i64, (coo_event_sum_entry<double, uint64_t, true>))
+
+BPL_DEFINE(gpu_coo_atomic_sum_homo_f32_i32, (coo_atomic_sum_entry<float, uint32_t, false>))
+BPL_DEFINE(gpu_coo_atomic_sum_homo_f32_i64, (coo_atomic_sum_entry<float, uint64_t, false>))
+BPL_DEFINE(gpu_coo_atomic_sum_homo_f64_i32, (coo_atomic_sum_entry<double, uint32_t, false>))
+BPL_DEFINE(gpu_coo_atomic_sum_homo_f64_i64, (coo_atomic_sum_entry<double, uint64_t, false>))
+BPL_DEFINE(gpu_coo_atomic_sum_heter_f32_i32, (coo_atomic_sum_entry<float, uint32_t, true>))
+BPL_DEFINE(gpu_coo_atomic_sum_heter_f32_i64, (coo_atomic_sum_entry<float, uint64_t, true>))
+BPL_DEFINE(gpu_coo_atomic_sum_heter_f64_i32, (coo_atomic_sum_entry<double, uint32_t, true>))
+BPL_DEFINE(gpu_coo_atomic_sum_heter_f64_i64, (coo_atomic_sum_entry<double, uint64_t, true>))

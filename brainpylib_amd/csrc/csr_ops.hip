@@ -966,9 +966,29 @@ void event_csr_batching_entry(const char *target, hipStream_t stream, void **buf
   }
 }
 
+// gpu_csr_event_sum_*_i32 (lib/gpu_event_sum.cu:48-118): the event scatter under its older name
+// and buffer order, buffers = [events, indices, indptr, values, result].
+template <typename F, bool HETER>
+void csr_event_sum_i32_entry(const char *target, hipStream_t stream, void **buffers, const char *opaque,
+                             size_t opaque_len) {
+  bpl_csr_event_sum_descriptor d;
+  if (!unpack(target, opaque, opaque_len, &d)) return;
+  if (buffers == nullptr) {
+    set_error("%s: null buffer table", target);
+    return;
+  }
+  launch_scatter<F, uint8_t, HETER, kEvent>(stream, static_cast<const F *>(buffers[3]),
+                                            static_cast<const uint32_t *>(buffers[1]),
+                                            static_cast<const uint32_t *>(buffers[2]),
+                                            static_cast<const uint8_t *>(buffers[0]), static_cast<F *>(buffers[4]),
+                                            d.pre_size, d.post_size);
+  check_launch(target);
+}
+
 }  // namespace
 }  // namespace bpl
 
+using bpl::csr_event_sum_i32_entry;
 using bpl::csr_matvec_entry;
 using bpl::event_csr_batching_entry;
 using bpl::event_csr_matvec_entry;
@@ -1015,3 +1035,8 @@ BPL_DEFINE(event_csr_matvec_batching_homo_float_bool, (event_csr_batching_entry<
 BPL_DEFINE(event_csr_matvec_batching_homo_float_float, (event_csr_batching_entry<float, float, false>(__func__, s, buffers, opaque, opaque_len)))
 BPL_DEFINE(event_csr_matvec_batching_homo_double_bool, (event_csr_batching_entry<double, uint8_t, false>(__func__, s, buffers, opaque, opaque_len)))
 BPL_DEFINE(event_csr_matvec_batching_homo_double_double, (event_csr_batching_entry<double, double, false>(__func__, s, buffers, opaque, opaque_len)))
+
+BPL_DEFINE(gpu_csr_event_sum_homo_f32_i32, (csr_event_sum_i32_entry<float, false>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(gpu_csr_event_sum_homo_f64_i32, (csr_event_sum_i32_entry<double, false>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(gpu_csr_event_sum_heter_f32_i32, (csr_event_sum_i32_entry<float, true>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(gpu_csr_event_sum_heter_f64_i32, (csr_event_sum_i32_entry<double, true>(__func__, s, buffers, opaque, opaque_len)))

@@ -42,6 +42,12 @@ PYBIND11_MODULE(gpu_ops, m) {
           return BPL_PACK(bpl_build_event_csr_batching_descriptor, n_row, n_col, batch_size, values_batch,
                           indices_batch, indptr_batch, events_batch, nnz, transpose ? 1 : 0);
         });
+  m.def("build_csr_event_sum_descriptor",
+        [](uint32_t pre_size, uint32_t post_size) { return BPL_PACK(bpl_build_csr_event_sum_descriptor, pre_size, post_size); });
+  m.def("build_coo_event_sum_descriptor",
+        [](uint32_t conn_size, uint32_t post_size) { return BPL_PACK(bpl_build_coo_event_sum_descriptor, conn_size, post_size); });
+  m.def("build_coo_atomic_sum_descriptor",
+        [](uint32_t conn_size, uint32_t post_size) { return BPL_PACK(bpl_build_coo_atomic_sum_descriptor, conn_size, post_size); });
   m.def("build_twouint_onebool_descriptor", [](uint32_t x, uint32_t y, bool b) {
     return BPL_PACK(bpl_build_twouint_onebool_descriptor, x, y, b ? 1 : 0);
   });

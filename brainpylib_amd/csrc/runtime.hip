@@ -127,6 +127,8 @@ uint32_t *stream_counters(hipStream_t stream) {
 static_assert(sizeof(bpl_twouint_onebool_descriptor) == 12, "TwoUintOneBoolDescriptor is 12 bytes");
 static_assert(offsetof(bpl_twouint_onebool_descriptor, transpose) == 8, "bool at offset 8");
 static_assert(sizeof(bpl_event_csr_batching_descriptor) == 36, "batching descriptor is 36 bytes");
+static_assert(sizeof(bpl_csr_event_sum_descriptor) == 8 && sizeof(bpl_coo_sum_descriptor) == 8,
+              "CSREventSumDescriptor / COOEventSumDescriptor / COOAtomicSumDescriptor are 8 bytes");
 static_assert(sizeof(bpl_double_size_descriptor) == 8, "DoubleSizeDescriptor is 8 bytes");
 static_assert(sizeof(bpl_nonzero_descriptor) == 8, "NonZeroDescriptor is 8 bytes");
 static_assert(sizeof(bpl_jitconn_prob_homo_descriptor) == 24, "JITConnProbHomoDescriptor is 24 bytes");
@@ -172,6 +174,21 @@ size_t bpl_build_event_csr_batching_descriptor(uint32_t n_row, uint32_t n_col, u
   d.events_batch = events_batch;
   d.nnz = nnz;
   d.transpose = transpose ? 1 : 0;
+  return pack(d, out, cap);
+}
+
+size_t bpl_build_csr_event_sum_descriptor(uint32_t pre_size, uint32_t post_size, char *out, size_t cap) {
+  bpl_csr_event_sum_descriptor d{pre_size, post_size};
+  return pack(d, out, cap);
+}
+
+size_t bpl_build_coo_event_sum_descriptor(uint32_t conn_size, uint32_t post_size, char *out, size_t cap) {
+  bpl_coo_sum_descriptor d{conn_size, post_size};
+  return pack(d, out, cap);
+}
+
+size_t bpl_build_coo_atomic_sum_descriptor(uint32_t conn_size, uint32_t post_size, char *out, size_t cap) {
+  bpl_coo_sum_descriptor d{conn_size, post_size};
   return pack(d, out, cap);
 }
 

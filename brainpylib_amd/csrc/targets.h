@@ -91,10 +91,37 @@
   X(event_csr_matvec_batching_homo_double_bool)      \
   X(event_csr_matvec_batching_homo_double_double)
 
+#define BPL_COMPAT_TARGETS(X) \
+  X(gpu_csr_event_sum_homo_f32_i32) \
+  X(gpu_csr_event_sum_homo_f32_i64) \
+  X(gpu_csr_event_sum_homo_f64_i32) \
+  X(gpu_csr_event_sum_homo_f64_i64) \
+  X(gpu_csr_event_sum_heter_f32_i32) \
+  X(gpu_csr_event_sum_heter_f32_i64) \
+  X(gpu_csr_event_sum_heter_f64_i32) \
+  X(gpu_csr_event_sum_heter_f64_i64) \
+  X(gpu_coo_event_sum_homo_f32_i32) \
+  X(gpu_coo_event_sum_homo_f32_i64) \
+  X(gpu_coo_event_sum_homo_f64_i32) \
+  X(gpu_coo_event_sum_homo_f64_i64) \
+  X(gpu_coo_event_sum_heter_f32_i32) \
+  X(gpu_coo_event_sum_heter_f32_i64) \
+  X(gpu_coo_event_sum_heter_f64_i32) \
+  X(gpu_coo_event_sum_heter_f64_i64) \
+  X(gpu_coo_atomic_sum_homo_f32_i32) \
+  X(gpu_coo_atomic_sum_homo_f32_i64) \
+  X(gpu_coo_atomic_sum_homo_f64_i32) \
+  X(gpu_coo_atomic_sum_homo_f64_i64) \
+  X(gpu_coo_atomic_sum_heter_f32_i32) \
+  X(gpu_coo_atomic_sum_heter_f32_i64) \
+  X(gpu_coo_atomic_sum_heter_f64_i32) \
+  X(gpu_coo_atomic_sum_heter_f64_i64)
+
 #define BPL_ALL_TARGETS(X)  \
   BPL_EVENT_CSR_TARGETS(X)  \
   BPL_EVENT_CSR_BATCHING_TARGETS(X) \
   BPL_CSR_TARGETS(X)        \
   BPL_JITCONN_TARGETS(X)    \
   BPL_MATMAT_TARGETS(X)     \
-  BPL_NONZERO_TARGETS(X)
+  BPL_NONZERO_TARGETS(X)    \
+  BPL_COMPAT_TARGETS(X)

@@ -69,6 +69,19 @@ typedef struct {
   uint8_t transpose;      /* 3 bytes of padding follow */
 } bpl_event_csr_batching_descriptor;
 
+/* lib/gpu_event_sum.cuh:10-13 (CSREventSumDescriptor): gpu_csr_event_sum_*. */
+typedef struct {
+  uint32_t pre_size;  /* rows of the CSR structure = length of events */
+  uint32_t post_size; /* length of the result */
+} bpl_csr_event_sum_descriptor;
+
+/* lib/gpu_event_sum.cuh:38-41 (COOEventSumDescriptor) and lib/gpu_atomic_sum.cuh:10-13
+ * (COOAtomicSumDescriptor): gpu_coo_event_sum_*, gpu_coo_atomic_sum_*. */
+typedef struct {
+  uint32_t conn_size; /* number of connections (length of post_ids) */
+  uint32_t post_size; /* length of the result */
+} bpl_coo_sum_descriptor;
+
 /* lib/kernel_helper_descriptor.cuh:120-123 (DoubleSizeDescriptor): csr_matvec. */
 typedef struct {
   uint32_t n_row;
@@ -124,6 +137,10 @@ size_t bpl_build_event_csr_batching_descriptor(uint32_t n_row, uint32_t n_col, u
                                                uint32_t values_batch, uint32_t indices_batch,
                                                uint32_t indptr_batch, uint32_t events_batch, uint32_t nnz,
                                                int transpose, char *out, size_t cap);
+/* lib/gpu_event_sum.cu:215-218,282-285, lib/gpu_atomic_sum.cu (build_*_descriptor) */
+size_t bpl_build_csr_event_sum_descriptor(uint32_t pre_size, uint32_t post_size, char *out, size_t cap);
+size_t bpl_build_coo_event_sum_descriptor(uint32_t conn_size, uint32_t post_size, char *out, size_t cap);
+size_t bpl_build_coo_atomic_sum_descriptor(uint32_t conn_size, uint32_t post_size, char *out, size_t cap);
 size_t bpl_build_twouint_onebool_descriptor(uint32_t n_row, uint32_t n_col, int transpose,
                                             char *out, size_t cap);
 size_t bpl_build_double_size_descriptor(uint32_t n_row, uint32_t n_col, char *out, size_t cap);
@@ -201,6 +218,48 @@ BPL_TARGET(event_csr_matvec_batching_homo_float_bool);
 BPL_TARGET(event_csr_matvec_batching_homo_float_float);
 BPL_TARGET(event_csr_matvec_batching_homo_double_bool);
 BPL_TARGET(event_csr_matvec_batching_homo_double_double);
+
+/* ------------------------------------------------------------------------------------------
+ * The older operator family kept by brainpylib/_src/compat (lib/gpu_ops.cc:27-58).
+ *   gpu_csr_event_sum_{homo,heter}_{f32,f64}_{i32,i64}  (lib/gpu_event_sum.cu:27-118,222-279)
+ *     buffers = [events bool[pre_size], indices I[nnz], indptr I[pre_size + 1],
+ *                values F[1] | F[nnz], result F[post_size]];  opaque = bpl_csr_event_sum_descriptor
+ *     result[indices[j]] += values[j] for every j in row r, for every r with events[r]
+ *   gpu_coo_event_sum_{homo,heter}_{f32,f64}_{i32,i64}  (lib/gpu_event_sum.cu:121-210,288-345)
+ *     buffers = [events bool[.], pre_ids I[conn_size], post_ids I[conn_size],
+ *                values F[1] | F[conn_size], result F[post_size]];  opaque = bpl_coo_sum_descriptor
+ *     result[post_ids[i]] += values[i] for every connection i with events[pre_ids[i]]
+ *   gpu_coo_atomic_sum_homo_{f32,f64}_{i32,i64}  (lib/gpu_atomic_sum.cu:27-60)
+ *     buffers = [values F[1], post_ids I[conn_size], result F[post_size]]
+ *   gpu_coo_atomic_sum_heter_{f32,f64}_{i32,i64}  (lib/gpu_atomic_sum.cu:62-98)
+ *     buffers = [values F[.], post_ids I[conn_size], pre_ids I[conn_size], result F[post_size]]
+ *     result[post_ids[i]] += values[pre_ids[i]];  opaque = bpl_coo_sum_descriptor
+ *   I is a 32- or 64-bit integer read as unsigned.  The result is zeroed by the call.
+ * ---------------------------------------------------------------------------------------- */
+BPL_TARGET(gpu_csr_event_sum_homo_f32_i32);
+BPL_TARGET(gpu_csr_event_sum_homo_f32_i64);
+BPL_TARGET(gpu_csr_event_sum_homo_f64_i32);
+BPL_TARGET(gpu_csr_event_sum_homo_f64_i64);
+BPL_TARGET(gpu_csr_event_sum_heter_f32_i32);
+BPL_TARGET(gpu_csr_event_sum_heter_f32_i64);
+BPL_TARGET(gpu_csr_event_sum_heter_f64_i32);
+BPL_TARGET(gpu_csr_event_sum_heter_f64_i64);
+BPL_TARGET(gpu_coo_event_sum_homo_f32_i32);
+BPL_TARGET(gpu_coo_event_sum_homo_f32_i64);
+BPL_TARGET(gpu_coo_event_sum_homo_f64_i32);
+BPL_TARGET(gpu_coo_event_sum_homo_f64_i64);
+BPL_TARGET(gpu_coo_event_sum_heter_f32_i32);
+BPL_TARGET(gpu_coo_event_sum_heter_f32_i64);
+BPL_TARGET(gpu_coo_event_sum_heter_f64_i32);
+BPL_TARGET(gpu_coo_event_sum_heter_f64_i64);
+BPL_TARGET(gpu_coo_atomic_sum_homo_f32_i32);
+BPL_TARGET(gpu_coo_atomic_sum_homo_f32_i64);
+BPL_TARGET(gpu_coo_atomic_sum_homo_f64_i32);
+BPL_TARGET(gpu_coo_atomic_sum_homo_f64_i64);
+BPL_TARGET(gpu_coo_atomic_sum_heter_f32_i32);
+BPL_TARGET(gpu_coo_atomic_sum_heter_f32_i64);
+BPL_TARGET(gpu_coo_atomic_sum_heter_f64_i32);
+BPL_TARGET(gpu_coo_atomic_sum_heter_f64_i64);
 
 /* ------------------------------------------------------------------------------------------
  * csr_matvec  (lib/gpu_csr_matvec.cu:563-621; launchers :84-135,:195-246,:505-560)

@@ -248,6 +248,47 @@ def csr_matvec(data, indices, indptr, vector, *, shape, transpose=False):
   return out
 
 
+def _wide(ids):
+  ids = np.ascontiguousarray(ids)
+  if ids.dtype == np.int32:
+    ids = ids.view(np.uint32)
+  return ids.astype(np.uint64)
+
+
+def coo_atomic_sum(values, post_ids, post_num, pre_ids=None):
+  values = np.atleast_1d(np.ascontiguousarray(values))
+  assert values.dtype in (np.float32, np.float64)
+  post = _wide(post_ids)
+  pre = post if values.shape[0] == 1 else _wide(pre_ids)
+  assert pre.shape == post.shape
+  out = np.empty(post_num, dtype=values.dtype)
+  fn = lib().oracle_coo_atomic_sum_f32 if values.dtype == np.float32 else lib().oracle_coo_atomic_sum_f64
+  fn(_p(values), ctypes.c_uint32(values.shape[0]), _p(post), _p(pre), ctypes.c_uint32(post.shape[0]),
+     ctypes.c_uint32(post_num), _p(out))
+  return out
+
+
+def coo_event_sum(events, pre_ids, post_ids, post_num, values):
+  values = np.atleast_1d(np.ascontiguousarray(values))
+  assert values.dtype in (np.float32, np.float64)
+  events = np.ascontiguousarray(events)
+  assert events.dtype == np.bool_
+  pre, post = _wide(pre_ids), _wide(post_ids)
+  assert pre.shape == post.shape and values.shape[0] in (1, pre.shape[0])
+  out = np.empty(post_num, dtype=values.dtype)
+  fn = lib().oracle_coo_event_sum_f32 if values.dtype == np.float32 else lib().oracle_coo_event_sum_f64
+  fn(_p(events.view(np.uint8)), _p(pre), _p(post), _p(values), ctypes.c_uint32(values.shape[0]),
+     ctypes.c_uint32(pre.shape[0]), ctypes.c_uint32(post_num), _p(out))
+  return out
+
+
+def csr_event_sum(events, pre2post, post_num, values):
+  """The older name of the event scatter; 64-bit index arrays are narrowed (the index width of
+  lib/cpu_event_sum.cc's template does not enter the arithmetic)."""
+  indices, indptr = (np.ascontiguousarray(a).astype(np.uint32) for a in pre2post)
+  return event_csr_matvec(values, indices, indptr, events, shape=(len(events), post_num), transpose=True)
+
+
 _EVENT_KINDS = {np.dtype(np.bool_): 0, np.dtype(np.int32): 1, np.dtype(np.int64): 2,
                 np.dtype(np.float32): 3, np.dtype(np.float64): 4}
 

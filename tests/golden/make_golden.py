@@ -1,8 +1,10 @@
 """Writes the golden fixtures in this directory by running the reference's own CPU kernels
-(lib/cpu_jitconn_*.cpp, lib/cpu_event_sum.cc), compiled unmodified by `make -C oracle ref`.
-Runs only where the reference tree is mounted; the fixtures it writes are committed.
+(lib/cpu_jitconn_*.cpp, lib/cpu_event_sum.cc, lib/cpu_atomic_sum.cc), compiled unmodified by
+`make -C oracle ref`.  Runs only where the reference tree is mounted; the fixtures it writes are
+committed.
 
-    python tests/golden/make_golden.py
+    python tests/golden/make_golden.py            # all fixtures
+    python tests/golden/make_golden.py compat     # only compat_cpu_reference.npz
 
 jitconn_cpu_reference.npz
     the reference CPU backend as it ships: ONE sequential generator per matrix.  For every case
@@ -13,6 +15,9 @@ jitconn_cpu_reference_streams.npz
     generator contract of the HIP kernels.
 event_sum_cpu_reference.npz
     lib/cpu_event_sum.cc on seeded CSR matrices (event_csr_matvec, transpose=True, bool events).
+compat_cpu_reference.npz
+    lib/cpu_atomic_sum.cc (coo_atomic_sum, homogeneous and heterogeneous, 32- and 64-bit ids) and
+    the 64-bit instantiation of lib/cpu_event_sum.cc, on seeded random connections.
 """
 import json
 import os
@@ -66,7 +71,41 @@ def run_ref(inp, meta, *, n_row=None, n_col=None, seed=None, sub=None):
     dense=meta["dense"])
 
 
+def compat_fixture():
+  out = {}
+  i = 0
+  for pre, post, conn in [(200, 200, 20000), (50, 300, 4000), (300, 7, 5000), (1, 1, 10)]:
+    for homo in (True, False):
+      for dt in (np.float32, np.float64):
+        for wide in (False, True):
+          rng = np.random.default_rng(900 + i)
+          pre_ids = rng.integers(0, pre, size=conn).astype(np.int64 if wide else np.int32)
+          post_ids = rng.integers(0, post, size=conn).astype(np.int64 if wide else np.int32)
+          values = np.array([0.37], dtype=dt) if homo else rng.standard_normal(pre).astype(dt)
+          out["as_values_%d" % i], out["as_pre_%d" % i], out["as_post_%d" % i] = values, pre_ids, post_ids
+          out["as_num_%d" % i] = np.array(post)
+          out["as_out_%d" % i] = ref.coo_atomic_sum(values, post_ids, post, None if homo else pre_ids, wide=wide)
+          i += 1
+  j = 0
+  for shape in [(100, 200), (1000, 10), (2, 10000)]:
+    for homo in (True, False):
+      for dt in (np.float32, np.float64):
+        indices, indptr = synth.bernoulli_csr(shape[0], shape[1], 0.4, seed=300 + j)
+        rng = np.random.default_rng(700 + j)
+        data = np.array([1.5], dtype=dt) if homo else rng.standard_normal(indices.shape[0]).astype(dt)
+        events = rng.random(shape[0]) < 0.2
+        out["es_data_%d" % j], out["es_events_%d" % j], out["es_shape_%d" % j] = data, events, np.array(shape)
+        out["es_indices_%d" % j], out["es_indptr_%d" % j] = indices.astype(np.int64), indptr.astype(np.int64)
+        out["es_out_%d" % j] = ref.csr_event_sum(data, indices, indptr, events, shape=shape, wide=True)
+        j += 1
+  np.savez_compressed(os.path.join(HERE, "compat_cpu_reference.npz"), **out)
+  print("wrote", i, "coo_atomic_sum cases and", j, "64-bit csr_event_sum cases")
+
+
 def main():
+  compat_fixture()
+  if len(sys.argv) > 1 and sys.argv[1] == "compat":
+    return
   assert ref.available(), "run `make -C oracle ref` first"
   seq, streams = {}, {}
   for i, (inp, meta) in enumerate(jitconn_cases()):
