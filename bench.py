@@ -116,9 +116,10 @@ def main():
   ap.add_argument("--warmup", type=int, default=20)
   ap.add_argument("--skip-extra", action="store_true", help="only the headline workload")
   ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU baseline")
-  ap.add_argument("--pmc", choices=["gather", "jitconn"], default=None,
+  ap.add_argument("--pmc", choices=["gather", "scatter", "jitconn"], default=None,
                   help="counter-collection mode for rocprofv3 --pmc.  gather: three plain copies of 400 MB "
-                       "(the calibration kernel) and three calls of the headline kernel.  jitconn: three calls "
+                       "(the calibration kernel) and three calls of the headline kernel.  scatter: three calls of "
+                       "the same matrix with transpose=True.  jitconn: three calls "
                        "of jitconn event matvec (1e6 x 1e6, p=0.001) in both walks.  Nothing else runs.")
   ap.add_argument("--reference-shapes", action="store_true",
                   help="instead of the headline run: the shapes of the reference's own benchmark scripts "
@@ -176,6 +177,13 @@ def main():
                                   transpose=True)
   got_s = bpl.event_csr_matvec(data, indices, indptr, events, shape=c["shape"], transpose=True).cpu().numpy()
   check(got_s, want_s, "event_csr_matvec scatter 1e8 nnz", mag_s)
+
+  if args.pmc == "scatter":
+    for _ in range(3):
+      bpl.event_csr_matvec(data, indices, indptr, events, shape=c["shape"], transpose=True)
+    torch.cuda.synchronize()
+    log("pmc mode done")
+    return
 
   if args.pmc == "gather":
     src = torch.empty(100_000_000, dtype=torch.float32, device=dev).normal_()

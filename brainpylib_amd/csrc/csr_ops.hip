@@ -147,11 +147,64 @@ __global__ __launch_bounds__(kScatterThreads) void csr_scatter_kernel(
 constexpr int kWinThreads = 1024;
 constexpr int kWinMaxRows = 2048;  // rows per workgroup = capacity of the active-row list
 
+// Active rows of the whole matrix, gathered once into a list in device memory (any order):
+// (first nonzero, length) per row whose input is nonzero and that has nonzeros, plus the input
+// value in dense mode.  The window kernel's row groups then take equal shares of the LIST, so
+// their work does not depend on where in the matrix the activity is.  One atomic per workgroup
+// reserves the list positions.
+template <typename F, typename VT, int MODE>
+__global__ __launch_bounds__(kWinThreads) void collect_active_rows_kernel(
+    const uint32_t *__restrict__ indptr, const VT *__restrict__ x, uint32_t n_row, uint32_t *__restrict__ counter,
+    uint2 *__restrict__ list, F *__restrict__ scales, NnzGate gate) {
+  if (!gate.open(indptr, n_row)) return;
+  constexpr uint32_t kWaves = kWinThreads / kWave;
+  __shared__ uint32_t s_off[kWaves];
+  __shared__ uint32_t s_base;
+  const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const uint32_t r = blockIdx.x * kWinThreads + tid;
+  bool on = false;
+  uint32_t start = 0, len = 0;
+  F scale = F(1);
+  if (r < n_row) {
+    if (MODE == kEvent) {
+      on = is_event(x[r]);
+    } else {
+      scale = static_cast<F>(x[r]);
+      on = scale != F(0);  // a zero input adds nothing
+    }
+    if (on) {
+      start = indptr[r];
+      len = indptr[r + 1] - start;
+      on = len != 0;
+    }
+  }
+  const uint64_t mask = __ballot(on);
+  if (lane == 0) s_off[wave] = static_cast<uint32_t>(__popcll(mask));
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t total = 0;
+    for (uint32_t w = 0; w < kWaves; ++w) {
+      const uint32_t c = s_off[w];
+      s_off[w] = total;
+      total += c;
+    }
+    s_base = total ? atomicAdd(counter, total) : 0u;
+  }
+  __syncthreads();
+  if (on) {
+    const uint32_t k = s_base + s_off[wave] + static_cast<uint32_t>(__popcll(mask & ((1ull << lane) - 1ull)));
+    list[k] = make_uint2(start, len);
+    if (MODE == kDense) scales[k] = scale;
+  }
+}
+
 template <typename F, typename VT, bool HETER, int MODE>
 __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
     const VT *__restrict__ x, F *__restrict__ y, uint32_t n_row, uint32_t n_col, uint32_t rows_per_wg,
-    uint32_t win, uint32_t n_win, F *__restrict__ partial, uint32_t *__restrict__ done_counter, NnzGate gate) {
+    uint32_t win, uint32_t n_win, F *__restrict__ partial, uint32_t *__restrict__ done_counter, NnzGate gate,
+    const uint32_t *__restrict__ active_count, const uint2 *__restrict__ active_list,
+    const F *__restrict__ active_scales) {
   if (!gate.open(indptr, n_row)) return;
   extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
   F *window = reinterpret_cast<F *>(smem_raw);
@@ -163,22 +216,48 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid % kWave, wave = tid / kWave;
   constexpr uint32_t kWaves = kWinThreads / kWave;
-  const uint32_t b = blockIdx.x % n_win, g = blockIdx.x / n_win;
+  // Workgroups are dealt to the 8 XCDs round robin by blockIdx.  The n_win workgroups of one row
+  // group read the same index and weight runs, so they are renumbered to sit on one XCD and
+  // share its L2: ids [x * per_xcd, (x + 1) * per_xcd) belong to XCD x.
+  uint32_t id = blockIdx.x;
+  {
+    constexpr uint32_t kXcds = 8;
+    const uint32_t per_xcd = gridDim.x / kXcds;
+    if (id < per_xcd * kXcds) id = (id % kXcds) * per_xcd + id / kXcds;
+  }
+  const uint32_t b = id % n_win, g = id / n_win;
   const uint32_t c0 = b * win;
   const uint32_t width = (c0 + win <= n_col) ? win : n_col - c0;
 
   for (uint32_t i = tid; i < width; i += kWinThreads) window[i] = F(0);
   const F w_homo = HETER ? F(0) : data[0];
 
-  // The group's rows are taken kWinMaxRows at a time (the capacity of the active-row list).
-  for (uint32_t chunk0 = 0; chunk0 < rows_per_wg; chunk0 += kWinMaxRows) {
-  const uint32_t chunk_rows = (rows_per_wg - chunk0 < kWinMaxRows) ? rows_per_wg - chunk0 : kWinMaxRows;
-  if (static_cast<uint64_t>(g) * rows_per_wg + chunk0 >= n_row) break;  // uniform: no rows left
-  if (tid == 0) s_count = 0, s_next = kWaves;
+  // Source of the active rows: this group's share of the list made by collect_active_rows_kernel,
+  // or (active_list == nullptr) the group's own rows_per_wg rows, tested here.  Either way they are
+  // taken kWinMaxRows at a time, the capacity of the list in LDS.
+  uint32_t span_lo = 0, span_hi = rows_per_wg;
+  if (active_list != nullptr) {
+    const uint32_t total = *active_count;
+    const uint32_t groups = gridDim.x / n_win;
+    span_lo = static_cast<uint32_t>(static_cast<uint64_t>(g) * total / groups);
+    span_hi = static_cast<uint32_t>(static_cast<uint64_t>(g + 1) * total / groups);
+  }
+  for (uint32_t chunk0 = span_lo; chunk0 < span_hi; chunk0 += kWinMaxRows) {
+  const uint32_t chunk_rows = (span_hi - chunk0 < kWinMaxRows) ? span_hi - chunk0 : kWinMaxRows;
+  if (active_list == nullptr && static_cast<uint64_t>(g) * rows_per_wg + chunk0 >= n_row) break;  // uniform
+  if (tid == 0) s_count = (active_list != nullptr) ? chunk_rows : 0u, s_next = kWaves;
   __syncthreads();
 
-  // active rows of the chunk (order does not matter)
-  for (uint32_t t0 = 0; t0 < chunk_rows; t0 += kWinThreads) {
+  if (active_list != nullptr) {
+    for (uint32_t i = tid; i < chunk_rows; i += kWinThreads) {
+      const uint2 e = active_list[chunk0 + i];
+      s_start[i] = e.x;
+      s_len[i] = e.y;
+      if (MODE == kDense) s_scale[i] = active_scales[chunk0 + i];
+    }
+  }
+  // else: active rows of the chunk, tested here (order does not matter)
+  for (uint32_t t0 = 0; active_list == nullptr && t0 < chunk_rows; t0 += kWinThreads) {
     const uint32_t r = g * rows_per_wg + chunk0 + t0 + tid;
     bool on = false;
     uint32_t start = 0, len = 0;
@@ -210,19 +289,53 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
   __syncthreads();
   const uint32_t count = s_count;
 
-  // waves take active rows from a shared counter; full steps of U*64 nonzeros run unguarded
+  // Waves take active rows from a shared counter and walk them in steps of U*64 nonzeros.  The
+  // column indices of the next step (of this row or of the next row taken) are requested
+  // before this step's weights are loaded and added, so that the two latencies overlap.
   constexpr int U = 8;
-  auto step = [&](const uint32_t *ip, const F *dp, uint32_t b0, uint32_t len, F scale, bool guard) {
-    uint32_t rel[U];
+  auto load_rel = [&](const uint32_t *ip, uint32_t b0, uint32_t len, uint32_t (&rel)[U]) {
+    if (b0 + U * kWave <= len) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const uint32_t j = b0 + u * kWave + lane;
-      rel[u] = 0xffffffffu;  // outside every window
-      if (!guard || j < len) rel[u] = ip[j] - c0;
+      for (int u = 0; u < U; ++u) rel[u] = ip[b0 + u * kWave + lane] - c0;
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t j = b0 + u * kWave + lane;
+        rel[u] = 0xffffffffu;  // outside every window
+        if (j < len) rel[u] = ip[j] - c0;
+      }
     }
+  };
+  uint32_t k = wave;
+  uint32_t start = 0, len = 0, b0 = 0;
+  F scale = F(1);
+  uint32_t rel[U];
+  if (k < count) {
+    start = s_start[k], len = s_len[k];
+    if (MODE == kDense) scale = s_scale[k];
+    load_rel(indices + start, 0, len, rel);
+  }
+  while (k < count) {
+    // where the next step is
+    uint32_t nk = k, nstart = start, nlen = len, nb0 = b0 + U * kWave;
+    F nscale = scale;
+    if (nb0 >= len) {
+      uint32_t t = 0;
+      if (lane == 0) t = atomicAdd(&s_next, 1u);
+      nk = __builtin_amdgcn_readfirstlane(t);
+      nb0 = 0;
+      if (nk < count) {
+        nstart = s_start[nk], nlen = s_len[nk];
+        if (MODE == kDense) nscale = s_scale[nk];
+      }
+    }
+    uint32_t nrel[U];
+    if (nk < count) load_rel(indices + nstart, nb0, nlen, nrel);
+    // this step: all weight loads first, then the LDS atomics
+    const F *dp = data + (HETER ? start : 0u);
     F w[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {  // all data loads of the step first, then the LDS atomics
+    for (int u = 0; u < U; ++u) {
       w[u] = w_homo;
       if (HETER && rel[u] < width) w[u] = dp[b0 + u * kWave + lane];
     }
@@ -230,19 +343,9 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     for (int u = 0; u < U; ++u) {
       if (rel[u] < width) atomicAdd(&window[rel[u]], (MODE == kDense) ? static_cast<F>(scale * w[u]) : w[u]);
     }
-  };
-  uint32_t k = wave;
-  while (k < count) {
-    const uint32_t start = s_start[k], len = s_len[k];
-    const F scale = (MODE == kDense) ? s_scale[k] : F(1);
-    const uint32_t *ip = indices + start;
-    const F *dp = data + (HETER ? start : 0u);
-    uint32_t b0 = 0;
-    for (; b0 + U * kWave <= len; b0 += U * kWave) step(ip, dp, b0, len, scale, false);
-    if (b0 < len) step(ip, dp, b0, len, scale, true);
-    uint32_t nk = 0;
-    if (lane == 0) nk = atomicAdd(&s_next, 1u);
-    k = __builtin_amdgcn_readfirstlane(nk);
+    k = nk, start = nstart, len = nlen, b0 = nb0, scale = nscale;
+#pragma unroll
+    for (int u = 0; u < U; ++u) rel[u] = nrel[u];
   }
   __syncthreads();  // the lists and counters are reused by the next chunk; the window is complete after the last
   }
@@ -294,8 +397,10 @@ template <typename F>
 __global__ __launch_bounds__(256) void sum_partials_kernel(const F *__restrict__ partial, F *__restrict__ y,
                                                            uint32_t n_col, uint32_t groups,
                                                            const uint32_t *__restrict__ indptr, uint32_t n_row,
-                                                           NnzGate gate) {
+                                                           NnzGate gate, uint32_t *__restrict__ reset) {
   if (!gate.open(indptr, n_row)) return;
+  // the active-row counter of this call is left at zero for the next one
+  if (reset != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *reset = 0u;
   const uint32_t c = blockIdx.x * 256u + threadIdx.x;
   if (c >= n_col) return;
   F acc = F(0);
@@ -537,7 +642,10 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
     if (static_cast<size_t>(n_col) * 16 <= 131072 && n_row <= 16 * kWinMaxRows && want_groups > 16) want_groups = 16;
     uint32_t rows_per_wg = div_up(n_row, want_groups);
     if (rows_per_wg < 64) rows_per_wg = 64;
-    const unsigned groups = div_up(n_row, rows_per_wg);
+    // Large matrices: the active rows are first gathered into one list (a launch of its own) and
+    // the row groups share the list evenly; small ones find their active rows themselves.
+    const bool use_list = n_row > 16 * kWinMaxRows;
+    const unsigned groups = use_list ? want_groups : div_up(n_row, rows_per_wg);
     // The window kernel hands whole rows to waves, one after the other: with more than a few
     // windows it only beats the direct atomics when rows are long (64 nonzeros on average).
     NnzGate window_gate = kAlways;
@@ -565,20 +673,46 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
       // Per-row-group partial outputs in scratch memory, summed by a second kernel (no global
       // atomics, no zero fill), as long as they stay small; else atomics into the zeroed y.
       const size_t partial_bytes = static_cast<size_t>(groups) * n_col * sizeof(F);
-      F *partial = nullptr;
-      if (groups > 1 && partial_bytes <= (static_cast<size_t>(64) << 20))
-        partial = static_cast<F *>(stream_workspace(stream, partial_bytes));
+      const bool want_partial = groups > 1 && partial_bytes <= (static_cast<size_t>(64) << 20);
+      // workspace: [active-row list][dense mode: their input values][partial outputs]
+      auto round_up = [](size_t v) { return (v + 255) / 256 * 256; };
+      const size_t list_off = 0, list_sz = use_list ? round_up(static_cast<size_t>(n_row) * sizeof(uint2)) : 0;
+      const size_t scale_sz = (use_list && MODE == kDense) ? round_up(static_cast<size_t>(n_row) * sizeof(F)) : 0;
+      const size_t partial_off = list_sz + scale_sz;
+      const size_t ws_bytes = partial_off + (want_partial ? partial_bytes : 0);
+      unsigned char *ws = ws_bytes ? static_cast<unsigned char *>(stream_workspace(stream, ws_bytes)) : nullptr;
+      uint32_t *counters = use_list ? stream_counters(stream) : nullptr;
+      if (ws_bytes != 0 && (ws == nullptr || (use_list && counters == nullptr))) {
+        // no scratch memory: the direct kernel needs none
+        bpl_clear_error();
+        fill_zero(stream, y, n_col);
+        hipLaunchKernelGGL((csr_scatter_kernel<F, VT, HETER, MODE>), dim3(div_up(n_row, kScatterRows)),
+                           dim3(kScatterThreads), 0, stream, data, indices, indptr, x, y, n_row, kAlways);
+        return;
+      }
+      F *partial = want_partial ? reinterpret_cast<F *>(ws + partial_off) : nullptr;
+      uint2 *active_list = use_list ? reinterpret_cast<uint2 *>(ws + list_off) : nullptr;
+      F *active_scales = scale_sz ? reinterpret_cast<F *>(ws + list_sz) : nullptr;
+      uint32_t *active_count = use_list ? counters + 1 : nullptr;  // slot 0 is the last-workgroup counter
       const bool gated = n_win > 4;
-      if (partial == nullptr) bpl_clear_error();
       if (partial == nullptr || gated) fill_zero(stream, y, n_col);
+      if (use_list)
+        hipLaunchKernelGGL((collect_active_rows_kernel<F, VT, MODE>), dim3(div_up(n_row, kWinThreads)),
+                           dim3(kWinThreads), 0, stream, indptr, x, n_row, active_count, active_list, active_scales,
+                           window_gate);
       // small slices: the last workgroup of the same launch sums them (one launch instead of two)
       uint32_t *done_counter = nullptr;
-      if (partial != nullptr && static_cast<size_t>(groups) * n_col <= 131072) done_counter = stream_counters(stream);
+      if (partial != nullptr && !use_list && static_cast<size_t>(groups) * n_col <= 131072)
+        done_counter = stream_counters(stream);
       hipLaunchKernelGGL(kernel, dim3(groups * n_win), dim3(kWinThreads), lds, stream, data, indices, indptr, x, y,
-                         n_row, n_col, rows_per_wg, win, n_win, partial, done_counter, window_gate);
+                         n_row, n_col, rows_per_wg, win, n_win, partial, done_counter, window_gate, active_count,
+                         active_list, active_scales);
+      // the list's counter goes back to zero: by the summing kernel, else by a fill of its own
       if (partial != nullptr && done_counter == nullptr)
         hipLaunchKernelGGL(sum_partials_kernel<F>, dim3(div_up(n_col, 256)), dim3(256), 0, stream, partial, y, n_col,
-                           groups, indptr, n_row, window_gate);
+                           groups, indptr, n_row, window_gate, active_count);
+      else if (use_list)
+        fill_zero(stream, active_count, 1u);
       if (!gated) return;
     } else {
       direct_gate = kAlways;

@@ -278,3 +278,39 @@ def test_scatter_many_windows_and_row_chunks(cuda, oracle_mod):
       want = oracle_mod.event_csr_matvec(ones, indices, indptr, ev, shape=shape, transpose=True)
       got = bpl.event_csr_matvec(ones, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
       assert np.array_equal(got, want)  # integer counts are exact
+
+
+def test_scatter_through_the_active_row_list(cuda, oracle_mod):
+  # more than 32,768 rows: the active rows are first gathered into one list that the row groups
+  # share; both input kinds, activity concentrated in one corner of the matrix, twice in a row
+  # (the list's counter must be back at zero), silent input
+  rng = np.random.default_rng(31)
+  for n_row, n_col, mean in ((50_000, 3000, 20), (40_000, 150_000, 80), (70_000, 40_000, 5)):
+    counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_row)
+    data = rng.standard_normal(indices.shape[0]).astype(np.float32)
+    shape = (n_row, n_col)
+    print("shape", shape, flush=True)
+    for kind in ("uniform", "corner", "silent"):
+      ev = rng.random(n_row) < 0.05
+      if kind == "corner":
+        ev[n_row // 50:] = False
+        ev[:n_row // 50] = True
+      elif kind == "silent":
+        ev[:] = False
+      for _ in range(2):
+        want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True)
+        mag = oracle_mod.event_csr_matvec(np.abs(data), indices, indptr, ev, shape=shape, transpose=True)
+        got = bpl.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+        assert_close_reordered(got, want, mag, what="event scatter %s %s" % (shape, kind))
+      ones = np.ones(1, dtype=np.float32)
+      want = oracle_mod.event_csr_matvec(ones, indices, indptr, ev, shape=shape, transpose=True)
+      got = bpl.event_csr_matvec(ones, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+      assert np.array_equal(got, want)
+    if n_col <= 131072:  # dense input uses the windows up to four of them
+      v = rng.standard_normal(n_row).astype(np.float32)
+      v[rng.random(n_row) < 0.5] = 0
+      want = oracle_mod.csr_matvec(data, indices, indptr, v, shape=shape, transpose=True)
+      mag = oracle_mod.csr_matvec(np.abs(data), indices, indptr, np.abs(v), shape=shape, transpose=True)
+      got = bpl.cusparse_csr_matvec(data, indices, indptr, v, shape=shape, transpose=True).cpu().numpy()
+      assert_close_reordered(got, want, mag, what="dense scatter %s" % (shape,))
