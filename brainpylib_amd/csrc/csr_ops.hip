@@ -207,6 +207,10 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     const F *__restrict__ active_scales) {
   if (!gate.open(indptr, n_row)) return;
   extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
+  // The window accumulates in F.  (Measured on this device: the LDS unit adds 32-bit floats at
+  // about a third of a lane per clock and CU, 64-bit floats nine times and 32-bit integers
+  // thirty times faster.  A float64 window would halve the window and double the passes over the
+  // indices, which costs what the faster additions save at the sizes tried.)
   F *window = reinterpret_cast<F *>(smem_raw);
   F *s_scale = window + win;  // dense mode: x[r] per active row
   uint32_t *s_start = reinterpret_cast<uint32_t *>(s_scale + (MODE == kDense ? kWinMaxRows : 0));
