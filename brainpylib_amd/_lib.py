@@ -131,6 +131,12 @@ def build_coo_atomic_sum_descriptor(conn_size, post_size):
 
 
 @functools.lru_cache(maxsize=256)
+def build_csr_transpose_descriptor(n_row, n_col, nnz):
+  return _build("bpl_build_csr_transpose_descriptor", ctypes.c_uint32(n_row), ctypes.c_uint32(n_col),
+                ctypes.c_uint32(nnz))
+
+
+@functools.lru_cache(maxsize=256)
 def build_double_size_descriptor(size_x, size_y):
   return _build("bpl_build_double_size_descriptor", ctypes.c_uint32(size_x), ctypes.c_uint32(size_y))
 

@@ -50,6 +50,15 @@ void *stream_workspace(hipStream_t stream, size_t bytes);
 // workgroup.  Every user leaves them at zero again.  nullptr if the allocation fails.
 uint32_t *stream_counters(hipStream_t stream);
 
+// Transposed CSR times dense vector through coarse sorting of the products (csr_bin_scatter.hip),
+// for outputs much wider than LDS.  `nnz` must be the matrix's nonzero count (indptr[n_row]).
+// bin_scatter returns false, having enqueued nothing, if it cannot run (no scratch memory).
+template <typename F>
+bool bin_scatter_usable(uint32_t n_col, uint32_t nnz);
+template <typename F>
+bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool heter, const uint32_t *indices,
+                 const uint32_t *indptr, const F *vec, F *y, uint32_t n_row, uint32_t n_col, uint32_t nnz);
+
 inline unsigned div_up(unsigned long long a, unsigned long long b) {
   return static_cast<unsigned>((a + b - 1) / b);
 }

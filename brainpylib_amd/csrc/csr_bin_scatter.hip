@@ -1,0 +1,259 @@
+// Transposed CSR matrix times dense vector for wide outputs: y[c] = sum_j v[row(j)] * data[j]
+// over the nonzeros j of column c, when every row contributes and the output (hundreds of
+// thousands of columns or more) is far larger than LDS.  One random global atomic per nonzero
+// retires at about 21 G/s on this device; instead the products are first sorted coarsely:
+//
+//   bin kernel     persistent producer workgroups walk their rows, form (column, product)
+//                  pairs and append each pair to the bin of its 16,384-column output window,
+//                  in a region of scratch memory private to (producer, window): no global
+//                  atomics, the position comes from a counter in LDS that one lane per group
+//                  of equal windows advances for its whole wave.  A pair that does not fit its
+//                  region (a very uneven matrix) is added to y directly instead.
+//   window kernel  workgroup (window, part) adds the pairs of its window from a share of the
+//                  producers into a float64 window in LDS (64-bit LDS float adds run at
+//                  several lanes per clock) and adds the window to the zeroed y, contiguous.
+//
+// The arrays are read once, the pairs written and read once: HBM bound instead of atomic bound.
+#include "common.h"
+
+namespace bpl {
+namespace {
+
+constexpr int kBinThreads = 1024;
+constexpr uint32_t kTileRows = 1024;      // rows staged in LDS at a time by a producer
+constexpr uint32_t kWinShift = 14;        // output window = 16,384 columns (128 KB of float64)
+constexpr uint32_t kWinCols = 1u << kWinShift;
+constexpr uint32_t kMaxWindows = 128;     // 7-bit window ids
+constexpr uint32_t kRegionSlack = 128;    // pairs a region holds beyond 5/4 of its even share
+
+template <typename F>
+struct BinPair {
+  uint32_t rel;  // column within the window
+  F val;
+};
+
+// Where producer `p`, whose rows hold nonzeros [a0, a1), keeps the pairs of window b:
+// region_base + b * cap.  Both kernels evaluate the same expressions.
+__device__ __forceinline__ uint32_t region_cap(uint32_t a0, uint32_t a1, uint32_t n_win) {
+  const uint32_t share = (a1 - a0) / n_win;
+  return share + share / 4u + kRegionSlack;
+}
+__device__ __forceinline__ uint64_t region_base(uint32_t a0, uint32_t p, uint32_t n_win) {
+  return static_cast<uint64_t>(a0) + a0 / 4u + static_cast<uint64_t>(p) * n_win * kRegionSlack;
+}
+__device__ __forceinline__ void producer_rows(uint32_t p, uint32_t rows_per, uint32_t n_row, uint32_t *r0,
+                                              uint32_t *r1) {
+  const uint64_t lo = static_cast<uint64_t>(p) * rows_per, hi = lo + rows_per;
+  *r0 = lo < n_row ? static_cast<uint32_t>(lo) : n_row;
+  *r1 = hi < n_row ? static_cast<uint32_t>(hi) : n_row;
+}
+
+template <typename F, bool HETER>
+__global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
+    const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
+    const F *__restrict__ vec, F *__restrict__ y, uint32_t n_row, uint32_t rows_per, uint32_t n_win,
+    uint32_t win_bits, BinPair<F> *__restrict__ pairs, uint64_t n_pairs, uint32_t *__restrict__ counts) {
+  __shared__ uint32_t s_ptr[kTileRows + 1];
+  __shared__ F s_v[kTileRows];
+  __shared__ uint32_t s_cnt[kMaxWindows];
+  const uint32_t tid = threadIdx.x, lane = tid % kWave;
+  const uint32_t p = blockIdx.x;
+  uint32_t r0, r1;
+  producer_rows(p, rows_per, n_row, &r0, &r1);
+  if (tid < kMaxWindows) s_cnt[tid] = 0;
+  const uint32_t a0 = indptr[r0], a1 = indptr[r1];
+  const uint32_t cap = region_cap(a0, a1, n_win);
+  const uint64_t region_off = region_base(a0, p, n_win);
+  const F w_homo = HETER ? F(0) : data[0];
+  const uint64_t lanes_below = (1ull << lane) - 1ull;
+
+  for (uint32_t t0 = r0; t0 < r1; t0 += kTileRows) {
+    const uint32_t rows = (r1 - t0 < kTileRows) ? r1 - t0 : kTileRows;
+    __syncthreads();  // the previous tile is done with s_ptr / s_v (and s_cnt is cleared)
+    if (tid < rows) s_v[tid] = vec[t0 + tid];
+    if (tid <= rows) s_ptr[tid] = indptr[t0 + tid];
+    if (tid == 0 && rows == kTileRows) s_ptr[kTileRows] = indptr[t0 + kTileRows];
+    __syncthreads();
+    const uint32_t j0 = s_ptr[0], j1 = s_ptr[rows];
+    // whole waves take part in every round (the ballots below need all lanes present);
+    // U rounds of loads are in flight together
+    constexpr int U = 4;
+    for (uint32_t jb = j0 + (tid - lane); jb < j1; jb += U * kBinThreads) {
+      uint32_t col[U];
+      F val[U];
+      bool valid[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t j = jb + u * kBinThreads + lane;
+        valid[u] = j < j1;
+        col[u] = 0;
+        val[u] = F(0);
+        if (valid[u]) {
+          // row of nonzero j: largest k < rows with s_ptr[k] <= j
+          uint32_t k = 0;
+#pragma unroll
+          for (uint32_t step = kTileRows / 2; step > 0; step >>= 1) {
+            const uint32_t mid = k + step;
+            if (mid < rows && s_ptr[mid] <= j) k = mid;
+          }
+          col[u] = indices[j];
+          // v * values[j] (heter) or values * v (homo), as the reference's CPU loop multiplies
+          val[u] = HETER ? static_cast<F>(s_v[k] * data[j]) : static_cast<F>(w_homo * s_v[k]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t b = col[u] >> kWinShift;
+        // lanes of this wave with the same window (and a valid pair)
+        uint64_t same = __ballot(valid[u]);
+        for (uint32_t bit = 0; bit < win_bits; ++bit) {
+          const bool one = (b >> bit) & 1u;
+          const uint64_t bal = __ballot(one);
+          same &= one ? bal : ~bal;
+        }
+        if (valid[u]) {
+          const uint32_t leader = static_cast<uint32_t>(__ffsll(static_cast<long long>(same))) - 1u;
+          uint32_t base = 0;
+          if (lane == leader) base = atomicAdd(&s_cnt[b], static_cast<uint32_t>(__popcll(same)));
+          base = __shfl(base, static_cast<int>(leader), kWave);
+          const uint32_t slot = base + static_cast<uint32_t>(__popcll(same & lanes_below));
+          const uint64_t at = region_off + static_cast<uint64_t>(b) * cap + slot;
+          if (slot < cap && at < n_pairs) {
+            BinPair<F> e;
+            e.rel = col[u] & (kWinCols - 1u);
+            e.val = val[u];
+            pairs[at] = e;
+          } else {
+            atomic_add(y + col[u], val[u]);
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+  if (tid < n_win) {
+    const uint32_t c = s_cnt[tid];
+    counts[static_cast<size_t>(tid) * gridDim.x + p] = c < cap ? c : cap;
+  }
+}
+
+// grid = n_win * parts; workgroup (b, s) adds window b's pairs of producers [s * P / parts, ...)
+template <typename F>
+__global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *__restrict__ indptr,
+                                                               F *__restrict__ y, uint32_t n_row, uint32_t n_col,
+                                                               uint32_t rows_per, uint32_t n_win, uint32_t parts,
+                                                               uint32_t producers,
+                                                               const BinPair<F> *__restrict__ pairs,
+                                                               uint64_t n_pairs,
+                                                               const uint32_t *__restrict__ counts) {
+  extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
+  double *window = reinterpret_cast<double *>(smem_raw);
+  const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  constexpr uint32_t kWaves = kBinThreads / kWave;
+  const uint32_t b = blockIdx.x / parts, s = blockIdx.x % parts;
+  const uint32_t c0 = b << kWinShift;
+  const uint32_t width = (n_col - c0 < kWinCols) ? n_col - c0 : kWinCols;
+  for (uint32_t i = tid; i < width; i += kBinThreads) window[i] = 0.0;
+  __syncthreads();
+  const uint32_t p_lo = static_cast<uint32_t>(static_cast<uint64_t>(s) * producers / parts);
+  const uint32_t p_hi = static_cast<uint32_t>(static_cast<uint64_t>(s + 1) * producers / parts);
+  // one producer's bin per wave at a time, 8 pairs per lane in flight
+  for (uint32_t p = p_lo + wave; p < p_hi; p += kWaves) {
+    uint32_t r0, r1;
+    producer_rows(p, rows_per, n_row, &r0, &r1);
+    const uint32_t a0 = indptr[r0], a1 = indptr[r1];
+    const uint32_t cap = region_cap(a0, a1, n_win);
+    const uint64_t bin_off = region_base(a0, p, n_win) + static_cast<uint64_t>(b) * cap;
+    const BinPair<F> *bin = pairs + bin_off;
+    uint32_t n = counts[static_cast<size_t>(b) * producers + p];
+    if (bin_off >= n_pairs) n = 0;  // (only if the caller's nonzero count was too small)
+    else if (n > n_pairs - bin_off) n = static_cast<uint32_t>(n_pairs - bin_off);
+    constexpr int U = 8;
+    for (uint32_t i0 = 0; i0 < n; i0 += U * kWave) {
+      BinPair<F> e[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t i = i0 + u * kWave + lane;
+        e[u].rel = 0xffffffffu;
+        e[u].val = F(0);
+        if (i < n) e[u] = bin[i];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (e[u].rel < width) atomicAdd(&window[e[u].rel], static_cast<double>(e[u].val));
+    }
+  }
+  __syncthreads();
+  for (uint32_t i = tid; i < width; i += kBinThreads) {
+    const F v = static_cast<F>(window[i]);
+    if (v != F(0)) atomic_add(y + c0 + i, v);
+  }
+}
+
+}  // namespace
+
+template <typename F>
+bool bin_scatter_usable(uint32_t n_col, uint32_t nnz) {
+  const uint32_t n_win = div_up(n_col, kWinCols);
+  return n_win >= 2 && n_win <= kMaxWindows && nnz >= (1u << 20);
+}
+
+template <typename F>
+bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool heter, const uint32_t *indices,
+                 const uint32_t *indptr, const F *vec, F *y, uint32_t n_row, uint32_t n_col, uint32_t nnz) {
+  const uint32_t n_win = div_up(n_col, kWinCols);
+  uint32_t win_bits = 0;
+  while ((1u << win_bits) < n_win) ++win_bits;
+  const unsigned num_cu = static_cast<unsigned>(device_info().num_cu);
+  // two producer workgroups per CU, at least 64 rows each
+  uint32_t producers = 2u * num_cu;
+  if (producers > div_up(n_row, 64)) producers = div_up(n_row, 64);
+  const uint32_t rows_per = div_up(n_row, producers);
+  producers = div_up(n_row, rows_per);
+  uint32_t parts = num_cu / n_win;
+  if (parts == 0) parts = 1;
+  if (parts > producers) parts = producers;
+
+  // the last region ends at or before nnz + nnz / 4 + producers * n_win * kRegionSlack
+  const size_t n_pairs = static_cast<size_t>(nnz) + nnz / 4u + static_cast<size_t>(producers) * n_win * kRegionSlack + 64u;
+  const size_t pair_bytes = (n_pairs * sizeof(BinPair<F>) + 255) / 256 * 256;
+  const size_t count_bytes = static_cast<size_t>(n_win) * producers * sizeof(uint32_t);
+  unsigned char *ws = static_cast<unsigned char *>(stream_workspace(stream, pair_bytes + count_bytes));
+  if (ws == nullptr) {
+    bpl_clear_error();
+    return false;
+  }
+  BinPair<F> *pairs = reinterpret_cast<BinPair<F> *>(ws);
+  uint32_t *counts = reinterpret_cast<uint32_t *>(ws + pair_bytes);
+
+  auto add_kernel = add_bins_kernel<F>;
+  const size_t lds = static_cast<size_t>(kWinCols) * sizeof(double);
+  static thread_local bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(add_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(lds)) != hipSuccess) {
+      (void)hipGetLastError();
+      return false;
+    }
+    attr_set = true;
+  }
+  fill_zero(stream, y, n_col);
+  if (heter)
+    hipLaunchKernelGGL((bin_products_kernel<F, true>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
+                       indptr, vec, y, n_row, rows_per, n_win, win_bits, pairs, static_cast<uint64_t>(n_pairs), counts);
+  else
+    hipLaunchKernelGGL((bin_products_kernel<F, false>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
+                       indptr, vec, y, n_row, rows_per, n_win, win_bits, pairs, static_cast<uint64_t>(n_pairs), counts);
+  hipLaunchKernelGGL(add_kernel, dim3(n_win * parts), dim3(kBinThreads), lds, stream, indptr, y, n_row, n_col, rows_per,
+                     n_win, parts, producers, pairs, static_cast<uint64_t>(n_pairs), counts);
+  return check_launch(target);
+}
+
+template bool bin_scatter_usable<float>(uint32_t, uint32_t);
+template bool bin_scatter_usable<double>(uint32_t, uint32_t);
+template bool bin_scatter<float>(const char *, hipStream_t, const float *, bool, const uint32_t *, const uint32_t *,
+                                 const float *, float *, uint32_t, uint32_t, uint32_t);
+template bool bin_scatter<double>(const char *, hipStream_t, const double *, bool, const uint32_t *, const uint32_t *,
+                                  const double *, double *, uint32_t, uint32_t, uint32_t);
+
+}  // namespace bpl

@@ -814,7 +814,14 @@ template <typename F, bool HETER, bool TRANSPOSE>
 void csr_matvec_entry(const char *target, hipStream_t stream, void **buffers, const char *opaque,
                       size_t opaque_len, int vector_slot) {
   bpl_double_size_descriptor d;
-  if (!unpack(target, opaque, opaque_len, &d)) return;
+  uint32_t nnz = 0;  // known only to the transposed targets' longer descriptor
+  if (TRANSPOSE && opaque != nullptr && opaque_len == sizeof(bpl_csr_transpose_descriptor)) {
+    bpl_csr_transpose_descriptor t;
+    std::memcpy(&t, opaque, sizeof(t));
+    d.n_row = t.n_row, d.n_col = t.n_col, nnz = t.nnz;
+  } else if (!unpack(target, opaque, opaque_len, &d)) {
+    return;
+  }
   if (buffers == nullptr) {
     set_error("%s: null buffer table", target);
     return;
@@ -825,6 +832,11 @@ void csr_matvec_entry(const char *target, hipStream_t stream, void **buffers, co
   const F *vec = static_cast<const F *>(buffers[vector_slot]);
   F *out = static_cast<F *>(buffers[vector_slot + 1]);
   if (TRANSPOSE) {
+    // outputs beyond four LDS windows: sort the products coarsely instead of one global atomic each
+    const uint32_t plain_windows = div_up(d.n_col, static_cast<uint32_t>((128u * 1024u) / sizeof(F)));
+    if (plain_windows > 4 && d.n_row > 0 && bin_scatter_usable<F>(d.n_col, nnz) &&
+        bin_scatter<F>(target, stream, data, HETER, indices, indptr, vec, out, d.n_row, d.n_col, nnz))
+      return;
     launch_scatter<F, F, HETER, kDense>(stream, data, indices, indptr, vec, out, d.n_row, d.n_col);
     check_launch(target);
   } else {

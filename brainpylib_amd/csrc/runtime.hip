@@ -192,6 +192,11 @@ size_t bpl_build_coo_atomic_sum_descriptor(uint32_t conn_size, uint32_t post_siz
   return pack(d, out, cap);
 }
 
+size_t bpl_build_csr_transpose_descriptor(uint32_t n_row, uint32_t n_col, uint32_t nnz, char *out, size_t cap) {
+  bpl_csr_transpose_descriptor d{n_row, n_col, nnz};
+  return pack(d, out, cap);
+}
+
 size_t bpl_build_double_size_descriptor(uint32_t n_row, uint32_t n_col, char *out, size_t cap) {
   bpl_double_size_descriptor d{n_row, n_col};
   return pack(d, out, cap);

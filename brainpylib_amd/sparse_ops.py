@@ -93,6 +93,7 @@ def _launch(data, indices, indptr, vector, shape, transpose, method='vector'):
   opaque = _lib.build_double_size_descriptor(shape[0], shape[1])
   out = torch.empty(shape[1] if transpose else shape[0], dtype=data.dtype, device=device)
   if transpose:
+    opaque = _lib.build_csr_transpose_descriptor(shape[0], shape[1], indices.shape[0])
     _lib.custom_call('csr_matvec_transpose_' + data_name + '_' + type_name, [data, indices, indptr, vector, out],
                      opaque)
     return out

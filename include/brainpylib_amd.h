@@ -88,6 +88,16 @@ typedef struct {
   uint32_t n_col;
 } bpl_double_size_descriptor;
 
+/* Descriptor of the csr_matvec_transpose_* targets (own targets: the reference hands the
+ * transposed product to cuSPARSE, brainpylib/_src/sparse_ops/cusparse_matvec.py:266-278).  The
+ * 8-byte bpl_double_size_descriptor is accepted too; with the nonzero count the library can
+ * size scratch memory for its sorted scatter of wide outputs. */
+typedef struct {
+  uint32_t n_row;
+  uint32_t n_col;
+  uint32_t nnz; /* length of indices = indptr[n_row] */
+} bpl_csr_transpose_descriptor;
+
 /* lib/kernel_helper_descriptor.cuh:42-45 (NonZeroDescriptor): event_info. */
 typedef struct {
   uint32_t event_size;
@@ -141,6 +151,7 @@ size_t bpl_build_event_csr_batching_descriptor(uint32_t n_row, uint32_t n_col, u
 size_t bpl_build_csr_event_sum_descriptor(uint32_t pre_size, uint32_t post_size, char *out, size_t cap);
 size_t bpl_build_coo_event_sum_descriptor(uint32_t conn_size, uint32_t post_size, char *out, size_t cap);
 size_t bpl_build_coo_atomic_sum_descriptor(uint32_t conn_size, uint32_t post_size, char *out, size_t cap);
+size_t bpl_build_csr_transpose_descriptor(uint32_t n_row, uint32_t n_col, uint32_t nnz, char *out, size_t cap);
 size_t bpl_build_twouint_onebool_descriptor(uint32_t n_row, uint32_t n_col, int transpose,
                                             char *out, size_t cap);
 size_t bpl_build_double_size_descriptor(uint32_t n_row, uint32_t n_col, char *out, size_t cap);

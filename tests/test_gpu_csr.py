@@ -314,3 +314,32 @@ def test_scatter_through_the_active_row_list(cuda, oracle_mod):
       mag = oracle_mod.csr_matvec(np.abs(data), indices, indptr, np.abs(v), shape=shape, transpose=True)
       got = bpl.cusparse_csr_matvec(data, indices, indptr, v, shape=shape, transpose=True).cpu().numpy()
       assert_close_reordered(got, want, mag, what="dense scatter %s" % (shape,))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_transposed_csr_matvec_wide_output_sorted_scatter(cuda, oracle_mod, dtype):
+  # outputs beyond a few LDS windows with at least 2^20 nonzeros: products are binned by output
+  # window first.  Even rows, one very long row (its bins overflow into direct atomics), few
+  # rows, twice in a row, homogeneous weight.
+  rng = np.random.default_rng(41)
+  for n_row, n_col, mean, long_row in ((30_000, 300_000, 50, 0), (50_000, 400_000, 25, 250_000),
+                                       (1500, 2_000_000, 1000, 0), (200_000, 140_000, 8, 0)):
+    counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
+    if long_row:
+      counts[7] = long_row
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_row)
+    assert indices.shape[0] >= 1 << 20
+    data = rng.random(indices.shape[0]).astype(dtype)
+    shape = (n_row, n_col)
+    print("shape", shape, dtype.__name__, flush=True)
+    v = rng.standard_normal(n_row).astype(dtype)
+    for _ in range(2):
+      want = oracle_mod.csr_matvec(data, indices, indptr, v, shape=shape, transpose=True)
+      mag = oracle_mod.csr_matvec(data, indices, indptr, np.abs(v), shape=shape, transpose=True)  # data >= 0
+      got = bpl.cusparse_csr_matvec(data, indices, indptr, v, shape=shape, transpose=True).cpu().numpy()
+      assert_close_reordered(got, want, mag, dtype, what="sorted scatter %s" % (shape,))
+    vi = rng.integers(-2, 3, size=n_row).astype(dtype)
+    w = np.array([0.5], dtype=dtype)
+    want = oracle_mod.csr_matvec(w, indices, indptr, vi, shape=shape, transpose=True)
+    got = bpl.cusparse_csr_matvec(w, indices, indptr, vi, shape=shape, transpose=True).cpu().numpy()
+    assert np.array_equal(got, want)  # multiples of 0.5: exact in any order
