@@ -6,8 +6,8 @@
 //   bin kernel     persistent producer workgroups walk their rows, form (column, product)
 //                  pairs and append each pair to the bin of its 16,384-column output window,
 //                  in a region of scratch memory private to (producer, window): no global
-//                  atomics, the position comes from a counter in LDS that one lane per group
-//                  of equal windows advances for its whole wave.  A pair that does not fit its
+//                  atomics, the position comes from a counter in LDS (32-bit integer LDS
+//                  atomics are cheap even when lanes meet).  A pair that does not fit its
 //                  region (a very uneven matrix) is added to y directly instead.
 //   window kernel  workgroup (window, part) adds the pairs of its window from a share of the
 //                  producers into a float64 window in LDS (64-bit LDS float adds run at
@@ -48,24 +48,43 @@ __device__ __forceinline__ void producer_rows(uint32_t p, uint32_t rows_per, uin
   *r1 = hi < n_row ? static_cast<uint32_t>(hi) : n_row;
 }
 
+constexpr uint32_t kHintShift = 8;                       // one row hint per 256 nonzeros
+constexpr uint32_t kSegment = kBinThreads << kHintShift;  // nonzeros covered by one set of hints
+
 template <typename F, bool HETER>
 __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
     const F *__restrict__ vec, F *__restrict__ y, uint32_t n_row, uint32_t rows_per, uint32_t n_win,
-    uint32_t win_bits, BinPair<F> *__restrict__ pairs, uint64_t n_pairs, uint32_t *__restrict__ counts) {
+    BinPair<F> *__restrict__ pairs, uint64_t n_pairs, uint32_t *__restrict__ counts) {
   __shared__ uint32_t s_ptr[kTileRows + 1];
   __shared__ F s_v[kTileRows];
-  __shared__ uint32_t s_cnt[kMaxWindows];
-  const uint32_t tid = threadIdx.x, lane = tid % kWave;
+  __shared__ uint32_t s_hint[kBinThreads + 1];  // row (within the tile) of every 256th nonzero of the segment
+  __shared__ uint32_t s_cnt[kMaxWindows];       // pairs of the current round, per window
+  __shared__ uint32_t s_off[kMaxWindows + 1];   // their offsets in the sorted round
+  __shared__ uint32_t s_total[kMaxWindows];     // pairs already in this producer's bin, per window
+  constexpr int U = (sizeof(F) == 4) ? 4 : 2;
+  constexpr uint32_t kRound = U * kBinThreads;
+  __shared__ BinPair<F> s_sorted[kRound];
+  __shared__ uint8_t s_window[kRound];
+  const uint32_t tid = threadIdx.x;
   const uint32_t p = blockIdx.x;
   uint32_t r0, r1;
   producer_rows(p, rows_per, n_row, &r0, &r1);
-  if (tid < kMaxWindows) s_cnt[tid] = 0;
+  if (tid < kMaxWindows) s_cnt[tid] = 0, s_total[tid] = 0;
   const uint32_t a0 = indptr[r0], a1 = indptr[r1];
   const uint32_t cap = region_cap(a0, a1, n_win);
   const uint64_t region_off = region_base(a0, p, n_win);
   const F w_homo = HETER ? F(0) : data[0];
-  const uint64_t lanes_below = (1ull << lane) - 1ull;
+
+  // largest k < rows with s_ptr[k] <= j, searched in [lo, hi]
+  auto row_of = [&](uint32_t j, uint32_t lo, uint32_t hi) {
+    while (lo < hi) {
+      const uint32_t mid = (lo + hi + 1u) >> 1;
+      if (s_ptr[mid] <= j) lo = mid;
+      else hi = mid - 1u;
+    }
+    return lo;
+  };
 
   for (uint32_t t0 = r0; t0 < r1; t0 += kTileRows) {
     const uint32_t rows = (r1 - t0 < kTileRows) ? r1 - t0 : kTileRows;
@@ -75,64 +94,84 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
     if (tid == 0 && rows == kTileRows) s_ptr[kTileRows] = indptr[t0 + kTileRows];
     __syncthreads();
     const uint32_t j0 = s_ptr[0], j1 = s_ptr[rows];
-    // whole waves take part in every round (the ballots below need all lanes present);
-    // U rounds of loads are in flight together
-    constexpr int U = 4;
-    for (uint32_t jb = j0 + (tid - lane); jb < j1; jb += U * kBinThreads) {
-      uint32_t col[U];
-      F val[U];
-      bool valid[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const uint32_t j = jb + u * kBinThreads + lane;
-        valid[u] = j < j1;
-        col[u] = 0;
-        val[u] = F(0);
-        if (valid[u]) {
-          // row of nonzero j: largest k < rows with s_ptr[k] <= j
-          uint32_t k = 0;
-#pragma unroll
-          for (uint32_t step = kTileRows / 2; step > 0; step >>= 1) {
-            const uint32_t mid = k + step;
-            if (mid < rows && s_ptr[mid] <= j) k = mid;
-          }
-          col[u] = indices[j];
-          // v * values[j] (heter) or values * v (homo), as the reference's CPU loop multiplies
-          val[u] = HETER ? static_cast<F>(s_v[k] * data[j]) : static_cast<F>(w_homo * s_v[k]);
-        }
+    for (uint32_t seg = j0; seg < j1; seg += kSegment) {
+      const uint32_t seg_end = (j1 - seg < kSegment) ? j1 : seg + kSegment;
+      // hints: the row of nonzero seg + 256 q, for every q up to the end of the segment
+      __syncthreads();  // the previous segment is done with s_hint
+      {
+        const uint32_t j = seg + (tid << kHintShift);
+        s_hint[tid] = (j < seg_end) ? row_of(j, 0u, rows - 1u) : rows - 1u;
+        if (tid == 0) s_hint[kBinThreads] = rows - 1u;
       }
+      __syncthreads();
+      // Rounds of kRound nonzeros.  The round's pairs are first sorted by window in LDS (rank within
+      // the window from an LDS counter, window offsets from a scan of the counters), then written
+      // out in that order: pairs of one window go to consecutive addresses of its bin, so the
+      // stores of neighbouring lanes merge instead of arriving as single 8-byte requests.
+      for (uint32_t jb = seg + tid; jb - tid < seg_end; jb += kRound) {
+        uint32_t rank[U], win[U], rel[U];
+        F val[U];
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const uint32_t b = col[u] >> kWinShift;
-        // lanes of this wave with the same window (and a valid pair)
-        uint64_t same = __ballot(valid[u]);
-        for (uint32_t bit = 0; bit < win_bits; ++bit) {
-          const bool one = (b >> bit) & 1u;
-          const uint64_t bal = __ballot(one);
-          same &= one ? bal : ~bal;
-        }
-        if (valid[u]) {
-          const uint32_t leader = static_cast<uint32_t>(__ffsll(static_cast<long long>(same))) - 1u;
-          uint32_t base = 0;
-          if (lane == leader) base = atomicAdd(&s_cnt[b], static_cast<uint32_t>(__popcll(same)));
-          base = __shfl(base, static_cast<int>(leader), kWave);
-          const uint32_t slot = base + static_cast<uint32_t>(__popcll(same & lanes_below));
-          const uint64_t at = region_off + static_cast<uint64_t>(b) * cap + slot;
-          if (slot < cap && at < n_pairs) {
-            BinPair<F> e;
-            e.rel = col[u] & (kWinCols - 1u);
-            e.val = val[u];
-            pairs[at] = e;
-          } else {
-            atomic_add(y + col[u], val[u]);
+        for (int u = 0; u < U; ++u) {
+          const uint32_t j = jb + u * kBinThreads;
+          win[u] = 0xffffffffu;  // no pair
+          rel[u] = 0;
+          val[u] = F(0);
+          rank[u] = 0;
+          if (j < seg_end) {
+            const uint32_t q = (j - seg) >> kHintShift;
+            const uint32_t k = row_of(j, s_hint[q], s_hint[q + 1]);
+            const uint32_t col = indices[j];
+            // v * values[j] (heter) or values * v (homo), as the reference's CPU loop multiplies
+            val[u] = HETER ? static_cast<F>(s_v[k] * data[j]) : static_cast<F>(w_homo * s_v[k]);
+            win[u] = col >> kWinShift;
+            rel[u] = col & (kWinCols - 1u);
           }
         }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (win[u] != 0xffffffffu) rank[u] = atomicAdd(&s_cnt[win[u]], 1u);
+        __syncthreads();
+        if (tid < kWave) {  // offsets of the windows within the round: two counters per lane
+          const uint32_t c0 = s_cnt[2 * tid], c1 = s_cnt[2 * tid + 1];
+          const uint32_t incl = wave_inclusive_scan_u32(c0 + c1);
+          s_off[2 * tid] = incl - (c0 + c1);
+          s_off[2 * tid + 1] = incl - c1;
+          if (tid == kWave - 1) s_off[kMaxWindows] = incl;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (win[u] != 0xffffffffu) {
+            const uint32_t pos = s_off[win[u]] + rank[u];
+            BinPair<F> e;
+            e.rel = rel[u];
+            e.val = val[u];
+            s_sorted[pos] = e;
+            s_window[pos] = static_cast<uint8_t>(win[u]);
+          }
+        }
+        __syncthreads();
+        const uint32_t round_total = s_off[kMaxWindows];
+        for (uint32_t i = tid; i < round_total; i += kBinThreads) {
+          const uint32_t w = s_window[i];
+          const BinPair<F> e = s_sorted[i];
+          const uint32_t slot = s_total[w] + (i - s_off[w]);
+          const uint64_t at = region_off + static_cast<uint64_t>(w) * cap + slot;
+          if (slot < cap && at < n_pairs) pairs[at] = e;
+          else atomic_add(y + ((w << kWinShift) | e.rel), e.val);
+        }
+        __syncthreads();
+        if (tid < kMaxWindows) {
+          s_total[tid] += s_cnt[tid];
+          s_cnt[tid] = 0;
+        }
+        __syncthreads();
       }
     }
   }
-  __syncthreads();
   if (tid < n_win) {
-    const uint32_t c = s_cnt[tid];
+    const uint32_t c = s_total[tid];
     counts[static_cast<size_t>(tid) * gridDim.x + p] = c < cap ? c : cap;
   }
 }
@@ -169,7 +208,16 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
     if (bin_off >= n_pairs) n = 0;  // (only if the caller's nonzero count was too small)
     else if (n > n_pairs - bin_off) n = static_cast<uint32_t>(n_pairs - bin_off);
     constexpr int U = 8;
-    for (uint32_t i0 = 0; i0 < n; i0 += U * kWave) {
+    uint32_t i0 = 0;
+    for (; i0 + U * kWave <= n; i0 += U * kWave) {  // full steps: plain loads, all in flight
+      BinPair<F> e[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) e[u] = bin[i0 + u * kWave + lane];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (e[u].rel < width) atomicAdd(&window[e[u].rel], static_cast<double>(e[u].val));
+    }
+    if (i0 < n) {
       BinPair<F> e[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
@@ -202,8 +250,6 @@ template <typename F>
 bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool heter, const uint32_t *indices,
                  const uint32_t *indptr, const F *vec, F *y, uint32_t n_row, uint32_t n_col, uint32_t nnz) {
   const uint32_t n_win = div_up(n_col, kWinCols);
-  uint32_t win_bits = 0;
-  while ((1u << win_bits) < n_win) ++win_bits;
   const unsigned num_cu = static_cast<unsigned>(device_info().num_cu);
   // two producer workgroups per CU, at least 64 rows each
   uint32_t producers = 2u * num_cu;
@@ -240,10 +286,10 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
   fill_zero(stream, y, n_col);
   if (heter)
     hipLaunchKernelGGL((bin_products_kernel<F, true>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
-                       indptr, vec, y, n_row, rows_per, n_win, win_bits, pairs, static_cast<uint64_t>(n_pairs), counts);
+                       indptr, vec, y, n_row, rows_per, n_win, pairs, static_cast<uint64_t>(n_pairs), counts);
   else
     hipLaunchKernelGGL((bin_products_kernel<F, false>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
-                       indptr, vec, y, n_row, rows_per, n_win, win_bits, pairs, static_cast<uint64_t>(n_pairs), counts);
+                       indptr, vec, y, n_row, rows_per, n_win, pairs, static_cast<uint64_t>(n_pairs), counts);
   hipLaunchKernelGGL(add_kernel, dim3(n_win * parts), dim3(kBinThreads), lds, stream, indptr, y, n_row, n_col, rows_per,
                      n_win, parts, producers, pairs, static_cast<uint64_t>(n_pairs), counts);
   return check_launch(target);
