@@ -119,22 +119,23 @@ __device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t str
       mt_generate<2>(st, pos, lane, kWave, w);
       const PolarF32 a = polar_attempt(w[0], w[1]);
       const uint64_t okm = __ballot(a.ok);
+      // Roles of the batch's 64 units (scalar work: one round per accepted group, not per unit).
+      // An accepted attempt at unit q makes q + 1 the first and q + 2 the second skip; the
+      // search for the next accepted attempt resumes at q + 3.  Shifts past bit 63 drop out,
+      // which is exactly a role that falls into the next batch (remembered in `state`).
       uint64_t k1 = 0, k2 = 0;
-      for (int p = 0; p < kWave;) {
-        if (state == 0) {
-          const uint64_t m = okm >> p;
-          if (m == 0) break;  // only rejected attempts remain in this batch
-          p += __ffsll(static_cast<unsigned long long>(m));
-          state = 1;
-        } else if (state == 1) {
-          k1 |= 1ull << p;
-          ++p;
-          state = 2;
-        } else {
-          k2 |= 1ull << p;
-          ++p;
-          state = 0;
-        }
+      int p = 0;
+      if (state == 1) k1 = 1ull, k2 = 2ull, p = 2;
+      else if (state == 2) k2 = 1ull, p = 1;
+      state = 0;
+      while (p < kWave) {
+        const uint64_t m = okm >> p;
+        if (m == 0) break;  // only rejected attempts remain in this batch
+        const int q = p + __ffsll(static_cast<unsigned long long>(m)) - 1;
+        k1 |= 2ull << q;
+        k2 |= 4ull << q;
+        state = (q == kWave - 1) ? 1 : (q == kWave - 2) ? 2 : 0;
+        p = q + 3;
       }
       const bool is_k1 = (k1 >> lane) & 1ull;
       const bool is_k2 = (k2 >> lane) & 1ull;
