@@ -46,8 +46,8 @@ const DeviceInfo &device_info();
 // time a size is requested (hipMalloc is not capturable).
 void *stream_workspace(hipStream_t stream, size_t bytes);
 
-// A few zero-initialised 32-bit counters per (device, stream) for kernels that elect a last
-// workgroup.  Every user leaves them at zero again.  nullptr if the allocation fails.
+// A few zero-initialised 32-bit counters per (device, stream) (the scatter's active-row count).
+// Every user leaves them at zero again.  nullptr if the allocation fails.
 uint32_t *stream_counters(hipStream_t stream);
 
 // Transposed CSR times dense vector through coarse sorting of the products (csr_bin_scatter.hip),

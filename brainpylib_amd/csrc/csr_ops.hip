@@ -202,7 +202,7 @@ template <typename F, typename VT, bool HETER, int MODE>
 __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
     const VT *__restrict__ x, F *__restrict__ y, uint32_t n_row, uint32_t n_col, uint32_t rows_per_wg,
-    uint32_t win, uint32_t n_win, F *__restrict__ partial, uint32_t *__restrict__ done_counter, NnzGate gate,
+    uint32_t win, uint32_t n_win, F *__restrict__ partial, NnzGate gate,
     const uint32_t *__restrict__ active_count, const uint2 *__restrict__ active_list,
     const F *__restrict__ active_scales) {
   if (!gate.open(indptr, n_row)) return;
@@ -359,35 +359,6 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     // kernel sums the slices
     F *dst = partial + static_cast<size_t>(g) * n_col + c0;
     for (uint32_t i = tid; i < width; i += kWinThreads) dst[i] = window[i];
-    if (done_counter != nullptr) {
-      // Small outputs: no second kernel.  The workgroup that finishes last sums the slices.
-      // Stores are published device-wide (release), the last arrival acquires before reading.
-      __shared__ uint32_t s_last;
-      __threadfence();
-      __syncthreads();
-      if (tid == 0) {
-        const uint32_t prev = __hip_atomic_fetch_add(done_counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (prev + 1 == gridDim.x) ? 1u : 0u;
-      }
-      __syncthreads();
-      if (s_last) {
-        __threadfence();
-        const uint32_t groups = gridDim.x / n_win;
-        for (uint32_t c = tid; c < n_col; c += kWinThreads) {
-          F acc = F(0);
-          for (uint32_t g0 = 0; g0 < groups; g0 += 8) {  // 8 independent loads in flight
-            F v[8];
-#pragma unroll
-            for (uint32_t u = 0; u < 8; ++u)
-              v[u] = (g0 + u < groups) ? partial[static_cast<size_t>(g0 + u) * n_col + c] : F(0);
-#pragma unroll
-            for (uint32_t u = 0; u < 8; ++u) acc += v[u];
-          }
-          y[c] = acc;
-        }
-        if (tid == 0) __hip_atomic_store(done_counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
   } else {
     for (uint32_t i = tid; i < width; i += kWinThreads) {
       const F v = window[i];
@@ -642,7 +613,7 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
     // about one workgroup per CU in total, at least 64 rows each
     unsigned want_groups = static_cast<unsigned>(device_info().num_cu) / n_win;
     if (want_groups == 0) want_groups = 1;
-    // small outputs: at most 16 row groups, so that the last workgroup can sum their slices itself
+    // small outputs: at most 16 row groups (their slices are summed by the second kernel)
     if (static_cast<size_t>(n_col) * 16 <= 131072 && n_row <= 16 * kWinMaxRows && want_groups > 16) want_groups = 16;
     uint32_t rows_per_wg = div_up(n_row, want_groups);
     if (rows_per_wg < 64) rows_per_wg = 64;
@@ -697,22 +668,18 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
       F *partial = want_partial ? reinterpret_cast<F *>(ws + partial_off) : nullptr;
       uint2 *active_list = use_list ? reinterpret_cast<uint2 *>(ws + list_off) : nullptr;
       F *active_scales = scale_sz ? reinterpret_cast<F *>(ws + list_sz) : nullptr;
-      uint32_t *active_count = use_list ? counters + 1 : nullptr;  // slot 0 is the last-workgroup counter
+      uint32_t *active_count = use_list ? counters : nullptr;
       const bool gated = n_win > 4;
       if (partial == nullptr || gated) fill_zero(stream, y, n_col);
       if (use_list)
         hipLaunchKernelGGL((collect_active_rows_kernel<F, VT, MODE>), dim3(div_up(n_row, kWinThreads)),
                            dim3(kWinThreads), 0, stream, indptr, x, n_row, active_count, active_list, active_scales,
                            window_gate);
-      // small slices: the last workgroup of the same launch sums them (one launch instead of two)
-      uint32_t *done_counter = nullptr;
-      if (partial != nullptr && !use_list && static_cast<size_t>(groups) * n_col <= 131072)
-        done_counter = stream_counters(stream);
       hipLaunchKernelGGL(kernel, dim3(groups * n_win), dim3(kWinThreads), lds, stream, data, indices, indptr, x, y,
-                         n_row, n_col, rows_per_wg, win, n_win, partial, done_counter, window_gate, active_count,
+                         n_row, n_col, rows_per_wg, win, n_win, partial, window_gate, active_count,
                          active_list, active_scales);
       // the list's counter goes back to zero: by the summing kernel, else by a fill of its own
-      if (partial != nullptr && done_counter == nullptr)
+      if (partial != nullptr)
         hipLaunchKernelGGL(sum_partials_kernel<F>, dim3(div_up(n_col, 256)), dim3(256), 0, stream, partial, y, n_col,
                            groups, indptr, n_row, window_gate, active_count);
       else if (use_list)
