@@ -51,6 +51,22 @@ def time_calls(fn, steps, warmup):
   return dur_ms, wall
 
 
+def back_to_back_us(fn, calls):
+  """Microseconds per call when `calls` calls are enqueued with nothing between them (one pair of
+  events around all of them): what a time-stepping loop pays per call once the queue is fed."""
+  import torch
+  for _ in range(20):
+    fn()
+  torch.cuda.synchronize()
+  e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+  e0.record()
+  for _ in range(calls):
+    fn()
+  e1.record()
+  torch.cuda.synchronize()
+  return e0.elapsed_time(e1) * 1e3 / calls
+
+
 def stats(dur_ms):
   return dict(mean_us=float(dur_ms.mean() * 1e3), median_us=float(np.median(dur_ms) * 1e3),
               p95_us=float(np.percentile(dur_ms, 95) * 1e3), min_us=float(dur_ms.min() * 1e3))
@@ -285,8 +301,9 @@ def main():
     got = bpl.event_csr_matvec(sd["data"], sd["indices"], sd["indptr"], sd["events"], shape=s["shape"], transpose=True)
     want = oracle.event_csr_matvec(s["data"], s["indices"], s["indptr"], s["events"], shape=s["shape"], transpose=True)
     check(got.cpu().numpy(), want, "event_csr_matvec scatter 4,000")
-    dur_c1, wall_c1 = time_calls(lambda: bpl.event_csr_matvec(sd["data"], sd["indices"], sd["indptr"], sd["events"],
-                                                              shape=s["shape"], transpose=True), args.steps, args.warmup)
+    scatter_c1 = lambda: bpl.event_csr_matvec(sd["data"], sd["indices"], sd["indptr"], sd["events"],
+                                              shape=s["shape"], transpose=True)
+    dur_c1, wall_c1 = time_calls(scatter_c1, args.steps, args.warmup)
     deliv = int(np.diff(s["indptr"])[s["events"]].sum())
     extra["scatter_4000"] = dict(stats(dur_c1), delivered_synapses=deliv, wall_us_per_call=wall_c1 / args.steps * 1e6)
     if not args.skip_cpu:
@@ -314,6 +331,9 @@ def main():
     check(out_raw.cpu().numpy(), want, "event_csr_matvec scatter 4,000 (bare ABI)")
     extra["scatter_4000"]["bare_abi_wall_us_per_call"] = wall_r / 1000 * 1e6
     extra["scatter_4000"]["bare_abi_event_us"] = stats(dur_r)
+    extra["scatter_4000"]["bare_abi_back_to_back_us"] = back_to_back_us(raw, 1000)
+    extra["scatter_4000"]["wrapper_back_to_back_us"] = back_to_back_us(scatter_c1, 1000)
+    extra["scatter_4000"]["trivial_kernel_back_to_back_us"] = back_to_back_us(lambda: xs.add_(1.0), 1000)
     # the same call replayed from a HIP graph: what a simulation loop that captures its time step pays
     gs = torch.cuda.Stream()
     gs.wait_stream(torch.cuda.current_stream())

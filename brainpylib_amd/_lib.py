@@ -74,6 +74,9 @@ def last_error():
   return lib().bpl_last_error().decode()
 
 
+_PTR_ARRAYS = {}
+
+
 def custom_call(name, buffers, opaque, stream=None):
   """Enqueue custom-call target ``name`` on ``stream`` (default: torch's current stream).
 
@@ -82,12 +85,16 @@ def custom_call(name, buffers, opaque, stream=None):
   fn = target(name)
   if stream is None:
     stream = torch.cuda.current_stream().cuda_stream
-  ptrs = (ctypes.c_void_p * len(buffers))(*[ctypes.c_void_p(b.data_ptr()) for b in buffers])
-  l = lib()
-  l.bpl_clear_error()
-  fn(ctypes.c_void_p(stream), ptrs, opaque, len(opaque))
-  err = l.bpl_last_error()
+  n = len(buffers)
+  array_type = _PTR_ARRAYS.get(n)
+  if array_type is None:
+    array_type = _PTR_ARRAYS[n] = ctypes.c_void_p * n
+  ptrs = array_type(*[b.data_ptr() for b in buffers])
+  fn(stream, ptrs, opaque, len(opaque))
+  # the error string is per thread and empty unless a target has just failed
+  err = lib().bpl_last_error()
   if err:
+    lib().bpl_clear_error()
     raise RuntimeError(err.decode())
 
 
