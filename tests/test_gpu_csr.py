@@ -343,3 +343,38 @@ def test_transposed_csr_matvec_wide_output_sorted_scatter(cuda, oracle_mod, dtyp
     want = oracle_mod.csr_matvec(w, indices, indptr, vi, shape=shape, transpose=True)
     got = bpl.cusparse_csr_matvec(w, indices, indptr, vi, shape=shape, transpose=True).cpu().numpy()
     assert np.array_equal(got, want)  # multiples of 0.5: exact in any order
+
+
+def test_full_size_csr_matvec_both_orientations(cuda, oracle_mod):
+  # 1,000,000 x 1,000,000, ~1e8 nnz (the transposed product runs the sorted scatter):
+  #  * against the oracle on the configuration's own data,
+  #  * <u, A v> == <A^T u, v> exactly with small integer data and vectors,
+  #  * A^T 1 with unit weight gives the column counts exactly.
+  c = synth.config_csr_matvec()
+  shape = c["shape"]
+  n = shape[0]
+  dev = cuda
+  data = torch.from_numpy(c["data"]).to(dev)
+  indices = torch.from_numpy(c["indices"]).to(dev)
+  indptr = torch.from_numpy(c["indptr"]).to(dev)
+  vec = torch.from_numpy(c["vector"]).to(dev)
+  print("full size csr_matvec", indices.shape[0], flush=True)
+  want = oracle_mod.csr_matvec(c["data"], c["indices"], c["indptr"], c["vector"], shape=shape)
+  got = bpl.csr_matvec(data, indices, indptr, vec, shape=shape).cpu().numpy()
+  assert_close(got, want, what="csr_matvec full size")
+  want = oracle_mod.csr_matvec(c["data"], c["indices"], c["indptr"], c["vector"], shape=shape, transpose=True)
+  mag = oracle_mod.csr_matvec(c["data"], c["indices"], c["indptr"], np.abs(c["vector"]), shape=shape, transpose=True)
+  got = bpl.cusparse_csr_matvec(data, indices, indptr, vec, shape=shape, transpose=True).cpu().numpy()
+  assert_close_reordered(got, want, mag, what="csr_matvec transposed full size")
+  rng = np.random.default_rng(5)
+  di = torch.from_numpy(rng.integers(0, 3, size=indices.shape[0]).astype(np.float32)).to(dev)
+  u = torch.from_numpy(rng.integers(-2, 3, size=n).astype(np.float32)).to(dev)
+  v = torch.from_numpy(rng.integers(-2, 3, size=n).astype(np.float32)).to(dev)
+  Av = bpl.csr_matvec(di, indices, indptr, v, shape=shape)
+  ATu = bpl.cusparse_csr_matvec(di, indices, indptr, u, shape=shape, transpose=True)
+  lhs = float((Av.double() * u.double()).sum())
+  rhs = float((ATu.double() * v.double()).sum())
+  assert lhs == rhs and lhs != 0
+  ones = torch.ones(n, dtype=torch.float32, device=dev)
+  cnt = bpl.cusparse_csr_matvec(torch.ones(1, device=dev), indices, indptr, ones, shape=shape, transpose=True)
+  assert np.array_equal(cnt.cpu().numpy(), np.bincount(c["indices"], minlength=n).astype(np.float32))

@@ -101,3 +101,24 @@ def test_batching_edge_cases(cuda, oracle_mod):
     bpl.event_csr_matvec_batching(data[0], indices, indptr, np.ones((1, 5), bool), batch_size=1, shape=shape)
   with pytest.raises(ValueError):
     bpl.event_csr_matvec_batching(data, indices, indptr, np.ones((1, 4), bool), batch_size=1, shape=shape)
+
+
+def test_full_size_batching_rows_equal_single_operator(cuda):
+  # 100,000 x 100,000, ~1e8 nnz, nine event vectors (two tiles of eight): every row of the batched
+  # result against the single operator; the homogeneous weight bit for bit
+  c = synth.config_event_csr_large()
+  shape = c["shape"]
+  dev = cuda
+  data = torch.from_numpy(c["data"]).to(dev)
+  indices = torch.from_numpy(c["indices"]).to(dev)
+  indptr = torch.from_numpy(c["indptr"]).to(dev)
+  rng = np.random.default_rng(17)
+  events = torch.from_numpy(rng.random((9, shape[1])) < 0.05).to(dev)
+  w = torch.full((1, 1), 0.6, dtype=torch.float32, device=dev)
+  het = bpl.event_csr_matvec_batching(data[None], indices[None], indptr[None], events, batch_size=9, shape=shape)
+  hom = bpl.event_csr_matvec_batching(w, indices[None], indptr[None], events, batch_size=9, shape=shape)
+  for bi in range(9):
+    single = bpl.event_csr_matvec(data, indices, indptr, events[bi], shape=shape)
+    assert_close(het[bi].cpu().numpy(), single.cpu().numpy(), what="heter entry %d" % bi)
+    single = bpl.event_csr_matvec(w[0], indices, indptr, events[bi], shape=shape)
+    assert torch.equal(hom[bi], single)
