@@ -59,6 +59,13 @@ template <typename F>
 bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool heter, const uint32_t *indices,
                  const uint32_t *indptr, const F *vec, F *y, uint32_t n_row, uint32_t n_col, uint32_t nnz);
 
+// Second half of the coarse-sorted scatter for producers other than the CSR one: adds bins laid
+// out uniformly, bin (p, b) = pairs + (p * n_win + b) * cap with counts[b * producers + p]
+// BinPair<F> entries (bins.h), n_win = ceil(n_out / 16,384), into the zeroed y.
+template <typename F>
+bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_out, uint32_t producers, uint32_t cap,
+                      const void *pairs, const uint32_t *counts);
+
 inline unsigned div_up(unsigned long long a, unsigned long long b) {
   return static_cast<unsigned>((a + b - 1) / b);
 }

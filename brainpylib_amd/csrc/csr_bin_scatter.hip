@@ -14,6 +14,7 @@
 //                  several lanes per clock) and adds the window to the zeroed y, contiguous.
 //
 // The arrays are read once, the pairs written and read once: HBM bound instead of atomic bound.
+#include "bins.h"
 #include "common.h"
 
 namespace bpl {
@@ -21,16 +22,10 @@ namespace {
 
 constexpr int kBinThreads = 1024;
 constexpr uint32_t kTileRows = 1024;      // rows staged in LDS at a time by a producer
-constexpr uint32_t kWinShift = 14;        // output window = 16,384 columns (128 KB of float64)
-constexpr uint32_t kWinCols = 1u << kWinShift;
-constexpr uint32_t kMaxWindows = 128;     // 7-bit window ids
+constexpr uint32_t kWinShift = kBinWinShift;
+constexpr uint32_t kWinCols = kBinWinCols;
+constexpr uint32_t kMaxWindows = kBinMaxWindows;
 constexpr uint32_t kRegionSlack = 128;    // pairs a region holds beyond 5/4 of its even share
-
-template <typename F>
-struct BinPair {
-  uint32_t rel;  // column within the window
-  F val;
-};
 
 // Where producer `p`, whose rows hold nonzeros [a0, a1), keeps the pairs of window b:
 // region_base + b * cap.  Both kernels evaluate the same expressions.
@@ -176,7 +171,9 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
   }
 }
 
-// grid = n_win * parts; workgroup (b, s) adds window b's pairs of producers [s * P / parts, ...)
+// grid = n_win * parts; workgroup (b, s) adds window b's pairs of producers [s * P / parts, ...).
+// Bin of (producer p, window b): derived from indptr as in bin_products_kernel, or, with
+// indptr == nullptr, the uniform layout pairs + (p * n_win + b) * uniform_cap.
 template <typename F>
 __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *__restrict__ indptr,
                                                                F *__restrict__ y, uint32_t n_row, uint32_t n_col,
@@ -184,7 +181,8 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
                                                                uint32_t producers,
                                                                const BinPair<F> *__restrict__ pairs,
                                                                uint64_t n_pairs,
-                                                               const uint32_t *__restrict__ counts) {
+                                                               const uint32_t *__restrict__ counts,
+                                                               uint32_t uniform_cap) {
   extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
   double *window = reinterpret_cast<double *>(smem_raw);
   const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
@@ -198,11 +196,15 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
   const uint32_t p_hi = static_cast<uint32_t>(static_cast<uint64_t>(s + 1) * producers / parts);
   // one producer's bin per wave at a time, 8 pairs per lane in flight
   for (uint32_t p = p_lo + wave; p < p_hi; p += kWaves) {
-    uint32_t r0, r1;
-    producer_rows(p, rows_per, n_row, &r0, &r1);
-    const uint32_t a0 = indptr[r0], a1 = indptr[r1];
-    const uint32_t cap = region_cap(a0, a1, n_win);
-    const uint64_t bin_off = region_base(a0, p, n_win) + static_cast<uint64_t>(b) * cap;
+    uint64_t bin_off;
+    if (indptr != nullptr) {
+      uint32_t r0, r1;
+      producer_rows(p, rows_per, n_row, &r0, &r1);
+      const uint32_t a0 = indptr[r0], a1 = indptr[r1];
+      bin_off = region_base(a0, p, n_win) + static_cast<uint64_t>(b) * region_cap(a0, a1, n_win);
+    } else {
+      bin_off = (static_cast<uint64_t>(p) * n_win + b) * uniform_cap;
+    }
     const BinPair<F> *bin = pairs + bin_off;
     uint32_t n = counts[static_cast<size_t>(b) * producers + p];
     if (bin_off >= n_pairs) n = 0;  // (only if the caller's nonzero count was too small)
@@ -291,10 +293,41 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
     hipLaunchKernelGGL((bin_products_kernel<F, false>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
                        indptr, vec, y, n_row, rows_per, n_win, pairs, static_cast<uint64_t>(n_pairs), counts);
   hipLaunchKernelGGL(add_kernel, dim3(n_win * parts), dim3(kBinThreads), lds, stream, indptr, y, n_row, n_col, rows_per,
-                     n_win, parts, producers, pairs, static_cast<uint64_t>(n_pairs), counts);
+                     n_win, parts, producers, pairs, static_cast<uint64_t>(n_pairs), counts, 0u);
   return check_launch(target);
 }
 
+// Adds uniformly laid out bins (filled by another producer, e.g. the jitconn column walk) to
+// the zeroed y of n_out elements: bin (p, b) = pairs + (p * n_win + b) * cap with counts[b * producers + p] pairs.
+template <typename F>
+bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_out, uint32_t producers, uint32_t cap,
+                      const void *pairs, const uint32_t *counts) {
+  const uint32_t n_win = div_up(n_out, kWinCols);
+  auto add_kernel = add_bins_kernel<F>;
+  const size_t lds = static_cast<size_t>(kWinCols) * sizeof(double);
+  static thread_local bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(add_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(lds)) != hipSuccess) {
+      (void)hipGetLastError();
+      return false;
+    }
+    attr_set = true;
+  }
+  uint32_t parts = static_cast<uint32_t>(device_info().num_cu) / n_win;
+  if (parts == 0) parts = 1;
+  if (parts > producers) parts = producers;
+  const uint64_t n_pairs = static_cast<uint64_t>(producers) * n_win * cap;
+  hipLaunchKernelGGL(add_kernel, dim3(n_win * parts), dim3(kBinThreads), lds, stream,
+                     static_cast<const uint32_t *>(nullptr), y, 0u, n_out, 0u, n_win, parts, producers,
+                     static_cast<const BinPair<F> *>(pairs), n_pairs, counts, cap);
+  return check_launch(target);
+}
+
+template bool add_uniform_bins<float>(const char *, hipStream_t, float *, uint32_t, uint32_t, uint32_t, const void *,
+                                      const uint32_t *);
+template bool add_uniform_bins<double>(const char *, hipStream_t, double *, uint32_t, uint32_t, uint32_t, const void *,
+                                       const uint32_t *);
 template bool bin_scatter_usable<float>(uint32_t, uint32_t);
 template bool bin_scatter_usable<double>(uint32_t, uint32_t);
 template bool bin_scatter<float>(const char *, hipStream_t, const float *, bool, const uint32_t *, const uint32_t *,

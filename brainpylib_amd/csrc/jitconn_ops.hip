@@ -19,6 +19,7 @@
 // lib/gpu_jitconn_matvec_atomic.cu:53-77 (buffers = [input, out]; descriptors; target names).
 #include <cmath>
 
+#include "bins.h"
 #include "common.h"
 #include "jitconn_stream.h"
 #include "targets.h"
@@ -130,6 +131,88 @@ __global__ __launch_bounds__(kColThreads) void jitconn_colwalk_kernel(const VT *
         atomic_add(&out[idx], add);
       }
     });
+  }
+}
+
+// Column walk that appends its (output, value) pairs to bins instead of adding them to `out` one
+// global atomic at a time (about 21 G/s on this device).  Persistent producer workgroup p owns the
+// columns [p * cols_per, (p + 1) * cols_per); a pair for output window b (16,384 outputs) goes to
+// pairs[(p * n_win + b) * cap + position], the position from a 32-bit counter in LDS; a pair that
+// finds its bin full is added directly.  add_uniform_bins() then adds the bins window by window.
+template <typename T1, typename VT, int IN, int W>
+__global__ __launch_bounds__(kColThreads) void jitconn_colwalk_bins_kernel(
+    const VT *__restrict__ in, T1 *__restrict__ out, uint32_t n_out, uint32_t n_in, uint32_t seed, double log_p, T1 wa,
+    T1 wb, uint32_t cols_per, uint32_t n_win, uint32_t cap, BinPair<T1> *__restrict__ pairs,
+    uint32_t *__restrict__ counts) {
+  constexpr int kWaves = kColThreads / kWave;
+  constexpr int kWords = StreamLds<T1, W>::words;
+  __shared__ __attribute__((aligned(8))) uint32_t s_state[kWaves * kWords];
+  __shared__ uint32_t s_col[kColThreads];
+  __shared__ T1 s_val[kColThreads];
+  __shared__ uint32_t s_wave_cnt[kWaves];
+  __shared__ uint32_t s_cnt[kBinMaxWindows];
+
+  const int lane = lane_id();
+  const uint32_t wave = threadIdx.x / kWave;
+  const uint32_t p = blockIdx.x;
+  const uint64_t c_lo64 = static_cast<uint64_t>(p) * cols_per;
+  const uint32_t c_lo = c_lo64 < n_in ? static_cast<uint32_t>(c_lo64) : n_in;
+  const uint32_t c_hi = (n_in - c_lo < cols_per) ? n_in : c_lo + cols_per;
+  if (threadIdx.x < kBinMaxWindows) s_cnt[threadIdx.x] = 0;
+  BinPair<T1> *region = pairs + static_cast<uint64_t>(p) * n_win * cap;
+  uint32_t *st = s_state + wave * kWords;
+
+  for (uint32_t tile = c_lo; tile < c_hi; tile += kColThreads) {
+    __syncthreads();  // the previous tile's column list is no longer read (and s_cnt is cleared)
+    const uint32_t c = tile + threadIdx.x;
+    T1 v = T1(0);
+    bool on = false;
+    if (c < c_hi) {
+      const VT x = in[c];
+      on = is_event(x);
+      v = static_cast<T1>(x);
+    }
+    const uint64_t mask = __ballot(on);
+    if (lane == 0) s_wave_cnt[wave] = static_cast<uint32_t>(__popcll(mask));
+    __syncthreads();
+    uint32_t base = 0, count = 0;
+#pragma unroll
+    for (uint32_t i = 0; i < kWaves; ++i) {
+      if (i < wave) base += s_wave_cnt[i];
+      count += s_wave_cnt[i];
+    }
+    if (on) {
+      const uint32_t k = base + static_cast<uint32_t>(__popcll(mask & ((1ull << lane) - 1ull)));
+      s_col[k] = c;
+      s_val[k] = v;
+    }
+    __syncthreads();
+    for (uint32_t k = wave; k < count; k += kWaves) {
+      const uint32_t col = s_col[k];
+      const T1 val = s_val[k];
+      walk_stream<T1, W>(st, lane, seed + col, nullptr, n_out, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
+        if (valid) {
+          T1 add;
+          if (IN == kInDense) add = (W == kHomo) ? val : static_cast<T1>(w * val);
+          else add = w;  // homo: w == 1
+          const uint32_t b = idx >> kBinWinShift;
+          const uint32_t slot = atomicAdd(&s_cnt[b], 1u);
+          if (slot < cap) {
+            BinPair<T1> e;
+            e.rel = idx & (kBinWinCols - 1u);
+            e.val = add;
+            region[static_cast<uint64_t>(b) * cap + slot] = e;
+          } else {
+            atomic_add(&out[idx], add);
+          }
+        }
+      });
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < n_win) {
+    const uint32_t c = s_cnt[threadIdx.x];
+    counts[static_cast<size_t>(threadIdx.x) * gridDim.x + p] = c < cap ? c : cap;
   }
 }
 
@@ -246,6 +329,40 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
                     double log_p, T1 wa, T1 wb) {
   fill_zero(stream, out, n_out);
   if (n_in == 0 || n_out == 0) return;
+  // Many pairs and an output far wider than LDS: bins.  The number of pairs is n_in * n_out * p for a
+  // dense input; for events it depends on the activity, which the host does not know: bins are sized
+  // for one column in eight being active (fuller bins overflow into direct atomics) and used when
+  // one active column in a hundred already means half a million pairs.
+  const uint32_t n_win = div_up(n_out, kBinWinCols);
+  const double p_conn = -std::expm1(log_p);
+  const double full = static_cast<double>(n_in) * static_cast<double>(n_out) * p_conn;
+  if (n_win >= 2 && n_win <= kBinMaxWindows && full >= (IN == kInDense ? 1048576.0 : 5.0e7)) {
+    uint32_t producers = 4u * static_cast<uint32_t>(device_info().num_cu);
+    if (producers > div_up(n_in, kColThreads)) producers = div_up(n_in, kColThreads);
+    const uint32_t cols_per = div_up(n_in, producers);
+    producers = div_up(n_in, cols_per);
+    const double per_bin = static_cast<double>(cols_per) * kBinWinCols * p_conn;  // every column active
+    double cap_d = 1.25 * per_bin + 6.0 * std::sqrt(per_bin) + 128.0;
+    if (IN == kInEvent) cap_d = cap_d / 8.0 < 512.0 ? 512.0 : cap_d / 8.0;
+    const size_t total_pairs = static_cast<size_t>(producers) * n_win * static_cast<size_t>(cap_d);
+    const size_t pair_bytes = (total_pairs * sizeof(BinPair<T1>) + 255) / 256 * 256;
+    if (cap_d < 4.0e9 && pair_bytes <= (static_cast<size_t>(32) << 30)) {
+      const uint32_t cap = static_cast<uint32_t>(cap_d);
+      unsigned char *ws = static_cast<unsigned char *>(
+        stream_workspace(stream, pair_bytes + static_cast<size_t>(n_win) * producers * sizeof(uint32_t)));
+      if (ws != nullptr) {
+        BinPair<T1> *pairs = reinterpret_cast<BinPair<T1> *>(ws);
+        uint32_t *counts = reinterpret_cast<uint32_t *>(ws + pair_bytes);
+        hipLaunchKernelGGL((jitconn_colwalk_bins_kernel<T1, VT, IN, W>), dim3(producers), dim3(kColThreads), 0, stream,
+                           in, out, n_out, n_in, seed, log_p, wa, wb, cols_per, n_win, cap, pairs, counts);
+        if (add_uniform_bins<T1>("jitconn column walk", stream, out, n_out, producers, cap, pairs, counts)) return;
+        // (the bins could not be added: nothing reached `out` yet except overflow pairs; start over)
+        fill_zero(stream, out, n_out);
+      } else {
+        bpl_clear_error();
+      }
+    }
+  }
   hipLaunchKernelGGL((jitconn_colwalk_kernel<T1, VT, IN, W>), dim3(div_up(n_in, kColThreads)), dim3(kColThreads), 0,
                      stream, in, out, n_out, n_in, seed, log_p, wa, wb);
 }

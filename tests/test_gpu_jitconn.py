@@ -313,3 +313,45 @@ def test_config_jitconn_matmat_full_size(cuda, oracle_mod):
   err = np.abs(got[rows].astype(np.float64) - want)
   bound = 1e-6 + 1e-5 * np.abs(want) + 4 * np.finfo(np.float32).eps * 0.05 * 1000
   assert (err <= bound).all(), float(err.max())
+
+
+@pytest.mark.parametrize("w_kind,a,b", [("homo", 0.0, 0.0), ("uniform", 0.25, 1.75), ("normal", 0.5, 2.0)])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_column_walk_through_bins_dense(cuda, oracle_mod, w_kind, a, b, dtype):
+  # dense input, output wider than one 16,384-element window, > 2^20 pairs: the column walk appends
+  # its pairs to bins that a second kernel adds.  Against the oracle's column walk (integer input:
+  # homogeneous sums are exact) and against the row walk of the transposed flags (adjoint).
+  n_out, n_in = 40_000, 2_500
+  lp = oracle_mod.log_p_of(0.05)
+  rng = np.random.default_rng(8)
+  x = rng.integers(-3, 4, n_in).astype(dtype)
+  got = kernel_call(x, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=21, n_row=n_out, n_col=n_in, col_walk=True,
+                    dense=True)
+  want = oracle_mod.jitconn_matvec(x, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=21, n_row=n_out, n_col=n_in,
+                                   col_walk=True, dense=True)
+  if w_kind == "homo":
+    assert np.array_equal(got, want)
+  else:
+    # bound on the sum of |addends| per output: |x| <= 3, |w| <= |a| + 5 |b| (5 sigma / the uniform range),
+    # about n_in * p addends, doubled
+    mag = np.full(n_out, 3.0 * (abs(a) + 5 * abs(b)) * n_in * 0.05 * 2)
+    assert_close_reordered(got, want, mag, dtype, what="binned column walk %s" % w_kind)
+  y = rng.integers(-3, 4, n_out).astype(np.float64)
+  x64 = x.astype(np.float64)
+  Mx = kernel_call(x64, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=21, n_row=n_out, n_col=n_in, col_walk=True, dense=True)
+  MTy = kernel_call(y, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=21, n_row=n_in, n_col=n_out, col_walk=False, dense=True)
+  assert abs(y @ Mx - MTy @ x64) <= 1e-9 * max(1.0, abs(y @ Mx))
+
+
+def test_column_walk_through_bins_events_and_overflow(cuda, oracle_mod):
+  # event input with n_in * n_out * p >= 5e7: bins sized for one active column in eight.  At 2 % activity
+  # everything fits; with every column active most pairs overflow into direct atomics.  Counts are exact.
+  n_out, n_in = 60_000, 90_000
+  lp = oracle_mod.log_p_of(0.01)
+  rng = np.random.default_rng(9)
+  for rate in (0.02, 1.0):
+    ev = rng.random(n_in) < rate
+    print("rate", rate, flush=True)
+    got = kernel_call(ev, w_kind="homo", log_p=lp, seed=5, n_row=n_out, n_col=n_in, col_walk=True, dense=False)
+    want = oracle_mod.jitconn_matvec(ev, w_kind="homo", log_p=lp, seed=5, n_row=n_out, n_col=n_in, col_walk=True)
+    assert np.array_equal(got, want)
