@@ -182,8 +182,10 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
                                                                const BinPair<F> *__restrict__ pairs,
                                                                uint64_t n_pairs,
                                                                const uint32_t *__restrict__ counts,
-                                                               uint32_t uniform_cap) {
+                                                               uint32_t uniform_cap, uint32_t *__restrict__ reset) {
   extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
+  // (a counter of the producer's, left at zero for the next call)
+  if (reset != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *reset = 0u;
   double *window = reinterpret_cast<double *>(smem_raw);
   const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   constexpr uint32_t kWaves = kBinThreads / kWave;
@@ -194,43 +196,59 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
   __syncthreads();
   const uint32_t p_lo = static_cast<uint32_t>(static_cast<uint64_t>(s) * producers / parts);
   const uint32_t p_hi = static_cast<uint32_t>(static_cast<uint64_t>(s + 1) * producers / parts);
-  // one producer's bin per wave at a time, 8 pairs per lane in flight
-  for (uint32_t p = p_lo + wave; p < p_hi; p += kWaves) {
-    uint64_t bin_off;
-    if (indptr != nullptr) {
-      uint32_t r0, r1;
-      producer_rows(p, rows_per, n_row, &r0, &r1);
-      const uint32_t a0 = indptr[r0], a1 = indptr[r1];
-      bin_off = region_base(a0, p, n_win) + static_cast<uint64_t>(b) * region_cap(a0, a1, n_win);
-    } else {
-      bin_off = (static_cast<uint64_t>(p) * n_win + b) * uniform_cap;
-    }
-    const BinPair<F> *bin = pairs + bin_off;
-    uint32_t n = counts[static_cast<size_t>(b) * producers + p];
-    if (bin_off >= n_pairs) n = 0;  // (only if the caller's nonzero count was too small)
-    else if (n > n_pairs - bin_off) n = static_cast<uint32_t>(n_pairs - bin_off);
-    constexpr int U = 8;
-    uint32_t i0 = 0;
-    for (; i0 + U * kWave <= n; i0 += U * kWave) {  // full steps: plain loads, all in flight
-      BinPair<F> e[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) e[u] = bin[i0 + u * kWave + lane];
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-        if (e[u].rel < width) atomicAdd(&window[e[u].rel], static_cast<double>(e[u].val));
-    }
-    if (i0 < n) {
-      BinPair<F> e[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const uint32_t i = i0 + u * kWave + lane;
-        e[u].rel = 0xffffffffu;
-        e[u].val = F(0);
-        if (i < n) e[u] = bin[i];
+  // One producer's bin per wave at a time, 8 pairs per lane in flight.  Where the bins are and how
+  // many pairs they hold is fetched for 64 bins at once (one per lane), so that the walk over the
+  // bins waits for pairs only.
+  for (uint32_t g0 = p_lo + wave; g0 < p_hi; g0 += kWaves * kWave) {
+    uint64_t my_off = 0;
+    uint32_t my_n = 0;
+    {
+      const uint64_t p64 = static_cast<uint64_t>(g0) + static_cast<uint64_t>(lane) * kWaves;
+      if (p64 < p_hi) {
+        const uint32_t p = static_cast<uint32_t>(p64);
+        if (indptr != nullptr) {
+          uint32_t r0, r1;
+          producer_rows(p, rows_per, n_row, &r0, &r1);
+          const uint32_t a0 = indptr[r0], a1 = indptr[r1];
+          my_off = region_base(a0, p, n_win) + static_cast<uint64_t>(b) * region_cap(a0, a1, n_win);
+        } else {
+          my_off = (static_cast<uint64_t>(p) * n_win + b) * uniform_cap;
+        }
+        my_n = counts[static_cast<size_t>(b) * producers + p];
+        if (indptr == nullptr && my_n > uniform_cap) my_n = uniform_cap;  // the producer counts what it could not store too
+        if (my_off >= n_pairs) my_n = 0;  // (only if the caller's nonzero count was too small)
+        else if (my_n > n_pairs - my_off) my_n = static_cast<uint32_t>(n_pairs - my_off);
       }
+    }
+    for (uint32_t j = 0; j < kWave && static_cast<uint64_t>(g0) + static_cast<uint64_t>(j) * kWaves < p_hi; ++j) {
+      const uint32_t n = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(my_n), j));
+      if (n == 0) continue;
+      const uint32_t off_lo = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(my_off), j));
+      const uint32_t off_hi = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(my_off >> 32), j));
+      const BinPair<F> *bin = pairs + ((static_cast<uint64_t>(off_hi) << 32) | off_lo);
+      constexpr int U = 8;
+      uint32_t i0 = 0;
+      for (; i0 + U * kWave <= n; i0 += U * kWave) {  // full steps: plain loads, all in flight
+        BinPair<F> e[U];
 #pragma unroll
-      for (int u = 0; u < U; ++u)
-        if (e[u].rel < width) atomicAdd(&window[e[u].rel], static_cast<double>(e[u].val));
+        for (int u = 0; u < U; ++u) e[u] = bin[i0 + u * kWave + lane];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (e[u].rel < width) atomicAdd(&window[e[u].rel], static_cast<double>(e[u].val));
+      }
+      if (i0 < n) {
+        BinPair<F> e[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t i = i0 + u * kWave + lane;
+          e[u].rel = 0xffffffffu;
+          e[u].val = F(0);
+          if (i < n) e[u] = bin[i];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (e[u].rel < width) atomicAdd(&window[e[u].rel], static_cast<double>(e[u].val));
+      }
     }
   }
   __syncthreads();
@@ -293,7 +311,8 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
     hipLaunchKernelGGL((bin_products_kernel<F, false>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
                        indptr, vec, y, n_row, rows_per, n_win, pairs, static_cast<uint64_t>(n_pairs), counts);
   hipLaunchKernelGGL(add_kernel, dim3(n_win * parts), dim3(kBinThreads), lds, stream, indptr, y, n_row, n_col, rows_per,
-                     n_win, parts, producers, pairs, static_cast<uint64_t>(n_pairs), counts, 0u);
+                     n_win, parts, producers, pairs, static_cast<uint64_t>(n_pairs), counts, 0u,
+                     static_cast<uint32_t *>(nullptr));
   return check_launch(target);
 }
 
@@ -301,7 +320,7 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
 // the zeroed y of n_out elements: bin (p, b) = pairs + (p * n_win + b) * cap with counts[b * producers + p] pairs.
 template <typename F>
 bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_out, uint32_t producers, uint32_t cap,
-                      const void *pairs, const uint32_t *counts) {
+                      const void *pairs, const uint32_t *counts, uint32_t *reset) {
   const uint32_t n_win = div_up(n_out, kWinCols);
   auto add_kernel = add_bins_kernel<F>;
   const size_t lds = static_cast<size_t>(kWinCols) * sizeof(double);
@@ -320,14 +339,14 @@ bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_o
   const uint64_t n_pairs = static_cast<uint64_t>(producers) * n_win * cap;
   hipLaunchKernelGGL(add_kernel, dim3(n_win * parts), dim3(kBinThreads), lds, stream,
                      static_cast<const uint32_t *>(nullptr), y, 0u, n_out, 0u, n_win, parts, producers,
-                     static_cast<const BinPair<F> *>(pairs), n_pairs, counts, cap);
+                     static_cast<const BinPair<F> *>(pairs), n_pairs, counts, cap, reset);
   return check_launch(target);
 }
 
 template bool add_uniform_bins<float>(const char *, hipStream_t, float *, uint32_t, uint32_t, uint32_t, const void *,
-                                      const uint32_t *);
+                                      const uint32_t *, uint32_t *);
 template bool add_uniform_bins<double>(const char *, hipStream_t, double *, uint32_t, uint32_t, uint32_t, const void *,
-                                       const uint32_t *);
+                                       const uint32_t *, uint32_t *);
 template bool bin_scatter_usable<float>(uint32_t, uint32_t);
 template bool bin_scatter_usable<double>(uint32_t, uint32_t);
 template bool bin_scatter<float>(const char *, hipStream_t, const float *, bool, const uint32_t *, const uint32_t *,

@@ -134,99 +134,138 @@ __global__ __launch_bounds__(kColThreads) void jitconn_colwalk_kernel(const VT *
   }
 }
 
-// Column walk that appends its (output, value) pairs to bins instead of adding them to `out` one
-// global atomic at a time (about 21 G/s on this device).  Persistent producer workgroup p owns the
-// columns [p * cols_per, (p + 1) * cols_per); a pair for output window b (16,384 outputs) goes to
-// pairs[(p * n_win + b) * cap + position], the position from a 32-bit counter in LDS; a pair that
-// finds its bin full is added directly.  add_uniform_bins() then adds the bins window by window.
-template <typename T1, typename VT, int IN, int W>
-__global__ __launch_bounds__(kColThreads) void jitconn_colwalk_bins_kernel(
-    const VT *__restrict__ in, T1 *__restrict__ out, uint32_t n_out, uint32_t n_in, uint32_t seed, double log_p, T1 wa,
-    T1 wb, uint32_t cols_per, uint32_t n_win, uint32_t cap, BinPair<T1> *__restrict__ pairs,
-    uint32_t *__restrict__ counts) {
-  constexpr int kWaves = kColThreads / kWave;
-  constexpr int kWords = StreamLds<T1, W>::words;
-  __shared__ __attribute__((aligned(8))) uint32_t s_state[kWaves * kWords];
-  __shared__ uint32_t s_col[kColThreads];
-  __shared__ T1 s_val[kColThreads];
-  __shared__ uint32_t s_wave_cnt[kWaves];
-  __shared__ uint32_t s_cnt[kBinMaxWindows];
+// Active input columns of an event vector, gathered into a list in device memory (any order): the
+// column and its value.  A workgroup lists the active ones among its kCollectCols columns in LDS
+// first, so that one atomic reserves all their positions (atomics of many workgroups on the one
+// counter are served one after the other).
+constexpr uint32_t kCollectCols = 4096;
 
-  const int lane = lane_id();
-  const uint32_t wave = threadIdx.x / kWave;
-  const uint32_t p = blockIdx.x;
-  const uint64_t c_lo64 = static_cast<uint64_t>(p) * cols_per;
-  const uint32_t c_lo = c_lo64 < n_in ? static_cast<uint32_t>(c_lo64) : n_in;
-  const uint32_t c_hi = (n_in - c_lo < cols_per) ? n_in : c_lo + cols_per;
-  if (threadIdx.x < kBinMaxWindows) s_cnt[threadIdx.x] = 0;
-  BinPair<T1> *region = pairs + static_cast<uint64_t>(p) * n_win * cap;
-  uint32_t *st = s_state + wave * kWords;
-
-  for (uint32_t tile = c_lo; tile < c_hi; tile += kColThreads) {
-    __syncthreads();  // the previous tile's column list is no longer read (and s_cnt is cleared)
-    const uint32_t c = tile + threadIdx.x;
-    T1 v = T1(0);
+template <typename T1, typename VT>
+__global__ __launch_bounds__(1024) void collect_active_columns_kernel(const VT *__restrict__ in, uint32_t n_in,
+                                                                      uint32_t *__restrict__ counter,
+                                                                      uint32_t *__restrict__ list_col,
+                                                                      T1 *__restrict__ list_val) {
+  __shared__ uint32_t s_col[kCollectCols];
+  __shared__ T1 s_val[kCollectCols];
+  __shared__ uint32_t s_count, s_base;
+  const uint32_t tid = threadIdx.x, lane = tid % kWave;
+  if (tid == 0) s_count = 0;
+  __syncthreads();
+  const uint32_t c0 = blockIdx.x * kCollectCols;
+  for (uint32_t t = 0; t < kCollectCols; t += 1024) {
+    const uint32_t c = c0 + t + tid;
     bool on = false;
-    if (c < c_hi) {
+    T1 v = T1(0);
+    if (c < n_in) {
       const VT x = in[c];
       on = is_event(x);
       v = static_cast<T1>(x);
     }
     const uint64_t mask = __ballot(on);
-    if (lane == 0) s_wave_cnt[wave] = static_cast<uint32_t>(__popcll(mask));
-    __syncthreads();
-    uint32_t base = 0, count = 0;
-#pragma unroll
-    for (uint32_t i = 0; i < kWaves; ++i) {
-      if (i < wave) base += s_wave_cnt[i];
-      count += s_wave_cnt[i];
-    }
+    uint32_t base = 0;
+    if (lane == 0 && mask) base = atomicAdd(&s_count, static_cast<uint32_t>(__popcll(mask)));
+    base = __builtin_amdgcn_readfirstlane(base);
     if (on) {
       const uint32_t k = base + static_cast<uint32_t>(__popcll(mask & ((1ull << lane) - 1ull)));
       s_col[k] = c;
       s_val[k] = v;
     }
-    __syncthreads();
-    for (uint32_t k = wave; k < count; k += kWaves) {
-      const uint32_t col = s_col[k];
-      const T1 val = s_val[k];
-      walk_stream<T1, W>(st, lane, seed + col, nullptr, n_out, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
-        if (valid) {
-          T1 add;
-          if (IN == kInDense) add = (W == kHomo) ? val : static_cast<T1>(w * val);
-          else add = w;  // homo: w == 1
-          const uint32_t b = idx >> kBinWinShift;
-          const uint32_t slot = atomicAdd(&s_cnt[b], 1u);
-          if (slot < cap) {
-            BinPair<T1> e;
-            e.rel = idx & (kBinWinCols - 1u);
-            e.val = add;
-            region[static_cast<uint64_t>(b) * cap + slot] = e;
-          } else {
-            atomic_add(&out[idx], add);
-          }
-        }
-      });
-    }
   }
   __syncthreads();
-  if (threadIdx.x < n_win) {
-    const uint32_t c = s_cnt[threadIdx.x];
-    counts[static_cast<size_t>(threadIdx.x) * gridDim.x + p] = c < cap ? c : cap;
+  const uint32_t count = s_count;
+  if (tid == 0) s_base = count ? atomicAdd(counter, count) : 0u;
+  __syncthreads();
+  const uint32_t base = s_base;
+  for (uint32_t i = tid; i < count; i += 1024) {
+    list_col[base + i] = s_col[i];
+    list_val[base + i] = s_val[i];
   }
+}
+
+// Column walk that appends its (output, value) pairs to bins instead of adding them to `out` one
+// global atomic at a time (about 21 G/s on this device).  The streams to walk are entries
+// [0, n_list) of a list: column list_col[k] with value list_val[k] (event input: the active
+// columns), or, without a list, column first + k with value in[first + k] (dense input).  Waves
+// take entries round robin over the whole grid, so every wave walks the same number of streams.
+// The generators of the first n_seeded entries were seeded ahead on the vector unit (`states`);
+// a wave seeding its own generator does it on the CU's one scalar unit, about 2 us each, and a
+// CU's waves queue up for it.  A pair for output window b (16,384 outputs) of workgroup p goes to
+// pairs[(p * n_win + b) * cap + position]; the positions continue from `counts` (zero before the
+// first launch of a call), so that a call may be split into several launches; a pair that finds
+// its bin full is added to `out` directly.  add_uniform_bins() then adds the bins window by window.
+constexpr int kColBinThreads = 1024;  // 16 waves share one set of bins: 4 times fewer, 4 times larger bins
+
+template <typename T1, typename VT, int IN, int W>
+__global__ __launch_bounds__(kColBinThreads) void jitconn_colwalk_bins_kernel(
+    const VT *__restrict__ in, T1 *__restrict__ out, uint32_t n_out, uint32_t seed, double log_p, T1 wa, T1 wb,
+    uint32_t first, uint32_t n_list_host, const uint32_t *__restrict__ n_list_dev,
+    const uint32_t *__restrict__ list_col, const T1 *__restrict__ list_val, const uint32_t *__restrict__ states,
+    uint32_t n_seeded, uint32_t n_win, uint32_t cap, BinPair<T1> *__restrict__ pairs, uint32_t *__restrict__ counts) {
+  constexpr int kWaves = kColBinThreads / kWave;
+  constexpr int kWords = StreamLds<T1, W>::words;
+  __shared__ __attribute__((aligned(8))) uint32_t s_state[kWaves * kWords];
+  __shared__ uint32_t s_cnt[kBinMaxWindows];
+
+  const int lane = lane_id();
+  const uint32_t wave = threadIdx.x / kWave;
+  const uint32_t p = blockIdx.x;
+  if (threadIdx.x < n_win) s_cnt[threadIdx.x] = counts[static_cast<size_t>(threadIdx.x) * gridDim.x + p];
+  __syncthreads();
+  BinPair<T1> *region = pairs + static_cast<uint64_t>(p) * n_win * cap;
+  uint32_t *st = s_state + wave * kWords;
+  const uint32_t n_list = n_list_dev ? *n_list_dev : n_list_host;
+
+  for (uint32_t k = wave * gridDim.x + p; k < n_list; k += gridDim.x * kWaves) {
+    uint32_t col;
+    T1 val;
+    if (list_col != nullptr) {
+      col = list_col[k];
+      val = list_val[k];
+    } else {
+      col = first + k;
+      val = static_cast<T1>(in[col]);
+      if (!is_event(val)) continue;  // a zero input adds nothing (wave uniform)
+    }
+    const uint32_t *pre = (k < n_seeded) ? states + static_cast<size_t>(k) * kMtN : nullptr;
+    walk_stream<T1, W>(st, lane, seed + col, pre, n_out, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
+      if (valid) {
+        T1 add;
+        if (IN == kInDense) add = (W == kHomo) ? val : static_cast<T1>(w * val);
+        else add = w;  // homo: w == 1
+        const uint32_t b = idx >> kBinWinShift;
+        const uint32_t slot = atomicAdd(&s_cnt[b], 1u);
+        if (slot < cap) {
+          BinPair<T1> e;
+          e.rel = idx & (kBinWinCols - 1u);
+          e.val = add;
+          region[static_cast<uint64_t>(b) * cap + slot] = e;
+        } else {
+          atomic_add(&out[idx], add);
+        }
+      }
+    });
+  }
+  __syncthreads();
+  if (threadIdx.x < n_win) counts[static_cast<size_t>(threadIdx.x) * gridDim.x + p] = s_cnt[threadIdx.x];
 }
 
 // ---- seeding ahead ------------------------------------------------------------------------------------
 constexpr int kSeedThreads = 128;
 
+// Stream s of the launch is seed + first + s, or, with a list, seed + ids[s]; `count_dev` (optional)
+// holds the number of list entries, of which at most `count` are seeded.
 __global__ __launch_bounds__(kSeedThreads) void mt_seed_streams_kernel(uint32_t seed, uint32_t first, uint32_t count,
-                                                                      uint32_t *__restrict__ states) {
+                                                                      uint32_t *__restrict__ states,
+                                                                      const uint32_t *__restrict__ ids,
+                                                                      const uint32_t *__restrict__ count_dev) {
   __shared__ uint32_t s_tile[kSeedThreads / kWave][kWave][kWave + 1];
   const uint32_t lane = static_cast<uint32_t>(lane_id()), wave = threadIdx.x / kWave;
   const uint32_t base = (blockIdx.x * (kSeedThreads / kWave) + wave) * kWave;  // first stream of this wave
+  if (count_dev != nullptr && *count_dev < count) count = *count_dev;
   if (base >= count) return;
   uint32_t (*tile)[kWave + 1] = s_tile[wave];
   uint32_t x = seed + first + base + lane;  // lane l seeds stream base + l
+  if (ids != nullptr) x = seed + ((base + lane < count) ? ids[base + lane] : 0u);
   for (uint32_t w0 = 0; w0 < kMtN; w0 += kWave) {
     const uint32_t nw = (kMtN - w0 < kWave) ? kMtN - w0 : kWave;
     for (uint32_t i = 0; i < nw; ++i) {
@@ -244,7 +283,8 @@ __global__ __launch_bounds__(kSeedThreads) void mt_seed_streams_kernel(uint32_t 
 void launch_seed_streams(hipStream_t stream, uint32_t seed, uint32_t first, uint32_t count, uint32_t *states) {
   if (count == 0) return;
   hipLaunchKernelGGL(mt_seed_streams_kernel, dim3(div_up(count, kSeedThreads)), dim3(kSeedThreads), 0, stream, seed,
-                     first, count, states);
+                     first, count, states, static_cast<const uint32_t *>(nullptr),
+                     static_cast<const uint32_t *>(nullptr));
 }
 
 namespace {
@@ -337,26 +377,58 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
   const double p_conn = -std::expm1(log_p);
   const double full = static_cast<double>(n_in) * static_cast<double>(n_out) * p_conn;
   if (n_win >= 2 && n_win <= kBinMaxWindows && full >= (IN == kInDense ? 1048576.0 : 5.0e7)) {
-    uint32_t producers = 4u * static_cast<uint32_t>(device_info().num_cu);
-    if (producers > div_up(n_in, kColThreads)) producers = div_up(n_in, kColThreads);
-    const uint32_t cols_per = div_up(n_in, producers);
-    producers = div_up(n_in, cols_per);
-    const double per_bin = static_cast<double>(cols_per) * kBinWinCols * p_conn;  // every column active
+    uint32_t producers = 2u * static_cast<uint32_t>(device_info().num_cu);
+    if (producers > div_up(n_in, kColBinThreads / kWave)) producers = div_up(n_in, kColBinThreads / kWave);
+    const double per_bin = full / (static_cast<double>(producers) * n_win);  // every column active
     double cap_d = 1.25 * per_bin + 6.0 * std::sqrt(per_bin) + 128.0;
     if (IN == kInEvent) cap_d = cap_d / 8.0 < 512.0 ? 512.0 : cap_d / 8.0;
+    auto round_up = [](size_t v) { return (v + 255) / 256 * 256; };
     const size_t total_pairs = static_cast<size_t>(producers) * n_win * static_cast<size_t>(cap_d);
-    const size_t pair_bytes = (total_pairs * sizeof(BinPair<T1>) + 255) / 256 * 256;
-    if (cap_d < 4.0e9 && pair_bytes <= (static_cast<size_t>(32) << 30)) {
+    const size_t pair_bytes = round_up(total_pairs * sizeof(BinPair<T1>));
+    const size_t count_bytes = round_up(static_cast<size_t>(n_win) * producers * sizeof(uint32_t));
+    const uint32_t seeded_max = n_in < kSeedChunk ? n_in : kSeedChunk;
+    const size_t state_bytes = round_up(static_cast<size_t>(seeded_max) * kMtN * 4);
+    const size_t list_bytes = (IN == kInEvent) ? round_up(static_cast<size_t>(n_in) * 4) : 0;
+    const size_t val_bytes = (IN == kInEvent) ? round_up(static_cast<size_t>(n_in) * sizeof(T1)) : 0;
+    uint32_t *list_count = (IN == kInEvent) ? stream_counters(stream) : nullptr;
+    if (cap_d < 4.0e9 && pair_bytes <= (static_cast<size_t>(32) << 30) && (IN == kInDense || list_count != nullptr)) {
       const uint32_t cap = static_cast<uint32_t>(cap_d);
       unsigned char *ws = static_cast<unsigned char *>(
-        stream_workspace(stream, pair_bytes + static_cast<size_t>(n_win) * producers * sizeof(uint32_t)));
+        stream_workspace(stream, pair_bytes + count_bytes + state_bytes + list_bytes + val_bytes));
       if (ws != nullptr) {
         BinPair<T1> *pairs = reinterpret_cast<BinPair<T1> *>(ws);
         uint32_t *counts = reinterpret_cast<uint32_t *>(ws + pair_bytes);
-        hipLaunchKernelGGL((jitconn_colwalk_bins_kernel<T1, VT, IN, W>), dim3(producers), dim3(kColThreads), 0, stream,
-                           in, out, n_out, n_in, seed, log_p, wa, wb, cols_per, n_win, cap, pairs, counts);
-        if (add_uniform_bins<T1>("jitconn column walk", stream, out, n_out, producers, cap, pairs, counts)) return;
+        uint32_t *states = reinterpret_cast<uint32_t *>(ws + pair_bytes + count_bytes);
+        uint32_t *list_col = list_bytes ? reinterpret_cast<uint32_t *>(ws + pair_bytes + count_bytes + state_bytes) : nullptr;
+        T1 *list_val = val_bytes ? reinterpret_cast<T1 *>(ws + pair_bytes + count_bytes + state_bytes + list_bytes) : nullptr;
+        fill_zero(stream, counts, n_win * producers);
+        auto walk = jitconn_colwalk_bins_kernel<T1, VT, IN, W>;
+        if (IN == kInEvent) {
+          // the active columns, their generators seeded ahead (those beyond kSeedChunk seed themselves), one walk
+          hipLaunchKernelGGL((collect_active_columns_kernel<T1, VT>), dim3(div_up(n_in, kCollectCols)), dim3(1024), 0, stream,
+                             in, n_in, list_count, list_col, list_val);
+          hipLaunchKernelGGL(mt_seed_streams_kernel, dim3(div_up(seeded_max, kSeedThreads)), dim3(kSeedThreads), 0,
+                             stream, seed, 0u, seeded_max, states, static_cast<const uint32_t *>(list_col),
+                             static_cast<const uint32_t *>(list_count));
+          hipLaunchKernelGGL(walk, dim3(producers), dim3(kColBinThreads), 0, stream, in, out, n_out, seed, log_p, wa, wb,
+                             0u, 0u, static_cast<const uint32_t *>(list_count), static_cast<const uint32_t *>(list_col),
+                             static_cast<const T1 *>(list_val), static_cast<const uint32_t *>(states), seeded_max,
+                             n_win, cap, pairs, counts);
+        } else {
+          // every column, a chunk of seeded generators at a time
+          for (uint32_t first = 0; first < n_in; first += kSeedChunk) {
+            const uint32_t count = (n_in - first < kSeedChunk) ? n_in - first : kSeedChunk;
+            launch_seed_streams(stream, seed, first, count, states);
+            hipLaunchKernelGGL(walk, dim3(producers), dim3(kColBinThreads), 0, stream, in, out, n_out, seed, log_p, wa,
+                               wb, first, count, static_cast<const uint32_t *>(nullptr),
+                               static_cast<const uint32_t *>(nullptr), static_cast<const T1 *>(nullptr),
+                               static_cast<const uint32_t *>(states), count, n_win, cap, pairs, counts);
+          }
+        }
+        if (add_uniform_bins<T1>("jitconn column walk", stream, out, n_out, producers, cap, pairs, counts, list_count))
+          return;
         // (the bins could not be added: nothing reached `out` yet except overflow pairs; start over)
+        if (list_count != nullptr) fill_zero(stream, list_count, 1u);
         fill_zero(stream, out, n_out);
       } else {
         bpl_clear_error();
