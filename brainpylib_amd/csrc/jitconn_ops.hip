@@ -369,14 +369,14 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
                     double log_p, T1 wa, T1 wb) {
   fill_zero(stream, out, n_out);
   if (n_in == 0 || n_out == 0) return;
-  // Many pairs and an output far wider than LDS: bins.  The number of pairs is n_in * n_out * p for a
+  // Many pairs: bins (also for a narrow output: seeding ahead and the even spread of the streams pay).  The number of pairs is n_in * n_out * p for a
   // dense input; for events it depends on the activity, which the host does not know: bins are sized
   // for one column in eight being active (fuller bins overflow into direct atomics) and used when
   // one active column in a hundred already means half a million pairs.
   const uint32_t n_win = div_up(n_out, kBinWinCols);
   const double p_conn = -std::expm1(log_p);
   const double full = static_cast<double>(n_in) * static_cast<double>(n_out) * p_conn;
-  if (n_win >= 2 && n_win <= kBinMaxWindows && full >= (IN == kInDense ? 1048576.0 : 5.0e7)) {
+  if (n_win <= kBinMaxWindows && full >= (IN == kInDense ? 1048576.0 : 5.0e7)) {
     uint32_t producers = 2u * static_cast<uint32_t>(device_info().num_cu);
     if (producers > div_up(n_in, kColBinThreads / kWave)) producers = div_up(n_in, kColBinThreads / kWave);
     const double per_bin = full / (static_cast<double>(producers) * n_win);  // every column active
