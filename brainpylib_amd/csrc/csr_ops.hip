@@ -211,7 +211,11 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
   // about a third of a lane per clock and CU, 64-bit floats nine times and 32-bit integers
   // thirty times faster.  A float64 window would halve the window and double the passes over the
   // indices, which costs what the faster additions save at the sizes tried.)
+  // With a homogeneous weight and event input the window counts synapses instead (32-bit integer
+  // LDS adds, exact) and the weight is multiplied in once per output at the end.
+  constexpr bool kCount = !HETER && MODE == kEvent;
   F *window = reinterpret_cast<F *>(smem_raw);
+  uint32_t *cwindow = reinterpret_cast<uint32_t *>(smem_raw);
   F *s_scale = window + win;  // dense mode: x[r] per active row
   uint32_t *s_start = reinterpret_cast<uint32_t *>(s_scale + (MODE == kDense ? kWinMaxRows : 0));
   uint32_t *s_len = s_start + kWinMaxRows;
@@ -233,8 +237,15 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
   const uint32_t c0 = b * win;
   const uint32_t width = (c0 + win <= n_col) ? win : n_col - c0;
 
-  for (uint32_t i = tid; i < width; i += kWinThreads) window[i] = F(0);
   const F w_homo = HETER ? F(0) : data[0];
+  // n synapses of weight w: n * w rounded once (nothing, not 0 * w, where no synapse arrived)
+  auto counted = [&](uint32_t n) {
+    return n ? static_cast<F>(static_cast<double>(w_homo) * static_cast<double>(n)) : F(0);
+  };
+  for (uint32_t i = tid; i < width; i += kWinThreads) {
+    if (kCount) cwindow[i] = 0u;
+    else window[i] = F(0);
+  }
 
   // Source of the active rows: this group's share of the list made by collect_active_rows_kernel,
   // or (active_list == nullptr) the group's own rows_per_wg rows, tested here.  Either way they are
@@ -345,7 +356,10 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      if (rel[u] < width) atomicAdd(&window[rel[u]], (MODE == kDense) ? static_cast<F>(scale * w[u]) : w[u]);
+      if (rel[u] < width) {
+        if (kCount) atomicAdd(&cwindow[rel[u]], 1u);
+        else atomicAdd(&window[rel[u]], (MODE == kDense) ? static_cast<F>(scale * w[u]) : w[u]);
+      }
     }
     k = nk, start = nstart, len = nlen, b0 = nb0, scale = nscale;
 #pragma unroll
@@ -358,10 +372,11 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     // plain contiguous stores of the whole window into this row group's slice; a second
     // kernel sums the slices
     F *dst = partial + static_cast<size_t>(g) * n_col + c0;
-    for (uint32_t i = tid; i < width; i += kWinThreads) dst[i] = window[i];
+    for (uint32_t i = tid; i < width; i += kWinThreads)
+      dst[i] = kCount ? counted(cwindow[i]) : window[i];
   } else {
     for (uint32_t i = tid; i < width; i += kWinThreads) {
-      const F v = window[i];
+      const F v = kCount ? counted(cwindow[i]) : window[i];
       if (v != F(0)) atomic_add(&y[c0 + i], v);
     }
   }
