@@ -7,9 +7,16 @@
 
 namespace bpl {
 
-constexpr uint32_t kBinWinShift = 14;  // output window = 16,384 elements (128 KB of float64)
-constexpr uint32_t kBinWinCols = 1u << kBinWinShift;
+constexpr uint32_t kBinMaxShift = 14;     // largest output window: 16,384 elements (128 KB of float64)
 constexpr uint32_t kBinMaxWindows = 128;  // 7-bit window ids
+
+// log2 of the output window for n_out outputs: about 64 windows (many LDS counters for the
+// producers to spread over, enough consumer workgroups), at most 16,384 elements each.
+inline uint32_t bin_window_shift(uint32_t n_out) {
+  uint32_t shift = 8;
+  while (shift < kBinMaxShift && (n_out >> shift) > 64u) ++shift;
+  return shift;
+}
 
 template <typename F>
 struct BinPair {

@@ -61,11 +61,11 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
 
 // Second half of the coarse-sorted scatter for producers other than the CSR one: adds bins laid
 // out uniformly, bin (p, b) = pairs + (p * n_win + b) * cap with counts[b * producers + p]
-// BinPair<F> entries (bins.h; counts above cap mean cap), n_win = ceil(n_out / 16,384), into the
+// BinPair<F> entries (bins.h; counts above cap mean cap), n_win = ceil(n_out / 2^shift), into the
 // zeroed y.  `reset` (optional): a device counter of the producer's that the kernel sets to zero.
 template <typename F>
-bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_out, uint32_t producers, uint32_t cap,
-                      const void *pairs, const uint32_t *counts, uint32_t *reset);
+bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_out, uint32_t shift, uint32_t producers,
+                      uint32_t cap, const void *pairs, const uint32_t *counts, uint32_t *reset);
 
 inline unsigned div_up(unsigned long long a, unsigned long long b) {
   return static_cast<unsigned>((a + b - 1) / b);

@@ -4,7 +4,8 @@
 // retires at about 21 G/s on this device; instead the products are first sorted coarsely:
 //
 //   bin kernel     persistent producer workgroups walk their rows, form (column, product)
-//                  pairs and append each pair to the bin of its 16,384-column output window,
+//                  pairs and append each pair to the bin of its output window (a power of two of
+//                  columns, at most 16,384, chosen so that there are about 64 windows),
 //                  in a region of scratch memory private to (producer, window): no global
 //                  atomics, the position comes from a counter in LDS (32-bit integer LDS
 //                  atomics are cheap even when lanes meet).  A pair that does not fit its
@@ -22,8 +23,6 @@ namespace {
 
 constexpr int kBinThreads = 1024;
 constexpr uint32_t kTileRows = 1024;      // rows staged in LDS at a time by a producer
-constexpr uint32_t kWinShift = kBinWinShift;
-constexpr uint32_t kWinCols = kBinWinCols;
 constexpr uint32_t kMaxWindows = kBinMaxWindows;
 constexpr uint32_t kRegionSlack = 128;    // pairs a region holds beyond 5/4 of its even share
 
@@ -49,7 +48,7 @@ constexpr uint32_t kSegment = kBinThreads << kHintShift;  // nonzeros covered by
 template <typename F, bool HETER>
 __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
-    const F *__restrict__ vec, F *__restrict__ y, uint32_t n_row, uint32_t rows_per, uint32_t n_win,
+    const F *__restrict__ vec, F *__restrict__ y, uint32_t n_row, uint32_t rows_per, uint32_t n_win, uint32_t shift,
     BinPair<F> *__restrict__ pairs, uint64_t n_pairs, uint32_t *__restrict__ counts) {
   __shared__ uint32_t s_ptr[kTileRows + 1];
   __shared__ F s_v[kTileRows];
@@ -119,8 +118,8 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
             const uint32_t col = indices[j];
             // v * values[j] (heter) or values * v (homo), as the reference's CPU loop multiplies
             val[u] = HETER ? static_cast<F>(s_v[k] * data[j]) : static_cast<F>(w_homo * s_v[k]);
-            win[u] = col >> kWinShift;
-            rel[u] = col & (kWinCols - 1u);
+            win[u] = col >> shift;
+            rel[u] = col & ((1u << shift) - 1u);
           }
         }
 #pragma unroll
@@ -154,7 +153,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
           const uint32_t slot = s_total[w] + (i - s_off[w]);
           const uint64_t at = region_off + static_cast<uint64_t>(w) * cap + slot;
           if (slot < cap && at < n_pairs) pairs[at] = e;
-          else atomic_add(y + ((w << kWinShift) | e.rel), e.val);
+          else atomic_add(y + ((w << shift) | e.rel), e.val);
         }
         __syncthreads();
         if (tid < kMaxWindows) {
@@ -177,7 +176,8 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
 template <typename F>
 __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *__restrict__ indptr,
                                                                F *__restrict__ y, uint32_t n_row, uint32_t n_col,
-                                                               uint32_t rows_per, uint32_t n_win, uint32_t parts,
+                                                               uint32_t rows_per, uint32_t n_win, uint32_t shift,
+                                                               uint32_t parts,
                                                                uint32_t producers,
                                                                const BinPair<F> *__restrict__ pairs,
                                                                uint64_t n_pairs,
@@ -190,8 +190,8 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
   const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   constexpr uint32_t kWaves = kBinThreads / kWave;
   const uint32_t b = blockIdx.x / parts, s = blockIdx.x % parts;
-  const uint32_t c0 = b << kWinShift;
-  const uint32_t width = (n_col - c0 < kWinCols) ? n_col - c0 : kWinCols;
+  const uint32_t c0 = b << shift;
+  const uint32_t width = (n_col - c0 < (1u << shift)) ? n_col - c0 : (1u << shift);
   for (uint32_t i = tid; i < width; i += kBinThreads) window[i] = 0.0;
   __syncthreads();
   const uint32_t p_lo = static_cast<uint32_t>(static_cast<uint64_t>(s) * producers / parts);
@@ -262,14 +262,15 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
 
 template <typename F>
 bool bin_scatter_usable(uint32_t n_col, uint32_t nnz) {
-  const uint32_t n_win = div_up(n_col, kWinCols);
+  const uint32_t n_win = div_up(n_col, 1u << bin_window_shift(n_col));
   return n_win >= 2 && n_win <= kMaxWindows && nnz >= (1u << 20);
 }
 
 template <typename F>
 bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool heter, const uint32_t *indices,
                  const uint32_t *indptr, const F *vec, F *y, uint32_t n_row, uint32_t n_col, uint32_t nnz) {
-  const uint32_t n_win = div_up(n_col, kWinCols);
+  const uint32_t shift = bin_window_shift(n_col);
+  const uint32_t n_win = div_up(n_col, 1u << shift);
   const unsigned num_cu = static_cast<unsigned>(device_info().num_cu);
   // two producer workgroups per CU, at least 64 rows each
   uint32_t producers = 2u * num_cu;
@@ -293,9 +294,9 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
   uint32_t *counts = reinterpret_cast<uint32_t *>(ws + pair_bytes);
 
   auto add_kernel = add_bins_kernel<F>;
-  const size_t lds = static_cast<size_t>(kWinCols) * sizeof(double);
+  const size_t lds = sizeof(double) << shift;
   static thread_local bool attr_set = false;
-  if (!attr_set) {
+  if (!attr_set && lds > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(add_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             static_cast<int>(lds)) != hipSuccess) {
       (void)hipGetLastError();
@@ -306,12 +307,12 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
   fill_zero(stream, y, n_col);
   if (heter)
     hipLaunchKernelGGL((bin_products_kernel<F, true>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
-                       indptr, vec, y, n_row, rows_per, n_win, pairs, static_cast<uint64_t>(n_pairs), counts);
+                       indptr, vec, y, n_row, rows_per, n_win, shift, pairs, static_cast<uint64_t>(n_pairs), counts);
   else
     hipLaunchKernelGGL((bin_products_kernel<F, false>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
-                       indptr, vec, y, n_row, rows_per, n_win, pairs, static_cast<uint64_t>(n_pairs), counts);
+                       indptr, vec, y, n_row, rows_per, n_win, shift, pairs, static_cast<uint64_t>(n_pairs), counts);
   hipLaunchKernelGGL(add_kernel, dim3(n_win * parts), dim3(kBinThreads), lds, stream, indptr, y, n_row, n_col, rows_per,
-                     n_win, parts, producers, pairs, static_cast<uint64_t>(n_pairs), counts, 0u,
+                     n_win, shift, parts, producers, pairs, static_cast<uint64_t>(n_pairs), counts, 0u,
                      static_cast<uint32_t *>(nullptr));
   return check_launch(target);
 }
@@ -319,13 +320,13 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
 // Adds uniformly laid out bins (filled by another producer, e.g. the jitconn column walk) to
 // the zeroed y of n_out elements: bin (p, b) = pairs + (p * n_win + b) * cap with counts[b * producers + p] pairs.
 template <typename F>
-bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_out, uint32_t producers, uint32_t cap,
-                      const void *pairs, const uint32_t *counts, uint32_t *reset) {
-  const uint32_t n_win = div_up(n_out, kWinCols);
+bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_out, uint32_t shift, uint32_t producers,
+                      uint32_t cap, const void *pairs, const uint32_t *counts, uint32_t *reset) {
+  const uint32_t n_win = div_up(n_out, 1u << shift);
   auto add_kernel = add_bins_kernel<F>;
-  const size_t lds = static_cast<size_t>(kWinCols) * sizeof(double);
+  const size_t lds = sizeof(double) << shift;
   static thread_local bool attr_set = false;
-  if (!attr_set) {
+  if (!attr_set && lds > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(add_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             static_cast<int>(lds)) != hipSuccess) {
       (void)hipGetLastError();
@@ -338,14 +339,15 @@ bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_o
   if (parts > producers) parts = producers;
   const uint64_t n_pairs = static_cast<uint64_t>(producers) * n_win * cap;
   hipLaunchKernelGGL(add_kernel, dim3(n_win * parts), dim3(kBinThreads), lds, stream,
-                     static_cast<const uint32_t *>(nullptr), y, 0u, n_out, 0u, n_win, parts, producers,
+                     static_cast<const uint32_t *>(nullptr), y, 0u, n_out, 0u, n_win, shift, parts, producers,
                      static_cast<const BinPair<F> *>(pairs), n_pairs, counts, cap, reset);
   return check_launch(target);
 }
 
-template bool add_uniform_bins<float>(const char *, hipStream_t, float *, uint32_t, uint32_t, uint32_t, const void *,
+template bool add_uniform_bins<float>(const char *, hipStream_t, float *, uint32_t, uint32_t, uint32_t, uint32_t, const void *,
                                       const uint32_t *, uint32_t *);
-template bool add_uniform_bins<double>(const char *, hipStream_t, double *, uint32_t, uint32_t, uint32_t, const void *,
+template bool add_uniform_bins<double>(const char *, hipStream_t, double *, uint32_t, uint32_t, uint32_t, uint32_t,
+                                       const void *,
                                        const uint32_t *, uint32_t *);
 template bool bin_scatter_usable<float>(uint32_t, uint32_t);
 template bool bin_scatter_usable<double>(uint32_t, uint32_t);

@@ -21,6 +21,8 @@
 //
 // Reference boundary: lib/gpu_event_csr_matvec.cu:148-260, lib/gpu_csr_matvec.cu:84-135,195-246,
 // 505-621 (buffer order, descriptor, target names).
+#include <type_traits>
+
 #include "common.h"
 #include "targets.h"
 
@@ -198,7 +200,9 @@ __global__ __launch_bounds__(kWinThreads) void collect_active_rows_kernel(
   }
 }
 
-template <typename F, typename VT, bool HETER, int MODE>
+// A = type of the window's accumulators: F, or double where every lane adds (dense input):
+// 64-bit LDS float adds retire nine times faster than 32-bit ones on this device.
+template <typename F, typename VT, bool HETER, int MODE, typename A>
 __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
     const VT *__restrict__ x, F *__restrict__ y, uint32_t n_row, uint32_t n_col, uint32_t rows_per_wg,
@@ -207,16 +211,16 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     const F *__restrict__ active_scales) {
   if (!gate.open(indptr, n_row)) return;
   extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
-  // The window accumulates in F.  (Measured on this device: the LDS unit adds 32-bit floats at
-  // about a third of a lane per clock and CU, 64-bit floats nine times and 32-bit integers
-  // thirty times faster.  A float64 window would halve the window and double the passes over the
-  // indices, which costs what the faster additions save at the sizes tried.)
+  // (Measured on this device: the LDS unit adds 32-bit floats at about a third of a lane per clock
+  // and CU, 64-bit floats nine times and 32-bit integers thirty times faster.  For sparse event
+  // input a float64 window would halve the window and double the passes over the indices, which
+  // costs what the faster additions save at the sizes tried: A = F there.)
   // With a homogeneous weight and event input the window counts synapses instead (32-bit integer
   // LDS adds, exact) and the weight is multiplied in once per output at the end.
   constexpr bool kCount = !HETER && MODE == kEvent;
-  F *window = reinterpret_cast<F *>(smem_raw);
+  A *window = reinterpret_cast<A *>(smem_raw);
   uint32_t *cwindow = reinterpret_cast<uint32_t *>(smem_raw);
-  F *s_scale = window + win;  // dense mode: x[r] per active row
+  F *s_scale = reinterpret_cast<F *>(window + win);  // dense mode: x[r] per active row
   uint32_t *s_start = reinterpret_cast<uint32_t *>(s_scale + (MODE == kDense ? kWinMaxRows : 0));
   uint32_t *s_len = s_start + kWinMaxRows;
   __shared__ uint32_t s_count, s_next;
@@ -244,7 +248,7 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
   };
   for (uint32_t i = tid; i < width; i += kWinThreads) {
     if (kCount) cwindow[i] = 0u;
-    else window[i] = F(0);
+    else window[i] = A(0);
   }
 
   // Source of the active rows: this group's share of the list made by collect_active_rows_kernel,
@@ -358,7 +362,7 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     for (int u = 0; u < U; ++u) {
       if (rel[u] < width) {
         if (kCount) atomicAdd(&cwindow[rel[u]], 1u);
-        else atomicAdd(&window[rel[u]], (MODE == kDense) ? static_cast<F>(scale * w[u]) : w[u]);
+        else atomicAdd(&window[rel[u]], static_cast<A>((MODE == kDense) ? static_cast<F>(scale * w[u]) : w[u]));
       }
     }
     k = nk, start = nstart, len = nlen, b0 = nb0, scale = nscale;
@@ -373,10 +377,10 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     // kernel sums the slices
     F *dst = partial + static_cast<size_t>(g) * n_col + c0;
     for (uint32_t i = tid; i < width; i += kWinThreads)
-      dst[i] = kCount ? counted(cwindow[i]) : window[i];
+      dst[i] = kCount ? counted(cwindow[i]) : static_cast<F>(window[i]);
   } else {
     for (uint32_t i = tid; i < width; i += kWinThreads) {
-      const F v = kCount ? counted(cwindow[i]) : window[i];
+      const F v = kCount ? counted(cwindow[i]) : static_cast<F>(window[i]);
       if (v != F(0)) atomic_add(&y[c0 + i], v);
     }
   }
@@ -619,8 +623,9 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
   // rows again, which is still far cheaper than one random global atomic per nonzero (about
   // 21 G/s) up to a few dozen windows when the activity is sparse (event input) and the rows are
   // long.  With a dense input every row is active and only a handful of windows pay off.
+  using A = typename std::conditional<MODE == kDense, double, F>::type;  // window accumulators
   const size_t list_bytes = kWinMaxRows * (8 + (MODE == kDense ? sizeof(F) : 0));
-  const uint32_t win_cap = static_cast<uint32_t>((static_cast<size_t>(128) * 1024) / sizeof(F));
+  const uint32_t win_cap = static_cast<uint32_t>((static_cast<size_t>(128) * 1024) / sizeof(A));
   const uint32_t n_win = div_up(n_col, win_cap);
   NnzGate direct_gate = kAlways;
   if (n_win <= (MODE == kEvent ? 32u : 4u)) {
@@ -649,8 +654,8 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
         direct_gate = {0u, static_cast<uint32_t>(min_nnz) - 1u};
       }
     }
-    const size_t lds = static_cast<size_t>(win) * sizeof(F) + list_bytes;
-    auto kernel = csr_scatter_window_kernel<F, VT, HETER, MODE>;
+    const size_t lds = static_cast<size_t>(win) * sizeof(A) + list_bytes;
+    auto kernel = csr_scatter_window_kernel<F, VT, HETER, MODE, A>;
     static thread_local size_t attr_set_for = 0;
     if (usable && lds > 64 * 1024 && attr_set_for < lds) {
       if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -814,9 +819,11 @@ void csr_matvec_entry(const char *target, hipStream_t stream, void **buffers, co
   const F *vec = static_cast<const F *>(buffers[vector_slot]);
   F *out = static_cast<F *>(buffers[vector_slot + 1]);
   if (TRANSPOSE) {
-    // outputs beyond four LDS windows: sort the products coarsely instead of one global atomic each
-    const uint32_t plain_windows = div_up(d.n_col, static_cast<uint32_t>((128u * 1024u) / sizeof(F)));
-    if (plain_windows > 4 && d.n_row > 0 && bin_scatter_usable<F>(d.n_col, nnz) &&
+    // Outputs beyond one float64 LDS window: sort the products coarsely.  (With every row active each
+    // further window means another pass over the whole matrix; the windows remain for matrices too
+    // small to sort or of unknown size, direct atomics beyond four windows.)
+    const uint32_t plain_windows = div_up(d.n_col, static_cast<uint32_t>((128u * 1024u) / sizeof(double)));
+    if (plain_windows > 1 && d.n_row > 0 && bin_scatter_usable<F>(d.n_col, nnz) &&
         bin_scatter<F>(target, stream, data, HETER, indices, indptr, vec, out, d.n_row, d.n_col, nnz))
       return;
     launch_scatter<F, F, HETER, kDense>(stream, data, indices, indptr, vec, out, d.n_row, d.n_col);

@@ -189,7 +189,7 @@ __global__ __launch_bounds__(1024) void collect_active_columns_kernel(const VT *
 // take entries round robin over the whole grid, so every wave walks the same number of streams.
 // The generators of the first n_seeded entries were seeded ahead on the vector unit (`states`);
 // a wave seeding its own generator does it on the CU's one scalar unit, about 2 us each, and a
-// CU's waves queue up for it.  A pair for output window b (16,384 outputs) of workgroup p goes to
+// CU's waves queue up for it.  A pair for output window b (2^shift outputs) of workgroup p goes to
 // pairs[(p * n_win + b) * cap + position]; the positions continue from `counts` (zero before the
 // first launch of a call), so that a call may be split into several launches; a pair that finds
 // its bin full is added to `out` directly.  add_uniform_bins() then adds the bins window by window.
@@ -200,7 +200,8 @@ __global__ __launch_bounds__(kColBinThreads) void jitconn_colwalk_bins_kernel(
     const VT *__restrict__ in, T1 *__restrict__ out, uint32_t n_out, uint32_t seed, double log_p, T1 wa, T1 wb,
     uint32_t first, uint32_t n_list_host, const uint32_t *__restrict__ n_list_dev,
     const uint32_t *__restrict__ list_col, const T1 *__restrict__ list_val, const uint32_t *__restrict__ states,
-    uint32_t n_seeded, uint32_t n_win, uint32_t cap, BinPair<T1> *__restrict__ pairs, uint32_t *__restrict__ counts) {
+    uint32_t n_seeded, uint32_t n_win, uint32_t shift, uint32_t cap, BinPair<T1> *__restrict__ pairs,
+    uint32_t *__restrict__ counts) {
   constexpr int kWaves = kColBinThreads / kWave;
   constexpr int kWords = StreamLds<T1, W>::words;
   __shared__ __attribute__((aligned(8))) uint32_t s_state[kWaves * kWords];
@@ -232,11 +233,11 @@ __global__ __launch_bounds__(kColBinThreads) void jitconn_colwalk_bins_kernel(
         T1 add;
         if (IN == kInDense) add = (W == kHomo) ? val : static_cast<T1>(w * val);
         else add = w;  // homo: w == 1
-        const uint32_t b = idx >> kBinWinShift;
+        const uint32_t b = idx >> shift;
         const uint32_t slot = atomicAdd(&s_cnt[b], 1u);
         if (slot < cap) {
           BinPair<T1> e;
-          e.rel = idx & (kBinWinCols - 1u);
+          e.rel = idx & ((1u << shift) - 1u);
           e.val = add;
           region[static_cast<uint64_t>(b) * cap + slot] = e;
         } else {
@@ -373,7 +374,8 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
   // dense input; for events it depends on the activity, which the host does not know: bins are sized
   // for one column in eight being active (fuller bins overflow into direct atomics) and used when
   // one active column in a hundred already means half a million pairs.
-  const uint32_t n_win = div_up(n_out, kBinWinCols);
+  const uint32_t shift = bin_window_shift(n_out);
+  const uint32_t n_win = div_up(n_out, 1u << shift);
   const double p_conn = -std::expm1(log_p);
   const double full = static_cast<double>(n_in) * static_cast<double>(n_out) * p_conn;
   if (n_win <= kBinMaxWindows && full >= (IN == kInDense ? 1048576.0 : 5.0e7)) {
@@ -413,7 +415,7 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
           hipLaunchKernelGGL(walk, dim3(producers), dim3(kColBinThreads), 0, stream, in, out, n_out, seed, log_p, wa, wb,
                              0u, 0u, static_cast<const uint32_t *>(list_count), static_cast<const uint32_t *>(list_col),
                              static_cast<const T1 *>(list_val), static_cast<const uint32_t *>(states), seeded_max,
-                             n_win, cap, pairs, counts);
+                             n_win, shift, cap, pairs, counts);
         } else {
           // every column, a chunk of seeded generators at a time
           for (uint32_t first = 0; first < n_in; first += kSeedChunk) {
@@ -422,10 +424,10 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
             hipLaunchKernelGGL(walk, dim3(producers), dim3(kColBinThreads), 0, stream, in, out, n_out, seed, log_p, wa,
                                wb, first, count, static_cast<const uint32_t *>(nullptr),
                                static_cast<const uint32_t *>(nullptr), static_cast<const T1 *>(nullptr),
-                               static_cast<const uint32_t *>(states), count, n_win, cap, pairs, counts);
+                               static_cast<const uint32_t *>(states), count, n_win, shift, cap, pairs, counts);
           }
         }
-        if (add_uniform_bins<T1>("jitconn column walk", stream, out, n_out, producers, cap, pairs, counts, list_count))
+        if (add_uniform_bins<T1>("jitconn column walk", stream, out, n_out, shift, producers, cap, pairs, counts, list_count))
           return;
         // (the bins could not be added: nothing reached `out` yet except overflow pairs; start over)
         if (list_count != nullptr) fill_zero(stream, list_count, 1u);
