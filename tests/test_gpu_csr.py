@@ -378,3 +378,33 @@ def test_full_size_csr_matvec_both_orientations(cuda, oracle_mod):
   ones = torch.ones(n, dtype=torch.float32, device=dev)
   cnt = bpl.cusparse_csr_matvec(torch.ones(1, device=dev), indices, indptr, ones, shape=shape, transpose=True)
   assert np.array_equal(cnt.cpu().numpy(), np.bincount(c["indices"], minlength=n).astype(np.float32))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_scatter_path_boundaries(cuda, oracle_mod, dtype):
+  # shapes on both sides of every rule that picks a scatter kernel: 32,768 rows (active-row list),
+  # 16,384 / 65,536 / 131,072 columns (one float64 window, four windows), 2^20 nonzeros (sorted
+  # scatter), 64 nonzeros per row on average (device-side gate), event and dense input
+  rng = np.random.default_rng(51)
+  cases = [(32_768, 16_384, 40), (32_769, 16_385, 40), (20_000, 65_536, 60), (20_000, 65_537, 60),
+           (9_000, 131_072, 130), (9_000, 131_073, 130), (40_000, 140_000, 63), (40_000, 140_000, 66),
+           (3_000, 20_000, 349), (3_000, 20_000, 351), (70_000, 500, 20)]
+  for n_row, n_col, mean in cases:
+    counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_row + mean)
+    data = rng.random(indices.shape[0]).astype(dtype)
+    shape = (n_row, n_col)
+    print("shape", shape, "nnz", indices.shape[0], dtype.__name__, flush=True)
+    ev = rng.random(n_row) < 0.1
+    want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True)
+    got = bpl.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+    assert_close_reordered(got, want, want, dtype, what="event scatter %s" % (shape,))  # data >= 0: want is the bound
+    w = np.array([0.3], dtype=dtype)
+    want = oracle_mod.event_csr_matvec(w, indices, indptr, ev, shape=shape, transpose=True)
+    got = bpl.event_csr_matvec(w, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+    assert_close(got, want, what="homogeneous event scatter %s" % (shape,))
+    v = rng.standard_normal(n_row).astype(dtype)
+    want = oracle_mod.csr_matvec(data, indices, indptr, v, shape=shape, transpose=True)
+    mag = oracle_mod.csr_matvec(data, indices, indptr, np.abs(v), shape=shape, transpose=True)
+    got = bpl.cusparse_csr_matvec(data, indices, indptr, v, shape=shape, transpose=True).cpu().numpy()
+    assert_close_reordered(got, want, mag, dtype, what="dense scatter %s" % (shape,))
