@@ -28,13 +28,18 @@ struct WeightWords {
   static constexpr int value = sizeof(T1) == 4 ? 1 : 2;  // mt19937 words per uniform weight
 };
 
-// LDS words one wave needs: the generator state, plus (double-precision normal weights only) a
-// 128-word staging buffer for the batch and 64 (index, weight) slots for the serial parser.
+// LDS words one wave needs: the generator state.
 template <typename T1, int W>
 struct StreamLds {
-  static constexpr bool serial = (W == kNormal && sizeof(T1) == 8);
-  static constexpr int words = serial ? (kMtStateWords + 128 + 64 + 128) : kMtStateWords;
+  static constexpr int words = kMtStateWords;
 };
+
+__device__ __forceinline__ double read_lane_f64(double v, int l) {
+  const unsigned long long b = static_cast<unsigned long long>(__double_as_longlong(v));
+  const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(b), l));
+  const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(b >> 32), l));
+  return __longlong_as_double(static_cast<long long>((static_cast<unsigned long long>(hi) << 32) | lo));
+}
 
 // std::normal_distribution<float> (libstdc++, Marsaglia polar): candidate pair from two words
 struct PolarF32 {
@@ -166,69 +171,80 @@ __device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t str
       prev_y63 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, yw), 63));
     }
   } else {
-    // std::normal_distribution<double>: every draw is one canonical double (2 words).  The wave
-    // generates 64 doubles at a time; lane 0 replays the reference loop over them and leaves the
-    // synapses it finds in LDS slots, which the whole wave then consumes.
-    uint32_t *buf = st + kMtStateWords;                                   // 128 words
-    uint32_t *slot_idx = buf + 128;                                       // 64 indices
-    double *slot_w = reinterpret_cast<double *>(slot_idx + 64);           // 64 weights (8-byte aligned)
-    int state = 0;  // 0: first skip, 1: x expected, 2: y expected, 3: skip expected
-    uint32_t col = 0;
-    double x = 0.0, saved = 0.0;
-    bool has_saved = false;
+    // std::normal_distribution<double>: every draw is one canonical double, so the stream again
+    // consists of 2-word units:  K  (X Y .. X Y K) (K) (X Y .. X Y K) (K) ...   X, Y = the two
+    // coordinates of a polar attempt, the last pair of a group is the accepted one; the first K
+    // after it belongs to the synapse that receives y*mult, the second K to the synapse that
+    // receives the cached x*mult.  Every lane evaluates its unit as a coordinate (and, with its
+    // left neighbour's, as the end of an attempt) and as a skip; the roles are assigned on the
+    // scalar unit, one round per accepted attempt.
+    uint32_t w0[2] = {1u, 1u};
+    mt_generate<2>(st, pos, lane, 1, w0);
+    uint32_t carry = __builtin_amdgcn_readfirstlane(skip_from_words(w0[0], w0[1], log_p));
+    int state = 0;  // 0: X expected, 1: Y expected (X was the last unit of the previous batch), 2: first skip, 3: second skip
+    double prev_v63 = 0.0, prev_x62 = 0.0, prev_x63 = 0.0, prev_y63 = 0.0;
     for (uint32_t b = 0; b < max_batches; ++b) {
       uint32_t w[2] = {1u, 1u};
       mt_generate<2>(st, pos, lane, kWave, w);
-      buf[2 * lane] = w[0];
-      buf[2 * lane + 1] = w[1];
-      int count = 0, finished = 0;
-      if (lane == 0) {
-        for (int i = 0; i < kWave && !finished; ++i) {
-          const double u = canonical_f64(buf[2 * i], buf[2 * i + 1]);
-          bool emit = false;
-          double wdraw = 0.0;
-          if (state == 0 || state == 3) {
-            const uint32_t skip = f64_to_u32_x86(ceil(log(u) / log_p.log_p));
-            col = (state == 0) ? skip : col + skip;
-            if (col >= n) {
-              finished = 1;
-            } else if (has_saved) {  // the next weight costs no draw
-              has_saved = false;
-              wdraw = saved;
-              emit = true;
-              state = 3;
-            } else {
-              state = 1;
-            }
-          } else if (state == 1) {
-            x = __dsub_rn(__dmul_rn(2.0, u), 1.0);
-            state = 2;
-          } else {
-            const double y = __dsub_rn(__dmul_rn(2.0, u), 1.0);
-            const double r2 = __dadd_rn(__dmul_rn(x, x), __dmul_rn(y, y));
-            if (r2 > 1.0 || r2 == 0.0) {
-              state = 1;
-            } else {
-              const double mult = sqrt(-2 * log(r2) / r2);
-              saved = __dmul_rn(x, mult);
-              has_saved = true;
-              wdraw = __dmul_rn(y, mult);
-              emit = true;
-              state = 3;
-            }
-          }
-          if (emit) {
-            slot_idx[count] = col;
-            slot_w[count] = __dadd_rn(__dmul_rn(wdraw, static_cast<double>(wb)), static_cast<double>(wa));
-            ++count;
-          }
-        }
+      const double v = __dsub_rn(__dmul_rn(2.0, canonical_f64(w[0], w[1])), 1.0);
+      double v_m1 = __shfl_up(v, 1, kWave);
+      if (lane == 0) v_m1 = prev_v63;
+      const double r2 = __dadd_rn(__dmul_rn(v_m1, v_m1), __dmul_rn(v, v));
+      const bool ok = !(r2 > 1.0 || r2 == 0.0);  // an attempt (lane - 1, lane) would be accepted
+      const uint64_t okm = __ballot(ok);
+      uint64_t k1 = 0, k2 = 0;
+      int p = 0;
+      if (state == 1) {  // unit 0 completes the attempt begun by the previous batch's last unit
+        if (okm & 1ull) k1 = 2ull, k2 = 4ull, p = 3;
+        else p = 1;
+      } else if (state == 2) {
+        k1 = 1ull, k2 = 2ull, p = 2;
+      } else if (state == 3) {
+        k2 = 1ull, p = 1;
       }
-      count = __builtin_amdgcn_readfirstlane(count);
-      finished = __builtin_amdgcn_readfirstlane(finished);
-      const bool valid = lane < count;
-      f(valid ? slot_idx[lane] : 0u, valid ? static_cast<T1>(slot_w[lane]) : T1(0), valid);
-      if (finished) break;
+      state = 0;
+      while (p < kWave) {
+        // attempts from unit p end at p + 1, p + 3, ...: the first accepted one
+        const uint64_t ends = (p & 1) ? 0x5555555555555555ull : 0xaaaaaaaaaaaaaaaaull;
+        const uint64_t m = (okm & ends) >> p;
+        if (m == 0) {  // only rejected attempts remain; an odd number of units leaves an X waiting for its Y
+          state = ((kWave - p) & 1) ? 1 : 0;
+          break;
+        }
+        const int q = p + __ffsll(static_cast<unsigned long long>(m)) - 1;
+        k1 |= 2ull << q;  // shifts past bit 63 drop out: that role falls into the next batch
+        k2 |= 4ull << q;
+        state = (q == kWave - 1) ? 2 : (q == kWave - 2) ? 3 : 0;
+        p = q + 3;
+      }
+      const bool is_k1 = (k1 >> lane) & 1ull;
+      const bool is_k2 = (k2 >> lane) & 1ull;
+      const bool is_k = is_k1 || is_k2;
+      double xw = 0.0, yw = 0.0;
+      if (ok) {
+        const double mult = sqrt(-2 * log(r2) / r2);
+        xw = __dmul_rn(v_m1, mult);
+        yw = __dmul_rn(v, mult);
+      }
+      double y_m1 = __shfl_up(yw, 1, kWave);
+      double x_m2 = __shfl_up(xw, 2, kWave);
+      if (lane == 0) y_m1 = prev_y63, x_m2 = prev_x62;
+      if (lane == 1) x_m2 = prev_x63;
+      const double raw = is_k1 ? y_m1 : x_m2;
+      const T1 weight = static_cast<T1>(__dadd_rn(__dmul_rn(raw, static_cast<double>(wb)), static_cast<double>(wa)));
+      const uint32_t skip_any = skip_from_words(w[0], w[1], log_p);  // wave-converged call
+      const uint32_t skip = is_k ? skip_any : 0u;
+      const uint32_t incl = wave_inclusive_scan_u32(skip);
+      const uint32_t idx = carry + incl - skip;
+      const uint64_t done = __ballot(is_k && idx >= n);
+      const int first = done ? (__ffsll(static_cast<unsigned long long>(done)) - 1) : kWave;
+      f(idx, weight, is_k && lane < first);
+      if (done) break;
+      carry += __builtin_amdgcn_readlane(incl, kWave - 1);
+      prev_v63 = read_lane_f64(v, kWave - 1);
+      prev_x62 = read_lane_f64(xw, kWave - 2);
+      prev_x63 = read_lane_f64(xw, kWave - 1);
+      prev_y63 = read_lane_f64(yw, kWave - 1);
     }
   }
 }
