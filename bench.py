@@ -268,6 +268,15 @@ def main():
         oracle.event_csr_matvec(c["data"], c["indices"], c["indptr"], c["events"], shape=c["shape"], transpose=True)
       t_cpu = (time.perf_counter() - t1) / 20
       extra["scatter_1e8"]["cpu_port_1core_us"] = t_cpu * 1e6
+      # the reference's own compiled kernel for this orientation (lib/cpu_event_sum.cc), where it was built
+      from oracle import ref
+      if ref.available():
+        got_ref = ref.csr_event_sum(c["data"], c["indices"], c["indptr"], c["events"], shape=c["shape"])
+        check(got_ref, want_s, "reference cpu_csr_event_sum_heter vs oracle (scatter 1e8 nnz)")
+        t1 = time.perf_counter()
+        for _ in range(20):
+          ref.csr_event_sum(c["data"], c["indices"], c["indptr"], c["events"], shape=c["shape"])
+        extra["scatter_1e8"]["cpu_reference_1core_us"] = (time.perf_counter() - t1) / 20 * 1e6
     log("scatter 1e8: %s" % extra["scatter_1e8"])
 
     # homogeneous weight, gather: only the index stream is read
