@@ -33,3 +33,23 @@ def test_event_info_edges_and_batch(cuda, oracle_mod):
   for b in range(7):
     w_ids, w_num = oracle_mod.event_info(ev[b])
     assert np.array_equal(ids[b].cpu().numpy(), w_ids) and int(num[b]) == int(w_num[0])
+
+
+@pytest.mark.parametrize("dtype", [np.bool_, np.float32])
+def test_event_info_tiles_alignment_and_density(cuda, oracle_mod, dtype):
+  # several 4,096-element tiles per row, rows that start at every alignment (one-byte events take a
+  # 16-byte vector path only where the tile start is aligned), event densities from empty to full
+  rng = np.random.default_rng(3)
+  for size in (4095, 4096, 4097, 12_301, 65_536):
+    for rate in (0.0, 0.03, 0.5, 1.0):
+      ev = (rng.random((5, size)) < rate).astype(dtype)
+      ids, num = bpl.event_info(ev)
+      for b in range(5):
+        w_ids, w_num = oracle_mod.event_info(ev[b])
+        assert np.array_equal(ids[b].cpu().numpy(), w_ids), (size, rate, b)
+        assert int(num[b]) == int(w_num[0])
+  # a vector that starts 3 bytes into an allocation
+  base = torch.from_numpy(rng.random(20_003) < 0.2).cuda()
+  ids, num = bpl.event_info(base[3:])
+  w_ids, w_num = oracle_mod.event_info(base[3:].cpu().numpy())
+  assert np.array_equal(ids.cpu().numpy(), w_ids) and int(num[0]) == int(w_num[0])
