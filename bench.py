@@ -456,6 +456,25 @@ def main():
                                            cpu_sample="2 of 128 rows of X, %.2f s" % t_cpu)
     log("jitconn matmat: %s" % extra["jitconn_matmat_1e4x128"])
 
+    # ---------------------------------------------------------------------------------------------
+    # event_info: 1,000 event vectors of 100,000 bool events, density 0.1 (the shape of the
+    # reference's event_info_VS_jax_operators.py, whose docstring reports 2.78 ms per call on its GPU)
+    # ---------------------------------------------------------------------------------------------
+    ev_np = np.random.default_rng(11).random((1000, 100_000)) < 0.1
+    ev_t = torch.from_numpy(ev_np).to(dev)
+    ids, num = bpl.event_info(ev_t)
+    w_ids, w_num = oracle.event_info(ev_np[17])
+    ok = bool(np.array_equal(ids[17].cpu().numpy(), w_ids)) and int(num[17]) == int(w_num[0]) and \
+        bool(np.array_equal(num.cpu().numpy(), ev_np.sum(axis=1)))
+    log("parity event_info (1000, 100000)          row 17 and all counts exact: %s" % ok)
+    if not ok:
+      raise SystemExit("event_info parity failed")
+    d_ei, _ = time_calls(lambda: bpl.event_info(ev_t), max(10, args.steps // 10), 3)
+    extra["event_info_1000x100000"] = dict(stats(d_ei), gb_per_s=(ev_np.size * 5 + 4000) / (d_ei.mean() * 1e-3) / 1e9,
+                                           reference_docstring_ms=2.782)
+    log("event_info: %s" % extra["event_info_1000x100000"])
+    del ev_t, ids, num
+
   result = {
     "metric": "GSOP/s + % HBM roofline, event_csr_matvec 1e8 nnz; jitconn GSOP/s at p=0.001",
     "value": value,
