@@ -163,6 +163,56 @@ __device__ __forceinline__ uint32_t pack_events32<uint8_t>(const uint8_t *__rest
   return m;
 }
 
+// An event vector already packed to one bit per element (32 per word), by pack_event_bitmap().
+struct PackedBits {
+  uint32_t w;
+  // (never evaluated: only to let the dense-vector branches of the shared kernels compile)
+  __host__ __device__ explicit operator float() const { return 0.f; }
+  __host__ __device__ explicit operator double() const { return 0.0; }
+};
+template <>
+__device__ __forceinline__ bool is_event<PackedBits>(PackedBits v) {
+  return v.w != 0u;
+}
+template <>
+__device__ __forceinline__ uint32_t pack_events32<PackedBits>(const PackedBits *__restrict__ ev, uint32_t base,
+                                                               uint32_t n) {
+  return ev[base >> 5].w;  // base is a multiple of 32; bits beyond n are zero
+}
+
+// Is element i of the event vector set?
+template <typename VT>
+__device__ __forceinline__ bool probe_event(const VT *__restrict__ ev, uint32_t i) {
+  return is_event(ev[i]);
+}
+template <>
+__device__ __forceinline__ bool probe_event<PackedBits>(const PackedBits *__restrict__ ev, uint32_t i) {
+  return (ev[i >> 5].w >> (i & 31u)) & 1u;
+}
+
+// bits[w] bit b = ev[32 w + b] != 0 (zero beyond n): coalesced loads, one ballot per 64 elements.
+template <typename VT>
+__global__ __launch_bounds__(256) void pack_event_bitmap_kernel(const VT *__restrict__ ev, uint32_t n,
+                                                                uint32_t *__restrict__ bits) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t waves = gridDim.x * (256 / kWave);
+  const uint32_t groups = (n + kWave - 1) / kWave;
+  for (uint32_t g = blockIdx.x * (256 / kWave) + threadIdx.x / kWave; g < groups; g += waves) {
+    const uint32_t i = g * kWave + lane;
+    const unsigned long long m = __ballot(i < n && is_event(ev[i]));
+    if (lane == 0) bits[2 * g] = static_cast<uint32_t>(m);
+    if (lane == 32 && 2 * g + 1 < (n + 31) / 32) bits[2 * g + 1] = static_cast<uint32_t>(m >> 32);
+  }
+}
+
+template <typename VT>
+inline void pack_event_bitmap(hipStream_t stream, const VT *ev, uint32_t n, uint32_t *bits) {
+  if (n == 0) return;
+  const unsigned groups = div_up(n, kWave);
+  const unsigned grid = div_up(groups, 256 / kWave);
+  hipLaunchKernelGGL(pack_event_bitmap_kernel<VT>, dim3(grid < 2048 ? grid : 2048), dim3(256), 0, stream, ev, n, bits);
+}
+
 __device__ __forceinline__ void atomic_add(float *p, float v) { unsafeAtomicAdd(p, v); }
 __device__ __forceinline__ void atomic_add(double *p, double v) { unsafeAtomicAdd(p, v); }
 

@@ -465,7 +465,7 @@ __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const ui
       if (MODE == kEvent) {
         bool hit;
         if (LDS_BITS) hit = (s_bits[col[u] >> 5] >> (col[u] & 31u)) & 1u;
-        else hit = is_event(x[col[u]]);
+        else hit = probe_event(x, col[u]);
         hit = hit && ok;
         use[u] = hit;
         val[u] = F(0);
@@ -536,7 +536,7 @@ __device__ __forceinline__ void gather_rows_wave(const F *__restrict__ data, con
       if (MODE == kEvent) {
         bool hit;
         if (LDS_BITS) hit = (s_bits[col[u] >> 5] >> (col[u] & 31u)) & 1u;
-        else hit = ok[u] && is_event(x[col[u]]);
+        else hit = ok[u] && probe_event(x, col[u]);
         hit = hit && ok[u];
         if (HETER) {
           val[u] = F(0);
@@ -763,6 +763,19 @@ template <typename F, typename VT, bool HETER, int MODE>
 void launch_gather(const char *target, hipStream_t stream, const F *data, const uint32_t *indices,
                    const uint32_t *indptr, const VT *x, F *y, uint32_t n_row, uint32_t n_col) {
   if (n_row == 0) return;
+  if constexpr (MODE == kEvent && sizeof(VT) > 1 && !std::is_same<VT, PackedBits>::value) {
+    // Wide event types: every persistent workgroup would read the whole vector (4 or 8 bytes per
+    // element) to build its bitmap; pack it once instead and hand the words to the kernels.
+    const size_t words = (static_cast<size_t>(n_col) + 31) / 32;
+    uint32_t *bits = static_cast<uint32_t *>(stream_workspace(stream, (words + 1) * sizeof(uint32_t)));
+    if (bits != nullptr) {
+      pack_event_bitmap<VT>(stream, x, n_col, bits);
+      launch_gather<F, PackedBits, HETER, MODE>(target, stream, data, indices, indptr,
+                                                reinterpret_cast<const PackedBits *>(bits), y, n_row, n_col);
+      return;
+    }
+    bpl_clear_error();
+  }
   if (MODE == kEvent) {
     const size_t lds_bytes = (static_cast<size_t>(n_col) + 31) / 32 * 4;
     const size_t lds_cap = static_cast<size_t>(160) * 1024 - 1024;

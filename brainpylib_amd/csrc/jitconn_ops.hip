@@ -19,6 +19,8 @@
 // lib/gpu_jitconn_matvec_atomic.cu:53-77 (buffers = [input, out]; descriptors; target names).
 #include <cmath>
 
+#include <type_traits>
+
 #include "bins.h"
 #include "common.h"
 #include "jitconn_stream.h"
@@ -63,7 +65,7 @@ __global__ __launch_bounds__(1024) void jitconn_rowwalk_kernel(const VT *__restr
         bool hit = false;
         if (valid) {
           if (LDS_BITS) hit = (bits[idx >> 5] >> (idx & 31u)) & 1u;
-          else hit = is_event(in[idx]);
+          else hit = probe_event(in, idx);
         }
         if (W == kHomo) cnt += static_cast<uint32_t>(__popcll(__ballot(hit)));
         else if (hit) acc += static_cast<double>(w);
@@ -344,6 +346,21 @@ template <typename T1, typename VT, int IN, int W>
 void launch_rowwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, uint32_t n_in, uint32_t seed,
                     double log_p, T1 wa, T1 wb) {
   if (n_out == 0) return;
+  if constexpr (IN == kInEvent && sizeof(VT) > 1 && !std::is_same<VT, PackedBits>::value) {
+    // Wide event types: pack the vector to one bit per element once, instead of once per workgroup.
+    // (The seeded generator states of large walks share the scratch buffer: the bitmap lies behind them.)
+    const size_t state_ws = (n_out >= kSeedAheadMin) ? static_cast<size_t>(kSeedChunk) * kMtN * 4 : 0;
+    const size_t words = (static_cast<size_t>(n_in) + 31) / 32;
+    unsigned char *ws = static_cast<unsigned char *>(stream_workspace(stream, state_ws + (words + 1) * 4));
+    if (ws != nullptr) {
+      uint32_t *bits = reinterpret_cast<uint32_t *>(ws + state_ws);
+      pack_event_bitmap<VT>(stream, in, n_in, bits);
+      launch_rowwalk<T1, PackedBits, IN, W>(stream, reinterpret_cast<const PackedBits *>(bits), out, n_out, n_in, seed,
+                                            log_p, wa, wb);
+      return;
+    }
+    bpl_clear_error();
+  }
   const size_t state_bytes = StreamLds<T1, W>::words * 4;
   const size_t cap = static_cast<size_t>(160) * 1024 - 512;
   if (IN == kInEvent) {
