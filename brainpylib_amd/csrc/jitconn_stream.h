@@ -55,6 +55,70 @@ __device__ __forceinline__ PolarF32 polar_attempt(uint32_t w0, uint32_t w1) {
   return a;
 }
 
+// Roles of the 64 two-word units of one batch of a normal-weight stream.  Which units are polar
+// attempts and which are skips follows from a small automaton over the units' "this attempt
+// would be accepted" bits; it runs on the scalar unit eight units at a time through a table:
+// entry [byte of accept bits] holds, for every state the automaton can enter the eight units in
+// (one byte per state), the units at which an attempt is accepted and 8 x the state it leaves in.
+struct RoleEntry {
+  uint32_t accept, next;
+};
+struct RoleTable {
+  RoleEntry e[256];
+};
+// float: 0 attempt expected, 1 first skip after an accepted attempt, 2 second skip.
+// double (kStates == 4; a unit is one coordinate): 0 X expected, 1 Y expected, 2 first skip, 3 second skip.
+template <int kStates>
+constexpr RoleTable make_role_table() {
+  RoleTable t{};
+  for (uint32_t b = 0; b < 256; ++b) {
+    uint32_t acc = 0, nxt = 0;
+    for (int s0 = 0; s0 < kStates; ++s0) {
+      int s = s0;
+      uint32_t e = 0;
+      for (int i = 0; i < 8; ++i) {
+        const bool ok = (b >> i) & 1u;
+        if (kStates == 3) {
+          if (s == 0) {
+            if (ok) e |= 1u << i, s = 1;
+          } else {
+            s = (s == 1) ? 2 : 0;
+          }
+        } else {
+          if (s == 0) s = 1;
+          else if (s == 1) {
+            if (ok) e |= 1u << i, s = 2;
+            else s = 0;
+          } else {
+            s = (s == 2) ? 3 : 0;
+          }
+        }
+      }
+      acc |= e << (8 * s0);
+      nxt |= static_cast<uint32_t>(8 * s) << (8 * s0);
+    }
+    t.e[b].accept = acc;
+    t.e[b].next = nxt;
+  }
+  return t;
+}
+static __constant__ const RoleTable kRolesF32 = make_role_table<3>();
+static __constant__ const RoleTable kRolesF64 = make_role_table<4>();
+
+// accept mask of a batch; `state8` = 8 x automaton state, carried from batch to batch
+__device__ __forceinline__ uint64_t accepted_units(const RoleTable &tab, uint64_t okm, uint32_t &state8) {
+  uint64_t acc = 0;
+  uint32_t sh = state8;
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    const RoleEntry t = tab.e[static_cast<uint32_t>(okm >> (8 * c)) & 0xffu];
+    acc |= static_cast<uint64_t>((t.accept >> sh) & 0xffu) << (8 * c);
+    sh = (t.next >> sh) & 0xffu;
+  }
+  state8 = sh;
+  return acc;
+}
+
 // Walks stream std::mt19937{stream_seed} over [0, n): calls f(index, weight, valid) once per
 // batch with the whole wave converged; `valid` marks the lanes that hold a synapse of the row.
 //
@@ -112,36 +176,23 @@ __device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t str
     // stream in 2-word units: K  (A..A K) (K) (A..A K) (K) ...   A = polar attempt (x word, y word),
     // the last A of a group is the accepted one; the first K after it belongs to the synapse
     // that receives y*mult, the second K to the synapse that receives the cached x*mult.
-    // Every lane evaluates its unit both ways; a scalar automaton over the accept mask
-    // assigns the roles.
+    // Every lane evaluates its unit both ways; accepted_units() assigns the roles.
     uint32_t w0[2] = {1u, 1u};
     mt_generate<2>(st, pos, lane, 1, w0);
     uint32_t carry = __builtin_amdgcn_readfirstlane(skip_from_words(w0[0], w0[1], log_p));
-    int state = 0;  // 0: attempt expected, 1: first skip after an accept, 2: second skip
+    uint32_t state8 = 0;
     float prev_x62 = 0.f, prev_x63 = 0.f, prev_y63 = 0.f;
     for (uint32_t b = 0; b < max_batches; ++b) {
       uint32_t w[2] = {1u, 1u};
       mt_generate<2>(st, pos, lane, kWave, w);
       const PolarF32 a = polar_attempt(w[0], w[1]);
       const uint64_t okm = __ballot(a.ok);
-      // Roles of the batch's 64 units (scalar work: one round per accepted group, not per unit).
-      // An accepted attempt at unit q makes q + 1 the first and q + 2 the second skip; the
-      // search for the next accepted attempt resumes at q + 3.  Shifts past bit 63 drop out,
-      // which is exactly a role that falls into the next batch (remembered in `state`).
-      uint64_t k1 = 0, k2 = 0;
-      int p = 0;
-      if (state == 1) k1 = 1ull, k2 = 2ull, p = 2;
-      else if (state == 2) k2 = 1ull, p = 1;
-      state = 0;
-      while (p < kWave) {
-        const uint64_t m = okm >> p;
-        if (m == 0) break;  // only rejected attempts remain in this batch
-        const int q = p + __ffsll(static_cast<unsigned long long>(m)) - 1;
-        k1 |= 2ull << q;
-        k2 |= 4ull << q;
-        state = (q == kWave - 1) ? 1 : (q == kWave - 2) ? 2 : 0;
-        p = q + 3;
-      }
+      // An accepted attempt at unit q makes q + 1 the first and q + 2 the second skip; a role
+      // that falls past unit 63 belongs to the next batch and comes back through `state8`.
+      const uint32_t entered = state8;
+      const uint64_t acc = accepted_units(kRolesF32, okm, state8);
+      const uint64_t k1 = (acc << 1) | (entered == 8u ? 1ull : 0ull);
+      const uint64_t k2 = (acc << 2) | (entered == 8u ? 2ull : entered == 16u ? 1ull : 0ull);
       const bool is_k1 = (k1 >> lane) & 1ull;
       const bool is_k2 = (k2 >> lane) & 1ull;
       const bool is_k = is_k1 || is_k2;
@@ -176,12 +227,11 @@ __device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t str
     // coordinates of a polar attempt, the last pair of a group is the accepted one; the first K
     // after it belongs to the synapse that receives y*mult, the second K to the synapse that
     // receives the cached x*mult.  Every lane evaluates its unit as a coordinate (and, with its
-    // left neighbour's, as the end of an attempt) and as a skip; the roles are assigned on the
-    // scalar unit, one round per accepted attempt.
+    // left neighbour's, as the end of an attempt) and as a skip; accepted_units() assigns the roles.
     uint32_t w0[2] = {1u, 1u};
     mt_generate<2>(st, pos, lane, 1, w0);
     uint32_t carry = __builtin_amdgcn_readfirstlane(skip_from_words(w0[0], w0[1], log_p));
-    int state = 0;  // 0: X expected, 1: Y expected (X was the last unit of the previous batch), 2: first skip, 3: second skip
+    uint32_t state8 = 0;
     double prev_v63 = 0.0, prev_x62 = 0.0, prev_x63 = 0.0, prev_y63 = 0.0;
     for (uint32_t b = 0; b < max_batches; ++b) {
       uint32_t w[2] = {1u, 1u};
@@ -192,31 +242,11 @@ __device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t str
       const double r2 = __dadd_rn(__dmul_rn(v_m1, v_m1), __dmul_rn(v, v));
       const bool ok = !(r2 > 1.0 || r2 == 0.0);  // an attempt (lane - 1, lane) would be accepted
       const uint64_t okm = __ballot(ok);
-      uint64_t k1 = 0, k2 = 0;
-      int p = 0;
-      if (state == 1) {  // unit 0 completes the attempt begun by the previous batch's last unit
-        if (okm & 1ull) k1 = 2ull, k2 = 4ull, p = 3;
-        else p = 1;
-      } else if (state == 2) {
-        k1 = 1ull, k2 = 2ull, p = 2;
-      } else if (state == 3) {
-        k2 = 1ull, p = 1;
-      }
-      state = 0;
-      while (p < kWave) {
-        // attempts from unit p end at p + 1, p + 3, ...: the first accepted one
-        const uint64_t ends = (p & 1) ? 0x5555555555555555ull : 0xaaaaaaaaaaaaaaaaull;
-        const uint64_t m = (okm & ends) >> p;
-        if (m == 0) {  // only rejected attempts remain; an odd number of units leaves an X waiting for its Y
-          state = ((kWave - p) & 1) ? 1 : 0;
-          break;
-        }
-        const int q = p + __ffsll(static_cast<unsigned long long>(m)) - 1;
-        k1 |= 2ull << q;  // shifts past bit 63 drop out: that role falls into the next batch
-        k2 |= 4ull << q;
-        state = (q == kWave - 1) ? 2 : (q == kWave - 2) ? 3 : 0;
-        p = q + 3;
-      }
+      // unit 0 may complete the attempt begun by the previous batch's last unit (state 1)
+      const uint32_t entered = state8;
+      const uint64_t acc = accepted_units(kRolesF64, okm, state8);
+      const uint64_t k1 = (acc << 1) | (entered == 16u ? 1ull : 0ull);
+      const uint64_t k2 = (acc << 2) | (entered == 16u ? 2ull : entered == 24u ? 1ull : 0ull);
       const bool is_k1 = (k1 >> lane) & 1ull;
       const bool is_k2 = (k2 >> lane) & 1ull;
       const bool is_k = is_k1 || is_k2;
