@@ -152,7 +152,7 @@ __device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t str
     // stream: K  (w K) (w K) ...   synapse s sits at K_0 + ... + K_s, its weight precedes K_{s+1}
     constexpr int WW = WeightWords<T1>::value;
     constexpr int K = WW + 2;
-    constexpr int NL = (K == 3) ? 64 : 32;  // K * NL <= 227
+    constexpr int NL = (K == 3) ? 64 : 56;  // K * NL <= 227
     uint32_t w0[2] = {1u, 1u};
     mt_generate<2>(st, pos, lane, 1, w0);
     uint32_t carry = __builtin_amdgcn_readfirstlane(skip_from_words(w0[0], w0[1], log_p));
