@@ -35,8 +35,22 @@ def device_of(*args):
   return torch.device("cuda", torch.cuda.current_device())
 
 
+_HOST_SCALARS = {}
+
+
 def to_device(t, device):
   if t.device != device:
+    if t.numel() == 1 and t.device.type == 'cpu' and not t.requires_grad:
+      # A one-element host operand (a homogeneous weight given as a Python number): its device copy
+      # is made once per value.  A pageable host-to-device copy per call would cost more than the
+      # kernels of a small network.  The operators only read their operands.
+      key = (t.item(), t.dtype, tuple(t.shape), device)
+      hit = _HOST_SCALARS.get(key)
+      if hit is None:
+        if len(_HOST_SCALARS) >= 256:
+          _HOST_SCALARS.clear()
+        hit = _HOST_SCALARS[key] = t.to(device).contiguous()
+      return hit
     t = t.to(device)
   return t.contiguous()
 

@@ -148,6 +148,19 @@ def test_edge_cases(cuda, oracle_mod):
   del t
 
 
+def test_python_number_weights_keep_their_values(cuda, oracle_mod):
+  # a homogeneous weight given as a Python number is copied to the device once per value:
+  # alternating values must not alias each other
+  shape = (50, 70)
+  _, indices, indptr = random_csr(shape, 0.3, seed=11, dtype=np.float32)
+  events = np.random.default_rng(3).random(shape[0]) < 0.5
+  ix, ip, ev = (torch.from_numpy(a).cuda() for a in (indices, indptr, events))
+  for w in (0.6, -1.25, 0.6, 3, -1.25, float("nan"), 0.6):
+    want = oracle_mod.event_csr_matvec(np.float32(w), indices, indptr, events, shape=shape, transpose=True)
+    got = bpl.event_csr_matvec(w, ix, ip, ev, shape=shape, transpose=True).cpu().numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6, equal_nan=True)
+
+
 def test_ragged_rows_and_all_row_length_modes(cuda, oracle_mod):
   # mean row lengths that select each lanes-per-row mode (8 / 16 / 32 / 64), with ragged rows,
   # empty rows and one very long row
