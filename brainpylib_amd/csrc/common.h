@@ -46,8 +46,9 @@ const DeviceInfo &device_info();
 // time a size is requested (hipMalloc is not capturable).
 void *stream_workspace(hipStream_t stream, size_t bytes);
 
-// A few zero-initialised 32-bit counters per (device, stream) (the scatter's active-row count).
-// Every user leaves them at zero again.  nullptr if the allocation fails.
+// A few zero-initialised 32-bit counters per (device, stream).  The first one (the scatter's
+// active-row count) is left at zero again by every user; the others carry nothing from call to
+// call.  nullptr if the allocation fails.
 uint32_t *stream_counters(hipStream_t stream);
 
 // Transposed CSR times dense vector through coarse sorting of the products (csr_bin_scatter.hip),
@@ -58,6 +59,21 @@ bool bin_scatter_usable(uint32_t n_col, uint32_t nnz);
 template <typename F>
 bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool heter, const uint32_t *indices,
                  const uint32_t *indptr, const F *vec, F *y, uint32_t n_row, uint32_t n_col, uint32_t nnz);
+
+// The same for event input (event_csr_matvec, transposed, wide outputs): the caller lists the
+// active rows on the device, (first nonzero, length) each in `active_list`, their number in
+// active_count[0]; `scratch` is device memory of bin_event_scatter_bytes() bytes whose first
+// kBinEventFillBytes are zero; y is zeroed.  Enqueues the two kernels; the second one sets
+// active_count[0] back to zero.  false (nothing enqueued) if it cannot run.
+constexpr size_t kBinEventFillBytes = 16384;
+template <typename F>
+bool bin_event_scatter_usable(uint32_t n_col);
+template <typename F>
+size_t bin_event_scatter_bytes(uint32_t n_row, uint32_t n_col);
+template <typename F>
+bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint32_t *indices, const uint32_t *indptr,
+                       F *y, uint32_t n_row, uint32_t n_col, uint32_t *active_count, const uint2 *active_list,
+                       void *scratch);
 
 // Second half of the coarse-sorted scatter for producers other than the CSR one: adds bins laid
 // out uniformly, bin (p, b) = pairs + (p * n_win + b) * cap with counts[b * producers + p]

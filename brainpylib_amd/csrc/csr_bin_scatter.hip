@@ -258,7 +258,262 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
   }
 }
 
+// ---- event input -------------------------------------------------------------------------------
+// Only the active rows contribute, how many is known on the device alone (a list made by the
+// caller: (first nonzero, length) per active row, their number in active_count[0]), and the
+// descriptor of the event operators does not carry the nonzero count.  So the bins are not private
+// to a producer here: window b owns ONE run of `cap` pairs, and a producer reserves room for the
+// pairs a round holds for a window with one global atomic on fill[b] (at most one per window and
+// round of 4,096 nonzeros; the event operators move far fewer pairs than the dense product, for
+// which that many same-address atomics would cost more than private regions).  Whatever the
+// distribution of the activity over rows and of the columns over windows, a run only overflows
+// (into direct atomics on y) when its window receives more than `cap` pairs.
+constexpr uint32_t kPairsPerProducer = 4096;  // a producer takes part per that many active nonzeros (estimated): one round
+constexpr uint32_t kFillStride = 32;          // words between the windows' fill counters: one 128-byte line each
+static_assert(kBinEventFillBytes == kMaxWindows * kFillStride * sizeof(uint32_t), "one fill counter per window");
+constexpr uint32_t kPairsPerPart = 8192;      // a consumer workgroup takes part per that many pairs of its window
+
+template <typename F, bool HETER>
+__global__ __launch_bounds__(kBinThreads) void bin_active_rows_kernel(
+    const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
+    uint32_t n_row, const uint32_t *__restrict__ active_count, const uint2 *__restrict__ active_list,
+    F *__restrict__ y, uint32_t shift, uint32_t cap, BinPair<F> *__restrict__ pairs, uint32_t *__restrict__ fill) {
+  __shared__ uint32_t s_ptr[kTileRows + 1];     // nonzeros of the tile's rows before row k
+  __shared__ uint32_t s_start[kTileRows];       // first nonzero of row k in the matrix
+  __shared__ uint32_t s_hint[kBinThreads + 1];
+  __shared__ uint32_t s_cnt[kMaxWindows];
+  __shared__ uint32_t s_off[kMaxWindows + 1];
+  __shared__ uint32_t s_base[kMaxWindows];      // where the round's pairs of a window go in its run
+  __shared__ uint32_t s_wave[kBinThreads / kWave];
+  constexpr int U = (sizeof(F) == 4) ? 4 : 2;
+  constexpr uint32_t kRound = U * kBinThreads;
+  __shared__ BinPair<F> s_sorted[kRound];
+  __shared__ uint8_t s_window[kRound];
+  const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const uint32_t total = active_count[0];
+  const uint32_t nnz = indptr[n_row];
+  // with little activity a few producers finish sooner than a chip full of them
+  const uint64_t want = (static_cast<uint64_t>(total) * (nnz / n_row + 1u) + kPairsPerProducer - 1u) / kPairsPerProducer;
+  const uint32_t producers = want < 1u ? 1u : want > gridDim.x ? gridDim.x : static_cast<uint32_t>(want);
+  const uint32_t p = blockIdx.x;
+  if (p >= producers) return;
+  const uint32_t lo = static_cast<uint32_t>(static_cast<uint64_t>(p) * total / producers);
+  const uint32_t hi = static_cast<uint32_t>(static_cast<uint64_t>(p + 1) * total / producers);
+  if (tid < kMaxWindows) s_cnt[tid] = 0;
+  const F w_homo = HETER ? F(0) : data[0];
+
+  auto row_of = [&](uint32_t j, uint32_t a, uint32_t b) {  // largest k in [a, b] with s_ptr[k] <= j
+    while (a < b) {
+      const uint32_t mid = (a + b + 1u) >> 1;
+      if (s_ptr[mid] <= j) a = mid;
+      else b = mid - 1u;
+    }
+    return a;
+  };
+
+  for (uint32_t t0 = lo; t0 < hi; t0 += kTileRows) {
+    const uint32_t rows = (hi - t0 < kTileRows) ? hi - t0 : kTileRows;
+    __syncthreads();  // the previous tile is done with s_ptr / s_start (and s_cnt is cleared)
+    uint2 e = make_uint2(0u, 0u);
+    if (tid < rows) e = active_list[t0 + tid];
+    const uint32_t incl = wave_inclusive_scan_u32(e.y);
+    if (lane == kWave - 1) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t before = 0;
+    for (uint32_t w = 0; w < wave; ++w) before += s_wave[w];
+    if (tid < rows) s_ptr[tid] = before + incl - e.y, s_start[tid] = e.x;
+    if (tid == rows - 1u) s_ptr[rows] = before + incl;
+    __syncthreads();
+    const uint32_t j1 = s_ptr[rows];  // the tile's nonzeros, numbered from 0 (listed rows are never empty)
+    for (uint32_t seg = 0; seg < j1; seg += kSegment) {
+      const uint32_t seg_end = (j1 - seg < kSegment) ? j1 : seg + kSegment;
+      __syncthreads();  // the previous segment is done with s_hint
+      {
+        const uint32_t j = seg + (tid << kHintShift);
+        s_hint[tid] = (j < seg_end) ? row_of(j, 0u, rows - 1u) : rows - 1u;
+        if (tid == 0) s_hint[kBinThreads] = rows - 1u;
+      }
+      __syncthreads();
+      for (uint32_t jb = seg + tid; jb - tid < seg_end; jb += kRound) {
+        uint32_t rank[U], win[U], rel[U];
+        F val[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t j = jb + u * kBinThreads;
+          win[u] = 0xffffffffu;  // no pair
+          rel[u] = 0;
+          val[u] = F(0);
+          rank[u] = 0;
+          if (j < seg_end) {
+            const uint32_t q = (j - seg) >> kHintShift;
+            const uint32_t k = row_of(j, s_hint[q], s_hint[q + 1]);
+            const uint32_t at = s_start[k] + (j - s_ptr[k]);
+            const uint32_t col = indices[at];
+            val[u] = HETER ? data[at] : w_homo;
+            win[u] = col >> shift;
+            rel[u] = col & ((1u << shift) - 1u);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (win[u] != 0xffffffffu) rank[u] = atomicAdd(&s_cnt[win[u]], 1u);
+        __syncthreads();
+        if (tid < kWave) {  // two windows per lane: offsets within the round, room in the windows' runs
+          const uint32_t c0 = s_cnt[2 * tid], c1 = s_cnt[2 * tid + 1];
+          const uint32_t sum = wave_inclusive_scan_u32(c0 + c1);
+          s_off[2 * tid] = sum - (c0 + c1);
+          s_off[2 * tid + 1] = sum - c1;
+          if (tid == kWave - 1) s_off[kMaxWindows] = sum;
+          s_base[2 * tid] = c0 ? atomicAdd(&fill[2 * tid * kFillStride], c0) : 0u;
+          s_base[2 * tid + 1] = c1 ? atomicAdd(&fill[(2 * tid + 1) * kFillStride], c1) : 0u;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (win[u] != 0xffffffffu) {
+            const uint32_t pos = s_off[win[u]] + rank[u];
+            BinPair<F> o;
+            o.rel = rel[u];
+            o.val = val[u];
+            s_sorted[pos] = o;
+            s_window[pos] = static_cast<uint8_t>(win[u]);
+          }
+        }
+        __syncthreads();
+        const uint32_t round_total = s_off[kMaxWindows];
+        for (uint32_t i = tid; i < round_total; i += kBinThreads) {
+          const uint32_t w = s_window[i];
+          const BinPair<F> o = s_sorted[i];
+          const uint32_t slot = s_base[w] + (i - s_off[w]);
+          if (slot < cap) pairs[static_cast<uint64_t>(w) * cap + slot] = o;
+          else atomic_add(y + ((w << shift) | o.rel), o.val);
+        }
+        __syncthreads();
+        if (tid < kMaxWindows) s_cnt[tid] = 0;
+        __syncthreads();
+      }
+    }
+  }
+}
+
+// grid = n_win * parts; workgroup (b, s) adds share s of window b's run to the zeroed y.
+template <typename F>
+__global__ __launch_bounds__(kBinThreads) void add_window_runs_kernel(F *__restrict__ y, uint32_t n_col, uint32_t shift,
+                                                                      uint32_t parts, uint32_t cap,
+                                                                      const BinPair<F> *__restrict__ pairs,
+                                                                      const uint32_t *__restrict__ fill,
+                                                                      uint32_t *__restrict__ reset) {
+  extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
+  // (the caller's active-row counter, left at zero for the next call)
+  if (reset != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *reset = 0u;
+  double *window = reinterpret_cast<double *>(smem_raw);
+  const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  constexpr uint32_t kWaves = kBinThreads / kWave;
+  const uint32_t b = blockIdx.x / parts, s = blockIdx.x % parts;
+  uint32_t n = fill[b * kFillStride];
+  if (n > cap) n = cap;  // the producers count what they could not store too
+  // every workgroup that takes part adds a whole window to y: few pairs, few workgroups
+  const uint32_t want = (n + kPairsPerPart - 1u) / kPairsPerPart;
+  if (want < parts) parts = want;
+  if (s >= parts) return;
+  const uint32_t lo = static_cast<uint32_t>(static_cast<uint64_t>(s) * n / parts);
+  const uint32_t hi = static_cast<uint32_t>(static_cast<uint64_t>(s + 1) * n / parts);
+  const uint32_t c0 = b << shift;
+  const uint32_t width = (n_col - c0 < (1u << shift)) ? n_col - c0 : (1u << shift);
+  for (uint32_t i = tid; i < width; i += kBinThreads) window[i] = 0.0;
+  __syncthreads();
+  const BinPair<F> *run = pairs + static_cast<uint64_t>(b) * cap;
+  constexpr int U = 8;
+  for (uint32_t i0 = lo + wave * (U * kWave); i0 < hi; i0 += kWaves * U * kWave) {
+    BinPair<F> e[U];
+    if (i0 + U * kWave <= hi) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) e[u] = run[i0 + u * kWave + lane];
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t i = i0 + u * kWave + lane;
+        e[u].rel = 0xffffffffu;
+        e[u].val = F(0);
+        if (i < hi) e[u] = run[i];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (e[u].rel < width) atomicAdd(&window[e[u].rel], static_cast<double>(e[u].val));
+  }
+  __syncthreads();
+  for (uint32_t i = tid; i < width; i += kBinThreads) {
+    const F v = static_cast<F>(window[i]);
+    if (v != F(0)) atomic_add(y + c0 + i, v);
+  }
+}
+
+// pairs all windows' runs hold together: 32 per row or column, between 2^22 and 2^26
+// log2 of the output window with event input: as many windows as the 7-bit ids allow (every
+// consumer workgroup adds a whole window to y, so small windows and few workgroups per window)
+inline uint32_t event_window_shift(uint32_t n_out) {
+  uint32_t shift = 8;
+  while (shift < kBinMaxShift && (n_out >> shift) >= kMaxWindows) ++shift;
+  return shift;
+}
+
+inline uint64_t event_run_pairs(uint32_t n_row, uint32_t n_col) {
+  uint64_t t = 32ull * (n_row > n_col ? n_row : n_col);
+  if (t < (1ull << 22)) t = 1ull << 22;
+  if (t > (1ull << 26)) t = 1ull << 26;
+  return t;
+}
+
 }  // namespace
+
+template <typename F>
+bool bin_event_scatter_usable(uint32_t n_col) {
+  const uint32_t n_win = div_up(n_col, 1u << event_window_shift(n_col));
+  return n_win >= 2 && n_win <= kMaxWindows;
+}
+
+template <typename F>
+size_t bin_event_scatter_bytes(uint32_t n_row, uint32_t n_col) {
+  const uint32_t n_win = div_up(n_col, 1u << event_window_shift(n_col));
+  const uint64_t cap = event_run_pairs(n_row, n_col) / n_win;
+  return kBinEventFillBytes + static_cast<size_t>(cap) * n_win * sizeof(BinPair<F>);
+}
+
+template <typename F>
+bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint32_t *indices, const uint32_t *indptr,
+                       F *y, uint32_t n_row, uint32_t n_col, uint32_t *active_count, const uint2 *active_list,
+                       void *scratch) {
+  const uint32_t shift = event_window_shift(n_col);
+  const uint32_t n_win = div_up(n_col, 1u << shift);
+  const uint32_t cap = static_cast<uint32_t>(event_run_pairs(n_row, n_col) / n_win);
+  uint32_t *fill = static_cast<uint32_t *>(scratch);
+  BinPair<F> *pairs = reinterpret_cast<BinPair<F> *>(static_cast<unsigned char *>(scratch) + kBinEventFillBytes);
+  const unsigned num_cu = static_cast<unsigned>(device_info().num_cu);
+  uint32_t parts = num_cu / n_win;
+  if (parts == 0) parts = 1;
+  auto add_kernel = add_window_runs_kernel<F>;
+  const size_t lds = sizeof(double) << shift;
+  static thread_local bool attr_set = false;
+  if (!attr_set && lds > 64 * 1024) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(add_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(lds)) != hipSuccess) {
+      (void)hipGetLastError();
+      return false;
+    }
+    attr_set = true;
+  }
+  const uint32_t producers = 2u * num_cu;
+  if (heter)
+    hipLaunchKernelGGL((bin_active_rows_kernel<F, true>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
+                       indptr, n_row, active_count, active_list, y, shift, cap, pairs, fill);
+  else
+    hipLaunchKernelGGL((bin_active_rows_kernel<F, false>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
+                       indptr, n_row, active_count, active_list, y, shift, cap, pairs, fill);
+  hipLaunchKernelGGL(add_kernel, dim3(n_win * parts), dim3(kBinThreads), lds, stream, y, n_col, shift, parts, cap, pairs,
+                     fill, active_count);
+  return true;
+}
 
 template <typename F>
 bool bin_scatter_usable(uint32_t n_col, uint32_t nnz) {
@@ -349,6 +604,14 @@ template bool add_uniform_bins<float>(const char *, hipStream_t, float *, uint32
 template bool add_uniform_bins<double>(const char *, hipStream_t, double *, uint32_t, uint32_t, uint32_t, uint32_t,
                                        const void *,
                                        const uint32_t *, uint32_t *);
+template bool bin_event_scatter_usable<float>(uint32_t);
+template bool bin_event_scatter_usable<double>(uint32_t);
+template size_t bin_event_scatter_bytes<float>(uint32_t, uint32_t);
+template size_t bin_event_scatter_bytes<double>(uint32_t, uint32_t);
+template bool bin_event_scatter<float>(hipStream_t, const float *, bool, const uint32_t *, const uint32_t *, float *, uint32_t,
+                                       uint32_t, uint32_t *, const uint2 *, void *);
+template bool bin_event_scatter<double>(hipStream_t, const double *, bool, const uint32_t *, const uint32_t *, double *,
+                                        uint32_t, uint32_t, uint32_t *, const uint2 *, void *);
 template bool bin_scatter_usable<float>(uint32_t, uint32_t);
 template bool bin_scatter_usable<double>(uint32_t, uint32_t);
 template bool bin_scatter<float>(const char *, hipStream_t, const float *, bool, const uint32_t *, const uint32_t *,

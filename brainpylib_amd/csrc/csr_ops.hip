@@ -151,53 +151,98 @@ constexpr int kWinMaxRows = 2048;  // rows per workgroup = capacity of the activ
 
 // Active rows of the whole matrix, gathered once into a list in device memory (any order):
 // (first nonzero, length) per row whose input is nonzero and that has nonzeros, plus the input
-// value in dense mode.  The window kernel's row groups then take equal shares of the LIST, so
-// their work does not depend on where in the matrix the activity is.  One atomic per workgroup
-// reserves the list positions.
-template <typename F, typename VT, int MODE>
+// value in dense mode.  The kernels that follow take equal shares of the LIST, so their work does
+// not depend on where in the matrix the activity is.  A workgroup tests 1,024 rows per unit of
+// kCollectPerThread and reserves its list positions with one atomic (atomics on one address
+// retire at about 15 ns each, whoever issues them: one per 1,024 rows cost 14 us for a million rows).
+// Optional chores for the kernels that follow: `clear[0 .. n_clear)` and `zero[0 .. n_zero)` are set to zero.
+template <typename F, typename VT, int MODE, int kCollectPerThread>
 __global__ __launch_bounds__(kWinThreads) void collect_active_rows_kernel(
     const uint32_t *__restrict__ indptr, const VT *__restrict__ x, uint32_t n_row, uint32_t *__restrict__ counter,
-    uint2 *__restrict__ list, F *__restrict__ scales, NnzGate gate) {
+    uint2 *__restrict__ list, F *__restrict__ scales, NnzGate gate, uint32_t *__restrict__ clear, uint32_t n_clear,
+    F *__restrict__ zero, uint32_t n_zero) {
   if (!gate.open(indptr, n_row)) return;
-  constexpr uint32_t kWaves = kWinThreads / kWave;
-  __shared__ uint32_t s_off[kWaves];
-  __shared__ uint32_t s_base;
-  const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  const uint32_t r = blockIdx.x * kWinThreads + tid;
-  bool on = false;
-  uint32_t start = 0, len = 0;
-  F scale = F(1);
-  if (r < n_row) {
-    if (MODE == kEvent) {
-      on = is_event(x[r]);
-    } else {
-      scale = static_cast<F>(x[r]);
-      on = scale != F(0);  // a zero input adds nothing
-    }
-    if (on) {
-      start = indptr[r];
-      len = indptr[r + 1] - start;
-      on = len != 0;
-    }
-  }
-  const uint64_t mask = __ballot(on);
-  if (lane == 0) s_off[wave] = static_cast<uint32_t>(__popcll(mask));
+  __shared__ uint32_t s_count, s_base;
+  const uint32_t tid = threadIdx.x, lane = tid % kWave;
+  if (tid == 0) s_count = 0;
+  if (blockIdx.x == 0)
+    for (uint32_t i = tid; i < n_clear; i += kWinThreads) clear[i] = 0u;
+  for (uint32_t i = blockIdx.x * kWinThreads + tid; i < n_zero; i += gridDim.x * kWinThreads) zero[i] = F(0);
   __syncthreads();
-  if (tid == 0) {
-    uint32_t total = 0;
-    for (uint32_t w = 0; w < kWaves; ++w) {
-      const uint32_t c = s_off[w];
-      s_off[w] = total;
-      total += c;
+  const uint32_t r0 = blockIdx.x * (kWinThreads * kCollectPerThread) + tid;
+  bool on[kCollectPerThread];
+  uint32_t start[kCollectPerThread], len[kCollectPerThread], at[kCollectPerThread];
+  F scale[kCollectPerThread];
+#pragma unroll
+  for (int e = 0; e < kCollectPerThread; ++e) {
+    const uint32_t r = r0 + e * kWinThreads;
+    on[e] = false;
+    scale[e] = F(1);
+    if (r < n_row) {
+      if (MODE == kEvent) {
+        on[e] = is_event(x[r]);
+      } else {
+        scale[e] = static_cast<F>(x[r]);
+        on[e] = scale[e] != F(0);  // a zero input adds nothing
+      }
     }
-    s_base = total ? atomicAdd(counter, total) : 0u;
+  }
+#pragma unroll
+  for (int e = 0; e < kCollectPerThread; ++e) {
+    start[e] = len[e] = at[e] = 0;
+    if (on[e]) {
+      const uint32_t r = r0 + e * kWinThreads;
+      start[e] = indptr[r];
+      len[e] = indptr[r + 1] - start[e];
+      on[e] = len[e] != 0;
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < kCollectPerThread; ++e) {
+    const uint64_t mask = __ballot(on[e]);
+    uint32_t base = 0;
+    if (lane == 0 && mask) base = atomicAdd(&s_count, static_cast<uint32_t>(__popcll(mask)));
+    base = __builtin_amdgcn_readfirstlane(base);
+    at[e] = base + static_cast<uint32_t>(__popcll(mask & ((1ull << lane) - 1ull)));
   }
   __syncthreads();
-  if (on) {
-    const uint32_t k = s_base + s_off[wave] + static_cast<uint32_t>(__popcll(mask & ((1ull << lane) - 1ull)));
-    list[k] = make_uint2(start, len);
-    if (MODE == kDense) scales[k] = scale;
+  if (tid == 0) s_base = s_count ? atomicAdd(counter, s_count) : 0u;
+  __syncthreads();
+  const uint32_t base = s_base;
+#pragma unroll
+  for (int e = 0; e < kCollectPerThread; ++e) {
+    if (on[e]) {
+      list[base + at[e]] = make_uint2(start[e], len[e]);
+      if (MODE == kDense) scales[base + at[e]] = scale[e];
+    }
   }
+}
+
+template <typename F, typename VT, int MODE>
+unsigned collect_workgroups(uint32_t n_row) {
+  return n_row > 262144u ? div_up(n_row, 4 * kWinThreads) : div_up(n_row, kWinThreads);
+}
+template <typename F, typename VT, int MODE>
+void launch_collect(hipStream_t stream, const uint32_t *indptr, const VT *x, uint32_t n_row, uint32_t *counter,
+                    uint2 *list, F *scales, NnzGate gate, uint32_t *clear, uint32_t n_clear, F *zero, uint32_t n_zero) {
+  const unsigned wgs = collect_workgroups<F, VT, MODE>(n_row);
+  if (n_row > 262144u)
+    hipLaunchKernelGGL((collect_active_rows_kernel<F, VT, MODE, 4>), dim3(wgs), dim3(kWinThreads), 0, stream, indptr, x,
+                       n_row, counter, list, scales, gate, clear, n_clear, zero, n_zero);
+  else
+    hipLaunchKernelGGL((collect_active_rows_kernel<F, VT, MODE, 1>), dim3(wgs), dim3(kWinThreads), 0, stream, indptr, x,
+                       n_row, counter, list, scales, gate, clear, n_clear, zero, n_zero);
+}
+
+// Row groups that take part in a launch whose active rows are listed in device memory: one per
+// 32,768 active nonzeros (estimated from the mean row length), at least one, at most the launched
+// number.  Every group writes a slice of partial outputs that the summing kernel reads again, so
+// with little activity a few groups finish sooner than a chip full of them.
+__device__ __forceinline__ uint32_t groups_in_use(uint32_t active_rows, uint32_t nnz, uint32_t n_row,
+                                                 uint32_t launched) {
+  const uint64_t work = static_cast<uint64_t>(active_rows) * (nnz / n_row + 1u);
+  const uint64_t want = (work + 32767u) / 32768u;
+  return want < 1u ? 1u : want > launched ? launched : static_cast<uint32_t>(want);
 }
 
 // A = type of the window's accumulators: F, or double where every lane adds (dense input):
@@ -207,7 +252,7 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
     const VT *__restrict__ x, F *__restrict__ y, uint32_t n_row, uint32_t n_col, uint32_t rows_per_wg,
     uint32_t win, uint32_t n_win, F *__restrict__ partial, NnzGate gate,
-    const uint32_t *__restrict__ active_count, const uint2 *__restrict__ active_list,
+    uint32_t *__restrict__ active_count, const uint2 *__restrict__ active_list,
     const F *__restrict__ active_scales) {
   if (!gate.open(indptr, n_row)) return;
   extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
@@ -237,7 +282,19 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
     const uint32_t per_xcd = gridDim.x / kXcds;
     if (id < per_xcd * kXcds) id = (id % kXcds) * per_xcd + id / kXcds;
   }
-  const uint32_t b = id % n_win, g = id / n_win;
+  const uint32_t b = id % n_win;
+  uint32_t g = id / n_win;
+  // With a device list only the first groups_in_use() groups work, in an order that deals
+  // consecutive groups to different XCDs; the choice goes to the summing kernel through the
+  // stream's second counter.
+  uint32_t groups = gridDim.x / n_win;
+  if (active_list != nullptr) {
+    const uint32_t launched = groups;
+    if (launched % 8u == 0) g = (g % (launched / 8u)) * 8u + g / (launched / 8u);
+    groups = groups_in_use(active_count[0], indptr[n_row], n_row, launched);
+    if (g == 0 && b == 0 && threadIdx.x == 0) active_count[1] = groups;
+    if (g >= groups) return;
+  }
   const uint32_t c0 = b * win;
   const uint32_t width = (c0 + win <= n_col) ? win : n_col - c0;
 
@@ -256,8 +313,7 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
   // taken kWinMaxRows at a time, the capacity of the list in LDS.
   uint32_t span_lo = 0, span_hi = rows_per_wg;
   if (active_list != nullptr) {
-    const uint32_t total = *active_count;
-    const uint32_t groups = gridDim.x / n_win;
+    const uint32_t total = active_count[0];
     span_lo = static_cast<uint32_t>(static_cast<uint64_t>(g) * total / groups);
     span_hi = static_cast<uint32_t>(static_cast<uint64_t>(g + 1) * total / groups);
   }
@@ -393,8 +449,12 @@ __global__ __launch_bounds__(256) void sum_partials_kernel(const F *__restrict__
                                                            const uint32_t *__restrict__ indptr, uint32_t n_row,
                                                            NnzGate gate, uint32_t *__restrict__ reset) {
   if (!gate.open(indptr, n_row)) return;
-  // the active-row counter of this call is left at zero for the next one
-  if (reset != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *reset = 0u;
+  // with a device list of active rows: the groups that took part, as the window kernel left them
+  // in the second counter; the active-row counter itself goes back to zero for the next call
+  if (reset != nullptr) {
+    groups = reset[1];
+    if (blockIdx.x == 0 && threadIdx.x == 0) reset[0] = 0u;
+  }
   const uint32_t c = blockIdx.x * 256u + threadIdx.x;
   if (c >= n_col) return;
   F acc = F(0);
@@ -631,6 +691,33 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
   const uint32_t win_cap = static_cast<uint32_t>((static_cast<size_t>(128) * 1024) / sizeof(A));
   const uint32_t n_win = div_up(n_col, win_cap);
   NnzGate direct_gate = kAlways;
+  // Event input and an output wider than a few windows: the active rows' nonzeros are sorted
+  // coarsely by output window instead (csr_bin_scatter.hip), at a cost that does not grow with
+  // the number of windows.
+  if (MODE == kEvent && n_win > 4 && bin_event_scatter_usable<F>(n_col)) {
+    const size_t list_sz = (static_cast<size_t>(n_row) * sizeof(uint2) + 255) / 256 * 256;
+    unsigned char *ws =
+        static_cast<unsigned char *>(stream_workspace(stream, list_sz + bin_event_scatter_bytes<F>(n_row, n_col)));
+    uint32_t *counters = ws ? stream_counters(stream) : nullptr;
+    if (ws != nullptr && counters != nullptr) {
+      uint2 *active_list = reinterpret_cast<uint2 *>(ws);
+      // the kernel that lists the active rows also zeroes the windows' fill counters and, unless
+      // the output is much longer than the input, y
+      const unsigned collectors = collect_workgroups<F, VT, MODE>(n_row);
+      const bool fold_zero = n_col <= 32ull * collectors * kWinThreads;
+      if (!fold_zero) fill_zero(stream, y, n_col);
+      launch_collect<F, VT, MODE>(stream, indptr, x, n_row, counters, active_list, static_cast<F *>(nullptr), kAlways,
+                                  reinterpret_cast<uint32_t *>(ws + list_sz),
+                                  static_cast<uint32_t>(kBinEventFillBytes / sizeof(uint32_t)), y,
+                                  fold_zero ? n_col : 0u);
+      if (bin_event_scatter<F>(stream, data, HETER, indices, indptr, y, n_row, n_col, counters, active_list,
+                               ws + list_sz))
+        return;
+      fill_zero(stream, counters, 1u);  // (the sort could not run: the list is not used)
+    } else {
+      bpl_clear_error();  // no scratch memory: the paths below need less or none
+    }
+  }
   if (n_win <= (MODE == kEvent ? 32u : 4u)) {
     const uint32_t win = div_up(n_col, n_win);
     // about one workgroup per CU in total, at least 64 rows each
@@ -695,9 +782,8 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
       const bool gated = n_win > 4;
       if (partial == nullptr || gated) fill_zero(stream, y, n_col);
       if (use_list)
-        hipLaunchKernelGGL((collect_active_rows_kernel<F, VT, MODE>), dim3(div_up(n_row, kWinThreads)),
-                           dim3(kWinThreads), 0, stream, indptr, x, n_row, active_count, active_list, active_scales,
-                           window_gate);
+        launch_collect<F, VT, MODE>(stream, indptr, x, n_row, active_count, active_list, active_scales, window_gate,
+                                    static_cast<uint32_t *>(nullptr), 0u, static_cast<F *>(nullptr), 0u);
       hipLaunchKernelGGL(kernel, dim3(groups * n_win), dim3(kWinThreads), lds, stream, data, indices, indptr, x, y,
                          n_row, n_col, rows_per_wg, win, n_win, partial, window_gate, active_count,
                          active_list, active_scales);

@@ -293,6 +293,41 @@ def test_scatter_many_windows_and_row_chunks(cuda, oracle_mod):
       assert np.array_equal(got, want)  # integer counts are exact
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_event_scatter_sorted_by_output_window(cuda, oracle_mod, dtype):
+  # event input and outputs wider than 131,072: the active rows' nonzeros are sorted coarsely by
+  # output window.  Cases: more than 1,024 active rows per producer workgroup (several row tiles);
+  # all columns in one window, more of them than the window's run holds (the rest goes through
+  # direct atomics); float events; silent input; calls repeated (the counters are back at zero).
+  rng = np.random.default_rng(41)
+  cases = []
+  counts = np.minimum(rng.poisson(3, size=1_200_000), 50)
+  cases.append(("tiles", (1_200_000, 200_000), synth.counted_csr(counts, 200_000, seed=1), 0.9))
+  ix, ip = synth.counted_csr(np.full(3000, 100), 4000, seed=2)   # columns < 4,096: one window of 4,096
+  cases.append(("one window", (3000, 200_000), (ix, ip), 1.0))
+  counts = rng.poisson(120, size=30_000)
+  cases.append(("plain", (30_000, 1_000_000), synth.counted_csr(counts, 1_000_000, seed=3), 0.05))
+  for name, shape, (indices, indptr), rate in cases:
+    print("case", name, shape, dtype.__name__, flush=True)
+    data = rng.standard_normal(indices.shape[0]).astype(dtype)
+    for kind in ("bool", "float", "silent"):
+      ev = rng.random(shape[0]) < rate
+      if kind == "silent":
+        ev[:] = False
+      elif kind == "float":
+        ev = (ev * rng.uniform(0.5, 2.0, shape[0])).astype(dtype)
+      for _ in range(2):
+        want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True)
+        mag = oracle_mod.event_csr_matvec(np.abs(data), indices, indptr, ev, shape=shape, transpose=True)
+        got = bpl.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+        assert got.dtype == dtype
+        assert_close_reordered(got, want, mag, what="sorted event scatter %s %s" % (name, kind))
+      ones = np.ones(1, dtype=dtype)
+      want = oracle_mod.event_csr_matvec(ones, indices, indptr, ev, shape=shape, transpose=True)
+      got = bpl.event_csr_matvec(ones, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+      assert np.array_equal(got, want)  # integer counts are exact
+
+
 def test_scatter_through_the_active_row_list(cuda, oracle_mod):
   # more than 32,768 rows: the active rows are first gathered into one list that the row groups
   # share; both input kinds, activity concentrated in one corner of the matrix, twice in a row
