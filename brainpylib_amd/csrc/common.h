@@ -65,7 +65,7 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
 // active_count[0]; `scratch` is device memory of bin_event_scatter_bytes() bytes whose first
 // kBinEventFillBytes are zero; y is zeroed.  Enqueues the two kernels; the second one sets
 // active_count[0] back to zero.  false (nothing enqueued) if it cannot run.
-constexpr size_t kBinEventFillBytes = 16384;
+constexpr size_t kBinEventFillBytes = 131072;
 template <typename F>
 bool bin_event_scatter_usable(uint32_t n_col);
 template <typename F>

@@ -262,15 +262,19 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
 // Only the active rows contribute, how many is known on the device alone (a list made by the
 // caller: (first nonzero, length) per active row, their number in active_count[0]), and the
 // descriptor of the event operators does not carry the nonzero count.  So the bins are not private
-// to a producer here: window b owns ONE run of `cap` pairs, and a producer reserves room for the
-// pairs a round holds for a window with one global atomic on fill[b] (at most one per window and
-// round of 4,096 nonzeros; the event operators move far fewer pairs than the dense product, for
-// which that many same-address atomics would cost more than private regions).  Whatever the
-// distribution of the activity over rows and of the columns over windows, a run only overflows
-// (into direct atomics on y) when its window receives more than `cap` pairs.
+// to a producer here: window b owns 8 runs of `cap` pairs each, shared by the producers p with the
+// same p % 8, and a producer reserves room for the pairs a round holds for a window with one
+// global atomic on the run's fill counter (at most one per window and round of 4,096 nonzeros;
+// the event operators move far fewer pairs than the dense product, for which that many
+// same-address atomics would cost more than private regions).  Whatever the distribution of the
+// activity over rows and of the columns over windows, a run only overflows (into direct atomics
+// on y) when it receives more than `cap` pairs.
 constexpr uint32_t kPairsPerProducer = 4096;  // a producer takes part per that many active nonzeros (estimated): one round
-constexpr uint32_t kFillStride = 32;          // words between the windows' fill counters: one 128-byte line each
-static_assert(kBinEventFillBytes == kMaxWindows * kFillStride * sizeof(uint32_t), "one fill counter per window");
+constexpr uint32_t kSubRuns = 8;              // a window's run is split: producer p appends to sub-run p % 8, so that
+                                              // the atomics on one counter (about 15 ns each) stay few
+constexpr uint32_t kFillStride = 32;          // words between fill counters: one 128-byte line each
+static_assert(kBinEventFillBytes == kMaxWindows * kSubRuns * kFillStride * sizeof(uint32_t),
+              "one fill counter per window and sub-run");
 constexpr uint32_t kPairsPerPart = 8192;      // a consumer workgroup takes part per that many pairs of its window
 
 template <typename F, bool HETER>
@@ -297,6 +301,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_active_rows_kernel(
   const uint32_t producers = want < 1u ? 1u : want > gridDim.x ? gridDim.x : static_cast<uint32_t>(want);
   const uint32_t p = blockIdx.x;
   if (p >= producers) return;
+  const uint32_t sub = p % kSubRuns;
   const uint32_t lo = static_cast<uint32_t>(static_cast<uint64_t>(p) * total / producers);
   const uint32_t hi = static_cast<uint32_t>(static_cast<uint64_t>(p + 1) * total / producers);
   if (tid < kMaxWindows) s_cnt[tid] = 0;
@@ -334,24 +339,41 @@ __global__ __launch_bounds__(kBinThreads) void bin_active_rows_kernel(
         if (tid == 0) s_hint[kBinThreads] = rows - 1u;
       }
       __syncthreads();
-      for (uint32_t jb = seg + tid; jb - tid < seg_end; jb += kRound) {
-        uint32_t rank[U], win[U], rel[U];
-        F val[U];
+      // One round's column indices and weights are requested a round ahead, so that their latency
+      // overlaps the sort, the reservation and the stores of the round before.
+      auto fetch = [&](uint32_t jb, uint32_t (&col)[U], F (&val)[U]) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const uint32_t j = jb + u * kBinThreads;
-          win[u] = 0xffffffffu;  // no pair
-          rel[u] = 0;
+          col[u] = 0xffffffffu;  // no pair
           val[u] = F(0);
-          rank[u] = 0;
           if (j < seg_end) {
             const uint32_t q = (j - seg) >> kHintShift;
             const uint32_t k = row_of(j, s_hint[q], s_hint[q + 1]);
             const uint32_t at = s_start[k] + (j - s_ptr[k]);
-            const uint32_t col = indices[at];
+            col[u] = indices[at];
             val[u] = HETER ? data[at] : w_homo;
-            win[u] = col >> shift;
-            rel[u] = col & ((1u << shift) - 1u);
+          }
+        }
+      };
+      uint32_t col[U];
+      F val[U];
+      fetch(seg + tid, col, val);
+      for (uint32_t jb = seg + tid; jb - tid < seg_end; jb += kRound) {
+        uint32_t ncol[U];
+        F nval[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) ncol[u] = 0xffffffffu, nval[u] = F(0);
+        if (jb - tid + kRound < seg_end) fetch(jb + kRound, ncol, nval);
+        uint32_t rank[U], win[U], rel[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          rank[u] = 0;
+          win[u] = 0xffffffffu;
+          rel[u] = 0;
+          if (col[u] != 0xffffffffu) {
+            win[u] = col[u] >> shift;
+            rel[u] = col[u] & ((1u << shift) - 1u);
           }
         }
 #pragma unroll
@@ -364,8 +386,8 @@ __global__ __launch_bounds__(kBinThreads) void bin_active_rows_kernel(
           s_off[2 * tid] = sum - (c0 + c1);
           s_off[2 * tid + 1] = sum - c1;
           if (tid == kWave - 1) s_off[kMaxWindows] = sum;
-          s_base[2 * tid] = c0 ? atomicAdd(&fill[2 * tid * kFillStride], c0) : 0u;
-          s_base[2 * tid + 1] = c1 ? atomicAdd(&fill[(2 * tid + 1) * kFillStride], c1) : 0u;
+          s_base[2 * tid] = c0 ? atomicAdd(&fill[(2 * tid * kSubRuns + sub) * kFillStride], c0) : 0u;
+          s_base[2 * tid + 1] = c1 ? atomicAdd(&fill[((2 * tid + 1) * kSubRuns + sub) * kFillStride], c1) : 0u;
         }
         __syncthreads();
 #pragma unroll
@@ -385,18 +407,21 @@ __global__ __launch_bounds__(kBinThreads) void bin_active_rows_kernel(
           const uint32_t w = s_window[i];
           const BinPair<F> o = s_sorted[i];
           const uint32_t slot = s_base[w] + (i - s_off[w]);
-          if (slot < cap) pairs[static_cast<uint64_t>(w) * cap + slot] = o;
+          if (slot < cap) pairs[static_cast<uint64_t>(w * kSubRuns + sub) * cap + slot] = o;
           else atomic_add(y + ((w << shift) | o.rel), o.val);
         }
         __syncthreads();
         if (tid < kMaxWindows) s_cnt[tid] = 0;
         __syncthreads();
+#pragma unroll
+        for (int u = 0; u < U; ++u) col[u] = ncol[u], val[u] = nval[u];
       }
     }
   }
 }
 
-// grid = n_win * parts; workgroup (b, s) adds share s of window b's run to the zeroed y.
+// grid = n_win * parts; workgroup (b, s) adds share s of window b's pairs (its 8 runs taken as
+// one sequence) to the zeroed y.
 template <typename F>
 __global__ __launch_bounds__(kBinThreads) void add_window_runs_kernel(F *__restrict__ y, uint32_t n_col, uint32_t shift,
                                                                       uint32_t parts, uint32_t cap,
@@ -410,8 +435,16 @@ __global__ __launch_bounds__(kBinThreads) void add_window_runs_kernel(F *__restr
   const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   constexpr uint32_t kWaves = kBinThreads / kWave;
   const uint32_t b = blockIdx.x / parts, s = blockIdx.x % parts;
-  uint32_t n = fill[b * kFillStride];
-  if (n > cap) n = cap;  // the producers count what they could not store too
+  // pre[r] = pairs in the runs before run r (at most 2^27 in all)
+  uint32_t pre[kSubRuns + 1];
+  pre[0] = 0;
+#pragma unroll
+  for (uint32_t r = 0; r < kSubRuns; ++r) {
+    uint32_t c = fill[(b * kSubRuns + r) * kFillStride];
+    if (c > cap) c = cap;  // the producers count what they could not store too
+    pre[r + 1] = pre[r] + c;
+  }
+  const uint32_t n = pre[kSubRuns];
   // every workgroup that takes part adds a whole window to y: few pairs, few workgroups
   const uint32_t want = (n + kPairsPerPart - 1u) / kPairsPerPart;
   if (want < parts) parts = want;
@@ -422,20 +455,28 @@ __global__ __launch_bounds__(kBinThreads) void add_window_runs_kernel(F *__restr
   const uint32_t width = (n_col - c0 < (1u << shift)) ? n_col - c0 : (1u << shift);
   for (uint32_t i = tid; i < width; i += kBinThreads) window[i] = 0.0;
   __syncthreads();
-  const BinPair<F> *run = pairs + static_cast<uint64_t>(b) * cap;
+  const BinPair<F> *runs = pairs + static_cast<uint64_t>(b) * kSubRuns * cap;
+  // pair number v of the window's runs taken as one sequence
+  auto pair_at = [&](uint32_t v) {
+    uint32_t r = 0, first = 0;
+#pragma unroll
+    for (uint32_t k = 1; k < kSubRuns; ++k)
+      if (v >= pre[k]) r = k, first = pre[k];
+    return runs[static_cast<uint64_t>(r) * cap + (v - first)];
+  };
   constexpr int U = 8;
   for (uint32_t i0 = lo + wave * (U * kWave); i0 < hi; i0 += kWaves * U * kWave) {
     BinPair<F> e[U];
-    if (i0 + U * kWave <= hi) {
+    if (i0 + U * kWave <= hi) {  // full steps: plain loads, all in flight
 #pragma unroll
-      for (int u = 0; u < U; ++u) e[u] = run[i0 + u * kWave + lane];
+      for (int u = 0; u < U; ++u) e[u] = pair_at(i0 + u * kWave + lane);
     } else {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const uint32_t i = i0 + u * kWave + lane;
+        const uint32_t v = i0 + u * kWave + lane;
         e[u].rel = 0xffffffffu;
         e[u].val = F(0);
-        if (i < hi) e[u] = run[i];
+        if (v < hi) e[u] = pair_at(v);
       }
     }
 #pragma unroll
@@ -449,7 +490,6 @@ __global__ __launch_bounds__(kBinThreads) void add_window_runs_kernel(F *__restr
   }
 }
 
-// pairs all windows' runs hold together: 32 per row or column, between 2^22 and 2^26
 // log2 of the output window with event input: as many windows as the 7-bit ids allow (every
 // consumer workgroup adds a whole window to y, so small windows and few workgroups per window)
 inline uint32_t event_window_shift(uint32_t n_out) {
@@ -459,9 +499,9 @@ inline uint32_t event_window_shift(uint32_t n_out) {
 }
 
 inline uint64_t event_run_pairs(uint32_t n_row, uint32_t n_col) {
-  uint64_t t = 32ull * (n_row > n_col ? n_row : n_col);
+  uint64_t t = 64ull * (n_row > n_col ? n_row : n_col);
   if (t < (1ull << 22)) t = 1ull << 22;
-  if (t > (1ull << 26)) t = 1ull << 26;
+  if (t > (1ull << 27)) t = 1ull << 27;
   return t;
 }
 
@@ -476,8 +516,8 @@ bool bin_event_scatter_usable(uint32_t n_col) {
 template <typename F>
 size_t bin_event_scatter_bytes(uint32_t n_row, uint32_t n_col) {
   const uint32_t n_win = div_up(n_col, 1u << event_window_shift(n_col));
-  const uint64_t cap = event_run_pairs(n_row, n_col) / n_win;
-  return kBinEventFillBytes + static_cast<size_t>(cap) * n_win * sizeof(BinPair<F>);
+  const uint64_t cap = event_run_pairs(n_row, n_col) / (n_win * kSubRuns);
+  return kBinEventFillBytes + static_cast<size_t>(cap) * n_win * kSubRuns * sizeof(BinPair<F>);
 }
 
 template <typename F>
@@ -486,7 +526,7 @@ bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint
                        void *scratch) {
   const uint32_t shift = event_window_shift(n_col);
   const uint32_t n_win = div_up(n_col, 1u << shift);
-  const uint32_t cap = static_cast<uint32_t>(event_run_pairs(n_row, n_col) / n_win);
+  const uint32_t cap = static_cast<uint32_t>(event_run_pairs(n_row, n_col) / (n_win * kSubRuns));
   uint32_t *fill = static_cast<uint32_t *>(scratch);
   BinPair<F> *pairs = reinterpret_cast<BinPair<F> *>(static_cast<unsigned char *>(scratch) + kBinEventFillBytes);
   const unsigned num_cu = static_cast<unsigned>(device_info().num_cu);

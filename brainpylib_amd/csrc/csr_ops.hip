@@ -165,8 +165,7 @@ __global__ __launch_bounds__(kWinThreads) void collect_active_rows_kernel(
   __shared__ uint32_t s_count, s_base;
   const uint32_t tid = threadIdx.x, lane = tid % kWave;
   if (tid == 0) s_count = 0;
-  if (blockIdx.x == 0)
-    for (uint32_t i = tid; i < n_clear; i += kWinThreads) clear[i] = 0u;
+  for (uint32_t i = blockIdx.x * kWinThreads + tid; i < n_clear; i += gridDim.x * kWinThreads) clear[i] = 0u;
   for (uint32_t i = blockIdx.x * kWinThreads + tid; i < n_zero; i += gridDim.x * kWinThreads) zero[i] = F(0);
   __syncthreads();
   const uint32_t r0 = blockIdx.x * (kWinThreads * kCollectPerThread) + tid;
