@@ -389,6 +389,23 @@ def main():
     extra["csr_matvec_transposed_1e8"] = dict(stats(dur3t), gsop_per_s=nnz3 / (dur3t.mean() * 1e-3) / 1e9,
                                               algorithmic_gb_per_s=bytes3 / (dur3t.mean() * 1e-3) / 1e9)
     log("csr_matvec transposed 1e8: %s" % extra["csr_matvec_transposed_1e8"])
+    # the same 1,000,000 x 1,000,000 matrix (100 nonzeros per row) driven by events, 1 % and 5 % of
+    # the rows active: the shape of a million-neuron network's synaptic update (output far wider than LDS)
+    wide = {}
+    for rate in (0.01, 0.05):
+      ev_np = np.random.default_rng(17).random(m["shape"][0]) < rate
+      ev_w = torch.from_numpy(ev_np).to(dev)
+      want = oracle.event_csr_matvec(m["data"], m["indices"], m["indptr"], ev_np, shape=m["shape"], transpose=True)
+      mag = oracle.event_csr_matvec(np.abs(m["data"]), m["indices"], m["indptr"], ev_np, shape=m["shape"], transpose=True)
+      got = bpl.event_csr_matvec(md["data"], md["indices"], md["indptr"], ev_w, shape=m["shape"], transpose=True)
+      check(got.cpu().numpy(), want, "event_csr_matvec scatter 1e6 x 1e6 at %g" % rate, mag)
+      dur_w, _ = time_calls(lambda: bpl.event_csr_matvec(md["data"], md["indices"], md["indptr"], ev_w, shape=m["shape"],
+                                                         transpose=True), args.steps, 5)
+      delivered = int(np.diff(m["indptr"])[ev_np].sum())
+      wide["events_%g" % rate] = dict(stats(dur_w), delivered_synapses=delivered,
+                                      gsop_per_s=delivered / (dur_w.mean() * 1e-3) / 1e9)
+    extra["scatter_1e6x1e6_100_per_row"] = wide
+    log("event scatter 1e6 x 1e6: %s" % wide)
 
   if not args.skip_extra:
     del md
