@@ -660,6 +660,17 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
   }
   // lanes per row from the mean row length
   const uint32_t mean = nnz / n_row;
+  if constexpr (MODE == kEvent && LDS_BITS) {
+    // An event bitmap above 80 KB leaves room for one workgroup (16 waves) per CU only: every lane
+    // then keeps 16 (rows under 24 nonzeros: 8) loads in flight instead of 2 to 8, in groups of
+    // 16, 8 or 4 lanes per row, or HBM sees too few requests (1e6 columns, 100 per row: 424 -> 167 us).
+    if (n_col > 655360u) {
+      if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, LDS_BITS, 8>(data, indices, indptr, x, y, n_row, s_bits);
+      else if (mean >= 48) gather_rows<F, VT, HETER, MODE, LDS_BITS, 8, 16>(data, indices, indptr, x, y, n_row, s_bits);
+      else gather_rows<F, VT, HETER, MODE, LDS_BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits);
+      return;
+    }
+  }
   if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, LDS_BITS, 8>(data, indices, indptr, x, y, n_row, s_bits);
   // (a dense vector is gathered from L2: for rows of 48 .. 191 nonzeros the pipelined 32-lane walk keeps more
   // of those gathers in flight than a wave per row does)

@@ -208,6 +208,32 @@ def test_unaligned_event_vector_and_large_bitmap(cuda, oracle_mod):
     assert_close(got, want)
 
 
+def test_gather_row_length_modes_with_a_bitmap_that_fills_lds(cuda, oracle_mod):
+  # more than 655,360 columns: the event bitmap leaves room for one workgroup per CU, and the
+  # lanes-per-row modes of that regime are used (rows under 48 / 48 .. 383 / from 384 nonzeros)
+  rng = np.random.default_rng(14)
+  n_col = 700_000
+  for n_row, mean in ((20_000, 5), (20_000, 40), (18_000, 120), (3000, 120), (17_000, 500)):
+    counts = rng.poisson(mean, size=n_row)
+    counts[::7] = 0
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_row + mean)
+    data = rng.standard_normal(indices.shape[0]).astype(np.float32)
+    ev = rng.random(n_col) < 0.2
+    shape = (n_row, n_col)
+    print("shape", shape, "mean", mean, flush=True)
+    want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape)
+    got = bpl.event_csr_matvec(data, indices, indptr, ev, shape=shape).cpu().numpy()
+    assert_close(got, want)
+    w = np.float32(0.37)
+    want = oracle_mod.event_csr_matvec(w, indices, indptr, ev, shape=shape)
+    got = bpl.event_csr_matvec(w, indices, indptr, ev, shape=shape).cpu().numpy()
+    assert_close(got, want)
+    evf = (ev * rng.uniform(0.5, 2.0, n_col)).astype(np.float32)
+    got = bpl.event_csr_matvec(data, indices, indptr, evf, shape=shape).cpu().numpy()
+    want = oracle_mod.event_csr_matvec(data, indices, indptr, evf, shape=shape)
+    assert_close(got, want)
+
+
 def test_config_event_csr_small(cuda, oracle_mod):
   # 4,000 x 4,000, 80 per row, homogeneous 0.6, events 2 %, transpose
   c = synth.config_event_csr_small()
