@@ -640,12 +640,16 @@ __device__ __forceinline__ void gather_rows_wave(const F *__restrict__ data, con
   }
 }
 
-template <typename F, typename VT, bool HETER, int MODE, bool LDS_BITS>
+// BITS: where the event probes go.  0: the event vector in global memory; 1: a bitmap in LDS;
+// 2: a bitmap in LDS of more than 80 KB (one workgroup per CU; a kernel of its own, so that the
+// code of the other cases does not depend on it).
+template <typename F, typename VT, bool HETER, int MODE, int BITS>
 __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ data,
                                                           const uint32_t *__restrict__ indices,
                                                           const uint32_t *__restrict__ indptr,
                                                           const VT *__restrict__ x, F *__restrict__ y,
                                                           uint32_t n_row, uint32_t n_col) {
+  constexpr bool LDS_BITS = BITS != 0;
   extern __shared__ uint32_t s_bits[];
   if (LDS_BITS) {
     const uint32_t words = (n_col + 31u) >> 5;
@@ -660,25 +664,23 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
   }
   // lanes per row from the mean row length
   const uint32_t mean = nnz / n_row;
-  if constexpr (MODE == kEvent && LDS_BITS) {
+  if constexpr (MODE == kEvent && BITS == 2) {
     // An event bitmap above 80 KB leaves room for one workgroup (16 waves) per CU only: every lane
-    // then keeps 16 (rows under 24 nonzeros: 8) loads in flight instead of 2 to 8, in groups of
-    // 16, 8 or 4 lanes per row, or HBM sees too few requests (1e6 columns, 100 per row: 424 -> 167 us).
-    if (n_col > 655360u) {
-      if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, LDS_BITS, 8>(data, indices, indptr, x, y, n_row, s_bits);
-      else if (mean >= 48) gather_rows<F, VT, HETER, MODE, LDS_BITS, 8, 16>(data, indices, indptr, x, y, n_row, s_bits);
-      else gather_rows<F, VT, HETER, MODE, LDS_BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits);
-      return;
-    }
+    // then keeps 16 (rows under 48 nonzeros: 8) loads in flight instead of 2 to 8, in groups of
+    // 8 or 4 lanes per row, or HBM sees too few requests (1e6 columns, 100 per row: 424 -> 164 us).
+    if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, LDS_BITS, 8>(data, indices, indptr, x, y, n_row, s_bits);
+    else if (mean >= 48) gather_rows<F, VT, HETER, MODE, LDS_BITS, 8, 16>(data, indices, indptr, x, y, n_row, s_bits);
+    else gather_rows<F, VT, HETER, MODE, LDS_BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits);
+  } else {
+    if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, LDS_BITS, 8>(data, indices, indptr, x, y, n_row, s_bits);
+    // (a dense vector is gathered from L2: for rows of 48 .. 191 nonzeros the pipelined 32-lane walk keeps more
+    // of those gathers in flight than a wave per row does)
+    else if (mean >= (MODE == kDense ? 192u : 48u)) gather_rows_wave<F, VT, HETER, MODE, LDS_BITS, 2>(data, indices, indptr, x, y, n_row, s_bits);
+    else if (mean >= 48) gather_rows<F, VT, HETER, MODE, LDS_BITS, 32, 4>(data, indices, indptr, x, y, n_row, s_bits);
+    else if (mean >= 24) gather_rows<F, VT, HETER, MODE, LDS_BITS, 32, 2>(data, indices, indptr, x, y, n_row, s_bits);
+    else if (mean >= 12) gather_rows<F, VT, HETER, MODE, LDS_BITS, 16, 2>(data, indices, indptr, x, y, n_row, s_bits);
+    else gather_rows<F, VT, HETER, MODE, LDS_BITS, 8, 2>(data, indices, indptr, x, y, n_row, s_bits);
   }
-  if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, LDS_BITS, 8>(data, indices, indptr, x, y, n_row, s_bits);
-  // (a dense vector is gathered from L2: for rows of 48 .. 191 nonzeros the pipelined 32-lane walk keeps more
-  // of those gathers in flight than a wave per row does)
-  else if (mean >= (MODE == kDense ? 192u : 48u)) gather_rows_wave<F, VT, HETER, MODE, LDS_BITS, 2>(data, indices, indptr, x, y, n_row, s_bits);
-  else if (mean >= 48) gather_rows<F, VT, HETER, MODE, LDS_BITS, 32, 4>(data, indices, indptr, x, y, n_row, s_bits);
-  else if (mean >= 24) gather_rows<F, VT, HETER, MODE, LDS_BITS, 32, 2>(data, indices, indptr, x, y, n_row, s_bits);
-  else if (mean >= 12) gather_rows<F, VT, HETER, MODE, LDS_BITS, 16, 2>(data, indices, indptr, x, y, n_row, s_bits);
-  else gather_rows<F, VT, HETER, MODE, LDS_BITS, 8, 2>(data, indices, indptr, x, y, n_row, s_bits);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -815,11 +817,11 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
                      dim3(kScatterThreads), 0, stream, data, indices, indptr, x, y, n_row, direct_gate);
 }
 
-template <typename F, typename VT, bool HETER, int MODE, bool LDS_BITS>
+template <typename F, typename VT, bool HETER, int MODE, int BITS>
 bool launch_gather_impl(const char *target, hipStream_t stream, const F *data, const uint32_t *indices,
                         const uint32_t *indptr, const VT *x, F *y, uint32_t n_row, uint32_t n_col,
                         size_t lds_bytes) {
-  auto kernel = csr_gather_kernel<F, VT, HETER, MODE, LDS_BITS>;
+  auto kernel = csr_gather_kernel<F, VT, HETER, MODE, BITS>;
   // Small problems: 256-thread workgroups, one wave per row at most.  Large ones: 1024-thread
   // persistent workgroups so that few copies of the event bitmap are built.
   const int block = (n_row >= 16384) ? 1024 : 256;
@@ -876,13 +878,16 @@ void launch_gather(const char *target, hipStream_t stream, const F *data, const 
     const size_t lds_bytes = (static_cast<size_t>(n_col) + 31) / 32 * 4;
     const size_t lds_cap = static_cast<size_t>(160) * 1024 - 1024;
     if (lds_bytes <= lds_cap) {
-      if (launch_gather_impl<F, VT, HETER, MODE, true>(target, stream, data, indices, indptr, x, y, n_row, n_col,
-                                                       lds_bytes))
-        return;
+      const bool ok = lds_bytes > 80 * 1024
+                          ? launch_gather_impl<F, VT, HETER, MODE, 2>(target, stream, data, indices, indptr, x, y, n_row,
+                                                                      n_col, lds_bytes)
+                          : launch_gather_impl<F, VT, HETER, MODE, 1>(target, stream, data, indices, indptr, x, y, n_row,
+                                                                      n_col, lds_bytes);
+      if (ok) return;
       bpl_clear_error();
     }
   }
-  launch_gather_impl<F, VT, HETER, MODE, false>(target, stream, data, indices, indptr, x, y, n_row, n_col, 0);
+  launch_gather_impl<F, VT, HETER, MODE, 0>(target, stream, data, indices, indptr, x, y, n_row, n_col, 0);
 }
 
 // event_csr_matvec: buffers = [data, indices, indptr, events, out]
