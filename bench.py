@@ -132,11 +132,12 @@ def main():
   ap.add_argument("--warmup", type=int, default=20)
   ap.add_argument("--skip-extra", action="store_true", help="only the headline workload")
   ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU baseline")
-  ap.add_argument("--pmc", choices=["gather", "scatter", "jitconn"], default=None,
+  ap.add_argument("--pmc", choices=["gather", "scatter", "jitconn", "jitconn-normal"], default=None,
                   help="counter-collection mode for rocprofv3 --pmc.  gather: three plain copies of 400 MB "
                        "(the calibration kernel) and three calls of the headline kernel.  scatter: three calls of "
                        "the same matrix with transpose=True.  jitconn: three calls "
-                       "of jitconn event matvec (1e6 x 1e6, p=0.001) in both walks.  Nothing else runs.")
+                       "of jitconn event matvec (1e6 x 1e6, p=0.001) in both walks.  jitconn-normal: three "
+                       "row walks of the same matrix with normal weights.  Nothing else runs.")
   ap.add_argument("--reference-shapes", action="store_true",
                   help="instead of the headline run: the shapes of the reference's own benchmark scripts "
                        "(event_matvec_jitconn_performance.py, csr_matvec_VS_cusparse_csr_matvec.py), with the "
@@ -167,6 +168,16 @@ def main():
       for _ in range(3):
         bpl.event_matvec_prob_conn_homo_weight(ev, j["weight"], conn_prob=j["conn_prob"], shape=j["shape"],
                                                seed=j["seed"], outdim_parallel=odp)
+    torch.cuda.synchronize()
+    log("pmc mode done")
+    return
+
+  if args.pmc == "jitconn-normal":
+    j = synth.config_jitconn_event()
+    ev = torch.from_numpy(j["events"]).to(dev)
+    for _ in range(3):
+      bpl.event_matvec_prob_conn_normal_weight(ev, w_mu=0.0, w_sigma=1.0, conn_prob=j["conn_prob"], shape=j["shape"],
+                                               seed=j["seed"], outdim_parallel=True)
     torch.cuda.synchronize()
     log("pmc mode done")
     return
