@@ -84,7 +84,12 @@ def custom_call(name, buffers, opaque, stream=None):
   import torch
   fn = target(name)
   if stream is None:
-    stream = torch.cuda.current_stream().cuda_stream
+    # (the raw handle; torch.cuda.current_stream() builds a Stream object first, which costs
+    # several microseconds per call)
+    try:
+      stream = torch._C._cuda_getCurrentRawStream(buffers[0].device.index)
+    except (AttributeError, TypeError):
+      stream = torch.cuda.current_stream(buffers[0].device).cuda_stream
   n = len(buffers)
   array_type = _PTR_ARRAYS.get(n)
   if array_type is None:

@@ -7,6 +7,9 @@ FLOAT_DTYPES = (torch.float32, torch.float64)
 _INDEX_DTYPES = (torch.int32, torch.uint32)
 
 
+_PY_SCALARS = {}  # host tensors of Python numbers seen as operands (read-only)
+
+
 def as_tensor(a):
   """Unwraps brainpy-like arrays (objects with `.value`) and wraps numpy / python data as a torch
   tensor WITHOUT moving it, so that argument checks can run before a device is needed.
@@ -16,7 +19,15 @@ def as_tensor(a):
   if isinstance(a, torch.Tensor):
     return a
   if isinstance(a, (bool, int, float)):
-    return torch.tensor(a, dtype=torch.bool if isinstance(a, bool) else torch.float32)
+    if a == 0:  # (0.0 and -0.0 compare equal: not cached)
+      return torch.tensor(a, dtype=torch.bool if isinstance(a, bool) else torch.float32)
+    key = (type(a), a)
+    t = _PY_SCALARS.get(key)
+    if t is None:
+      if len(_PY_SCALARS) >= 256:
+        _PY_SCALARS.clear()
+      t = _PY_SCALARS[key] = torch.tensor(a, dtype=torch.bool if isinstance(a, bool) else torch.float32)
+    return t
   arr = np.asarray(a)
   if arr.dtype == np.uint32:
     return torch.from_numpy(np.ascontiguousarray(arr).view(np.int32)).view(torch.uint32)
