@@ -420,11 +420,13 @@ __global__ __launch_bounds__(kBinThreads) void bin_active_rows_kernel(
   }
 }
 
-// grid = n_win * parts; workgroup (b, s) adds share s of window b's pairs (its 8 runs taken as
-// one sequence) to the zeroed y.
+// grid = n_win * slices * parts; workgroup (b, q, s) adds share s of window b's pairs (its 8 runs
+// taken as one sequence) to the zeroed y.  A window wider than the 2^lds_shift float64 accumulators
+// in LDS is cut into `slices` = 2^(shift - lds_shift) slices: the workgroups of slice q read the
+// same pairs and keep those that fall into their slice.
 template <typename F>
 __global__ __launch_bounds__(kBinThreads) void add_window_runs_kernel(F *__restrict__ y, uint32_t n_col, uint32_t shift,
-                                                                      uint32_t parts, uint32_t cap,
+                                                                      uint32_t lds_shift, uint32_t parts, uint32_t cap,
                                                                       const BinPair<F> *__restrict__ pairs,
                                                                       const uint32_t *__restrict__ fill,
                                                                       uint32_t *__restrict__ reset) {
@@ -434,7 +436,8 @@ __global__ __launch_bounds__(kBinThreads) void add_window_runs_kernel(F *__restr
   double *window = reinterpret_cast<double *>(smem_raw);
   const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   constexpr uint32_t kWaves = kBinThreads / kWave;
-  const uint32_t b = blockIdx.x / parts, s = blockIdx.x % parts;
+  const uint32_t slices = 1u << (shift - lds_shift);
+  const uint32_t b = blockIdx.x / (parts * slices), q = (blockIdx.x / parts) % slices, s = blockIdx.x % parts;
   // pre[r] = pairs in the runs before run r (at most 2^27 in all)
   uint32_t pre[kSubRuns + 1];
   pre[0] = 0;
@@ -451,8 +454,10 @@ __global__ __launch_bounds__(kBinThreads) void add_window_runs_kernel(F *__restr
   if (s >= parts) return;
   const uint32_t lo = static_cast<uint32_t>(static_cast<uint64_t>(s) * n / parts);
   const uint32_t hi = static_cast<uint32_t>(static_cast<uint64_t>(s + 1) * n / parts);
-  const uint32_t c0 = b << shift;
-  const uint32_t width = (n_col - c0 < (1u << shift)) ? n_col - c0 : (1u << shift);
+  const uint32_t r0 = q << lds_shift;  // first column of the slice within the window
+  const uint32_t c0 = (b << shift) + r0;
+  if (c0 >= n_col) return;
+  const uint32_t width = (n_col - c0 < (1u << lds_shift)) ? n_col - c0 : (1u << lds_shift);
   for (uint32_t i = tid; i < width; i += kBinThreads) window[i] = 0.0;
   __syncthreads();
   const BinPair<F> *runs = pairs + static_cast<uint64_t>(b) * kSubRuns * cap;
@@ -481,7 +486,7 @@ __global__ __launch_bounds__(kBinThreads) void add_window_runs_kernel(F *__restr
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (e[u].rel < width) atomicAdd(&window[e[u].rel], static_cast<double>(e[u].val));
+      if (e[u].rel - r0 < width) atomicAdd(&window[e[u].rel - r0], static_cast<double>(e[u].val));  // (wraps below r0)
   }
   __syncthreads();
   for (uint32_t i = tid; i < width; i += kBinThreads) {
@@ -491,10 +496,13 @@ __global__ __launch_bounds__(kBinThreads) void add_window_runs_kernel(F *__restr
 }
 
 // log2 of the output window with event input: as many windows as the 7-bit ids allow (every
-// consumer workgroup adds a whole window to y, so small windows and few workgroups per window)
+// consumer workgroup adds a whole window to y, so small windows and few workgroups per window).
+// Up to 2^14 columns a window has its accumulators in LDS at once; wider ones (outputs above two
+// million columns) are added in slices of 2^14, each slice reading the window's pairs again.
+constexpr uint32_t kEventMaxShift = 17;
 inline uint32_t event_window_shift(uint32_t n_out) {
   uint32_t shift = 8;
-  while (shift < kBinMaxShift && (n_out >> shift) >= kMaxWindows) ++shift;
+  while (shift < kEventMaxShift && (n_out >> shift) >= kMaxWindows) ++shift;
   return shift;
 }
 
@@ -533,7 +541,10 @@ bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint
   uint32_t parts = num_cu / n_win;
   if (parts == 0) parts = 1;
   auto add_kernel = add_window_runs_kernel<F>;
-  const size_t lds = sizeof(double) << shift;
+  const uint32_t lds_shift = shift < kBinMaxShift ? shift : kBinMaxShift;
+  const uint32_t slices = 1u << (shift - lds_shift);
+  if (slices > 1) parts = 1;
+  const size_t lds = sizeof(double) << lds_shift;
   static thread_local bool attr_set = false;
   if (!attr_set && lds > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(add_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -550,8 +561,8 @@ bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint
   else
     hipLaunchKernelGGL((bin_active_rows_kernel<F, false>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
                        indptr, n_row, active_count, active_list, y, shift, cap, pairs, fill);
-  hipLaunchKernelGGL(add_kernel, dim3(n_win * parts), dim3(kBinThreads), lds, stream, y, n_col, shift, parts, cap, pairs,
-                     fill, active_count);
+  hipLaunchKernelGGL(add_kernel, dim3(n_win * slices * parts), dim3(kBinThreads), lds, stream, y, n_col, shift,
+                     lds_shift, parts, cap, pairs, fill, active_count);
   return true;
 }
 

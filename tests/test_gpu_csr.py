@@ -333,6 +333,9 @@ def test_event_scatter_sorted_by_output_window(cuda, oracle_mod, dtype):
   cases.append(("one window", (3000, 200_000), (ix, ip), 1.0))
   counts = rng.poisson(120, size=30_000)
   cases.append(("plain", (30_000, 1_000_000), synth.counted_csr(counts, 1_000_000, seed=3), 0.05))
+  # above 2^21 columns a window is wider than its accumulators in LDS and is added in slices
+  counts = rng.poisson(60, size=20_000)
+  cases.append(("sliced windows", (20_000, 5_000_001), synth.counted_csr(counts, 5_000_001, seed=4), 0.3))
   for name, shape, (indices, indptr), rate in cases:
     print("case", name, shape, dtype.__name__, flush=True)
     data = rng.standard_normal(indices.shape[0]).astype(dtype)
