@@ -221,6 +221,43 @@ __global__ __launch_bounds__(256) void pack_event_bitmap_kernel(const VT *__rest
   }
 }
 
+// Two-level bitmap for event vectors whose bitmap does not fit LDS.  Behind the exact bitmap
+// (ceil(n / 32) words, padded to coarse_offset_words(n)) sits a coarse one: bit c = any of the
+// elements [c << g, (c + 1) << g) is set, with g = coarse_shift(n) the smallest shift for which
+// the coarse bitmap fits kLdsBitmapCap bytes.  A kernel keeps the coarse bitmap in LDS and looks
+// at the exact one, in global memory, only where the coarse bit is set.
+constexpr uint32_t kLdsBitmapCap = 160u * 1024u - 1024u;
+__host__ __device__ inline uint32_t coarse_bits(uint32_t n, uint32_t g) { return n ? ((n - 1u) >> g) + 1u : 0u; }
+__host__ __device__ inline uint32_t coarse_shift(uint32_t n) {
+  uint32_t g = 0;
+  while ((coarse_bits(n, g) + 31u) / 32u * 4u > kLdsBitmapCap) ++g;
+  return g;
+}
+__host__ __device__ inline uint32_t coarse_offset_words(uint32_t n) { return ((n + 31u) / 32u + 63u) / 64u * 64u; }
+
+static __global__ __launch_bounds__(256) void coarsen_bitmap_kernel(const uint32_t *__restrict__ bits, uint32_t n_words,
+                                                             uint32_t g, uint32_t *__restrict__ coarse,
+                                                             uint32_t n_coarse_words) {
+  const uint32_t w = blockIdx.x * 256u + threadIdx.x;
+  if (w >= n_coarse_words) return;
+  uint32_t out = 0;
+  for (uint32_t i = 0; i < 32u; ++i) {
+    const uint64_t c = static_cast<uint64_t>(w) * 32u + i;
+    uint32_t any = 0;
+    if (g >= 5u) {
+      const uint64_t first = c << (g - 5u);
+      for (uint64_t k = 0; k < (1ull << (g - 5u)) && first + k < n_words; ++k) any |= bits[first + k];
+    } else {
+      const uint64_t word = c >> (5u - g);
+      const uint32_t sub = static_cast<uint32_t>(c) & ((1u << (5u - g)) - 1u);
+      const uint32_t v = word < n_words ? bits[word] : 0u;
+      any = (v >> (sub << g)) & ((1u << (1u << g)) - 1u);
+    }
+    out |= (any != 0u ? 1u : 0u) << i;
+  }
+  coarse[w] = out;
+}
+
 template <typename VT>
 inline void pack_event_bitmap(hipStream_t stream, const VT *ev, uint32_t n, uint32_t *bits) {
   if (n == 0) return;

@@ -478,10 +478,48 @@ __global__ __launch_bounds__(256) void sum_partials_kernel(const F *__restrict__
 // before the loads that depend on the current step's indices are consumed, so a row change
 // does not drain the pipeline.  Loads are unconditional (out-of-row lanes re-read a valid
 // element and are masked out of the sum); only the `data` fetch of an event hit is predicated.
-template <typename F, typename VT, bool HETER, int MODE, bool LDS_BITS, int G, int U>
+// Is column `col` an event?  BITS 0: the event vector in global memory; 1, 2: the bitmap in LDS;
+// 3: a coarse bitmap in LDS (one bit per 2^g columns), then the exact packed one in global memory.
+template <int BITS, typename VT>
+__device__ __forceinline__ bool event_hit(const uint32_t *s_bits, const VT *__restrict__ x, uint32_t col, uint32_t g) {
+  if constexpr (BITS == 0) {
+    return probe_event(x, col);
+  } else if constexpr (BITS == 3) {
+    const uint32_t c = col >> g;
+    return ((s_bits[c >> 5] >> (c & 31u)) & 1u) && probe_event(x, col);
+  } else {
+    return (s_bits[col >> 5] >> (col & 31u)) & 1u;
+  }
+}
+
+// The same for the U columns of a step.  With the two-level bitmap the loads of the exact words are
+// issued for all U columns before any is looked at (lanes whose coarse bit is clear read word 0),
+// so that they are in flight together instead of one behind the other.
+template <int BITS, int U, typename VT>
+__device__ __forceinline__ void event_hits(const uint32_t *s_bits, const VT *__restrict__ x, const uint32_t (&col)[U],
+                                           uint32_t g, bool (&hit)[U]) {
+  if constexpr (BITS == 3) {
+    uint32_t word[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t c = col[u] >> g;
+      hit[u] = (s_bits[c >> 5] >> (c & 31u)) & 1u;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) word[u] = x[hit[u] ? col[u] >> 5 : 0u].w;
+#pragma unroll
+    for (int u = 0; u < U; ++u) hit[u] = hit[u] && ((word[u] >> (col[u] & 31u)) & 1u);
+  } else {
+#pragma unroll
+    for (int u = 0; u < U; ++u) hit[u] = event_hit<BITS>(s_bits, x, col[u], g);
+  }
+}
+
+template <typename F, typename VT, bool HETER, int MODE, int BITS, int G, int U>
 __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const uint32_t *__restrict__ indices,
                                             const uint32_t *__restrict__ indptr, const VT *__restrict__ x,
-                                            F *__restrict__ y, uint32_t n_row, const uint32_t *s_bits) {
+                                            F *__restrict__ y, uint32_t n_row, const uint32_t *s_bits,
+                                            uint32_t coarse_g) {
   const uint32_t groups_per_block = blockDim.x / G;
   const uint32_t gl = threadIdx.x % G;
   const uint32_t total_groups = gridDim.x * groups_per_block;
@@ -517,14 +555,16 @@ __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const ui
     // loads that depend on this step's indices
     F val[U];
     bool use[U];
+    bool hits_u[U];
+    if constexpr (MODE == kEvent && BITS == 3) event_hits<BITS, U>(s_bits, x, col, coarse_g, hits_u);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t j = base + u * G + gl;
       const bool ok = j < end;
       if (MODE == kEvent) {
         bool hit;
-        if (LDS_BITS) hit = (s_bits[col[u] >> 5] >> (col[u] & 31u)) & 1u;
-        else hit = probe_event(x, col[u]);
+        if constexpr (BITS == 3) hit = hits_u[u];
+        else hit = event_hit<BITS>(s_bits, x, col[u], coarse_g);
         hit = hit && ok;
         use[u] = hit;
         val[u] = F(0);
@@ -570,10 +610,11 @@ __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const ui
 // Long rows: one wave per row.  Row bounds and base pointers are wave uniform (scalar
 // registers), lanes address their elements as base + small offset, full steps of U*64 nonzeros
 // run without guards and only the last step of a row is predicated.
-template <typename F, typename VT, bool HETER, int MODE, bool LDS_BITS, int U>
+template <typename F, typename VT, bool HETER, int MODE, int BITS, int U>
 __device__ __forceinline__ void gather_rows_wave(const F *__restrict__ data, const uint32_t *__restrict__ indices,
                                                  const uint32_t *__restrict__ indptr, const VT *__restrict__ x,
-                                                 F *__restrict__ y, uint32_t n_row, const uint32_t *s_bits) {
+                                                 F *__restrict__ y, uint32_t n_row, const uint32_t *s_bits,
+                                                 uint32_t coarse_g) {
   const uint32_t lane = static_cast<uint32_t>(lane_id());
   const uint32_t waves_per_block = blockDim.x / kWave;
   const uint32_t total_waves = gridDim.x * waves_per_block;
@@ -589,13 +630,16 @@ __device__ __forceinline__ void gather_rows_wave(const F *__restrict__ data, con
       col[u] = ok[u] ? ip[off] : 0u;
     }
     F val[U];
+    bool hits_u[U];
+    if constexpr (MODE == kEvent && BITS == 3) event_hits<BITS, U>(s_bits, x, col, coarse_g, hits_u);  // (col 0 where !ok)
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t off = b + u * kWave + lane;
       if (MODE == kEvent) {
         bool hit;
-        if (LDS_BITS) hit = (s_bits[col[u] >> 5] >> (col[u] & 31u)) & 1u;
-        else hit = ok[u] && probe_event(x, col[u]);
+        if constexpr (BITS == 3) hit = hits_u[u];
+        else if (BITS == 1 || BITS == 2) hit = event_hit<BITS>(s_bits, x, col[u], coarse_g);
+        else hit = ok[u] && event_hit<BITS>(s_bits, x, col[u], coarse_g);
         hit = hit && ok[u];
         if (HETER) {
           val[u] = F(0);
@@ -649,9 +693,16 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
                                                           const uint32_t *__restrict__ indptr,
                                                           const VT *__restrict__ x, F *__restrict__ y,
                                                           uint32_t n_row, uint32_t n_col) {
-  constexpr bool LDS_BITS = BITS != 0;
   extern __shared__ uint32_t s_bits[];
-  if (LDS_BITS) {
+  uint32_t coarse_g = 0;
+  if constexpr (BITS == 3) {
+    // x is the exact packed bitmap; the coarse one behind it goes to LDS
+    coarse_g = coarse_shift(n_col);
+    const uint32_t words = (coarse_bits(n_col, coarse_g) + 31u) >> 5;
+    const uint32_t *coarse = reinterpret_cast<const uint32_t *>(x) + coarse_offset_words(n_col);
+    for (uint32_t w = threadIdx.x; w < words; w += blockDim.x) s_bits[w] = coarse[w];
+    __syncthreads();
+  } else if constexpr (BITS != 0) {
     const uint32_t words = (n_col + 31u) >> 5;
     for (uint32_t w = threadIdx.x; w < words; w += blockDim.x) s_bits[w] = pack_events32<VT>(x, w << 5, n_col);
     __syncthreads();
@@ -664,22 +715,22 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
   }
   // lanes per row from the mean row length
   const uint32_t mean = nnz / n_row;
-  if constexpr (MODE == kEvent && BITS == 2) {
+  if constexpr (MODE == kEvent && (BITS == 2 || BITS == 3)) {
     // An event bitmap above 80 KB leaves room for one workgroup (16 waves) per CU only: every lane
     // then keeps 16 (rows under 48 nonzeros: 8) loads in flight instead of 2 to 8, in groups of
     // 8 or 4 lanes per row, or HBM sees too few requests (1e6 columns, 100 per row: 424 -> 164 us).
-    if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, LDS_BITS, 8>(data, indices, indptr, x, y, n_row, s_bits);
-    else if (mean >= 48) gather_rows<F, VT, HETER, MODE, LDS_BITS, 8, 16>(data, indices, indptr, x, y, n_row, s_bits);
-    else gather_rows<F, VT, HETER, MODE, LDS_BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits);
+    if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    else if (mean >= 48) gather_rows<F, VT, HETER, MODE, BITS, 8, 16>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    else gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
   } else {
-    if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, LDS_BITS, 8>(data, indices, indptr, x, y, n_row, s_bits);
+    if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
     // (a dense vector is gathered from L2: for rows of 48 .. 191 nonzeros the pipelined 32-lane walk keeps more
     // of those gathers in flight than a wave per row does)
-    else if (mean >= (MODE == kDense ? 192u : 48u)) gather_rows_wave<F, VT, HETER, MODE, LDS_BITS, 2>(data, indices, indptr, x, y, n_row, s_bits);
-    else if (mean >= 48) gather_rows<F, VT, HETER, MODE, LDS_BITS, 32, 4>(data, indices, indptr, x, y, n_row, s_bits);
-    else if (mean >= 24) gather_rows<F, VT, HETER, MODE, LDS_BITS, 32, 2>(data, indices, indptr, x, y, n_row, s_bits);
-    else if (mean >= 12) gather_rows<F, VT, HETER, MODE, LDS_BITS, 16, 2>(data, indices, indptr, x, y, n_row, s_bits);
-    else gather_rows<F, VT, HETER, MODE, LDS_BITS, 8, 2>(data, indices, indptr, x, y, n_row, s_bits);
+    else if (mean >= (MODE == kDense ? 192u : 48u)) gather_rows_wave<F, VT, HETER, MODE, BITS, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    else if (mean >= 48) gather_rows<F, VT, HETER, MODE, BITS, 32, 4>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    else if (mean >= 24) gather_rows<F, VT, HETER, MODE, BITS, 32, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    else if (mean >= 12) gather_rows<F, VT, HETER, MODE, BITS, 16, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    else gather_rows<F, VT, HETER, MODE, BITS, 8, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
   }
 }
 
@@ -861,6 +912,27 @@ template <typename F, typename VT, bool HETER, int MODE>
 void launch_gather(const char *target, hipStream_t stream, const F *data, const uint32_t *indices,
                    const uint32_t *indptr, const VT *x, F *y, uint32_t n_row, uint32_t n_col) {
   if (n_row == 0) return;
+  if constexpr (MODE == kEvent && !std::is_same<VT, PackedBits>::value) {
+    // A bitmap that does not fit LDS (more than 1.3 million columns): two levels, the exact one in
+    // global memory and a coarse one (one bit per 2^g columns) for LDS, both built here.
+    if ((static_cast<size_t>(n_col) + 31) / 32 * 4 > kLdsBitmapCap) {
+      const uint32_t g = coarse_shift(n_col);
+      const uint32_t n_words = (n_col + 31u) / 32u, off = coarse_offset_words(n_col);
+      const uint32_t c_words = (coarse_bits(n_col, g) + 31u) / 32u;
+      uint32_t *bits = static_cast<uint32_t *>(
+          stream_workspace(stream, (static_cast<size_t>(off) + c_words + 1) * sizeof(uint32_t)));
+      if (bits != nullptr) {
+        pack_event_bitmap<VT>(stream, x, n_col, bits);
+        hipLaunchKernelGGL(coarsen_bitmap_kernel, dim3(div_up(c_words, 256)), dim3(256), 0, stream, bits, n_words, g,
+                           bits + off, c_words);
+        if (launch_gather_impl<F, PackedBits, HETER, MODE, 3>(target, stream, data, indices, indptr,
+                                                              reinterpret_cast<const PackedBits *>(bits), y, n_row,
+                                                              n_col, static_cast<size_t>(c_words) * 4))
+          return;
+      }
+      bpl_clear_error();
+    }
+  }
   if constexpr (MODE == kEvent && sizeof(VT) > 1 && !std::is_same<VT, PackedBits>::value) {
     // Wide event types: every persistent workgroup would read the whole vector (4 or 8 bytes per
     // element) to build its bitmap; pack it once instead and hand the words to the kernels.
@@ -876,7 +948,7 @@ void launch_gather(const char *target, hipStream_t stream, const F *data, const 
   }
   if (MODE == kEvent) {
     const size_t lds_bytes = (static_cast<size_t>(n_col) + 31) / 32 * 4;
-    const size_t lds_cap = static_cast<size_t>(160) * 1024 - 1024;
+    const size_t lds_cap = kLdsBitmapCap;
     if (lds_bytes <= lds_cap) {
       const bool ok = lds_bytes > 80 * 1024
                           ? launch_gather_impl<F, VT, HETER, MODE, 2>(target, stream, data, indices, indptr, x, y, n_row,
@@ -1197,7 +1269,7 @@ void event_csr_batching_entry(const char *target, hipStream_t stream, void **buf
     hipLaunchKernelGGL(pack_event_masks_kernel<VT>, dim3(div_up(d.n_col, 256), tiles), dim3(256), 0, stream, events,
                        masks, d.n_col, stride, d.batch_size, d.events_batch);
     const size_t lds_bytes = stride;
-    const size_t lds_cap = static_cast<size_t>(160) * 1024 - 1024;
+    const size_t lds_cap = kLdsBitmapCap;
     if (lds_bytes <= lds_cap &&
         launch_gather_batched_impl<F, HETER, true>(target, stream, values, indices, indptr, masks, out, d.n_row,
                                                    stride, d.batch_size, lds_bytes))

@@ -234,6 +234,34 @@ def test_gather_row_length_modes_with_a_bitmap_that_fills_lds(cuda, oracle_mod):
     assert_close(got, want)
 
 
+def test_gather_with_a_two_level_event_bitmap(cuda, oracle_mod):
+  # more columns than a bitmap in LDS can cover (1.3 million): a coarse bitmap (one bit per 2^g
+  # columns) in LDS and the exact one in global memory; g = 2, 4 and 6 (both ways the coarse
+  # bitmap is built), rows of all three length classes, bool and float events
+  rng = np.random.default_rng(15)
+  for n_col, n_row, mean in ((3_000_000, 20_000, 30), (3_000_000, 17_000, 450), (12_000_000, 3000, 120),
+                             (45_000_001, 2000, 60)):
+    counts = rng.poisson(mean, size=n_row)
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_row + mean)
+    data = rng.standard_normal(indices.shape[0]).astype(np.float32)
+    ev = rng.random(n_col) < 0.1
+    ev[indices[::3]] = True  # (make sure many nonzeros do hit)
+    shape = (n_row, n_col)
+    print("shape", shape, "mean", mean, flush=True)
+    want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape)
+    got = bpl.event_csr_matvec(data, indices, indptr, ev, shape=shape).cpu().numpy()
+    assert_close(got, want)
+    ones = np.ones(1, dtype=np.float32)
+    want = oracle_mod.event_csr_matvec(ones, indices, indptr, ev, shape=shape)
+    got = bpl.event_csr_matvec(ones, indices, indptr, ev, shape=shape).cpu().numpy()
+    assert np.array_equal(got, want)
+    if n_col <= 12_000_000:
+      evf = (ev * rng.uniform(0.5, 2.0, n_col)).astype(np.float32)
+      want = oracle_mod.event_csr_matvec(data, indices, indptr, evf, shape=shape)
+      got = bpl.event_csr_matvec(data, indices, indptr, evf, shape=shape).cpu().numpy()
+      assert_close(got, want)
+
+
 def test_config_event_csr_small(cuda, oracle_mod):
   # 4,000 x 4,000, 80 per row, homogeneous 0.6, events 2 %, transpose
   c = synth.config_event_csr_small()
