@@ -170,14 +170,16 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
   }
 }
 
-// grid = n_win * parts; workgroup (b, s) adds window b's pairs of producers [s * P / parts, ...).
+// grid = n_win * slices * parts; workgroup (b, q, s) adds window b's pairs of producers
+// [s * P / parts, ...) that fall into slice q of the window (slices = 2^(shift - lds_shift): a window
+// wider than the 2^lds_shift accumulators in LDS is added slice by slice, every slice reading the pairs).
 // Bin of (producer p, window b): derived from indptr as in bin_products_kernel, or, with
 // indptr == nullptr, the uniform layout pairs + (p * n_win + b) * uniform_cap.
 template <typename F>
 __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *__restrict__ indptr,
                                                                F *__restrict__ y, uint32_t n_row, uint32_t n_col,
                                                                uint32_t rows_per, uint32_t n_win, uint32_t shift,
-                                                               uint32_t parts,
+                                                               uint32_t lds_shift, uint32_t parts,
                                                                uint32_t producers,
                                                                const BinPair<F> *__restrict__ pairs,
                                                                uint64_t n_pairs,
@@ -189,9 +191,12 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
   double *window = reinterpret_cast<double *>(smem_raw);
   const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   constexpr uint32_t kWaves = kBinThreads / kWave;
-  const uint32_t b = blockIdx.x / parts, s = blockIdx.x % parts;
-  const uint32_t c0 = b << shift;
-  const uint32_t width = (n_col - c0 < (1u << shift)) ? n_col - c0 : (1u << shift);
+  const uint32_t slices = 1u << (shift - lds_shift);
+  const uint32_t b = blockIdx.x / (parts * slices), q = (blockIdx.x / parts) % slices, s = blockIdx.x % parts;
+  const uint32_t r0 = q << lds_shift;  // first column of the slice within the window
+  const uint32_t c0 = (b << shift) + r0;
+  if (c0 >= n_col) return;
+  const uint32_t width = (n_col - c0 < (1u << lds_shift)) ? n_col - c0 : (1u << lds_shift);
   for (uint32_t i = tid; i < width; i += kBinThreads) window[i] = 0.0;
   __syncthreads();
   const uint32_t p_lo = static_cast<uint32_t>(static_cast<uint64_t>(s) * producers / parts);
@@ -234,7 +239,7 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
         for (int u = 0; u < U; ++u) e[u] = bin[i0 + u * kWave + lane];
 #pragma unroll
         for (int u = 0; u < U; ++u)
-          if (e[u].rel < width) atomicAdd(&window[e[u].rel], static_cast<double>(e[u].val));
+          if (e[u].rel - r0 < width) atomicAdd(&window[e[u].rel - r0], static_cast<double>(e[u].val));  // (wraps below r0)
       }
       if (i0 < n) {
         BinPair<F> e[U];
@@ -247,7 +252,7 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
-          if (e[u].rel < width) atomicAdd(&window[e[u].rel], static_cast<double>(e[u].val));
+          if (e[u].rel - r0 < width) atomicAdd(&window[e[u].rel - r0], static_cast<double>(e[u].val));  // (wraps below r0)
       }
     }
   }
@@ -499,10 +504,9 @@ __global__ __launch_bounds__(kBinThreads) void add_window_runs_kernel(F *__restr
 // consumer workgroup adds a whole window to y, so small windows and few workgroups per window).
 // Up to 2^14 columns a window has its accumulators in LDS at once; wider ones (outputs above two
 // million columns) are added in slices of 2^14, each slice reading the window's pairs again.
-constexpr uint32_t kEventMaxShift = 17;
 inline uint32_t event_window_shift(uint32_t n_out) {
   uint32_t shift = 8;
-  while (shift < kEventMaxShift && (n_out >> shift) >= kMaxWindows) ++shift;
+  while (shift < kBinMaxShift && (n_out >> shift) >= kMaxWindows) ++shift;
   return shift;
 }
 
@@ -541,7 +545,7 @@ bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint
   uint32_t parts = num_cu / n_win;
   if (parts == 0) parts = 1;
   auto add_kernel = add_window_runs_kernel<F>;
-  const uint32_t lds_shift = shift < kBinMaxShift ? shift : kBinMaxShift;
+  const uint32_t lds_shift = bin_lds_shift(shift);
   const uint32_t slices = 1u << (shift - lds_shift);
   if (slices > 1) parts = 1;
   const size_t lds = sizeof(double) << lds_shift;
@@ -583,7 +587,9 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
   if (producers > div_up(n_row, 64)) producers = div_up(n_row, 64);
   const uint32_t rows_per = div_up(n_row, producers);
   producers = div_up(n_row, rows_per);
-  uint32_t parts = num_cu / n_win;
+  const uint32_t lds_shift = bin_lds_shift(shift);
+  const uint32_t slices = 1u << (shift - lds_shift);
+  uint32_t parts = num_cu / (n_win * slices);
   if (parts == 0) parts = 1;
   if (parts > producers) parts = producers;
 
@@ -600,7 +606,7 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
   uint32_t *counts = reinterpret_cast<uint32_t *>(ws + pair_bytes);
 
   auto add_kernel = add_bins_kernel<F>;
-  const size_t lds = sizeof(double) << shift;
+  const size_t lds = sizeof(double) << lds_shift;
   static thread_local bool attr_set = false;
   if (!attr_set && lds > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(add_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -617,8 +623,8 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
   else
     hipLaunchKernelGGL((bin_products_kernel<F, false>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
                        indptr, vec, y, n_row, rows_per, n_win, shift, pairs, static_cast<uint64_t>(n_pairs), counts);
-  hipLaunchKernelGGL(add_kernel, dim3(n_win * parts), dim3(kBinThreads), lds, stream, indptr, y, n_row, n_col, rows_per,
-                     n_win, shift, parts, producers, pairs, static_cast<uint64_t>(n_pairs), counts, 0u,
+  hipLaunchKernelGGL(add_kernel, dim3(n_win * slices * parts), dim3(kBinThreads), lds, stream, indptr, y, n_row, n_col,
+                     rows_per, n_win, shift, lds_shift, parts, producers, pairs, static_cast<uint64_t>(n_pairs), counts, 0u,
                      static_cast<uint32_t *>(nullptr));
   return check_launch(target);
 }
@@ -630,7 +636,9 @@ bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_o
                       uint32_t cap, const void *pairs, const uint32_t *counts, uint32_t *reset) {
   const uint32_t n_win = div_up(n_out, 1u << shift);
   auto add_kernel = add_bins_kernel<F>;
-  const size_t lds = sizeof(double) << shift;
+  const uint32_t lds_shift = bin_lds_shift(shift);
+  const uint32_t slices = 1u << (shift - lds_shift);
+  const size_t lds = sizeof(double) << lds_shift;
   static thread_local bool attr_set = false;
   if (!attr_set && lds > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(add_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -640,12 +648,12 @@ bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_o
     }
     attr_set = true;
   }
-  uint32_t parts = static_cast<uint32_t>(device_info().num_cu) / n_win;
+  uint32_t parts = static_cast<uint32_t>(device_info().num_cu) / (n_win * slices);
   if (parts == 0) parts = 1;
   if (parts > producers) parts = producers;
   const uint64_t n_pairs = static_cast<uint64_t>(producers) * n_win * cap;
-  hipLaunchKernelGGL(add_kernel, dim3(n_win * parts), dim3(kBinThreads), lds, stream,
-                     static_cast<const uint32_t *>(nullptr), y, 0u, n_out, 0u, n_win, shift, parts, producers,
+  hipLaunchKernelGGL(add_kernel, dim3(n_win * slices * parts), dim3(kBinThreads), lds, stream,
+                     static_cast<const uint32_t *>(nullptr), y, 0u, n_out, 0u, n_win, shift, lds_shift, parts, producers,
                      static_cast<const BinPair<F> *>(pairs), n_pairs, counts, cap, reset);
   return check_launch(target);
 }

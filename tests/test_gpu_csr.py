@@ -428,7 +428,9 @@ def test_transposed_csr_matvec_wide_output_sorted_scatter(cuda, oracle_mod, dtyp
   # rows, twice in a row, homogeneous weight.
   rng = np.random.default_rng(41)
   for n_row, n_col, mean, long_row in ((30_000, 300_000, 50, 0), (50_000, 400_000, 25, 250_000),
-                                       (1500, 2_000_000, 1000, 0), (200_000, 140_000, 8, 0)):
+                                       (1500, 2_000_000, 1000, 0), (200_000, 140_000, 8, 0),
+                                       # (above 2^21 columns: windows wider than their LDS accumulators, added in slices)
+                                       (4000, 5_000_001, 300, 0)):
     counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
     if long_row:
       counts[7] = long_row

@@ -343,6 +343,24 @@ def test_column_walk_through_bins_dense(cuda, oracle_mod, w_kind, a, b, dtype):
   assert abs(y @ Mx - MTy @ x64) <= 1e-9 * max(1.0, abs(y @ Mx))
 
 
+def test_column_walk_through_bins_sliced_windows(cuda, oracle_mod):
+  # more than 2^21 outputs: the bins' windows are wider than their accumulators in LDS and are
+  # added in slices
+  n_out, n_in = 3_000_001, 1_500
+  lp = oracle_mod.log_p_of(0.0004)
+  rng = np.random.default_rng(9)
+  x = rng.integers(-3, 4, n_in).astype(np.float32)
+  for w_kind, a, b in (("homo", 0.0, 0.0), ("uniform", 0.25, 1.75)):
+    got = kernel_call(x, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=5, n_row=n_out, n_col=n_in, col_walk=True, dense=True)
+    want = oracle_mod.jitconn_matvec(x, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=5, n_row=n_out, n_col=n_in,
+                                     col_walk=True, dense=True)
+    if w_kind == "homo":
+      assert np.array_equal(got, want)
+    else:
+      mag = np.full(n_out, 3.0 * (abs(a) + abs(b)) * 16)
+      assert_close_reordered(got, want, mag, np.float32, what="sliced binned column walk")
+
+
 def test_column_walk_through_bins_events_and_overflow(cuda, oracle_mod):
   # event input with n_in * n_out * p >= 5e7: bins sized for one active column in eight.  At 2 % activity
   # everything fits; with every column active most pairs overflow into direct atomics.  Counts are exact.
