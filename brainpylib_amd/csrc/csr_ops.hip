@@ -757,7 +757,7 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
   // Event input and an output wider than a few windows: the active rows' nonzeros are sorted
   // coarsely by output window instead (csr_bin_scatter.hip), at a cost that does not grow with
   // the number of windows.
-  if (MODE == kEvent && n_win > 1 && bin_event_scatter_usable<F>(n_col)) {
+  if (MODE == kEvent && n_col > 8192 && bin_event_scatter_usable<F>(n_col)) {
     const size_t list_sz = (static_cast<size_t>(n_row) * sizeof(uint2) + 255) / 256 * 256;
     unsigned char *ws =
         static_cast<unsigned char *>(stream_workspace(stream, list_sz + bin_event_scatter_bytes<F>(n_row, n_col)));
