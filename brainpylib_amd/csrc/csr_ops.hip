@@ -787,7 +787,10 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
     unsigned want_groups = static_cast<unsigned>(device_info().num_cu) / n_win;
     if (want_groups == 0) want_groups = 1;
     // small outputs: at most 16 row groups (their slices are summed by the second kernel)
-    if (static_cast<size_t>(n_col) * 16 <= 131072 && n_row <= 16 * kWinMaxRows && want_groups > 16) want_groups = 16;
+    // (dense input: every row is active and a wave walks its rows one after the other, so more groups)
+    const unsigned small_groups = MODE == kEvent ? 16 : 64;
+    if (static_cast<size_t>(n_col) * 16 <= 131072 && n_row <= 16 * kWinMaxRows && want_groups > small_groups)
+      want_groups = small_groups;
     uint32_t rows_per_wg = div_up(n_row, want_groups);
     if (rows_per_wg < 64) rows_per_wg = 64;
     // Large matrices: the active rows are first gathered into one list (a launch of its own) and
