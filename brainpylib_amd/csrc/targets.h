@@ -68,6 +68,14 @@
   X(gpu_matvec_atomic_prob_normal_v2_float) \
   X(gpu_matvec_atomic_prob_normal_v2_double)
 
+#define BPL_JITCONN_HASH_TARGETS(X) \
+  X(gpu_event_matvec_prob_homo_float) \
+  X(gpu_event_matvec_prob_homo_double) \
+  X(gpu_event_matvec_prob_uniform_float) \
+  X(gpu_event_matvec_prob_uniform_double) \
+  X(gpu_event_matvec_prob_normal_float) \
+  X(gpu_event_matvec_prob_normal_double)
+
 #define BPL_MATMAT_TARGETS(X) \
   X(gpu_matmat_prob_prob_normal_float_v1) \
   X(gpu_matmat_prob_prob_normal_double_v1) \
@@ -122,6 +130,7 @@
   BPL_EVENT_CSR_BATCHING_TARGETS(X) \
   BPL_CSR_TARGETS(X)        \
   BPL_JITCONN_TARGETS(X)    \
+  BPL_JITCONN_HASH_TARGETS(X) \
   BPL_MATMAT_TARGETS(X)     \
   BPL_NONZERO_TARGETS(X)    \
   BPL_COMPAT_TARGETS(X)

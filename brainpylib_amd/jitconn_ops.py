@@ -22,6 +22,7 @@ __all__ = [
   'event_matvec_prob_conn_normal_weight',
   'matvec_prob_conn_homo_weight', 'matvec_prob_conn_uniform_weight', 'matvec_prob_conn_normal_weight',
   'matmat_prob_conn_uniform_weight', 'matmat_prob_conn_normal_weight',
+  'event_matvec_prob_conn_hashed',
 ]
 
 
@@ -186,6 +187,41 @@ def _dense(vector):
   if vector.dtype not in FLOAT_DTYPES:
     raise TypeError(f'vector should be float32 or float64, got {vector.dtype}.')
   return vector
+
+
+def event_matvec_prob_conn_hashed(events, *, w_kind: str = 'homo', weight=1.0, w_low: float = 0.0,
+                                  w_high: float = 1.0, w_mu: float = 0.0, w_sigma: float = 1.0, conn_prob: float,
+                                  shape: Tuple[int, int], seed: int, transpose: bool = False,
+                                  dtype=torch.float32):
+  """``y = M @ events`` with the stateless connectivity of the reference's first GPU kernel
+  generation (targets ``gpu_event_matvec_prob_{homo,uniform,normal}_{float,double}``,
+  lib/gpu_jitconn_event_matvec.cu:10-79,138-215,281-362): synapse (row, col) exists iff a hash of
+  ``seed + n_col * row + col`` falls below ``conn_prob``.  The reference registers these targets
+  but none of its Python functions builds their names; this wrapper collects the event positions
+  with ``event_info`` and calls them.  A different matrix from ``event_matvec_prob_conn_*_weight``."""
+  from .event_ops import event_info
+  if w_kind not in ('homo', 'uniform', 'normal'):
+    raise ValueError(f'w_kind should be homo, uniform or normal, got {w_kind}.')
+  if dtype not in FLOAT_DTYPES:
+    raise TypeError(f'Only support float32 and float64. But we got {dtype}.')
+  events = as_tensor(events)
+  if events.ndim != 1:
+    raise ValueError('events should be a 1D vector.')
+  n_row, n_col = (shape[1], shape[0]) if transpose else (shape[0], shape[1])
+  if events.shape[0] != n_col:
+    raise ValueError(f'Shape mismatch, mat {(n_row, n_col)} @ vec ({events.shape[0]},).')
+  ids, num = event_info(events)
+  if w_kind == 'homo':
+    opaque = _lib.build_jitconn_prob_homo_descriptor(n_row, n_col, seed, float(conn_prob))
+  elif w_kind == 'uniform':
+    opaque = _lib.build_jitconn_prob_uniform_descriptor(n_row, n_col, seed, float(conn_prob), float(w_low),
+                                                        float(w_high) - float(w_low))
+  else:
+    opaque = _lib.build_jitconn_prob_normal_descriptor(n_row, n_col, seed, float(conn_prob), float(w_mu),
+                                                       float(w_sigma))
+  out = torch.empty(n_row, dtype=dtype, device=ids.device)
+  _lib.custom_call('gpu_event_matvec_prob_' + w_kind + _type_name(dtype), [ids, num, out], opaque)
+  return _apply_weight(out, weight) if w_kind == 'homo' else out
 
 
 def matvec_prob_conn_homo_weight(vector, weight, *, conn_prob: float, shape: Tuple[int, int],

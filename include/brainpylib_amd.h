@@ -366,6 +366,28 @@ BPL_TARGET(gpu_matvec_atomic_prob_normal_v2_float);
 BPL_TARGET(gpu_matvec_atomic_prob_normal_v2_double);
 
 /* ------------------------------------------------------------------------------------------
+ * jitconn event matvec, first kernel generation ("hash" connectivity)
+ *   (lib/gpu_jitconn_event_matvec.cu:10-79,138-215,281-362; names lib/gpu_ops.cc:107-112;
+ *   generators lib/kernel_helpers_random.cuh:12-71)
+ *   buffers = [event_ids (int32[n_col]: the positions of the events first, as nonzero_* lists
+ *              them), event_num (int32[1]), out (F[n_row])]
+ *   opaque = bpl_jitconn_prob_homo_descriptor (homo) or bpl_jitconn_prob_weight_descriptor
+ *            (uniform: w_a = low, w_b = high - low; normal: w_a = mean, w_b = stddev), with the
+ *            connection probability itself in the field `log_p` (the reference calls it `prob`)
+ *   Synapse (row, col) exists iff lfsr113(seed + n_col * row + col) * 2^-32 < prob in 32-bit
+ *   wrapping arithmetic (one step of LFSR113 from the state seed + {1, 7, 15, 127}); its weight
+ *   is 1, taus88 * w_b + w_a, or w_a + sqrt(-2 log u) cos(2 pi v) * w_b with u, v the first two
+ *   taus88 outputs from the state seed' + {1, 7, 15}.  out[row] adds the weights of the row's
+ *   synapses to the listed columns, in list order.  A different matrix from the _v2 targets'.
+ * ---------------------------------------------------------------------------------------- */
+BPL_TARGET(gpu_event_matvec_prob_homo_float);
+BPL_TARGET(gpu_event_matvec_prob_homo_double);
+BPL_TARGET(gpu_event_matvec_prob_uniform_float);
+BPL_TARGET(gpu_event_matvec_prob_uniform_double);
+BPL_TARGET(gpu_event_matvec_prob_normal_float);
+BPL_TARGET(gpu_event_matvec_prob_normal_double);
+
+/* ------------------------------------------------------------------------------------------
  * jitconn matmat: Y[m,n] = X[m,k] @ M[k,n], row-major X and Y, M regenerated on the fly
  *   (lib/gpu_jitconn_matmat.cu:279-317,364-455; names lib/gpu_ops.cc:161-174)
  *   buffers = [X (F[m*k]), Y (F[m*n])],  opaque = bpl_matmat_jit_prob_descriptor

@@ -28,6 +28,10 @@ event_csr_matvec                dense matmul brute force, scipy.sparse, homo == 
                                 bool events)
 csr_matvec                      dense matmul brute force, scipy.sparse (both orientations)
 event_info                      numpy.flatnonzero
+event_matvec_hash, lfsr113,     the reference holds this algorithm as CUDA only.  Maximal period
+taus88                          of every component recurrence (2^31-1, 2^29-1, 2^28-1, 2^25-1:
+                                no wrong shift or mask constant survives that), GF(2)-linearity,
+                                synapse fraction and weight moments, closed forms at prob 0 / 1
 ==============================  ==============================================================
 """
 import ctypes
@@ -61,6 +65,9 @@ def lib():
     _lib.oracle_jitconn_stream_weights_f32.restype = ctypes.c_uint32
     _lib.oracle_jitconn_stream_weights_f64.restype = ctypes.c_uint32
     _lib.oracle_get_threads.restype = ctypes.c_int
+    _lib.oracle_lfsr_component_step.restype = ctypes.c_uint32
+    _lib.oracle_lfsr_component_period.restype = ctypes.c_uint64
+    _lib.oracle_lfsr113_word.restype = ctypes.c_uint32
   return _lib
 
 
@@ -301,3 +308,38 @@ def event_info(events):
   lib().oracle_event_info(_p(buf), ctypes.c_int(_EVENT_KINDS[events.dtype]),
                           ctypes.c_uint32(events.shape[0]), _p(ids), _p(num))
   return ids, num
+
+
+# ---- stateless ("hash") jitconn event matvec: lib/gpu_jitconn_event_matvec.cu:10-51,138-183,281-331 ----
+def lfsr_component_step(gen, comp, z):
+  """One step of component ``comp`` of taus88 (gen 0) or LFSR113 (gen 1)."""
+  return int(lib().oracle_lfsr_component_step(ctypes.c_int(gen), ctypes.c_int(comp), ctypes.c_uint32(z)))
+
+
+def lfsr_component_period(gen, comp, start, limit):
+  return int(lib().oracle_lfsr_component_period(ctypes.c_int(gen), ctypes.c_int(comp), ctypes.c_uint32(start),
+                                                ctypes.c_uint64(limit)))
+
+
+def lfsr113_word(seed):
+  """lfsr113_double(seed) * 2^32 (lib/kernel_helpers_random.cuh:55-71)."""
+  return int(lib().oracle_lfsr113_word(ctypes.c_uint32(seed & 0xffffffff)))
+
+
+def taus88_words(seed, n=2):
+  out = (ctypes.c_uint32 * 2)()
+  lib().oracle_taus88_words(ctypes.c_uint32(seed & 0xffffffff), ctypes.c_int(n), out)
+  return [int(out[i]) for i in range(n)]
+
+
+def event_matvec_hash(event_ids, event_num, *, w_kind="homo", w_a=0.0, w_b=0.0, prob, seed, n_row, n_col,
+                      dtype=np.float32):
+  """out[row] = sum over the first ``event_num`` listed columns c with
+  lfsr113(seed + n_col * row + c) * 2^-32 < prob of the synapse's weight."""
+  ids = _c(event_ids, np.int32)
+  out = np.empty(n_row, dtype=dtype)
+  fn = lib().oracle_event_matvec_hash_f32 if np.dtype(dtype) == np.float32 else lib().oracle_event_matvec_hash_f64
+  fn(_p(ids), ctypes.c_int32(int(event_num)), ctypes.c_uint32(seed & 0xffffffff), ctypes.c_double(prob),
+     ctypes.c_int(_W_KINDS[w_kind]), ctypes.c_double(w_a), ctypes.c_double(w_b), ctypes.c_uint32(n_row),
+     ctypes.c_uint32(n_col), _p(out))
+  return out

@@ -19,6 +19,7 @@
  * Parity status of every exported function is listed in oracle/__init__.py next to its
  * Python binding.
  */
+#define _GNU_SOURCE /* M_PI */
 #include <math.h>
 #include <stdint.h>
 #include <stdlib.h>
@@ -251,6 +252,8 @@ ORACLE_API uint32_t oracle_jitconn_stream_indices(uint32_t seed, double log_p, u
 #include "csr_body.inc"
 #undef T1
 #undef T1SUF
+
+#include "hash_body.inc"
 
 /* ------------------------------------------------------------------------------------------ */
 /* event_info: ordered compaction of the nonzero positions, padded with -1, plus the count     */
