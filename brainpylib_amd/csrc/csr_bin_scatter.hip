@@ -1,6 +1,7 @@
-// Transposed CSR matrix times dense vector for wide outputs: y[c] = sum_j v[row(j)] * data[j]
-// over the nonzeros j of column c, when every row contributes and the output (hundreds of
-// thousands of columns or more) is far larger than LDS.  One random global atomic per nonzero
+// Transposed CSR matrix times vector through coarse sorting: y[c] = sum_j v[row(j)] * data[j] over
+// the nonzeros j of column c.  First half of the file: dense vector, every row contributes, output
+// (hundreds of thousands of columns or more) far larger than LDS.  Second half: event vector, only
+// the listed active rows contribute (from 8,192 columns).  One random global atomic per nonzero
 // retires at about 21 G/s on this device; instead the products are first sorted coarsely:
 //
 //   bin kernel     persistent producer workgroups walk their rows, form (column, product)

@@ -748,18 +748,18 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
     fill_zero(stream, y, n_col);
     return;
   }
-  // Output windows in LDS.  Every window's workgroup streams the column indices of the active
-  // rows again, which is still far cheaper than one random global atomic per nonzero (about
-  // 21 G/s) up to a few dozen windows when the activity is sparse (event input) and the rows are
-  // long.  With a dense input every row is active and only a handful of windows pay off.
+  // Output windows in LDS (the path for narrow outputs, and the fallback of the event input when
+  // the sorted scatter below has no scratch memory).  Every window's workgroup streams the column
+  // indices of the active rows again, which is still far cheaper than one random global atomic per
+  // nonzero (about 21 G/s) for a few windows; a wave walks its rows one after the other.
   using A = typename std::conditional<MODE == kDense, double, F>::type;  // window accumulators
   const size_t list_bytes = kWinMaxRows * (8 + (MODE == kDense ? sizeof(F) : 0));
   const uint32_t win_cap = static_cast<uint32_t>((static_cast<size_t>(128) * 1024) / sizeof(A));
   const uint32_t n_win = div_up(n_col, win_cap);
   NnzGate direct_gate = kAlways;
-  // Event input and an output wider than a few windows: the active rows' nonzeros are sorted
-  // coarsely by output window instead (csr_bin_scatter.hip), at a cost that does not grow with
-  // the number of windows.
+  // Event input and more than 8,192 outputs: the active rows' nonzeros are flattened and sorted
+  // coarsely by output window instead (csr_bin_scatter.hip), at a cost that neither grows with the
+  // number of windows nor with the number of rows a wave would have to walk in turn.
   if (MODE == kEvent && n_col > 8192 && bin_event_scatter_usable<F>(n_col)) {
     const size_t list_sz = (static_cast<size_t>(n_row) * sizeof(uint2) + 255) / 256 * 256;
     unsigned char *ws =
