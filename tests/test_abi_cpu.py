@@ -51,6 +51,42 @@ def test_reference_target_names_present():
         assert "csr_matvec_%s_%s_%s" % (data, m, t) in names
 
 
+def test_reference_registry_keys_of_the_other_operators_present():
+  # lib/gpu_ops.cc:27-58 (the older event / atomic sums), :72-174 (jitconn, matmat, nonzero)
+  names = set(_lib.target_names())
+  want = []
+  for w in ("homo", "uniform", "normal"):
+    for t in ("float_bool", "float_float", "double_bool", "double_double"):
+      want += ["gpu_event_matvec_prob_%s_v2_%s" % (w, t), "gpu_event_matvec_atomic_prob_%s_v2_%s" % (w, t)]
+    for t in ("float", "double"):
+      want += ["gpu_matvec_prob_%s_v2_%s" % (w, t), "gpu_matvec_atomic_prob_%s_v2_%s" % (w, t),
+               "gpu_event_matvec_prob_%s_%s" % (w, t)]  # (the last: first-generation event kernels)
+  for w in ("normal", "uniform"):
+    for t in ("float", "double"):
+      want.append("gpu_matmat_prob_prob_%s_%s_v1" % (w, t))
+  want += ["nonzero_" + t for t in ("bool", "int", "long", "float", "double")]
+  for op in ("gpu_csr_event_sum", "gpu_coo_event_sum", "gpu_coo_atomic_sum"):
+    for data in ("homo", "heter"):
+      for f in ("f32", "f64"):
+        for i in ("i32", "i64"):
+          want.append("%s_%s_%s_%s" % (op, data, f, i))
+  missing = [n for n in want if n not in names]
+  assert not missing, missing
+  assert len(want) == 36 + 6 + 4 + 5 + 24
+
+
+@pytest.mark.parametrize("name", sorted(_lib.target_names()))
+def test_every_target_refuses_a_malformed_call(name):
+  # wrong opaque size, then a null buffer table: the call returns, launches nothing, records an error
+  lib = _lib.lib()
+  fn = _lib.target(name)
+  bufs = (ctypes.c_void_p * 8)()
+  lib.bpl_clear_error()
+  fn(None, bufs, b"\x00" * 3, 3)
+  assert "invalid opaque object size" in _lib.last_error()
+  lib.bpl_clear_error()
+
+
 def test_descriptor_layouts():
   # lib/kernel_helper_descriptor.cuh: native alignment, little endian
   assert _lib.build_twouint_onebool_descriptor(3, 4, True) == struct.pack("<IIB3x", 3, 4, 1)
