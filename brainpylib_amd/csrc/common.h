@@ -228,9 +228,9 @@ __global__ __launch_bounds__(256) void pack_event_bitmap_kernel(const VT *__rest
 // at the exact one, in global memory, only where the coarse bit is set.
 constexpr uint32_t kLdsBitmapCap = 160u * 1024u - 1024u;
 __host__ __device__ inline uint32_t coarse_bits(uint32_t n, uint32_t g) { return n ? ((n - 1u) >> g) + 1u : 0u; }
-__host__ __device__ inline uint32_t coarse_shift(uint32_t n) {
+__host__ __device__ inline uint32_t coarse_shift(uint32_t n, uint32_t cap_bytes = kLdsBitmapCap) {
   uint32_t g = 0;
-  while ((coarse_bits(n, g) + 31u) / 32u * 4u > kLdsBitmapCap) ++g;
+  while ((coarse_bits(n, g) + 31u) / 32u * 4u > cap_bytes) ++g;
   return g;
 }
 __host__ __device__ inline uint32_t coarse_offset_words(uint32_t n) { return ((n + 31u) / 32u + 63u) / 64u * 64u; }

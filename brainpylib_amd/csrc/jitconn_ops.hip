@@ -30,7 +30,15 @@ namespace bpl {
 namespace {
 
 // ---- row walk -------------------------------------------------------------------------------------
-template <typename T1, typename VT, int IN, int W, bool LDS_BITS>
+// LDS the row walk gives to an event bitmap when it wants two 16-wave workgroups per CU (each wave
+// can issue one instruction every four cycles, so the number of resident waves bounds the VALU
+// utilisation: 32 waves per CU walk 290 G synapses/s, the 15 that fit beside a 125 KB bitmap 228).
+constexpr uint32_t kRowwalkCoarseBytes = 38912;
+
+// BITS: where the event probes go.  0: the event vector in global memory; 1: its bitmap in LDS;
+// 2: a coarse bitmap in LDS (one bit per 2^g inputs, at most kRowwalkCoarseBytes) and, where its
+// bit is set, the exact packed bitmap in global memory (`in`, the coarse one behind it).
+template <typename T1, typename VT, int IN, int W, int BITS>
 __global__ __launch_bounds__(1024) void jitconn_rowwalk_kernel(const VT *__restrict__ in, T1 *__restrict__ out,
                                                                uint32_t n_out, uint32_t n_in, uint32_t seed,
                                                                double log_p, T1 wa, T1 wb, uint32_t first,
@@ -44,7 +52,15 @@ __global__ __launch_bounds__(1024) void jitconn_rowwalk_kernel(const VT *__restr
   constexpr int kWords = StreamLds<T1, W>::words;
   uint32_t *st = smem + wave * kWords;
   const uint32_t *bits = smem + nwaves * kWords;
-  if (LDS_BITS) {
+  uint32_t coarse_g = 0;
+  if constexpr (BITS == 2) {
+    uint32_t *wbits = smem + nwaves * kWords;
+    coarse_g = coarse_shift(n_in, kRowwalkCoarseBytes);
+    const uint32_t words = (coarse_bits(n_in, coarse_g) + 31u) >> 5;
+    const uint32_t *coarse = reinterpret_cast<const uint32_t *>(in) + coarse_offset_words(n_in);
+    for (uint32_t i = threadIdx.x; i < words; i += blockDim.x) wbits[i] = coarse[i];
+    __syncthreads();
+  } else if constexpr (BITS == 1) {
     uint32_t *wbits = smem + nwaves * kWords;
     const uint32_t words = (n_in + 31u) >> 5;
     for (uint32_t i = threadIdx.x; i < words; i += blockDim.x) wbits[i] = pack_events32<VT>(in, i << 5, n_in);
@@ -55,7 +71,31 @@ __global__ __launch_bounds__(1024) void jitconn_rowwalk_kernel(const VT *__restr
     const uint32_t *pre = states ? states + static_cast<size_t>(i) * kMtN : nullptr;
     double acc = 0.0;
     uint32_t cnt = 0;
+    // two-level bitmap: the exact word of a batch is requested when the batch is drawn and looked
+    // at when the next one is, so that no wave waits for it
+    uint32_t late_word = 0, late_bit = 0;
+    bool late_coarse = false;
+    T1 late_w = T1(0);
+    auto settle = [&]() {
+      const bool hit = late_coarse && ((late_word >> late_bit) & 1u);
+      if (W == kHomo) cnt += static_cast<uint32_t>(__popcll(__ballot(hit)));
+      else if (hit) acc += static_cast<double>(late_w);
+    };
     walk_stream<T1, W>(st, lane, seed + o, pre, n_in, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
+      if constexpr (IN == kInEvent && BITS == 2) {
+        settle();
+        bool coarse = false;
+        if (valid) {
+          const uint32_t c = idx >> coarse_g;
+          coarse = (bits[c >> 5] >> (c & 31u)) & 1u;
+        }
+        // (lanes without a coarse hit read word 0 and ignore it: a plain load for the whole wave)
+        late_word = reinterpret_cast<const uint32_t *>(in)[coarse ? idx >> 5 : 0u];
+        late_bit = idx & 31u;
+        late_coarse = coarse;
+        late_w = w;
+        return;
+      }
       if (IN == kInDense) {
         if (valid) {
           const T1 v = static_cast<T1>(in[idx]);
@@ -64,13 +104,14 @@ __global__ __launch_bounds__(1024) void jitconn_rowwalk_kernel(const VT *__restr
       } else {
         bool hit = false;
         if (valid) {
-          if (LDS_BITS) hit = (bits[idx >> 5] >> (idx & 31u)) & 1u;
+          if (BITS == 1) hit = (bits[idx >> 5] >> (idx & 31u)) & 1u;
           else hit = probe_event(in, idx);
         }
         if (W == kHomo) cnt += static_cast<uint32_t>(__popcll(__ballot(hit)));
         else if (hit) acc += static_cast<double>(w);
       }
     });
+    if constexpr (IN == kInEvent && BITS == 2) settle();
     if (IN == kInEvent && W == kHomo) {
       if (lane == 0) out[o] = static_cast<T1>(cnt);
     } else {
@@ -301,10 +342,10 @@ bool valid_log_p(const char *target, double log_p) {
   return true;
 }
 
-template <typename T1, typename VT, int IN, int W, bool LDS_BITS>
+template <typename T1, typename VT, int IN, int W, int BITS>
 void launch_rowwalk_impl(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, uint32_t n_in, uint32_t seed,
                          double log_p, T1 wa, T1 wb, int nwaves, size_t lds_bytes) {
-  auto kernel = jitconn_rowwalk_kernel<T1, VT, IN, W, LDS_BITS>;
+  auto kernel = jitconn_rowwalk_kernel<T1, VT, IN, W, BITS>;
   const int block = nwaves * kWave;
   struct Cached {
     size_t lds_bytes;
@@ -346,6 +387,30 @@ template <typename T1, typename VT, int IN, int W>
 void launch_rowwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, uint32_t n_in, uint32_t seed,
                     double log_p, T1 wa, T1 wb) {
   if (n_out == 0) return;
+  if constexpr (IN == kInEvent && !std::is_same<VT, PackedBits>::value) {
+    // An event bitmap that would leave room for fewer than two 16-wave workgroups per CU: two
+    // levels instead, the exact bitmap packed into global memory and a coarse one made for LDS.
+    if ((static_cast<size_t>(n_in) + 31) / 32 * 4 > kRowwalkCoarseBytes) {
+      const size_t state_ws = (n_out >= kSeedAheadMin) ? static_cast<size_t>(kSeedChunk) * kMtN * 4 : 0;
+      const uint32_t g = coarse_shift(n_in, kRowwalkCoarseBytes);
+      const uint32_t n_words = (n_in + 31u) / 32u, off = coarse_offset_words(n_in);
+      const uint32_t c_words = (coarse_bits(n_in, g) + 31u) / 32u;
+      unsigned char *ws = static_cast<unsigned char *>(
+          stream_workspace(stream, state_ws + (static_cast<size_t>(off) + c_words + 1) * sizeof(uint32_t)));
+      if (ws != nullptr) {
+        uint32_t *bits = reinterpret_cast<uint32_t *>(ws + state_ws);
+        pack_event_bitmap<VT>(stream, in, n_in, bits);
+        hipLaunchKernelGGL(coarsen_bitmap_kernel, dim3(div_up(c_words, 256)), dim3(256), 0, stream, bits, n_words, g,
+                           bits + off, c_words);
+        const size_t state_bytes = StreamLds<T1, W>::words * 4;
+        launch_rowwalk_impl<T1, PackedBits, IN, W, 2>(stream, reinterpret_cast<const PackedBits *>(bits), out, n_out, n_in,
+                                                      seed, log_p, wa, wb, 16,
+                                                      static_cast<size_t>(c_words) * 4 + 16 * state_bytes);
+        return;
+      }
+      bpl_clear_error();
+    }
+  }
   if constexpr (IN == kInEvent && sizeof(VT) > 1 && !std::is_same<VT, PackedBits>::value) {
     // Wide event types: pack the vector to one bit per element once, instead of once per workgroup.
     // (The seeded generator states of large walks share the scratch buffer: the bitmap lies behind them.)
@@ -374,12 +439,12 @@ void launch_rowwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
         nw = static_cast<int>((cap - bitmap) / state_bytes);
         if (nw > 16) nw = 16;
       }
-      launch_rowwalk_impl<T1, VT, IN, W, true>(stream, in, out, n_out, n_in, seed, log_p, wa, wb, nw,
-                                               bitmap + nw * state_bytes);
+      launch_rowwalk_impl<T1, VT, IN, W, 1>(stream, in, out, n_out, n_in, seed, log_p, wa, wb, nw,
+                                            bitmap + nw * state_bytes);
       return;
     }
   }
-  launch_rowwalk_impl<T1, VT, IN, W, false>(stream, in, out, n_out, n_in, seed, log_p, wa, wb, 8, 8 * state_bytes);
+  launch_rowwalk_impl<T1, VT, IN, W, 0>(stream, in, out, n_out, n_in, seed, log_p, wa, wb, 8, 8 * state_bytes);
 }
 
 template <typename T1, typename VT, int IN, int W>

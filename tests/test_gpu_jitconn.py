@@ -108,6 +108,28 @@ def test_index_sets_bit_exact_via_integer_probes(cuda, oracle_mod, shape, p):
       assert np.array_equal(got, want), (shape, p, col_walk)
 
 
+@pytest.mark.parametrize("n_in", [320_000, 1_500_000, 5_000_000])
+def test_row_walk_with_a_two_level_event_bitmap(cuda, oracle_mod, n_in):
+  # more inputs than the 38 KB of LDS the row walk gives to a bitmap cover (311,296): a coarse
+  # bitmap in LDS (one bit per 2, 8 and 32 inputs here) and the exact one in global memory, whose
+  # word is looked at one batch late.  Bool and float events, all weight kinds; counts exact.
+  n_out = 300
+  rng = np.random.default_rng(n_in)
+  ev = rng.random(n_in) < 0.02
+  lp = oracle_mod.log_p_of(2000.0 / n_in)
+  for inp in (ev, (ev * rng.uniform(0.5, 2.0, n_in)).astype(np.float32)):
+    dense = None if inp.dtype == np.bool_ else False
+    want = oracle_mod.jitconn_matvec(inp, log_p=lp, seed=77, n_row=n_out, n_col=n_in, dense=dense)
+    got = kernel_call(inp, w_kind="homo", log_p=lp, seed=77, n_row=n_out, n_col=n_in, col_walk=False, dense=False)
+    assert want.sum() > 0 and np.array_equal(got, want)
+  for w_kind, a, b in (("uniform", 0.25, 1.75), ("normal", 0.5, 2.0)):
+    want = oracle_mod.jitconn_matvec(ev, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=77, n_row=n_out, n_col=n_in)
+    got = kernel_call(ev, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=77, n_row=n_out, n_col=n_in, col_walk=False,
+                      dense=False)
+    mag = np.full(n_out, (abs(a) + 5 * abs(b)) * 80)  # about 40 active synapses per row
+    assert_close_reordered(got, want, mag, np.float32, what="two-level row walk %s" % w_kind)
+
+
 def test_full_matrix_recovered_by_one_hot_events(cuda, oracle_mod):
   # every entry of a 100 x 200 implicit matrix, both walks, against the per-stream oracle's index lists
   n_row, n_col, seed = 100, 200, 77
