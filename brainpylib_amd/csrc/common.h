@@ -65,6 +65,9 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
 // active_count[0]; `scratch` is device memory of bin_event_scatter_bytes() bytes whose first
 // kBinEventFillBytes are zero; y is zeroed.  Enqueues the two kernels; the second one sets
 // active_count[0] back to zero.  false (nothing enqueued) if it cannot run.
+// Batched calls (several event vectors, one matrix) hand in one list over all batch entries, n_col
+// = batch * columns, and `active_colbase` = what to add to the columns of each listed row (its
+// batch entry * columns); n_row stays the matrix's row count (indptr has n_row + 1 entries).
 constexpr size_t kBinEventFillBytes = 131072;
 template <typename F>
 bool bin_event_scatter_usable(uint32_t n_col);
@@ -73,7 +76,7 @@ size_t bin_event_scatter_bytes(uint32_t n_row, uint32_t n_col);
 template <typename F>
 bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint32_t *indices, const uint32_t *indptr,
                        F *y, uint32_t n_row, uint32_t n_col, uint32_t *active_count, const uint2 *active_list,
-                       void *scratch);
+                       void *scratch, const uint32_t *active_colbase = nullptr);
 
 // Second half of the coarse-sorted scatter for producers other than the CSR one: adds bins laid
 // out uniformly, bin (p, b) = pairs + (p * n_win + b) * cap with counts[b * producers + p]

@@ -287,9 +287,11 @@ template <typename F, bool HETER>
 __global__ __launch_bounds__(kBinThreads) void bin_active_rows_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
     uint32_t n_row, const uint32_t *__restrict__ active_count, const uint2 *__restrict__ active_list,
-    F *__restrict__ y, uint32_t shift, uint32_t cap, BinPair<F> *__restrict__ pairs, uint32_t *__restrict__ fill) {
+    const uint32_t *__restrict__ active_colbase, F *__restrict__ y, uint32_t shift, uint32_t cap,
+    BinPair<F> *__restrict__ pairs, uint32_t *__restrict__ fill) {
   __shared__ uint32_t s_ptr[kTileRows + 1];     // nonzeros of the tile's rows before row k
   __shared__ uint32_t s_start[kTileRows];       // first nonzero of row k in the matrix
+  __shared__ uint32_t s_colbase[kTileRows];     // added to row k's columns (batched calls: batch entry * n_col)
   __shared__ uint32_t s_hint[kBinThreads + 1];
   __shared__ uint32_t s_cnt[kMaxWindows];
   __shared__ uint32_t s_off[kMaxWindows + 1];
@@ -332,7 +334,10 @@ __global__ __launch_bounds__(kBinThreads) void bin_active_rows_kernel(
     __syncthreads();
     uint32_t before = 0;
     for (uint32_t w = 0; w < wave; ++w) before += s_wave[w];
-    if (tid < rows) s_ptr[tid] = before + incl - e.y, s_start[tid] = e.x;
+    if (tid < rows) {
+      s_ptr[tid] = before + incl - e.y, s_start[tid] = e.x;
+      s_colbase[tid] = active_colbase ? active_colbase[t0 + tid] : 0u;
+    }
     if (tid == rows - 1u) s_ptr[rows] = before + incl;
     __syncthreads();
     const uint32_t j1 = s_ptr[rows];  // the tile's nonzeros, numbered from 0 (listed rows are never empty)
@@ -357,7 +362,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_active_rows_kernel(
             const uint32_t q = (j - seg) >> kHintShift;
             const uint32_t k = row_of(j, s_hint[q], s_hint[q + 1]);
             const uint32_t at = s_start[k] + (j - s_ptr[k]);
-            col[u] = indices[at];
+            col[u] = indices[at] + s_colbase[k];
             val[u] = HETER ? data[at] : w_homo;
           }
         }
@@ -540,7 +545,7 @@ size_t bin_event_scatter_bytes(uint32_t n_row, uint32_t n_col) {
 template <typename F>
 bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint32_t *indices, const uint32_t *indptr,
                        F *y, uint32_t n_row, uint32_t n_col, uint32_t *active_count, const uint2 *active_list,
-                       void *scratch) {
+                       void *scratch, const uint32_t *active_colbase) {
   const uint32_t shift = event_window_shift(n_col);
   const uint32_t n_win = div_up(n_col, 1u << shift);
   const uint32_t cap = static_cast<uint32_t>(event_run_pairs(n_row, n_col) / (n_win * kSubRuns));
@@ -566,10 +571,10 @@ bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint
   const uint32_t producers = 2u * num_cu;
   if (heter)
     hipLaunchKernelGGL((bin_active_rows_kernel<F, true>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
-                       indptr, n_row, active_count, active_list, y, shift, cap, pairs, fill);
+                       indptr, n_row, active_count, active_list, active_colbase, y, shift, cap, pairs, fill);
   else
     hipLaunchKernelGGL((bin_active_rows_kernel<F, false>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
-                       indptr, n_row, active_count, active_list, y, shift, cap, pairs, fill);
+                       indptr, n_row, active_count, active_list, active_colbase, y, shift, cap, pairs, fill);
   hipLaunchKernelGGL(add_kernel, dim3(n_win * slices * parts), dim3(kBinThreads), lds, stream, y, n_col, shift,
                      lds_shift, parts, cap, pairs, fill, active_count);
   return true;
@@ -673,9 +678,9 @@ template bool bin_event_scatter_usable<double>(uint32_t);
 template size_t bin_event_scatter_bytes<float>(uint32_t, uint32_t);
 template size_t bin_event_scatter_bytes<double>(uint32_t, uint32_t);
 template bool bin_event_scatter<float>(hipStream_t, const float *, bool, const uint32_t *, const uint32_t *, float *, uint32_t,
-                                       uint32_t, uint32_t *, const uint2 *, void *);
+                                       uint32_t, uint32_t *, const uint2 *, void *, const uint32_t *);
 template bool bin_event_scatter<double>(hipStream_t, const double *, bool, const uint32_t *, const uint32_t *, double *,
-                                        uint32_t, uint32_t, uint32_t *, const uint2 *, void *);
+                                        uint32_t, uint32_t, uint32_t *, const uint2 *, void *, const uint32_t *);
 template bool bin_scatter_usable<float>(uint32_t, uint32_t);
 template bool bin_scatter_usable<double>(uint32_t, uint32_t);
 template bool bin_scatter<float>(const char *, hipStream_t, const float *, bool, const uint32_t *, const uint32_t *,

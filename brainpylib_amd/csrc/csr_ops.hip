@@ -233,6 +233,67 @@ void launch_collect(hipStream_t stream, const uint32_t *indptr, const VT *x, uin
                        n_row, counter, list, scales, gate, clear, n_clear, zero, n_zero);
 }
 
+// The same list over the rows of every entry of a batch of event vectors that share one matrix:
+// virtual row v = entry * n_row + r; `colbase` receives entry * n_col for every listed row.
+// events: [events_batch][n_row]; entry bi of this launch is entry first_entry + bi of the whole
+// batch and reads row (first_entry + bi) % events_batch.
+template <typename F, typename VT>
+__global__ __launch_bounds__(kWinThreads) void collect_active_rows_batched_kernel(
+    const uint32_t *__restrict__ indptr, const VT *__restrict__ events, uint32_t n_row, uint32_t n_col,
+    uint32_t batch, uint32_t events_batch, uint32_t first_entry, uint32_t *__restrict__ counter,
+    uint2 *__restrict__ list,
+    uint32_t *__restrict__ colbase, uint32_t *__restrict__ clear, uint32_t n_clear, F *__restrict__ zero,
+    uint64_t n_zero) {
+  constexpr int kPer = 8;
+  __shared__ uint32_t s_count, s_base;
+  const uint32_t tid = threadIdx.x, lane = tid % kWave;
+  if (tid == 0) s_count = 0;
+  for (uint32_t i = blockIdx.x * kWinThreads + tid; i < n_clear; i += gridDim.x * kWinThreads) clear[i] = 0u;
+  for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kWinThreads + tid; i < n_zero;
+       i += static_cast<uint64_t>(gridDim.x) * kWinThreads)
+    zero[i] = F(0);
+  __syncthreads();
+  const uint64_t total = static_cast<uint64_t>(batch) * n_row;
+  const uint64_t v0 = static_cast<uint64_t>(blockIdx.x) * (kWinThreads * kPer) + tid;
+  bool on[kPer];
+  uint32_t start[kPer], len[kPer], at[kPer], base_col[kPer];
+#pragma unroll
+  for (int e = 0; e < kPer; ++e) {
+    const uint64_t v = v0 + static_cast<uint64_t>(e) * kWinThreads;
+    on[e] = false;
+    start[e] = len[e] = at[e] = base_col[e] = 0;
+    if (v < total) {
+      const uint32_t bi = static_cast<uint32_t>(v / n_row), r = static_cast<uint32_t>(v % n_row);
+      on[e] = is_event(events[static_cast<size_t>((first_entry + bi) % events_batch) * n_row + r]);
+      if (on[e]) {
+        start[e] = indptr[r];
+        len[e] = indptr[r + 1] - start[e];
+        on[e] = len[e] != 0;
+        base_col[e] = bi * n_col;
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < kPer; ++e) {
+    const uint64_t mask = __ballot(on[e]);
+    uint32_t base = 0;
+    if (lane == 0 && mask) base = atomicAdd(&s_count, static_cast<uint32_t>(__popcll(mask)));
+    base = __builtin_amdgcn_readfirstlane(base);
+    at[e] = base + static_cast<uint32_t>(__popcll(mask & ((1ull << lane) - 1ull)));
+  }
+  __syncthreads();
+  if (tid == 0) s_base = s_count ? atomicAdd(counter, s_count) : 0u;
+  __syncthreads();
+  const uint32_t base = s_base;
+#pragma unroll
+  for (int e = 0; e < kPer; ++e) {
+    if (on[e]) {
+      list[base + at[e]] = make_uint2(start[e], len[e]);
+      colbase[base + at[e]] = base_col[e];
+    }
+  }
+}
+
 // Row groups that take part in a launch whose active rows are listed in device memory: one per
 // 32,768 active nonzeros (estimated from the mean row length), at least one, at most the launched
 // number.  Every group writes a slice of partial outputs that the summing kernel reads again, so
@@ -1284,6 +1345,50 @@ void event_csr_batching_entry(const char *target, hipStream_t stream, void **buf
     launch_gather_batched_impl<F, HETER, false>(target, stream, values, indices, indptr, masks, out, d.n_row, stride,
                                                 d.batch_size, 0);
     return;
+  }
+  // Transposed, one matrix for all entries: groups of up to 8 entries go through ONE sorted scatter
+  // over a virtual output of group * n_col columns (entry g's columns shifted by g * n_col), fed by
+  // one list of the active rows of the group's entries.  (Larger groups gain nothing more and
+  // overflow the runs of the sort sooner.)
+  if (d.transpose && shared_matrix && d.batch_size > 1 && d.n_row > 0 && d.n_col > 0) {
+    uint32_t group = d.batch_size < 8 ? d.batch_size : 8;
+    while (group > 1 && (static_cast<uint64_t>(group) * d.n_col >= (1ull << 24) ||
+                         static_cast<uint64_t>(group) * d.n_row >= (1ull << 31)))
+      --group;
+    const uint32_t vcols = group * d.n_col;
+    if (group > 1 && vcols > 8192 && bin_event_scatter_usable<F>(vcols)) {
+      auto round_up = [](size_t v) { return (v + 255) / 256 * 256; };
+      const size_t vrows = static_cast<size_t>(group) * d.n_row;
+      const size_t list_sz = round_up(vrows * sizeof(uint2));
+      const size_t base_sz = round_up(vrows * sizeof(uint32_t));
+      unsigned char *ws = static_cast<unsigned char *>(
+          stream_workspace(stream, list_sz + base_sz + bin_event_scatter_bytes<F>(d.n_row, vcols)));
+      uint32_t *counters = ws ? stream_counters(stream) : nullptr;
+      if (ws != nullptr && counters != nullptr) {
+        uint2 *list = reinterpret_cast<uint2 *>(ws);
+        uint32_t *colbase = reinterpret_cast<uint32_t *>(ws + list_sz);
+        unsigned char *scratch = ws + list_sz + base_sz;
+        for (uint32_t b0 = 0; b0 < d.batch_size; b0 += group) {
+          const uint32_t g = (d.batch_size - b0 < group) ? d.batch_size - b0 : group;
+          // entry b0 + i reads event vector (b0 + i) % events_batch: hand the kernel the rotation
+          F *o = out + static_cast<size_t>(b0) * d.n_col;
+          hipLaunchKernelGGL((collect_active_rows_batched_kernel<F, VT>),
+                             dim3(div_up(static_cast<uint64_t>(g) * d.n_row, 8 * kWinThreads)), dim3(kWinThreads), 0,
+                             stream, indptr, events, d.n_row, d.n_col, g, d.events_batch, b0, counters, list, colbase,
+                             reinterpret_cast<uint32_t *>(scratch),
+                             static_cast<uint32_t>(kBinEventFillBytes / sizeof(uint32_t)), o,
+                             static_cast<uint64_t>(g) * d.n_col);
+          if (!bin_event_scatter<F>(stream, values, HETER, indices, indptr, o, d.n_row, g * d.n_col, counters, list,
+                                    scratch, colbase)) {
+            set_error("%s: the sorted scatter could not be enqueued", target);
+            return;
+          }
+        }
+        check_launch(target);
+        return;
+      }
+      bpl_clear_error();
+    }
   }
   for (uint32_t bi = 0; bi < d.batch_size; ++bi) {
     const F *v = values + static_cast<size_t>(bi % d.values_batch) * value_stride;

@@ -66,6 +66,28 @@ def test_batching_short_and_long_rows_and_wide_matrices(cuda, oracle_mod):
     assert np.array_equal(got, want), "homogeneous gather is bit-exact"
 
 
+def test_batching_transposed_through_one_sorted_scatter(cuda, oracle_mod):
+  # transpose=True with one matrix for all entries: the active rows of all entries go through one
+  # coarse sort over batch * n_col virtual columns.  Many virtual rows (several row tiles per
+  # producer), wide virtual outputs (sliced windows above 2^21), events broadcast (3 vectors for 6 entries).
+  rng = np.random.default_rng(13)
+  for n_row, n_col, mean, batch, eb, rate in ((20_000, 30_000, 30, 8, 8, 0.05), (300_000, 5000, 4, 6, 3, 0.6),
+                                              (2000, 1_500_000, 200, 4, 4, 0.3)):
+    counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_row)
+    data = rng.standard_normal(indices.shape[0]).astype(np.float32)
+    shape = (n_row, n_col)
+    print("shape", shape, "batch", batch, flush=True)
+    events = rng.random((eb, n_row)) < rate
+    _check(oracle_mod, data[None], indices[None], indptr[None], events, batch, shape, True, "heter")
+    one = np.ones((1, 1), dtype=np.float32)
+    got, want = _check(oracle_mod, one, indices[None], indptr[None], events, batch, shape, True, "counts")
+    assert np.array_equal(got, want)
+    # twice in a row (the list's counter is back at zero), float events
+    fev = (events * rng.uniform(0.5, 2.0, events.shape)).astype(np.float32)
+    _check(oracle_mod, data[None], indices[None], indptr[None], fev, batch, shape, True, "heter float events")
+
+
 def test_batching_equals_single_operator(cuda):
   # every row of the batched result is the single operator's result (exactly so for the
   # homogeneous weight, to rounding of one float64 sum otherwise)
