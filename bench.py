@@ -313,6 +313,24 @@ def main():
       del evb
     extra["gather_batched_1e8"] = batched
     log("gather batched 1e8: %s" % batched)
+    # the same in scatter orientation: 8 event vectors of 1 % and 5 % activity through one sorted scatter
+    batched_t = {}
+    for rate in (0.01, 0.05):
+      ev_np = rng_b.random((8, n_row)) < rate
+      evb = torch.from_numpy(ev_np).to(dev)
+      got = bpl.event_csr_matvec_batching(data[None], indices[None], indptr[None], evb, batch_size=8, shape=c["shape"],
+                                          transpose=True)[3].cpu().numpy()
+      want = oracle.event_csr_matvec(c["data"], c["indices"], c["indptr"], ev_np[3], shape=c["shape"], transpose=True)
+      mag = oracle.event_csr_matvec(np.abs(c["data"]), c["indices"], c["indptr"], ev_np[3], shape=c["shape"],
+                                    transpose=True)
+      check(got, want, "batched scatter 1e8 nnz, entry 3 at %g" % rate, mag)
+      dur_b, _ = time_calls(lambda: bpl.event_csr_matvec_batching(
+        data[None], indices[None], indptr[None], evb, batch_size=8, shape=c["shape"], transpose=True),
+        max(args.steps // 4, 5), max(args.warmup // 4, 2))
+      batched_t["x8_events_%g" % rate] = dict(stats(dur_b), us_per_event_vector=float(dur_b.mean() * 1e3 / 8))
+      del evb
+    extra["scatter_batched_1e8"] = batched_t
+    log("scatter batched 1e8: %s" % batched_t)
     del data, indices, indptr, events
 
     # 4,000 x 4,000, 80 per row, homogeneous 0.6, 2 % events, scatter (the reference's own CPU-sized case)
