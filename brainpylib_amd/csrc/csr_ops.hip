@@ -790,7 +790,8 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
     if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
     // (a dense vector is gathered from L2: for rows of 48 .. 191 nonzeros the pipelined 32-lane walk keeps more
     // of those gathers in flight than a wave per row does)
-    else if (mean >= (MODE == kDense ? 192u : 48u)) gather_rows_wave<F, VT, HETER, MODE, BITS, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    else if (MODE == kEvent && mean >= 48u) gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    else if (MODE == kDense && mean >= 192u) gather_rows_wave<F, VT, HETER, MODE, BITS, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
     else if (mean >= 48) gather_rows<F, VT, HETER, MODE, BITS, 32, 4>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
     else if (mean >= 24) gather_rows<F, VT, HETER, MODE, BITS, 32, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
     else if (mean >= 12) gather_rows<F, VT, HETER, MODE, BITS, 16, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
