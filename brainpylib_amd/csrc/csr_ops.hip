@@ -793,6 +793,9 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
     else if (MODE == kEvent && mean >= 48u) gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
     else if (MODE == kDense && mean >= 192u) gather_rows_wave<F, VT, HETER, MODE, BITS, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
     else if (mean >= 48) gather_rows<F, VT, HETER, MODE, BITS, 32, 4>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    else if (MODE == kEvent && mean >= 24) gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    else if (MODE == kEvent && mean >= 12) gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    else if (MODE == kEvent) gather_rows<F, VT, HETER, MODE, BITS, 4, 4>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
     else if (mean >= 24) gather_rows<F, VT, HETER, MODE, BITS, 32, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
     else if (mean >= 12) gather_rows<F, VT, HETER, MODE, BITS, 16, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
     else gather_rows<F, VT, HETER, MODE, BITS, 8, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
