@@ -749,8 +749,8 @@ __device__ __forceinline__ void gather_rows_wave(const F *__restrict__ data, con
 }
 
 // BITS: where the event probes go.  0: the event vector in global memory; 1: a bitmap in LDS;
-// 2: a bitmap in LDS of more than 80 KB (one workgroup per CU; a kernel of its own, so that the
-// code of the other cases does not depend on it).
+// 2: a bitmap in LDS of more than 80 KB (one workgroup per CU; a kernel of its own, because its
+// variants need more than the 64 registers that let two workgroups of the other cases share a CU).
 template <typename F, typename VT, bool HETER, int MODE, int BITS>
 __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ data,
                                                           const uint32_t *__restrict__ indices,
