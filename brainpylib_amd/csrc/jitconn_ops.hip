@@ -38,8 +38,10 @@ constexpr uint32_t kRowwalkCoarseBytes = 38912;
 // BITS: where the event probes go.  0: the event vector in global memory; 1: its bitmap in LDS;
 // 2: a coarse bitmap in LDS (one bit per 2^g inputs, at most kRowwalkCoarseBytes) and, where its
 // bit is set, the exact packed bitmap in global memory (`in`, the coarse one behind it).
+// (With the coarse bitmap two 16-wave workgroups are meant to share a CU: 8 waves per SIMD, which
+// the register allocation has to leave room for; the normal-weight walk needs 66 otherwise.)
 template <typename T1, typename VT, int IN, int W, int BITS>
-__global__ __launch_bounds__(1024) void jitconn_rowwalk_kernel(const VT *__restrict__ in, T1 *__restrict__ out,
+__global__ __launch_bounds__(1024, BITS == 2 ? 8 : 4) void jitconn_rowwalk_kernel(const VT *__restrict__ in, T1 *__restrict__ out,
                                                                uint32_t n_out, uint32_t n_in, uint32_t seed,
                                                                double log_p, T1 wa, T1 wb, uint32_t first,
                                                                const uint32_t *__restrict__ states) {
@@ -239,7 +241,7 @@ __global__ __launch_bounds__(1024) void collect_active_columns_kernel(const VT *
 constexpr int kColBinThreads = 1024;  // 16 waves share one set of bins: 4 times fewer, 4 times larger bins
 
 template <typename T1, typename VT, int IN, int W>
-__global__ __launch_bounds__(kColBinThreads) void jitconn_colwalk_bins_kernel(
+__global__ __launch_bounds__(kColBinThreads, sizeof(T1) == 4 ? 8 : 4) void jitconn_colwalk_bins_kernel(
     const VT *__restrict__ in, T1 *__restrict__ out, uint32_t n_out, uint32_t seed, double log_p, T1 wa, T1 wb,
     uint32_t first, uint32_t n_list_host, const uint32_t *__restrict__ n_list_dev,
     const uint32_t *__restrict__ list_col, const T1 *__restrict__ list_val, const uint32_t *__restrict__ states,
