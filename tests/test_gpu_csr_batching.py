@@ -31,7 +31,7 @@ def _check(oracle_mod, values, indices, indptr, events, batch, shape, transpose,
 def test_batching_broadcast_combinations(cuda, oracle_mod, shape, transpose, dtype):
   rng = np.random.default_rng(11)
   n_in = shape[0] if transpose else shape[1]
-  for dims, batch in (((1, 1, 1, 5), 5), ((1, 1, 1, 9), 9), ((1, 1, 1, 1), 1), ((1, 1, 1, 3), 20),
+  for dims, batch in (((1, 1, 1, 5), 5), ((1, 1, 1, 9), 9), ((1, 1, 1, 1), 1), ((1, 1, 1, 3), 20), ((1, 1, 1, 1), 4),
                       ((1, 3, 3, 1), 3), ((4, 1, 1, 4), 4), ((3, 3, 3, 3), 3), ((2, 1, 1, 3), 6)):
     vb, ib, pb, eb = dims
     print("case", shape, transpose, dtype.__name__, dims, batch, flush=True)
