@@ -515,3 +515,52 @@ def test_scatter_path_boundaries(cuda, oracle_mod, dtype):
     mag = oracle_mod.csr_matvec(data, indices, indptr, np.abs(v), shape=shape, transpose=True)
     got = bpl.cusparse_csr_matvec(data, indices, indptr, v, shape=shape, transpose=True).cpu().numpy()
     assert_close_reordered(got, want, mag, dtype, what="dense scatter %s" % (shape,))
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_random_shapes_all_operators_against_oracle(cuda, oracle_mod, seed):
+  # shapes, row lengths (with an occasional very long row), activity, dtypes and event kinds drawn
+  # at random over the ranges that select the different kernels; every operator of the family
+  # against the oracle
+  rng = np.random.default_rng(seed)
+  done = 0
+  for case in range(60):
+    n_row = int(10 ** rng.uniform(0, 5.3))
+    n_col = int(10 ** rng.uniform(0, 5.6))
+    mean = float(10 ** rng.uniform(-0.5, 2.3))
+    counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
+    if rng.random() < 0.3:
+      counts[rng.integers(0, n_row)] = min(n_col, int(10 ** rng.uniform(2, 4.5)))
+    if counts.sum() > 1e7:
+      continue
+    indices, indptr = synth.counted_csr(counts, n_col, seed=case)
+    dtype = np.float32 if rng.random() < 0.7 else np.float64
+    data = rng.standard_normal(indices.shape[0]).astype(dtype)
+    rate = float(rng.choice([0.0, 0.001, 0.02, 0.2, 1.0]))
+    shape = (n_row, n_col)
+    print("case", case, shape, "mean %.1f" % mean, "nnz", indices.shape[0], "rate", rate, dtype.__name__, flush=True)
+    for transpose in (True, False):
+      n_in = n_row if transpose else n_col
+      ev = rng.random(n_in) < rate
+      if rng.random() < 0.3:
+        ev = (ev * rng.uniform(0.5, 2, n_in)).astype(dtype)
+      for d in (data, np.array([0.75], dtype=dtype)):
+        want = oracle_mod.event_csr_matvec(d, indices, indptr, ev, shape=shape, transpose=transpose)
+        got = bpl.event_csr_matvec(d, indices, indptr, ev, shape=shape, transpose=transpose).cpu().numpy()
+        if transpose:
+          mag = oracle_mod.event_csr_matvec(np.abs(d), indices, indptr, ev, shape=shape, transpose=True)
+          assert_close_reordered(got, want, mag, dtype, what="event scatter %s" % (shape,))
+        else:
+          assert_close(got, want, what="event gather %s" % (shape,))
+      v = rng.standard_normal(n_in).astype(dtype)
+      want = oracle_mod.csr_matvec(data, indices, indptr, v, shape=shape, transpose=transpose)
+      if transpose:
+        got = bpl.cusparse_csr_matvec(data, indices, indptr, v, shape=shape, transpose=True).cpu().numpy()
+        mag = oracle_mod.csr_matvec(np.abs(data), indices, indptr, np.abs(v), shape=shape, transpose=True)
+        assert_close_reordered(got, want, mag, dtype, what="dense scatter %s" % (shape,))
+      else:
+        got = bpl.csr_matvec(data, indices, indptr, v, shape=shape).cpu().numpy()
+        assert_close(got, want, what="dense gather %s" % (shape,))
+    done += 1
+  assert done >= 40
+
