@@ -395,3 +395,41 @@ def test_column_walk_through_bins_events_and_overflow(cuda, oracle_mod):
     got = kernel_call(ev, w_kind="homo", log_p=lp, seed=5, n_row=n_out, n_col=n_in, col_walk=True, dense=False)
     want = oracle_mod.jitconn_matvec(ev, w_kind="homo", log_p=lp, seed=5, n_row=n_out, n_col=n_in, col_walk=True)
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_shapes_walks_weights_and_inputs_against_oracle(cuda, oracle_mod, seed):
+  # shapes up to two million inputs / outputs, both walks, all weight kinds, bool / float events and
+  # dense vectors drawn at random: every target of the family against the oracle
+  rng = np.random.default_rng(seed)
+  for case in range(100):
+    n_out = int(10 ** rng.uniform(0, 4.0))
+    n_in = int(10 ** rng.uniform(0, 6.3))
+    col_walk = bool(rng.random() < 0.5)
+    if col_walk:
+      n_out, n_in = int(10 ** rng.uniform(0, 6.3)), int(10 ** rng.uniform(0, 3.7))
+    syn = 10 ** rng.uniform(0, 2.5)
+    p = min(1.0, syn / max(n_out if col_walk else n_in, 1))
+    lp = oracle_mod.log_p_of(p)
+    w_kind = str(rng.choice(["homo", "uniform", "normal"]))
+    a, b = (0.0, 0.0) if w_kind == "homo" else (0.25, 1.75)
+    dtype = np.float32 if rng.random() < 0.7 else np.float64
+    kind = str(rng.choice(["bool", "float", "dense"]))
+    if kind == "bool":
+      inp, dense = rng.random(n_in) < rng.choice([0.0, 0.02, 0.5, 1.0]), False
+    elif kind == "float":
+      inp, dense = ((rng.random(n_in) < 0.3) * rng.uniform(0.5, 2, n_in)).astype(dtype), False
+    else:
+      inp, dense = rng.integers(-3, 4, n_in).astype(dtype), True
+    stream_seed = int(rng.integers(0, 2 ** 31))
+    print("case", case, n_out, n_in, col_walk, "%.2e" % p, w_kind, kind, dtype.__name__, flush=True)
+    want = oracle_mod.jitconn_matvec(inp, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=stream_seed, n_row=n_out,
+                                     n_col=n_in, col_walk=col_walk, dense=(None if kind == "bool" else dense))
+    got = kernel_call(inp, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=stream_seed, n_row=n_out, n_col=n_in,
+                      col_walk=col_walk, dense=dense)
+    if w_kind == "homo":
+      assert np.array_equal(got, want)  # counts / sums of small integers
+    else:
+      mag = np.full(n_out, 3.0 * (abs(a) + 5 * abs(b)) * (syn * 3 + 20))
+      assert_close_reordered(got, want, mag, np.float32 if kind == "bool" else dtype, what="case %d" % case)
+
