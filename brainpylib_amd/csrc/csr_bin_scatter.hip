@@ -518,10 +518,10 @@ inline uint32_t event_window_shift(uint32_t n_out) {
 
 // Pairs all windows' runs hold together.  The host knows neither the nonzero count nor the
 // activity, and what does not fit goes through direct atomics at a fortieth of the speed, so the
-// scratch memory is sized generously for this device: 1,024 pairs per row or column, between 2^24
+// scratch memory is sized generously for this device: 4,096 pairs per row or column, between 2^24
 // and 2^27 (1 GB of float pairs: every nonzero of a 1e8-nnz matrix active at once).
 inline uint64_t event_run_pairs(uint32_t n_row, uint32_t n_col) {
-  uint64_t t = 1024ull * (n_row > n_col ? n_row : n_col);
+  uint64_t t = 4096ull * (n_row > n_col ? n_row : n_col);
   if (t < (1ull << 24)) t = 1ull << 24;
   if (t > (1ull << 27)) t = 1ull << 27;
   return t;

@@ -357,7 +357,9 @@ def test_event_scatter_sorted_by_output_window(cuda, oracle_mod, dtype):
   cases = []
   counts = np.minimum(rng.poisson(3, size=1_200_000), 50)
   cases.append(("tiles", (1_200_000, 200_000), synth.counted_csr(counts, 200_000, seed=1), 0.9))
-  ix, ip = synth.counted_csr(np.full(3000, 100), 4000, seed=2)   # columns < 4,096: one window of 4,096
+  # columns < 2,000: all 1.8 million pairs fall into one window (2,048 columns at this width), more than
+  # its runs hold (8 x 171,000): the rest goes through direct atomics
+  ix, ip = synth.counted_csr(np.full(3000, 600), 2000, seed=2)
   cases.append(("one window", (3000, 200_000), (ix, ip), 1.0))
   counts = rng.poisson(120, size=30_000)
   cases.append(("plain", (30_000, 1_000_000), synth.counted_csr(counts, 1_000_000, seed=3), 0.05))
