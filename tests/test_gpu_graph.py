@@ -57,3 +57,33 @@ def test_jitconn_graph_replays(cuda):
   for odp in (True, False):
     _replay_check(lambda: bpl.event_matvec_prob_conn_homo_weight(ev, 0.5, conn_prob=0.01, shape=(n, n), seed=3,
                                                                  outdim_parallel=odp), new_events)
+
+
+def test_sorted_event_scatter_and_two_level_walk_graph_replays(cuda):
+  # the multi-kernel paths that pass counters and lists from kernel to kernel: the sorted event
+  # scatter (more than 8,192 outputs), its batched form, and the row walk with a two-level bitmap
+  rng = np.random.default_rng(2)
+  n_row, n_col = 30_000, 50_000
+  indices, indptr = synth.counted_csr(rng.poisson(40, size=n_row), n_col, seed=5)
+  data = torch.from_numpy(rng.standard_normal(indices.shape[0]).astype(np.float32)).to(cuda)
+  ix, ip = torch.from_numpy(indices).to(cuda), torch.from_numpy(indptr).to(cuda)
+  ev = torch.zeros(n_row, dtype=torch.bool, device=cuda)
+  evb = torch.zeros((5, n_row), dtype=torch.bool, device=cuda)
+
+  def new_events(i):
+    ev.copy_(torch.from_numpy(rng.random(n_row) < 0.03 * (i + 1)).to(cuda))
+    evb.copy_(torch.from_numpy(rng.random((5, n_row)) < 0.03 * (i + 1)).to(cuda))
+
+  new_events(0)
+  _replay_check(lambda: bpl.event_csr_matvec(data, ix, ip, ev, shape=(n_row, n_col), transpose=True), new_events)
+  _replay_check(lambda: bpl.event_csr_matvec_batching(data[None], ix[None], ip[None], evb, batch_size=5,
+                                                      shape=(n_row, n_col), transpose=True), new_events)
+  n_in = 400_000
+  evj = torch.zeros(n_in, dtype=torch.bool, device=cuda)
+
+  def new_inputs(i):
+    evj.copy_(torch.from_numpy(rng.random(n_in) < 0.02 * (i + 1)).to(cuda))
+
+  new_inputs(0)
+  _replay_check(lambda: bpl.event_matvec_prob_conn_homo_weight(evj, 0.5, conn_prob=0.001, shape=(500, n_in), seed=9),
+                new_inputs)
