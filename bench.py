@@ -51,6 +51,22 @@ def time_calls(fn, steps, warmup):
   return dur_ms, wall
 
 
+def single_call_us(fn, reps=20):
+  """Wall microseconds of ONE call with an idle queue before it and a synchronize after it: launch,
+  the kernels and the wait, as a caller that needs the result at once pays them.  Returns the first
+  (cold: whatever this call is the first to touch is loaded or allocated inside it) and the median
+  of `reps` further ones."""
+  import torch
+  out = []
+  for _ in range(reps + 1):
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    fn()
+    torch.cuda.synchronize()
+    out.append((time.perf_counter() - t0) * 1e6)
+  return dict(first=out[0], median=float(np.median(out[1:])))
+
+
 def back_to_back_us(fn, calls):
   """Microseconds per call when `calls` calls are enqueued with nothing between them (one pair of
   events around all of them): what a time-stepping loop pays per call once the queue is fed."""
@@ -197,7 +213,13 @@ def main():
 
   # parity gate at full size (the oracle's single-thread loops take well under a second each)
   want_g = oracle.event_csr_matvec(c["data"], c["indices"], c["indptr"], c["events"], shape=c["shape"])
-  got_g = bpl.event_csr_matvec(data, indices, indptr, events, shape=c["shape"]).cpu().numpy()
+  torch.cuda.synchronize()
+  t1 = time.perf_counter()
+  got_dev = bpl.event_csr_matvec(data, indices, indptr, events, shape=c["shape"])
+  torch.cuda.synchronize()
+  cold_gather_us = (time.perf_counter() - t1) * 1e6  # this process's first call of the operator
+  got_g = got_dev.cpu().numpy()
+  del got_dev
   check(got_g, want_g, "event_csr_matvec gather 1e8 nnz")
   want_s = oracle.event_csr_matvec(c["data"], c["indices"], c["indptr"], c["events"], shape=c["shape"], transpose=True)
   mag_s = oracle.event_csr_matvec(np.abs(c["data"]), c["indices"], c["indptr"], c["events"], shape=c["shape"],
@@ -244,6 +266,8 @@ def main():
     kernel_ms * 1e3, ms_per_step * 1e3, value, achieved))
 
   extra = {"gather_call_us": stats(dur), "nnz": nnz, "hits": hits, "active_rows": active}
+  one = single_call_us(gather)
+  extra["gather_single_call_wall_us"] = dict(cold_first_in_process=cold_gather_us, warm_median=one["median"])
 
   # ---------------------------------------------------------------------------------------------
   # CPU baseline: the oracle's restatement of the reference's CPU loop for this exact call
@@ -341,9 +365,11 @@ def main():
     check(got.cpu().numpy(), want, "event_csr_matvec scatter 4,000")
     scatter_c1 = lambda: bpl.event_csr_matvec(sd["data"], sd["indices"], sd["indptr"], sd["events"],
                                               shape=s["shape"], transpose=True)
+    one_c1 = single_call_us(scatter_c1)  # before any warm-up of this shape
     dur_c1, wall_c1 = time_calls(scatter_c1, args.steps, args.warmup)
     deliv = int(np.diff(s["indptr"])[s["events"]].sum())
-    extra["scatter_4000"] = dict(stats(dur_c1), delivered_synapses=deliv, wall_us_per_call=wall_c1 / args.steps * 1e6)
+    extra["scatter_4000"] = dict(stats(dur_c1), delivered_synapses=deliv, wall_us_per_call=wall_c1 / args.steps * 1e6,
+                                 single_call_wall_us=dict(first=one_c1["first"], warm_median=one_c1["median"]))
     if not args.skip_cpu:
       t1 = time.perf_counter()
       for _ in range(2000):
