@@ -143,6 +143,16 @@ def build_coo_atomic_sum_descriptor(conn_size, post_size):
 
 
 @functools.lru_cache(maxsize=256)
+def build_coo_atomic_prod_descriptor(conn_size, post_size):
+  return _build("bpl_build_coo_atomic_prod_descriptor", ctypes.c_uint32(conn_size), ctypes.c_uint32(post_size))
+
+
+@functools.lru_cache(maxsize=256)
+def build_csr_event_prod_descriptor(pre_size, post_size):
+  return _build("bpl_build_csr_event_prod_descriptor", ctypes.c_uint32(pre_size), ctypes.c_uint32(post_size))
+
+
+@functools.lru_cache(maxsize=256)
 def build_csr_transpose_descriptor(n_row, n_col, nnz):
   return _build("bpl_build_csr_transpose_descriptor", ctypes.c_uint32(n_row), ctypes.c_uint32(n_col),
                 ctypes.c_uint32(nnz))

@@ -1,14 +1,15 @@
 """The older operator names that brainpylib keeps for BrainPy models written against them
-(brainpylib/_src/compat): ``csr_event_sum``, ``coo_event_sum`` and ``coo_atomic_sum``, with the
-reference's signatures and argument checks, lowered to the custom-call targets its GPU
-translations name (event_sum.py:110-138,199-235, atomic_sum.py:93-131)."""
+(brainpylib/_src/compat): ``csr_event_sum``, ``coo_event_sum``, ``coo_atomic_sum`` and the product
+twins ``csr_event_prod`` and ``coo_atomic_prod``, with the reference's signatures and argument
+checks, lowered to the custom-call targets its GPU translations name (event_sum.py:110-138,199-235,
+atomic_sum.py:93-131, event_prod.py:107-127, atomic_prod.py:129-163)."""
 import torch
 
 from . import _lib
 from ._tensors import FLOAT_DTYPES, as_tensor, device_of, to_device
 from .event_ops import event_csr_matvec
 
-__all__ = ["csr_event_sum", "coo_event_sum", "coo_atomic_sum"]
+__all__ = ["csr_event_sum", "coo_event_sum", "coo_atomic_sum", "csr_event_prod", "coo_atomic_prod"]
 
 _INT_DTYPES = (torch.int32, torch.uint32, torch.int64, torch.uint64)
 
@@ -28,9 +29,9 @@ def _values(values):
   return values
 
 
-def csr_event_sum(events, pre2post, post_num, values):
-  """``out[post] += values`` over the synapses of every presynaptic neuron with an event
-  (event_sum.py:33-63).  ``pre2post = (indices, indptr)``."""
+def _csr_event_args(events, pre2post, post_num, values):
+  """The argument checks csr_event_sum and csr_event_prod share (event_sum.py:33-62,
+  event_prod.py:28-58)."""
   events = as_tensor(events)
   values = _values(values)
   indices, indptr = (as_tensor(a) for a in pre2post)
@@ -51,7 +52,14 @@ def csr_event_sum(events, pre2post, post_num, values):
   if values.numel() not in [1, indices.numel()]:
     raise ValueError(f'The size of "values" must be 1 (a scalar) or len(pre2post[0]) (a vector), '
                      f'while we got {values.numel()} != 1 != {indices.numel()}')
-  values = values.flatten()
+  return events, indices, indptr, post_num, values.flatten()
+
+
+def csr_event_sum(events, pre2post, post_num, values):
+  """``out[post] += values`` over the synapses of every presynaptic neuron with an event
+  (event_sum.py:33-63).  ``pre2post = (indices, indptr)``."""
+  events, indices, indptr, post_num, values = _csr_event_args(events, pre2post, post_num, values)
+  dtype = values.dtype
   if _i_type(indices.dtype) == '_i32':
     # the reference forwards to event_csr_matvec (event_sum.py:63)
     return event_csr_matvec(values, indices, indptr, events, shape=(events.shape[0], post_num), transpose=True)
@@ -62,6 +70,20 @@ def csr_event_sum(events, pre2post, post_num, values):
   name = 'gpu_csr_event_sum' + ('_homo' if values.shape[0] == 1 else '_heter') + _f_type(dtype) + '_i64'
   _lib.custom_call(name, [events, indices, indptr, values, out],
                    _lib.build_csr_event_sum_descriptor(events.shape[0], post_num))
+  return out
+
+
+def csr_event_prod(events, pre2post, post_num, values):
+  """``out[post] *= values`` on a vector of ones, over the synapses of every presynaptic neuron
+  with an event (event_prod.py:28-58; arithmetic of lib/cpu_event_prod.cc)."""
+  events, indices, indptr, post_num, values = _csr_event_args(events, pre2post, post_num, values)
+  device = device_of(values, indices, indptr, events)
+  events, indices, indptr, values = (to_device(t, device) for t in (events, indices, indptr, values))
+  out = torch.empty(post_num, dtype=values.dtype, device=device)
+  name = ('gpu_csr_event_prod' + ('_homo' if values.shape[0] == 1 else '_heter') + _f_type(values.dtype) +
+          _i_type(indices.dtype))
+  _lib.custom_call(name, [events, indices, indptr, values, out],
+                   _lib.build_csr_event_prod_descriptor(events.shape[0], post_num))
   return out
 
 
@@ -100,9 +122,9 @@ def coo_event_sum(events, pre_ids, post_ids, post_num, values):
   return out
 
 
-def coo_atomic_sum(values, post_ids, post_num, pre_ids=None):
-  """``out[post_ids[i]] += values[pre_ids[i]]`` over all connections, or ``+= values`` for a
-  scalar (atomic_sum.py:27-63)."""
+def _coo_atomic(op, values, post_ids, post_num, pre_ids):
+  """coo_atomic_sum and coo_atomic_prod: the same checks (atomic_sum.py:27-63,
+  atomic_prod.py:28-62) and buffer order."""
   values = _values(values)
   post_ids = as_tensor(post_ids)
   post_num = int(post_num)
@@ -131,7 +153,20 @@ def coo_atomic_sum(values, post_ids, post_num, pre_ids=None):
   device = device_of(values, post_ids, pre_ids)
   values, post_ids, pre_ids = (to_device(t, device) for t in (values, post_ids, pre_ids))
   out = torch.empty(post_num, dtype=values.dtype, device=device)
-  name = 'gpu_coo_atomic_sum' + ('_homo' if homo else '_heter') + _f_type(values.dtype) + _i_type(post_ids.dtype)
+  name = 'gpu_coo_atomic_' + op + ('_homo' if homo else '_heter') + _f_type(values.dtype) + _i_type(post_ids.dtype)
   buffers = [values, post_ids, out] if homo else [values, post_ids, pre_ids, out]
-  _lib.custom_call(name, buffers, _lib.build_coo_atomic_sum_descriptor(post_ids.shape[0], post_num))
+  build = _lib.build_coo_atomic_sum_descriptor if op == 'sum' else _lib.build_coo_atomic_prod_descriptor
+  _lib.custom_call(name, buffers, build(post_ids.shape[0], post_num))
   return out
+
+
+def coo_atomic_sum(values, post_ids, post_num, pre_ids=None):
+  """``out[post_ids[i]] += values[pre_ids[i]]`` over all connections, or ``+= values`` for a
+  scalar (atomic_sum.py:27-63)."""
+  return _coo_atomic('sum', values, post_ids, post_num, pre_ids)
+
+
+def coo_atomic_prod(values, post_ids, post_num, pre_ids=None):
+  """``out[post_ids[i]] *= values[pre_ids[i]]`` on a vector of ones, over all connections, or
+  ``*= values`` for a scalar (atomic_prod.py:28-62; arithmetic of lib/cpu_atomic_prod.cc)."""
+  return _coo_atomic('prod', values, post_ids, post_num, pre_ids)

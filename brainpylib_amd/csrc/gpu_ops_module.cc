@@ -48,6 +48,10 @@ PYBIND11_MODULE(gpu_ops, m) {
         [](uint32_t conn_size, uint32_t post_size) { return BPL_PACK(bpl_build_coo_event_sum_descriptor, conn_size, post_size); });
   m.def("build_coo_atomic_sum_descriptor",
         [](uint32_t conn_size, uint32_t post_size) { return BPL_PACK(bpl_build_coo_atomic_sum_descriptor, conn_size, post_size); });
+  m.def("build_coo_atomic_prod_descriptor",
+        [](uint32_t conn_size, uint32_t post_size) { return BPL_PACK(bpl_build_coo_atomic_prod_descriptor, conn_size, post_size); });
+  m.def("build_csr_event_prod_descriptor",
+        [](uint32_t pre_size, uint32_t post_size) { return BPL_PACK(bpl_build_csr_event_prod_descriptor, pre_size, post_size); });
   m.def("build_csr_transpose_descriptor", [](uint32_t n_row, uint32_t n_col, uint32_t nnz) {
     return BPL_PACK(bpl_build_csr_transpose_descriptor, n_row, n_col, nnz);
   });

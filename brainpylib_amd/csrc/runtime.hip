@@ -192,6 +192,16 @@ size_t bpl_build_coo_atomic_sum_descriptor(uint32_t conn_size, uint32_t post_siz
   return pack(d, out, cap);
 }
 
+size_t bpl_build_coo_atomic_prod_descriptor(uint32_t conn_size, uint32_t post_size, char *out, size_t cap) {
+  bpl_coo_sum_descriptor d{conn_size, post_size};
+  return pack(d, out, cap);
+}
+
+size_t bpl_build_csr_event_prod_descriptor(uint32_t pre_size, uint32_t post_size, char *out, size_t cap) {
+  bpl_csr_event_sum_descriptor d{pre_size, post_size};
+  return pack(d, out, cap);
+}
+
 size_t bpl_build_csr_transpose_descriptor(uint32_t n_row, uint32_t n_col, uint32_t nnz, char *out, size_t cap) {
   bpl_csr_transpose_descriptor d{n_row, n_col, nnz};
   return pack(d, out, cap);

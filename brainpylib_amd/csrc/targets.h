@@ -123,7 +123,23 @@
   X(gpu_coo_atomic_sum_heter_f32_i32) \
   X(gpu_coo_atomic_sum_heter_f32_i64) \
   X(gpu_coo_atomic_sum_heter_f64_i32) \
-  X(gpu_coo_atomic_sum_heter_f64_i64)
+  X(gpu_coo_atomic_sum_heter_f64_i64) \
+  X(gpu_coo_atomic_prod_homo_f32_i32) \
+  X(gpu_coo_atomic_prod_homo_f32_i64) \
+  X(gpu_coo_atomic_prod_homo_f64_i32) \
+  X(gpu_coo_atomic_prod_homo_f64_i64) \
+  X(gpu_coo_atomic_prod_heter_f32_i32) \
+  X(gpu_coo_atomic_prod_heter_f32_i64) \
+  X(gpu_coo_atomic_prod_heter_f64_i32) \
+  X(gpu_coo_atomic_prod_heter_f64_i64) \
+  X(gpu_csr_event_prod_homo_f32_i32) \
+  X(gpu_csr_event_prod_homo_f32_i64) \
+  X(gpu_csr_event_prod_homo_f64_i32) \
+  X(gpu_csr_event_prod_homo_f64_i64) \
+  X(gpu_csr_event_prod_heter_f32_i32) \
+  X(gpu_csr_event_prod_heter_f32_i64) \
+  X(gpu_csr_event_prod_heter_f64_i32) \
+  X(gpu_csr_event_prod_heter_f64_i64)
 
 #define BPL_ALL_TARGETS(X)  \
   BPL_EVENT_CSR_TARGETS(X)  \

@@ -151,6 +151,9 @@ size_t bpl_build_event_csr_batching_descriptor(uint32_t n_row, uint32_t n_col, u
 size_t bpl_build_csr_event_sum_descriptor(uint32_t pre_size, uint32_t post_size, char *out, size_t cap);
 size_t bpl_build_coo_event_sum_descriptor(uint32_t conn_size, uint32_t post_size, char *out, size_t cap);
 size_t bpl_build_coo_atomic_sum_descriptor(uint32_t conn_size, uint32_t post_size, char *out, size_t cap);
+/* lib/gpu_atomic_prod.cu:104-107; brainpylib/_src/compat/event_prod.py:113 */
+size_t bpl_build_coo_atomic_prod_descriptor(uint32_t conn_size, uint32_t post_size, char *out, size_t cap);
+size_t bpl_build_csr_event_prod_descriptor(uint32_t pre_size, uint32_t post_size, char *out, size_t cap);
 size_t bpl_build_csr_transpose_descriptor(uint32_t n_row, uint32_t n_col, uint32_t nnz, char *out, size_t cap);
 size_t bpl_build_twouint_onebool_descriptor(uint32_t n_row, uint32_t n_col, int transpose,
                                             char *out, size_t cap);
@@ -271,6 +274,39 @@ BPL_TARGET(gpu_coo_atomic_sum_heter_f32_i32);
 BPL_TARGET(gpu_coo_atomic_sum_heter_f32_i64);
 BPL_TARGET(gpu_coo_atomic_sum_heter_f64_i32);
 BPL_TARGET(gpu_coo_atomic_sum_heter_f64_i64);
+
+/* The product twins: the result starts as ones and is multiplied, following the reference's CPU
+ * kernels (lib/cpu_atomic_prod.cc:5-43, lib/cpu_event_prod.cc:5-55).
+ *   gpu_coo_atomic_prod_homo_{f32,f64}_{i32,i64}   (registered at lib/gpu_ops.cc:60-64)
+ *     buffers = [values F[1], post_ids I[conn_size], result F[post_size]]
+ *   gpu_coo_atomic_prod_heter_{f32,f64}_{i32,i64}  (registered at lib/gpu_ops.cc:65-69)
+ *     buffers = [values F[.], post_ids I[conn_size], pre_ids I[conn_size], result F[post_size]]
+ *     result[post_ids[i]] *= values[pre_ids[i]];  opaque = bpl_coo_sum_descriptor
+ *     (same layout as lib/gpu_atomic_prod.cuh:10-13; the reference's GPU kernels behind these
+ *     names, lib/gpu_atomic_prod.cu:26-98, fill the result's bytes with 1 and add: not followed)
+ *   gpu_csr_event_prod_{homo,heter}_{f32,f64}_{i32,i64}
+ *     buffers = [events bool[pre_size], indices I[nnz], indptr I[pre_size + 1],
+ *                values F[1] | F[nnz], result F[post_size]];  opaque = bpl_csr_event_sum_descriptor
+ *     result[indices[j]] *= values[j] for every j in row r, for every r with events[r].
+ *     The reference registers no such GPU target; these are the names its Python layer builds
+ *     (brainpylib/_src/compat/event_prod.py:107-127, with build_csr_event_prod_descriptor(pre, post)).
+ * ---------------------------------------------------------------------------------------- */
+BPL_TARGET(gpu_coo_atomic_prod_homo_f32_i32);
+BPL_TARGET(gpu_coo_atomic_prod_homo_f32_i64);
+BPL_TARGET(gpu_coo_atomic_prod_homo_f64_i32);
+BPL_TARGET(gpu_coo_atomic_prod_homo_f64_i64);
+BPL_TARGET(gpu_coo_atomic_prod_heter_f32_i32);
+BPL_TARGET(gpu_coo_atomic_prod_heter_f32_i64);
+BPL_TARGET(gpu_coo_atomic_prod_heter_f64_i32);
+BPL_TARGET(gpu_coo_atomic_prod_heter_f64_i64);
+BPL_TARGET(gpu_csr_event_prod_homo_f32_i32);
+BPL_TARGET(gpu_csr_event_prod_homo_f32_i64);
+BPL_TARGET(gpu_csr_event_prod_homo_f64_i32);
+BPL_TARGET(gpu_csr_event_prod_homo_f64_i64);
+BPL_TARGET(gpu_csr_event_prod_heter_f32_i32);
+BPL_TARGET(gpu_csr_event_prod_heter_f32_i64);
+BPL_TARGET(gpu_csr_event_prod_heter_f64_i32);
+BPL_TARGET(gpu_csr_event_prod_heter_f64_i64);
 
 /* ------------------------------------------------------------------------------------------
  * csr_matvec  (lib/gpu_csr_matvec.cu:563-621; launchers :84-135,:195-246,:505-560)

@@ -28,6 +28,11 @@ event_csr_matvec                dense matmul brute force, scipy.sparse, homo == 
                                 bool events)
 csr_matvec                      dense matmul brute force, scipy.sparse (both orientations)
 event_info                      numpy.flatnonzero
+coo_atomic_sum, csr_event_sum   compiled lib/cpu_atomic_sum.cc, lib/cpu_event_sum.cc (fixtures),
+(64-bit ids), coo_event_sum     the reference tests' known answers, numpy.bincount
+coo_atomic_prod,                compiled lib/cpu_atomic_prod.cc, lib/cpu_event_prod.cc
+csr_event_prod                  (fixtures), the reference tests' known answers, numpy
+                                multiply.at / powers of the weight
 event_matvec_hash, lfsr113,     the reference holds this algorithm as CUDA only.  Maximal period
 taus88                          of every component recurrence (2^31-1, 2^29-1, 2^28-1, 2^25-1:
                                 no wrong shift or mask constant survives that), GF(2)-linearity,
@@ -272,6 +277,33 @@ def coo_atomic_sum(values, post_ids, post_num, pre_ids=None):
   fn = lib().oracle_coo_atomic_sum_f32 if values.dtype == np.float32 else lib().oracle_coo_atomic_sum_f64
   fn(_p(values), ctypes.c_uint32(values.shape[0]), _p(post), _p(pre), ctypes.c_uint32(post.shape[0]),
      ctypes.c_uint32(post_num), _p(out))
+  return out
+
+
+def coo_atomic_prod(values, post_ids, post_num, pre_ids=None):
+  values = np.atleast_1d(np.ascontiguousarray(values))
+  assert values.dtype in (np.float32, np.float64)
+  post = _wide(post_ids)
+  pre = post if values.shape[0] == 1 else _wide(pre_ids)
+  assert pre.shape == post.shape
+  out = np.empty(post_num, dtype=values.dtype)
+  fn = lib().oracle_coo_atomic_prod_f32 if values.dtype == np.float32 else lib().oracle_coo_atomic_prod_f64
+  fn(_p(values), ctypes.c_uint32(values.shape[0]), _p(post), _p(pre), ctypes.c_uint32(post.shape[0]),
+     ctypes.c_uint32(post_num), _p(out))
+  return out
+
+
+def csr_event_prod(events, pre2post, post_num, values):
+  values = np.atleast_1d(np.ascontiguousarray(values))
+  assert values.dtype in (np.float32, np.float64)
+  events = np.ascontiguousarray(events)
+  assert events.dtype == np.bool_
+  indices, indptr = (_wide(a) for a in pre2post)
+  assert indptr.shape[0] == events.shape[0] + 1 and values.shape[0] in (1, indices.shape[0])
+  out = np.empty(post_num, dtype=values.dtype)
+  fn = lib().oracle_csr_event_prod_f32 if values.dtype == np.float32 else lib().oracle_csr_event_prod_f64
+  fn(_p(events.view(np.uint8)), _p(indices), _p(indptr), _p(values), ctypes.c_uint32(values.shape[0]),
+     ctypes.c_uint32(events.shape[0]), ctypes.c_uint32(post_num), _p(out))
   return out
 
 

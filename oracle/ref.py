@@ -99,6 +99,44 @@ def coo_atomic_sum(values, post_ids, post_num, pre_ids=None, *, wide=False):
   return out
 
 
+def coo_atomic_prod(values, post_ids, post_num, pre_ids=None, *, wide=False):
+  """lib/cpu_atomic_prod.cc: on ones, out[post_ids[i]] *= values[pre_ids[i]] (heter, :5-23) or
+  *= values[0] (homo, :25-43)."""
+  values = np.atleast_1d(np.ascontiguousarray(values))
+  post_ids = _ids(post_ids, wide)
+  f = "f32" if values.dtype == np.float32 else "f64"
+  i = "i64" if wide else "i32"
+  out = np.empty(post_num, dtype=values.dtype)
+  conn = np.array(post_ids.shape[0], dtype=np.uint32)
+  size = np.array(post_num, dtype=np.uint32)
+  if values.shape[0] == 1:
+    kind, ins = "homo", [values, post_ids, conn, size]
+  else:
+    kind, ins = "heter", [values, _ids(pre_ids, wide), post_ids, conn, size]
+  in_arr = (ctypes.c_void_p * len(ins))(*[_ptr(a) for a in ins])
+  _sym("cpu_coo_atomic_prod_%s_%s_%s" % (kind, f, i), tuple_out=False)(_ptr(out), in_arr)
+  return out
+
+
+def csr_event_prod(data, indices, indptr, events, *, shape, wide=False):
+  """lib/cpu_event_prod.cc: on ones, out[post] *= w for every synapse of every pre with
+  events[pre]."""
+  data = np.atleast_1d(np.ascontiguousarray(data))
+  events = np.ascontiguousarray(events)
+  assert events.dtype == np.bool_
+  indices = _ids(indices, wide)
+  indptr = _ids(indptr, wide)
+  kind = "homo" if data.shape[0] == 1 else "heter"
+  f = "f32" if data.dtype == np.float32 else "f64"
+  out = np.empty(shape[1], dtype=data.dtype)
+  pre = np.array(shape[0], dtype=np.uint32)
+  post = np.array(shape[1], dtype=np.uint32)
+  ins = [pre, post, events, indices, indptr, data]
+  in_arr = (ctypes.c_void_p * len(ins))(*[_ptr(a) for a in ins])
+  _sym("cpu_csr_event_prod_%s_%s_%s" % (kind, f, "i64" if wide else "i32"), tuple_out=False)(_ptr(out), in_arr)
+  return out
+
+
 def csr_event_sum(data, indices, indptr, events, *, shape, wide=False):
   """lib/cpu_event_sum.cc: out[post] += w for every synapse of every pre with events[pre]
   (the transpose=True, bool-event case of event_csr_matvec); `wide` selects the 64-bit index

@@ -1,10 +1,12 @@
 """Writes the golden fixtures in this directory by running the reference's own CPU kernels
-(lib/cpu_jitconn_*.cpp, lib/cpu_event_sum.cc, lib/cpu_atomic_sum.cc), compiled unmodified by
+(lib/cpu_jitconn_*.cpp, lib/cpu_event_sum.cc, lib/cpu_atomic_sum.cc, lib/cpu_event_prod.cc,
+lib/cpu_atomic_prod.cc), compiled unmodified by
 `make -C oracle ref`.  Runs only where the reference tree is mounted; the fixtures it writes are
 committed.
 
     python tests/golden/make_golden.py            # all fixtures
     python tests/golden/make_golden.py compat     # only compat_cpu_reference.npz
+    python tests/golden/make_golden.py prod       # only compat_prod_cpu_reference.npz
 
 jitconn_cpu_reference.npz
     the reference CPU backend as it ships: ONE sequential generator per matrix.  For every case
@@ -18,6 +20,9 @@ event_sum_cpu_reference.npz
 compat_cpu_reference.npz
     lib/cpu_atomic_sum.cc (coo_atomic_sum, homogeneous and heterogeneous, 32- and 64-bit ids) and
     the 64-bit instantiation of lib/cpu_event_sum.cc, on seeded random connections.
+compat_prod_cpu_reference.npz
+    lib/cpu_atomic_prod.cc (coo_atomic_prod) and lib/cpu_event_prod.cc (csr_event_prod), homogeneous
+    and heterogeneous, 32- and 64-bit ids, on seeded random connections with weights near 1.
 """
 import json
 import os
@@ -102,7 +107,46 @@ def compat_fixture():
   print("wrote", i, "coo_atomic_sum cases and", j, "64-bit csr_event_sum cases")
 
 
+def prod_fixture():
+  out = {}
+  i = 0
+  # weights near 1 keep products of a few hundred factors inside the normal range
+  for pre, post, conn in [(200, 200, 4000), (50, 300, 2000), (300, 7, 600), (1, 1, 10)]:
+    for homo in (True, False):
+      for dt in (np.float32, np.float64):
+        for wide in (False, True):
+          rng = np.random.default_rng(1900 + i)
+          pre_ids = rng.integers(0, pre, size=conn).astype(np.int64 if wide else np.int32)
+          post_ids = rng.integers(0, post, size=conn).astype(np.int64 if wide else np.int32)
+          values = np.array([0.97], dtype=dt) if homo else rng.uniform(0.9, 1.1, pre).astype(dt)
+          if not homo and i % 4 == 1:
+            values[rng.integers(0, pre, 3)] *= -1  # signs
+          out["ap_values_%d" % i], out["ap_pre_%d" % i], out["ap_post_%d" % i] = values, pre_ids, post_ids
+          out["ap_num_%d" % i] = np.array(post)
+          out["ap_out_%d" % i] = ref.coo_atomic_prod(values, post_ids, post, None if homo else pre_ids, wide=wide)
+          i += 1
+  j = 0
+  for shape in [(100, 200), (300, 10), (2, 3000)]:
+    for homo in (True, False):
+      for dt in (np.float32, np.float64):
+        for wide in (False, True):
+          indices, indptr = synth.bernoulli_csr(shape[0], shape[1], 0.3, seed=1300 + j)
+          rng = np.random.default_rng(1700 + j)
+          data = np.array([1.03], dtype=dt) if homo else rng.uniform(0.9, 1.1, indices.shape[0]).astype(dt)
+          events = rng.random(shape[0]) < 0.3
+          it = np.int64 if wide else np.int32
+          out["ep_data_%d" % j], out["ep_events_%d" % j], out["ep_shape_%d" % j] = data, events, np.array(shape)
+          out["ep_indices_%d" % j], out["ep_indptr_%d" % j] = indices.astype(it), indptr.astype(it)
+          out["ep_out_%d" % j] = ref.csr_event_prod(data, indices, indptr, events, shape=shape, wide=wide)
+          j += 1
+  np.savez_compressed(os.path.join(HERE, "compat_prod_cpu_reference.npz"), **out)
+  print("wrote", i, "coo_atomic_prod cases and", j, "csr_event_prod cases")
+
+
 def main():
+  if len(sys.argv) > 1 and sys.argv[1] == "prod":
+    prod_fixture()
+    return
   compat_fixture()
   if len(sys.argv) > 1 and sys.argv[1] == "compat":
     return

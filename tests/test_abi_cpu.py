@@ -52,7 +52,7 @@ def test_reference_target_names_present():
 
 
 def test_reference_registry_keys_of_the_other_operators_present():
-  # lib/gpu_ops.cc:27-58 (the older event / atomic sums), :72-174 (jitconn, matmat, nonzero)
+  # lib/gpu_ops.cc:27-69 (the older event / atomic sums and products), :72-174 (jitconn, matmat, nonzero)
   names = set(_lib.target_names())
   want = []
   for w in ("homo", "uniform", "normal"):
@@ -65,14 +65,14 @@ def test_reference_registry_keys_of_the_other_operators_present():
     for t in ("float", "double"):
       want.append("gpu_matmat_prob_prob_%s_%s_v1" % (w, t))
   want += ["nonzero_" + t for t in ("bool", "int", "long", "float", "double")]
-  for op in ("gpu_csr_event_sum", "gpu_coo_event_sum", "gpu_coo_atomic_sum"):
+  for op in ("gpu_csr_event_sum", "gpu_coo_event_sum", "gpu_coo_atomic_sum", "gpu_coo_atomic_prod"):
     for data in ("homo", "heter"):
       for f in ("f32", "f64"):
         for i in ("i32", "i64"):
           want.append("%s_%s_%s_%s" % (op, data, f, i))
   missing = [n for n in want if n not in names]
   assert not missing, missing
-  assert len(want) == 36 + 6 + 4 + 5 + 24
+  assert len(want) == 36 + 6 + 4 + 5 + 32
 
 
 @pytest.mark.parametrize("name", sorted(_lib.target_names()))
@@ -148,6 +148,8 @@ def test_gpu_ops_module_matches_reference_interface():
     assert api.PyCapsule_GetPointer(cap, b"xla._CUSTOM_CALL_TARGET") == lib.bpl_find_target(name.encode())
   assert gpu_ops.build_twouint_onebool_descriptor(3, 4, True) == struct.pack("<IIB3x", 3, 4, 1)
   assert gpu_ops.build_double_size_descriptor(5, 6) == struct.pack("<II", 5, 6)
+  assert gpu_ops.build_coo_atomic_prod_descriptor(5, 6) == struct.pack("<II", 5, 6)  # lib/gpu_atomic_prod.cuh:10-13
+  assert gpu_ops.build_csr_event_prod_descriptor(7, 8) == struct.pack("<II", 7, 8)
   assert gpu_ops.build_nonzero_descriptor(7, 8) == struct.pack("<II", 7, 8)
   assert gpu_ops.build_jitconn_prob_homo_descriptor(1, 2, 3, -0.25) == struct.pack("<III4xd", 1, 2, 3, -0.25)
   assert gpu_ops.build_jitconn_prob_uniform_descriptor(1, 2, 3, -0.25, 0.5, 1.0) == struct.pack(

@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 
 import brainpylib_amd as bpl
+from brainpylib_amd import synth
 from util import assert_close_reordered
 
 pytestmark = pytest.mark.gpu
@@ -85,3 +86,109 @@ def test_known_answers_and_argument_checks(cuda):
     bpl.coo_atomic_sum(np.ones(5, np.float32), post, 10, pre)  # values shorter than max(pre_ids)
   with pytest.raises(ValueError):
     bpl.csr_event_sum(np.ones(4, bool), (post, np.zeros(4, np.int32)), 10, 1.0)  # len(indptr) != len(events) + 1
+
+
+PROD_GOLD = os.path.join(os.path.dirname(__file__), "golden", "compat_prod_cpu_reference.npz")
+
+
+def _assert_close_product(got, want, count, dtype, what):
+  """A product of `count` factors rounds count - 1 times in either order (half an ulp each), so two
+  orders differ by at most (count - 1) eps relative; equal factors give the same bits."""
+  got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+  bound = np.abs(want) * np.finfo(dtype).eps * (count + 1)
+  bad = np.abs(got - want) > bound
+  assert not bad.any(), "%s: %d of %d off, worst %g" % (what, bad.sum(), bad.size, np.abs(got - want).max())
+
+
+def test_coo_atomic_prod_golden(cuda):
+  # lib/cpu_atomic_prod.cc, compiled
+  z = np.load(PROD_GOLD)
+  n = sum(1 for k in z.files if k.startswith("ap_out_"))
+  assert n == 32
+  for i in range(n):
+    values, pre, post, num = z["ap_values_%d" % i], z["ap_pre_%d" % i], z["ap_post_%d" % i], int(z["ap_num_%d" % i])
+    homo = values.shape[0] == 1
+    got = bpl.coo_atomic_prod(values, post, num, None if homo else pre).cpu().numpy()
+    want = z["ap_out_%d" % i]
+    assert got.dtype == want.dtype
+    if homo:
+      assert np.array_equal(got, want), "case %d" % i  # equal factors: the order cannot matter
+    else:
+      _assert_close_product(got, want, np.bincount(post, minlength=num), values.dtype, "coo_atomic_prod %d" % i)
+
+
+def test_csr_event_prod_golden(cuda):
+  # lib/cpu_event_prod.cc, compiled
+  z = np.load(PROD_GOLD)
+  n = sum(1 for k in z.files if k.startswith("ep_out_"))
+  assert n == 24
+  for i in range(n):
+    data, events, indices, indptr = (z["ep_%s_%d" % (k, i)] for k in ("data", "events", "indices", "indptr"))
+    post_n = int(z["ep_shape_%d" % i][1])
+    got = bpl.csr_event_prod(events, (indices, indptr), post_n, data).cpu().numpy()
+    want = z["ep_out_%d" % i]
+    assert got.dtype == want.dtype
+    if data.shape[0] == 1:
+      assert np.array_equal(got, want), "case %d" % i
+    else:
+      count = np.bincount(indices[np.repeat(events, np.diff(indptr))], minlength=post_n)
+      _assert_close_product(got, want, count, data.dtype, "csr_event_prod %d" % i)
+
+
+def test_prod_vs_oracle_larger(cuda, oracle_mod):
+  rng = np.random.default_rng(77)
+  for dtype in (np.float32, np.float64):
+    for wide in (False, True):
+      it = np.int64 if wide else np.int32
+      pre_n, post_n, conn = 3000, 5000, 200000
+      pre = rng.integers(0, pre_n, conn).astype(it)
+      post = rng.integers(0, post_n, conn).astype(it)
+      post[:2000] = 17  # one heavily shared target
+      values = rng.uniform(0.99, 1.01, pre_n).astype(dtype)
+      values[rng.integers(0, pre_n, 40)] *= -1
+      got = bpl.coo_atomic_prod(values, post, post_n, pre).cpu().numpy()
+      want = oracle_mod.coo_atomic_prod(values, post, post_n, pre)
+      _assert_close_product(got, want, np.bincount(post, minlength=post_n), dtype, "coo_atomic_prod")
+      assert np.array_equal(np.signbit(got), np.signbit(want))
+      w = np.array([1.0009765625], dtype)  # 2,000 equal factors on one target: bit for bit
+      got = bpl.coo_atomic_prod(w, post, post_n).cpu().numpy()
+      assert got.dtype == dtype and np.array_equal(got, oracle_mod.coo_atomic_prod(w, post, post_n))
+      indices, indptr = synth.bernoulli_csr(800, 1200, 0.1, seed=5)
+      events = rng.random(800) < 0.4
+      data = rng.uniform(0.98, 1.02, indices.shape[0]).astype(dtype)
+      got = bpl.csr_event_prod(events, (indices.astype(it), indptr.astype(it)), 1200, data).cpu().numpy()
+      want = oracle_mod.csr_event_prod(events, (indices, indptr), 1200, data)
+      count = np.bincount(indices[np.repeat(events, np.diff(indptr))], minlength=1200)
+      _assert_close_product(got, want, count, dtype, "csr_event_prod")
+      assert np.all(got[count == 0] == 1)
+
+
+def test_prod_known_answers_and_argument_checks(cuda):
+  # brainpylib/_src/compat/tests/test_atomic_prod_cpu.py:16-53
+  size = 200
+  ids = np.arange(size, dtype=np.uint32)
+  sps = np.random.default_rng(12345).integers(0, 2, size).astype(np.float32)
+  assert np.array_equal(bpl.coo_atomic_prod(sps, ids, size, ids).cpu().numpy(), sps)
+  assert np.all(bpl.coo_atomic_prod(2., ids, size).cpu().numpy() == 2.)
+  pre, post = np.divmod(np.arange(100, dtype=np.int32), 10)
+  assert np.all(bpl.coo_atomic_prod(2., post, 10).cpu().numpy() == 1024.)
+  assert np.all(bpl.coo_atomic_prod(np.full(10, 2., np.float32), post, 10, pre).cpu().numpy() == 1024.)
+  # a NaN weight reaches its target and nothing else
+  v = np.ones(10, np.float64)
+  v[3] = np.nan
+  got = bpl.coo_atomic_prod(v, np.arange(10, dtype=np.int32), 10, np.arange(10, dtype=np.int32)).cpu().numpy()
+  assert np.isnan(got[3]) and np.all(np.delete(got, 3) == 1)
+  # no connections, no events: ones
+  e = np.zeros(0, np.int32)
+  assert np.all(bpl.coo_atomic_prod(3., e, 6).cpu().numpy() == 1.)
+  indices = np.array([1, 2, 0, 2, 2], dtype=np.int32)
+  indptr = np.array([0, 2, 2, 4, 5], dtype=np.int32)
+  got = bpl.csr_event_prod(np.array([True, True, False, True]), (indices, indptr), 3, np.array([2., 3., 5., 7., 11.]))
+  assert np.array_equal(got.cpu().numpy(), [1., 2., 33.])
+  assert np.all(bpl.csr_event_prod(np.zeros(4, bool), (indices, indptr), 3, 3.).cpu().numpy() == 1.)
+  with pytest.raises(ValueError):
+    bpl.csr_event_prod(np.ones(4, np.float32), (indices, indptr), 3, 1.0)  # events must be bool
+  with pytest.raises(ValueError):
+    bpl.csr_event_prod(np.ones(3, bool), (indices, indptr), 3, 1.0)
+  with pytest.raises(ValueError):
+    bpl.coo_atomic_prod(np.ones(5, np.float32), post, 10, pre)  # values shorter than max(pre_ids)
