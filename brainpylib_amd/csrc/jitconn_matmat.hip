@@ -10,7 +10,8 @@
 // wave64 owns a column: X is first transposed into a scratch buffer XT[k][m] (rows padded to a
 // multiple of 64), then for every synapse (id, w) of the column the wave reads the contiguous
 // row XT[id][0..m) and each lane accumulates its own output rows, in stream order, with the same
-// multiply-then-add the CPU path performs.
+// multiply-then-add the CPU path performs.  The synapses of a batch pass from the lanes that drew
+// them to the whole wave through LDS (one broadcast read each).
 //
 // Reference boundary: lib/gpu_jitconn_matmat.cu:279-317,364-455 (buffers = [X, Y], descriptor
 // MatMatJITProbDescriptor1, target names lib/gpu_ops.cc:161-174).
@@ -41,20 +42,17 @@ __global__ __launch_bounds__(kTile * 8) void transpose_pad_kernel(const T *__res
   }
 }
 
-__device__ __forceinline__ float read_lane(float v, int l) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
-}
-__device__ __forceinline__ double read_lane(double v, int l) {
-  const long long b = __builtin_bit_cast(long long, v);
-  const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(b), l));
-  const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(b >> 32), l));
-  return __builtin_bit_cast(double, (static_cast<long long>(hi) << 32) | lo);
-}
-
 __device__ __forceinline__ float mul_rn(float a, float b) { return __fmul_rn(a, b); }
 __device__ __forceinline__ double mul_rn(double a, double b) { return __dmul_rn(a, b); }
 __device__ __forceinline__ float add_rn(float a, float b) { return __fadd_rn(a, b); }
 __device__ __forceinline__ double add_rn(double a, double b) { return __dadd_rn(a, b); }
+
+// one synapse of a batch: where its row of XT starts (bytes) and its weight
+template <typename T1>
+struct __attribute__((aligned(2 * sizeof(T1)))) Synapse {
+  uint32_t off;
+  T1 w;
+};
 
 // MT = 64-row tiles of Y one wave accumulates (m_pad / 64 per pass of blockIdx.y)
 template <typename T1, int W, int MT>
@@ -64,50 +62,59 @@ __global__ __launch_bounds__(256) void jitconn_matmat_kernel(const T1 *__restric
   constexpr int kWaves = 4;
   constexpr int kWords = StreamLds<T1, W>::words;
   __shared__ __attribute__((aligned(8))) uint32_t s_state[kWaves * kWords];
+  __shared__ Synapse<T1> s_syn[kWaves * kWave];
   const int lane = lane_id();
   const uint32_t wave = threadIdx.x / kWave;
   uint32_t *st = s_state + wave * kWords;
+  Synapse<T1> *syn = s_syn + wave * kWave;
   const uint32_t row_base = blockIdx.y * (MT * kWave);  // first row of Y of this pass
+  // byte offsets into XT fit 32 bits (checked by the host): one add per synapse instead of a 64-bit product
+  const uint32_t row_bytes = m_pad * static_cast<uint32_t>(sizeof(T1));
+  const char *xt_lane = reinterpret_cast<const char *>(XT + row_base + lane);
 
   for (uint32_t j = blockIdx.x * kWaves + wave; j < n; j += gridDim.x * kWaves) {
     T1 acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = T1(0);
     walk_stream<T1, W>(st, lane, seed + j, nullptr, k, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
-      uint64_t mask = __ballot(valid);
-      constexpr int U = 4;
-      while (mask) {
-        uint32_t id[U];
+      // Every valid lane leaves its synapse (the byte offset of its row of XT, its weight) in the
+      // wave's LDS slots, in lane order (which is stream order); every lane then reads the slots
+      // one after the other (one address per read: a broadcast), so a synapse costs one LDS read,
+      // one address add, MT loads and MT multiply-adds, with U synapses' loads in flight.
+      const uint64_t mask = __ballot(valid);
+      const uint32_t count = static_cast<uint32_t>(__popcll(mask));
+      const uint32_t slot = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32),
+                                                      __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u));
+      __builtin_amdgcn_wave_barrier();  // the reads of the batch before are done
+      if (valid) {
+        syn[slot].off = idx * row_bytes;
+        syn[slot].w = w;
+      }
+      __builtin_amdgcn_wave_barrier();
+      constexpr int U = (MT >= 4) ? 4 : 8;
+      uint32_t i = 0;
+      for (; i + U <= count; i += U) {
         T1 ws[U];
         T1 x[U][MT];
-        int got = 0;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-          if (mask) {
-            const int s = __ffsll(static_cast<unsigned long long>(mask)) - 1;
-            mask &= mask - 1;
-            ++got;
-            id[u] = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(idx), s));
-            ws[u] = read_lane(w, s);
-          } else {  // pad the group (loaded but not accumulated)
-            id[u] = 0u;
-            ws[u] = T1(0);
-          }
-        }
-        const int group = got;
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const T1 *row = XT + static_cast<size_t>(id[u]) * m_pad + row_base + lane;
+          const Synapse<T1> e = syn[i + u];
+          ws[u] = e.w;
+          const T1 *row = reinterpret_cast<const T1 *>(xt_lane + e.off);
 #pragma unroll
           for (int t = 0; t < MT; ++t) x[u][t] = row[t * kWave];
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-          if (u < group) {
 #pragma unroll
-            for (int t = 0; t < MT; ++t) acc[t] = add_rn(acc[t], mul_rn(ws[u], x[u][t]));
-          }
+          for (int t = 0; t < MT; ++t) acc[t] = add_rn(acc[t], mul_rn(ws[u], x[u][t]));
         }
+      }
+      for (; i < count; ++i) {
+        const Synapse<T1> e = syn[i];
+        const T1 *row = reinterpret_cast<const T1 *>(xt_lane + e.off);
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[t] = add_rn(acc[t], mul_rn(e.w, row[t * kWave]));
       }
     });
 #pragma unroll
@@ -140,6 +147,10 @@ void matmat_entry(const char *target, hipStream_t stream, void **buffers, const 
   if (k == 0) {
     fill_zero(stream, Y, m * n);  // m * n fits 32 bits whenever Y is addressable by the kernels below
     check_launch(target);
+    return;
+  }
+  if (static_cast<uint64_t>(k) * m_pad * sizeof(T1) > 0xffffffffull) {
+    set_error("%s: the transposed operand (%u x %u) exceeds 4 GiB", target, k, m_pad);
     return;
   }
   T1 *XT = static_cast<T1 *>(stream_workspace(stream, static_cast<size_t>(k) * m_pad * sizeof(T1)));
