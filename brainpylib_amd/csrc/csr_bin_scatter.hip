@@ -282,9 +282,18 @@ constexpr uint32_t kFillStride = 32;          // words between fill counters: on
 static_assert(kBinEventFillBytes == kMaxWindows * kSubRuns * kFillStride * sizeof(uint32_t),
               "one fill counter per window and sub-run");
 constexpr uint32_t kPairsPerPart = 8192;      // a consumer workgroup takes part per that many pairs of its window
+// Little activity (the usual state of a spiking network): up to this many active nonzeros
+// (estimated) skip the runs, because the chain list -> sort -> reserve -> store -> add costs more
+// than their atomics.  The producer only leaves the number of active rows in a spare word of the
+// fill area (zeroed with it before every call) and the consumer's waves add the rows to y directly.
+constexpr uint32_t kDirectPairs = 131072;
+constexpr uint32_t kDirectWord = 1;           // (fill counters sit at multiples of kFillStride)
 
+// (At most 80 scalar registers: measured on this device, a 1,024-thread workgroup whose waves hold
+// 81..96 of them is alone on its CU, as it would be with more than 64 vector registers; the
+// float producer crossed that line by one register and took 37 instead of 27 us.)
 template <typename F, bool HETER>
-__global__ __launch_bounds__(kBinThreads) void bin_active_rows_kernel(
+__global__ __launch_bounds__(kBinThreads) __attribute__((amdgpu_num_sgpr(80))) void bin_active_rows_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
     uint32_t n_row, const uint32_t *__restrict__ active_count, const uint2 *__restrict__ active_list,
     const uint32_t *__restrict__ active_colbase, F *__restrict__ y, uint32_t shift, uint32_t cap,
@@ -307,6 +316,10 @@ __global__ __launch_bounds__(kBinThreads) void bin_active_rows_kernel(
   // with little activity a few producers finish sooner than a chip full of them
   const uint64_t want = (static_cast<uint64_t>(total) * (nnz / n_row + 1u) + kPairsPerProducer - 1u) / kPairsPerProducer;
   const uint32_t producers = want < 1u ? 1u : want > gridDim.x ? gridDim.x : static_cast<uint32_t>(want);
+  if (static_cast<uint64_t>(total) * (nnz / n_row + 1u) <= kDirectPairs) {
+    if (blockIdx.x == 0 && tid == 0) fill[kDirectWord] = total;
+    return;
+  }
   const uint32_t p = blockIdx.x;
   if (p >= producers) return;
   const uint32_t sub = p % kSubRuns;
@@ -440,13 +453,34 @@ __global__ __launch_bounds__(kBinThreads) void add_window_runs_kernel(F *__restr
                                                                       uint32_t lds_shift, uint32_t parts, uint32_t cap,
                                                                       const BinPair<F> *__restrict__ pairs,
                                                                       const uint32_t *__restrict__ fill,
-                                                                      uint32_t *__restrict__ reset) {
+                                                                      uint32_t *__restrict__ reset,
+                                                                      const F *__restrict__ data, bool heter,
+                                                                      const uint32_t *__restrict__ indices,
+                                                                      const uint2 *__restrict__ active_list,
+                                                                      const uint32_t *__restrict__ active_colbase) {
   extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
   // (the caller's active-row counter, left at zero for the next call)
   if (reset != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *reset = 0u;
   double *window = reinterpret_cast<double *>(smem_raw);
   const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   constexpr uint32_t kWaves = kBinThreads / kWave;
+  const uint32_t direct_rows = fill[kDirectWord];
+  if (direct_rows != 0u) {
+    // k waves per active row (all the grid's waves when the rows are few), dealt over the
+    // workgroups first; wave `part` of a row takes every k-th group of 64 nonzeros
+    const F w_homo = heter ? F(0) : data[0];
+    const uint32_t total_waves = gridDim.x * kWaves;
+    const uint32_t k = direct_rows < total_waves ? total_waves / direct_rows : 1u;
+    const uint64_t items = static_cast<uint64_t>(direct_rows) * k;
+    for (uint64_t item = wave * gridDim.x + blockIdx.x; item < items; item += total_waves) {
+      const uint32_t r = static_cast<uint32_t>(item / k), part = static_cast<uint32_t>(item % k);
+      const uint2 e = active_list[r];  // (first nonzero, length)
+      F *out = y + (active_colbase ? active_colbase[r] : 0u);
+      for (uint32_t j = part * kWave + lane; j < e.y; j += k * kWave)
+        atomic_add(out + indices[e.x + j], heter ? data[e.x + j] : w_homo);
+    }
+    return;
+  }
   const uint32_t slices = 1u << (shift - lds_shift);
   const uint32_t b = blockIdx.x / (parts * slices), q = (blockIdx.x / parts) % slices, s = blockIdx.x % parts;
   // pre[r] = pairs in the runs before run r (at most 2^27 in all)
@@ -576,7 +610,8 @@ bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint
     hipLaunchKernelGGL((bin_active_rows_kernel<F, false>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
                        indptr, n_row, active_count, active_list, active_colbase, y, shift, cap, pairs, fill);
   hipLaunchKernelGGL(add_kernel, dim3(n_win * slices * parts), dim3(kBinThreads), lds, stream, y, n_col, shift,
-                     lds_shift, parts, cap, pairs, fill, active_count);
+                     lds_shift, parts, cap, pairs, fill, active_count, data, heter, indices, active_list,
+                     active_colbase);
   return true;
 }
 

@@ -40,8 +40,11 @@ constexpr uint32_t kRowwalkCoarseBytes = 38912;
 // bit is set, the exact packed bitmap in global memory (`in`, the coarse one behind it).
 // (With the coarse bitmap two 16-wave workgroups are meant to share a CU: 8 waves per SIMD, which
 // the register allocation has to leave room for; the normal-weight walk needs 66 otherwise.)
+// Register budget: eight waves per SIMD need at most 64 vector AND at most 80 scalar registers per
+// wave here (with 81..96 scalar registers only seven fit, so a second 16-wave workgroup does not).
 template <typename T1, typename VT, int IN, int W, int BITS>
-__global__ __launch_bounds__(1024, BITS == 2 ? 8 : 4) void jitconn_rowwalk_kernel(const VT *__restrict__ in, T1 *__restrict__ out,
+__global__ __launch_bounds__(1024, (BITS == 2 || (W == kNormal && sizeof(T1) == 4)) ? 8 : 4)
+    __attribute__((amdgpu_num_sgpr(80))) void jitconn_rowwalk_kernel(const VT *__restrict__ in, T1 *__restrict__ out,
                                                                uint32_t n_out, uint32_t n_in, uint32_t seed,
                                                                double log_p, T1 wa, T1 wb, uint32_t first,
                                                                const uint32_t *__restrict__ states) {

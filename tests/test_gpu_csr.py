@@ -352,7 +352,8 @@ def test_event_scatter_sorted_by_output_window(cuda, oracle_mod, dtype):
   # event input and outputs wider than 131,072: the active rows' nonzeros are sorted coarsely by
   # output window.  Cases: more than 1,024 active rows per producer workgroup (several row tiles);
   # all columns in one window, more of them than the window's run holds (the rest goes through
-  # direct atomics); float events; silent input; calls repeated (the counters are back at zero).
+  # direct atomics); float events; silent input; calls repeated (the counters are back at zero);
+  # so little activity that the sort is skipped.
   rng = np.random.default_rng(41)
   cases = []
   counts = np.minimum(rng.poisson(3, size=1_200_000), 50)
@@ -362,7 +363,10 @@ def test_event_scatter_sorted_by_output_window(cuda, oracle_mod, dtype):
   ix, ip = synth.counted_csr(np.full(3000, 600), 2000, seed=2)
   cases.append(("one window", (3000, 200_000), (ix, ip), 1.0))
   counts = rng.poisson(120, size=30_000)
-  cases.append(("plain", (30_000, 1_000_000), synth.counted_csr(counts, 1_000_000, seed=3), 0.05))
+  plain = synth.counted_csr(counts, 1_000_000, seed=3)
+  cases.append(("plain", (30_000, 1_000_000), plain, 0.05))
+  # some 7,000 active nonzeros: too few to be worth sorting, the active rows add them to y directly
+  cases.append(("little activity", (30_000, 1_000_000), plain, 0.002))
   # above 2^21 columns a window is wider than its accumulators in LDS and is added in slices
   counts = rng.poisson(60, size=20_000)
   cases.append(("sliced windows", (20_000, 5_000_001), synth.counted_csr(counts, 5_000_001, seed=4), 0.3))
