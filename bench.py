@@ -67,6 +67,17 @@ def single_call_us(fn, reps=20):
   return dict(first=out[0], median=float(np.median(out[1:])))
 
 
+def copy_bandwidth_gb_per_s(dev, n_bytes=1 << 30):
+  """What a plain device-to-device copy of `n_bytes` moves per second on this device (bytes read
+  plus bytes written): the HBM rate a streaming kernel can actually reach, to set beside the
+  published peak."""
+  import torch
+  a = torch.empty(n_bytes // 4, dtype=torch.float32, device=dev).normal_()
+  b = torch.empty_like(a)
+  dur, _ = time_calls(lambda: b.copy_(a), 20, 3)
+  return 2.0 * n_bytes / (float(np.median(dur)) * 1e-3) / 1e9
+
+
 def back_to_back_us(fn, calls):
   """Microseconds per call when `calls` calls are enqueued with nothing between them (one pair of
   events around all of them): what a time-stepping loop pays per call once the queue is fed."""
@@ -267,6 +278,12 @@ def main():
 
   extra = {"gather_call_us": stats(dur), "nnz": nnz, "hits": hits, "active_rows": active}
   one = single_call_us(gather)
+  copy_rate = copy_bandwidth_gb_per_s(dev)
+  extra["hbm_copy_gb_per_s"] = copy_rate  # 1 GiB device-to-device copy, read + write
+  if nnz == 100014049:
+    extra["gather_hbm_traffic_gb_per_s"] = GATHER_TRAFFIC_BYTES / (kernel_ms * 1e-3) / 1e9
+    extra["gather_traffic_over_copy_rate"] = extra["gather_hbm_traffic_gb_per_s"] / copy_rate
+  log("device-to-device copy of 1 GiB: %.0f GB/s (read + write)" % copy_rate)
   extra["gather_single_call_wall_us"] = dict(cold_first_in_process=cold_gather_us, warm_median=one["median"])
 
   # ---------------------------------------------------------------------------------------------
