@@ -576,6 +576,16 @@ __device__ __forceinline__ void event_hits(const uint32_t *s_bits, const VT *__r
   }
 }
 
+// Element `col` of the dense vector.  BITS == 2: its first `lds_n` elements are staged in LDS
+// (`s_x`), the rest is gathered from global memory.
+template <typename VT, int BITS>
+__device__ __forceinline__ VT dense_element(const VT *__restrict__ x, const uint32_t *s_x, uint32_t lds_n, uint32_t col) {
+  if constexpr (BITS == 2) {
+    if (col < lds_n) return reinterpret_cast<const VT *>(s_x)[col];
+  }
+  return x[col];
+}
+
 template <typename F, typename VT, bool HETER, int MODE, int BITS, int G, int U>
 __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const uint32_t *__restrict__ indices,
                                             const uint32_t *__restrict__ indptr, const VT *__restrict__ x,
@@ -634,7 +644,7 @@ __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const ui
         use[u] = ok;
         const F d = HETER ? data[ok ? j : (end ? end - 1 : 0u)] : w_homo;
         // product formed in F, then widened (the reference multiplies two F values)
-        val[u] = static_cast<F>(static_cast<F>(x[col[u]]) * d);
+        val[u] = static_cast<F>(static_cast<F>(dense_element<VT, BITS>(x, s_bits, coarse_g, col[u])) * d);
       }
     }
     // indices of the next step, and the row bounds one row further ahead
@@ -716,7 +726,7 @@ __device__ __forceinline__ void gather_rows_wave(const F *__restrict__ data, con
         if (ok[u]) {
           const F d = HETER ? dp[off] : w_homo;
           // product formed in F, then widened (the reference multiplies two F values)
-          val[u] = static_cast<F>(static_cast<F>(x[col[u]]) * d);
+          val[u] = static_cast<F>(static_cast<F>(dense_element<VT, BITS>(x, s_bits, coarse_g, col[u])) * d);
         }
       }
     }
@@ -757,9 +767,20 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
                                                           const uint32_t *__restrict__ indptr,
                                                           const VT *__restrict__ x, F *__restrict__ y,
                                                           uint32_t n_row, uint32_t n_col) {
-  extern __shared__ uint32_t s_bits[];
+  extern __shared__ __attribute__((aligned(16))) uint32_t s_bits[];
   uint32_t coarse_g = 0;
-  if constexpr (BITS == 3) {
+  if constexpr (MODE == kDense) {
+    // BITS == 1: the dense vector itself is staged in LDS (the host checked that it fits), so the
+    // per-nonzero gather is an LDS read instead of an L2 request and the kernel streams at HBM speed
+    // BITS == 2: as much of it as fits; the kernel gathers the rest from L2 as without LDS
+    if constexpr (BITS == 1 || BITS == 2) {
+      VT *s_x = reinterpret_cast<VT *>(s_bits);
+      const uint32_t fits = static_cast<uint32_t>(kLdsBitmapCap / sizeof(VT));
+      coarse_g = n_col < fits ? n_col : fits;  // (the walks take it as the number of staged elements)
+      for (uint32_t i = threadIdx.x; i < coarse_g; i += blockDim.x) s_x[i] = x[i];
+      __syncthreads();
+    }
+  } else if constexpr (BITS == 3) {
     // x is the exact packed bitmap; the coarse one behind it goes to LDS
     coarse_g = coarse_shift(n_col);
     const uint32_t words = (coarse_bits(n_col, coarse_g) + 31u) >> 5;
@@ -779,7 +800,18 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
   }
   // lanes per row from the mean row length
   const uint32_t mean = nnz / n_row;
-  if constexpr (MODE == kEvent && (BITS == 2 || BITS == 3)) {
+  if constexpr (MODE == kDense && BITS == 1) {
+    // (nothing left to hide but the index and weight streams: the walks of the event gather)
+    const VT *xs = reinterpret_cast<const VT *>(s_bits);
+    if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g);
+    else if (mean >= 24) gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g);
+    else if (mean >= 12) gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g);
+    else gather_rows<F, VT, HETER, MODE, BITS, 4, 4>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g);
+  } else if constexpr (MODE == kDense && BITS == 2) {
+    if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    else if (mean >= 24) gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    else gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+  } else if constexpr (MODE == kEvent && (BITS == 2 || BITS == 3)) {
     // An event bitmap above 80 KB leaves room for one workgroup (16 waves) per CU only: every lane
     // then keeps 16 (rows under 48 nonzeros: 8) loads in flight instead of 2 to 8, in groups of
     // 8 or 4 lanes per row, or HBM sees too few requests (1e6 columns, 100 per row: 424 -> 164 us).
@@ -1027,6 +1059,25 @@ void launch_gather(const char *target, hipStream_t stream, const F *data, const 
                           : launch_gather_impl<F, VT, HETER, MODE, 1>(target, stream, data, indices, indptr, x, y, n_row,
                                                                       n_col, lds_bytes);
       if (ok) return;
+      bpl_clear_error();
+    }
+  }
+  if constexpr (MODE == kDense) {
+    // A dense vector that fits LDS beside nothing else (up to 40,704 floats), under persistent
+    // workgroups (few copies): staged there.  Gathers from L2 cap the product at about 140 G nonzeros
+    // per second whatever the vector's size; from LDS the index and weight streams are the limit.
+    const size_t lds_bytes = static_cast<size_t>(n_col) * sizeof(VT);
+    if (n_row >= 16384 && n_col > 0 && lds_bytes <= kLdsBitmapCap) {
+      if (launch_gather_impl<F, VT, HETER, MODE, 1>(target, stream, data, indices, indptr, x, y, n_row, n_col,
+                                                    lds_bytes))
+        return;
+      bpl_clear_error();
+    } else if (n_row >= 16384 && lds_bytes <= 4 * kLdsBitmapCap) {
+      // up to four times that: the part that fits is staged (one workgroup per CU), which takes a
+      // quarter or more of the gathers off the L2
+      if (launch_gather_impl<F, VT, HETER, MODE, 2>(target, stream, data, indices, indptr, x, y, n_row, n_col,
+                                                    kLdsBitmapCap))
+        return;
       bpl_clear_error();
     }
   }

@@ -570,3 +570,28 @@ def test_random_shapes_all_operators_against_oracle(cuda, oracle_mod, seed):
     done += 1
   assert done >= 40
 
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_csr_matvec_with_the_vector_staged_in_lds(cuda, oracle_mod, dtype):
+  # at least 16,384 rows and a vector of at most 159 KB: the kernels gather it from LDS.  Every
+  # row-length mode of that path, the largest vector that fits and the first that does not
+  # (staged in part), empty rows, heterogeneous and homogeneous weights.
+  rng = np.random.default_rng(61)
+  limit = (160 * 1024 - 1024) // np.dtype(dtype).itemsize
+  for n_row, n_col, mean in ((20_000, 5_000, 30), (17_000, limit, 5), (16_384, limit + 1, 5), (40_000, 3_000, 100),
+                             (16_500, 20_000, 400), (30_000, 9_000, 14), (40_000, 1, 1),
+                             # up to four times as long: the part that fits is staged, the rest comes from L2
+                             (20_000, 100_000, 30), (17_000, 4 * limit, 8), (16_400, 70_000, 450)):
+    counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
+    counts[rng.integers(0, n_row, 50)] = 0
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_row)
+    data = rng.standard_normal(indices.shape[0]).astype(dtype)
+    v = rng.standard_normal(n_col).astype(dtype)
+    shape = (n_row, n_col)
+    print("shape", shape, flush=True)
+    for d in (data, np.array([0.75], dtype=dtype)):
+      want = oracle_mod.csr_matvec(d, indices, indptr, v, shape=shape)
+      got = bpl.csr_matvec(d, indices, indptr, v, shape=shape).cpu().numpy()
+      assert got.dtype == dtype
+      assert_close(got, want, what="csr_matvec %s" % (shape,))
