@@ -461,6 +461,19 @@ def main():
     extra["csr_matvec_transposed_1e8"] = dict(stats(dur3t), gsop_per_s=nnz3 / (dur3t.mean() * 1e-3) / 1e9,
                                               algorithmic_gb_per_s=bytes3 / (dur3t.mean() * 1e-3) / 1e9)
     log("csr_matvec transposed 1e8: %s" % extra["csr_matvec_transposed_1e8"])
+    # a dense vector short enough for LDS (up to 159 KB): 200,000 x 19,000, 100 per row, 2.0e7 nnz
+    rng_s = np.random.default_rng(23)
+    ix_s, ip_s = synth.counted_csr(np.full(200_000, 100), 19_000, seed=23)
+    d_s = rng_s.random(ix_s.shape[0], dtype=np.float32)
+    v_s = rng_s.standard_normal(19_000).astype(np.float32)
+    dev_s = [torch.from_numpy(a_).to(dev) for a_ in (d_s, ix_s, ip_s, v_s)]
+    got = bpl.csr_matvec(*dev_s, shape=(200_000, 19_000)).cpu().numpy()
+    check(got, oracle.csr_matvec(d_s, ix_s, ip_s, v_s, shape=(200_000, 19_000)), "csr_matvec vector in LDS")
+    dur_s, _ = time_calls(lambda: bpl.csr_matvec(*dev_s, shape=(200_000, 19_000)), max(20, args.steps // 4), 5)
+    extra["csr_matvec_2e7_vector_in_lds"] = dict(stats(dur_s), gsop_per_s=ix_s.shape[0] / (dur_s.mean() * 1e-3) / 1e9,
+                                                 algorithmic_gb_per_s=8.0 * ix_s.shape[0] / (dur_s.mean() * 1e-3) / 1e9)
+    log("csr_matvec 2e7, vector in LDS: %s" % extra["csr_matvec_2e7_vector_in_lds"])
+    del dev_s
     # the same 1,000,000 x 1,000,000 matrix (100 nonzeros per row) driven by events, 1 % and 5 % of
     # the rows active: the shape of a million-neuron network's synaptic update (output far wider than LDS)
     wide = {}
