@@ -21,6 +21,7 @@ VGPR_MAX, SGPR_MAX = 64, 80
 # (pattern on the demangled name, why it needs eight waves per SIMD)
 TWO_PER_CU = [
   (r"csr_gather_kernel<\w+, [\w:]+, (true|false), 0, 1>", "event gather with the bitmap in LDS (the headline kernel)"),
+  (r"csr_gather_kernel<float, float, (true|false), 1, 1>", "csr_matvec with the vector staged in LDS, float"),
   (r"csr_scatter_window_kernel<", "event scatter into LDS windows"),
   (r"bin_active_rows_kernel<", "producer of the sorted event scatter"),
   (r"jitconn_rowwalk_kernel<\w+, bpl::PackedBits, 0, \d, 2>", "jitconn row walk with the two-level bitmap"),
