@@ -41,15 +41,50 @@ const DeviceInfo &device_info();
 // Scratch device memory for operators that need a staging buffer (the custom-call ABI provides
 // none): one allocation per (device, stream), grown on demand and kept until the process ends.
 // Work enqueued on one stream is ordered, so calls on the same stream can share the buffer;
-// calls on different streams get different buffers.  Returns nullptr (and records an error) if
-// the allocation fails.  Not usable while the stream is being captured into a graph the first
-// time a size is requested (hipMalloc is not capturable).
+// calls on different streams get different buffers.  A buffer that has been handed out is never
+// freed: when a larger one is needed the old one is retired (kept allocated), because work that
+// was enqueued earlier, or a HIP graph captured earlier on the stream, may still use it.  Growing
+// needs hipMalloc, which cannot run while the stream is being captured into a graph: then the
+// call fails (nullptr, error recorded, nothing enqueued), so every size must have been used once
+// on the stream before it is captured.  nullptr (error recorded) also if the allocation fails.
 void *stream_workspace(hipStream_t stream, size_t bytes);
 
 // A few zero-initialised 32-bit counters per (device, stream).  The first one (the scatter's
 // active-row count) is left at zero again by every user; the others carry nothing from call to
-// call.  nullptr if the allocation fails.
+// call.  nullptr if the allocation fails (or would be needed during a capture).
 uint32_t *stream_counters(hipStream_t stream);
+constexpr size_t kStreamCounterBytes = 256;
+
+// True if the calling thread's most recent stream_workspace() / stream_counters() call failed
+// because the stream was being captured.  A launcher that would otherwise fall back to a path
+// that needs less scratch memory must then give up with the error standing: a graph that
+// silently records the slow path would replay it for good.
+bool scratch_refused_by_capture();
+
+// Where the launchers of one call take their scratch memory from: the cached allocation of the
+// call's stream (above), or a fixed arena that the entry point owns and that is never grown (the
+// allocation-free entry point's static device array).  Either way ONE buffer serves the whole
+// call: every request() of a call returns the same base address, and the launchers lay their
+// sub-buffers out inside it.
+struct ScratchSource {
+  hipStream_t stream = nullptr;
+  unsigned char *arena = nullptr;     // fixed arena (device memory), or nullptr: the cached allocation
+  size_t arena_bytes = 0;
+  uint32_t *arena_counters = nullptr;  // kStreamCounterBytes of device memory beside the arena
+
+  bool fixed() const { return arena != nullptr; }
+  // after a failed request(): must the call fail (true), or may it fall back to a path that needs
+  // less scratch memory (an allocation failed: false)?
+  bool failure_is_final() const { return fixed() || scratch_refused_by_capture(); }
+  // `want` bytes if they can be had, at least `need`; *got receives the size obtained.  nullptr,
+  // with an error recorded, if `need` bytes are not available.
+  void *request(size_t want, size_t need, size_t *got) const;
+  void *request(size_t bytes) const {
+    size_t got = 0;
+    return request(bytes, bytes, &got);
+  }
+  uint32_t *counters() const { return fixed() ? arena_counters : stream_counters(stream); }
+};
 
 // Transposed CSR times dense vector through coarse sorting of the products (csr_bin_scatter.hip),
 // for outputs much wider than LDS.  `nnz` must be the matrix's nonzero count (indptr[n_row]).
@@ -62,9 +97,12 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
 
 // The same for event input (event_csr_matvec, transposed, wide outputs): the caller lists the
 // active rows on the device, (first nonzero, length) each in `active_list`, their number in
-// active_count[0]; `scratch` is device memory of bin_event_scatter_bytes() bytes whose first
+// active_count[0] (the list has room for `list_cap` rows); `scratch` is device memory of `scratch_bytes` bytes whose first
 // kBinEventFillBytes are zero; y is zeroed.  Enqueues the two kernels; the second one sets
 // active_count[0] back to zero.  false (nothing enqueued) if it cannot run.
+// The scratch memory behind the fill counters holds the runs of (column, weight) pairs: the call
+// works with any size from bin_event_scatter_min_bytes() on (pairs that find their run full go
+// through direct atomics, far more slowly), and bin_event_scatter_bytes() is the size to ask for.
 // Batched calls (several event vectors, one matrix) hand in one list over all batch entries, n_col
 // = batch * columns, and `active_colbase` = what to add to the columns of each listed row (its
 // batch entry * columns); n_row stays the matrix's row count (indptr has n_row + 1 entries).
@@ -74,9 +112,12 @@ bool bin_event_scatter_usable(uint32_t n_col);
 template <typename F>
 size_t bin_event_scatter_bytes(uint32_t n_row, uint32_t n_col);
 template <typename F>
+size_t bin_event_scatter_min_bytes(uint32_t n_col);
+template <typename F>
 bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint32_t *indices, const uint32_t *indptr,
                        F *y, uint32_t n_row, uint32_t n_col, uint32_t *active_count, const uint2 *active_list,
-                       void *scratch, const uint32_t *active_colbase = nullptr);
+                       uint32_t list_cap, void *scratch, size_t scratch_bytes,
+                       const uint32_t *active_colbase = nullptr);
 
 // Second half of the coarse-sorted scatter for producers other than the CSR one: adds bins laid
 // out uniformly, bin (p, b) = pairs + (p * n_win + b) * cap with counts[b * producers + p]

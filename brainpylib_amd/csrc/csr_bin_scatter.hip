@@ -296,7 +296,7 @@ template <typename F, bool HETER>
 __global__ __launch_bounds__(kBinThreads) __attribute__((amdgpu_num_sgpr(80))) void bin_active_rows_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
     uint32_t n_row, const uint32_t *__restrict__ active_count, const uint2 *__restrict__ active_list,
-    const uint32_t *__restrict__ active_colbase, F *__restrict__ y, uint32_t shift, uint32_t cap,
+    uint32_t list_cap, const uint32_t *__restrict__ active_colbase, F *__restrict__ y, uint32_t shift, uint32_t cap,
     BinPair<F> *__restrict__ pairs, uint32_t *__restrict__ fill) {
   __shared__ uint32_t s_ptr[kTileRows + 1];     // nonzeros of the tile's rows before row k
   __shared__ uint32_t s_start[kTileRows];       // first nonzero of row k in the matrix
@@ -311,7 +311,7 @@ __global__ __launch_bounds__(kBinThreads) __attribute__((amdgpu_num_sgpr(80))) v
   __shared__ BinPair<F> s_sorted[kRound];
   __shared__ uint8_t s_window[kRound];
   const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  const uint32_t total = active_count[0];
+  const uint32_t total = active_count[0] < list_cap ? active_count[0] : list_cap;  // (never beyond the list)
   const uint32_t nnz = indptr[n_row];
   // with little activity a few producers finish sooner than a chip full of them
   const uint64_t want = (static_cast<uint64_t>(total) * (nnz / n_row + 1u) + kPairsPerProducer - 1u) / kPairsPerProducer;
@@ -576,13 +576,26 @@ size_t bin_event_scatter_bytes(uint32_t n_row, uint32_t n_col) {
   return kBinEventFillBytes + static_cast<size_t>(cap) * n_win * kSubRuns * sizeof(BinPair<F>);
 }
 
+// at least kMinRunPairs pairs per run
+constexpr uint32_t kMinRunPairs = 1024;
+template <typename F>
+size_t bin_event_scatter_min_bytes(uint32_t n_col) {
+  const uint32_t n_win = div_up(n_col, 1u << event_window_shift(n_col));
+  return kBinEventFillBytes + static_cast<size_t>(kMinRunPairs) * n_win * kSubRuns * sizeof(BinPair<F>);
+}
+
 template <typename F>
 bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint32_t *indices, const uint32_t *indptr,
                        F *y, uint32_t n_row, uint32_t n_col, uint32_t *active_count, const uint2 *active_list,
-                       void *scratch, const uint32_t *active_colbase) {
+                       uint32_t list_cap, void *scratch, size_t scratch_bytes, const uint32_t *active_colbase) {
   const uint32_t shift = event_window_shift(n_col);
   const uint32_t n_win = div_up(n_col, 1u << shift);
-  const uint32_t cap = static_cast<uint32_t>(event_run_pairs(n_row, n_col) / (n_win * kSubRuns));
+  if (scratch_bytes < bin_event_scatter_min_bytes<F>(n_col)) return false;
+  // pairs per run: what the scratch memory holds (a window's kSubRuns runs together stay below
+  // 2^28 pairs, which the consumer counts in 32 bits)
+  const uint64_t cap64 = (scratch_bytes - kBinEventFillBytes) / (static_cast<size_t>(n_win) * kSubRuns * sizeof(BinPair<F>));
+  const uint64_t cap_max = (1ull << 28) / kSubRuns;
+  const uint32_t cap = static_cast<uint32_t>(cap64 > cap_max ? cap_max : cap64);
   uint32_t *fill = static_cast<uint32_t *>(scratch);
   BinPair<F> *pairs = reinterpret_cast<BinPair<F> *>(static_cast<unsigned char *>(scratch) + kBinEventFillBytes);
   const unsigned num_cu = static_cast<unsigned>(device_info().num_cu);
@@ -605,10 +618,10 @@ bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint
   const uint32_t producers = 2u * num_cu;
   if (heter)
     hipLaunchKernelGGL((bin_active_rows_kernel<F, true>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
-                       indptr, n_row, active_count, active_list, active_colbase, y, shift, cap, pairs, fill);
+                       indptr, n_row, active_count, active_list, list_cap, active_colbase, y, shift, cap, pairs, fill);
   else
     hipLaunchKernelGGL((bin_active_rows_kernel<F, false>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
-                       indptr, n_row, active_count, active_list, active_colbase, y, shift, cap, pairs, fill);
+                       indptr, n_row, active_count, active_list, list_cap, active_colbase, y, shift, cap, pairs, fill);
   hipLaunchKernelGGL(add_kernel, dim3(n_win * slices * parts), dim3(kBinThreads), lds, stream, y, n_col, shift,
                      lds_shift, parts, cap, pairs, fill, active_count, data, heter, indices, active_list,
                      active_colbase);
@@ -644,7 +657,7 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
   const size_t count_bytes = static_cast<size_t>(n_win) * producers * sizeof(uint32_t);
   unsigned char *ws = static_cast<unsigned char *>(stream_workspace(stream, pair_bytes + count_bytes));
   if (ws == nullptr) {
-    bpl_clear_error();
+    if (!scratch_refused_by_capture()) bpl_clear_error();  // (an allocation failed: the caller has other paths)
     return false;
   }
   BinPair<F> *pairs = reinterpret_cast<BinPair<F> *>(ws);
@@ -712,10 +725,13 @@ template bool bin_event_scatter_usable<float>(uint32_t);
 template bool bin_event_scatter_usable<double>(uint32_t);
 template size_t bin_event_scatter_bytes<float>(uint32_t, uint32_t);
 template size_t bin_event_scatter_bytes<double>(uint32_t, uint32_t);
+template size_t bin_event_scatter_min_bytes<float>(uint32_t);
+template size_t bin_event_scatter_min_bytes<double>(uint32_t);
 template bool bin_event_scatter<float>(hipStream_t, const float *, bool, const uint32_t *, const uint32_t *, float *, uint32_t,
-                                       uint32_t, uint32_t *, const uint2 *, void *, const uint32_t *);
+                                       uint32_t, uint32_t *, const uint2 *, uint32_t, void *, size_t, const uint32_t *);
 template bool bin_event_scatter<double>(hipStream_t, const double *, bool, const uint32_t *, const uint32_t *, double *,
-                                        uint32_t, uint32_t, uint32_t *, const uint2 *, void *, const uint32_t *);
+                                        uint32_t, uint32_t, uint32_t *, const uint2 *, uint32_t, void *, size_t,
+                                        const uint32_t *);
 template bool bin_scatter_usable<float>(uint32_t, uint32_t);
 template bool bin_scatter_usable<double>(uint32_t, uint32_t);
 template bool bin_scatter<float>(const char *, hipStream_t, const float *, bool, const uint32_t *, const uint32_t *,

@@ -161,6 +161,8 @@ __global__ __launch_bounds__(kWinThreads) void collect_active_rows_kernel(
     const uint32_t *__restrict__ indptr, const VT *__restrict__ x, uint32_t n_row, uint32_t *__restrict__ counter,
     uint2 *__restrict__ list, F *__restrict__ scales, NnzGate gate, uint32_t *__restrict__ clear, uint32_t n_clear,
     F *__restrict__ zero, uint32_t n_zero) {
+  // (The list holds n_row entries.  The counter is zero when a call starts, so positions stay below
+  // n_row; should an earlier call have failed half way and left it set, nothing is written beyond.)
   if (!gate.open(indptr, n_row)) return;
   __shared__ uint32_t s_count, s_base;
   const uint32_t tid = threadIdx.x, lane = tid % kWave;
@@ -210,7 +212,7 @@ __global__ __launch_bounds__(kWinThreads) void collect_active_rows_kernel(
   const uint32_t base = s_base;
 #pragma unroll
   for (int e = 0; e < kCollectPerThread; ++e) {
-    if (on[e]) {
+    if (on[e] && base + at[e] < n_row) {
       list[base + at[e]] = make_uint2(start[e], len[e]);
       if (MODE == kDense) scales[base + at[e]] = scale[e];
     }
@@ -287,7 +289,7 @@ __global__ __launch_bounds__(kWinThreads) void collect_active_rows_batched_kerne
   const uint32_t base = s_base;
 #pragma unroll
   for (int e = 0; e < kPer; ++e) {
-    if (on[e]) {
+    if (on[e] && base + at[e] < total) {  // (the list holds batch * n_row entries)
       list[base + at[e]] = make_uint2(start[e], len[e]);
       colbase[base + at[e]] = base_col[e];
     }
@@ -351,7 +353,7 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
   if (active_list != nullptr) {
     const uint32_t launched = groups;
     if (launched % 8u == 0) g = (g % (launched / 8u)) * 8u + g / (launched / 8u);
-    groups = groups_in_use(active_count[0], indptr[n_row], n_row, launched);
+    groups = groups_in_use(active_count[0] < n_row ? active_count[0] : n_row, indptr[n_row], n_row, launched);
     if (g == 0 && b == 0 && threadIdx.x == 0) active_count[1] = groups;
     if (g >= groups) return;
   }
@@ -373,7 +375,7 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
   // taken kWinMaxRows at a time, the capacity of the list in LDS.
   uint32_t span_lo = 0, span_hi = rows_per_wg;
   if (active_list != nullptr) {
-    const uint32_t total = active_count[0];
+    const uint32_t total = active_count[0] < n_row ? active_count[0] : n_row;  // (the list's capacity)
     span_lo = static_cast<uint32_t>(static_cast<uint64_t>(g) * total / groups);
     span_hi = static_cast<uint32_t>(static_cast<uint64_t>(g + 1) * total / groups);
   }
@@ -837,9 +839,135 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
 // ------------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------------
+// ------------------------------------------------------------------------------------------------
+// scatter, small matrices with event input: one launch
+// ------------------------------------------------------------------------------------------------
+// Up to kSmallRows rows and kSmallCols columns (the synapses of one small population; the
+// reference's own benchmark network has 4,000 x 4,000) a call is bound by how many dependent
+// memory round trips and launches it needs, not by bandwidth.  One launch: workgroup b owns output
+// window b (at most 16 windows).  Every workgroup loads ALL events and ALL row bounds at once (one
+// round trip), lists the active rows in LDS, then groups of 16 lanes walk the listed rows (the
+// indices of the next step, which may belong to the group's next row, are requested before this
+// step's are used), add what falls into the window with LDS atomics (integer counts for a
+// homogeneous weight) and the window is stored straight to y: no partial outputs to sum, no
+// atomics on y, no zero fill.  Every workgroup streams all active nonzeros, so the time grows
+// with the activity; the launcher takes this path for small matrices only.
+constexpr uint32_t kSmallRows = 4096;
+constexpr uint32_t kSmallCols = 8192;
+constexpr uint32_t kSmallMaxWindows = 16;
+
+template <typename F, typename VT, bool HETER>
+__global__ __launch_bounds__(kWinThreads) void csr_scatter_small_kernel(
+    const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
+    const VT *__restrict__ x, F *__restrict__ y, uint32_t n_row, uint32_t n_col, uint32_t win) {
+  constexpr uint32_t kPer = kSmallRows / kWinThreads;  // rows tested per thread
+  constexpr uint32_t G = 16, U = 8;                    // lanes per row, nonzeros per lane and step
+  constexpr uint32_t kGroups = kWinThreads / G;
+  __shared__ uint32_t s_start[kSmallRows], s_len[kSmallRows];
+  __shared__ uint32_t s_count;
+  extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
+  F *window = reinterpret_cast<F *>(smem_raw);
+  uint32_t *cwindow = reinterpret_cast<uint32_t *>(smem_raw);
+  const uint32_t tid = threadIdx.x, lane = tid % kWave;
+  const uint32_t c0 = blockIdx.x * win;
+  const uint32_t width = (c0 + win <= n_col) ? win : n_col - c0;
+
+  // all events and row bounds: independent loads, issued together
+  VT ev[kPer];
+  uint32_t lo[kPer], hi[kPer];
+#pragma unroll
+  for (uint32_t k = 0; k < kPer; ++k) {
+    const uint32_t r = k * kWinThreads + tid;
+    ev[k] = VT(0);
+    lo[k] = hi[k] = 0;
+    if (r < n_row) {
+      ev[k] = x[r];
+      lo[k] = indptr[r];
+      hi[k] = indptr[r + 1];
+    }
+  }
+  const F w_homo = HETER ? F(0) : data[0];
+  if (tid == 0) s_count = 0;
+  for (uint32_t i = tid; i < width; i += kWinThreads) {
+    if (HETER) window[i] = F(0);
+    else cwindow[i] = 0u;
+  }
+  __syncthreads();
+#pragma unroll
+  for (uint32_t k = 0; k < kPer; ++k) {
+    const bool on = is_event(ev[k]) && hi[k] > lo[k];
+    const uint64_t mask = __ballot(on);
+    uint32_t base = 0;
+    if (lane == 0 && mask) base = atomicAdd(&s_count, static_cast<uint32_t>(__popcll(mask)));
+    base = __builtin_amdgcn_readfirstlane(base);
+    if (on) {
+      const uint32_t at = base + static_cast<uint32_t>(__popcll(mask & ((1ull << lane) - 1ull)));
+      s_start[at] = lo[k];
+      s_len[at] = hi[k] - lo[k];
+    }
+  }
+  __syncthreads();
+  const uint32_t count = s_count;
+
+  // group `gid` walks listed rows gid, gid + kGroups, ... in steps of G * U nonzeros
+  const uint32_t gid = tid / G, gl = tid % G;
+  auto load_rel = [&](uint32_t start, uint32_t b0, uint32_t len, uint32_t (&rel)[U]) {
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) {
+      const uint32_t j = b0 + u * G + gl;
+      rel[u] = 0xffffffffu;  // outside every window
+      if (j < len) rel[u] = indices[start + j] - c0;
+    }
+  };
+  uint32_t k = gid, start = 0, len = 0, b0 = 0;
+  uint32_t rel[U];
+  if (k < count) {
+    start = s_start[k], len = s_len[k];
+    load_rel(start, 0, len, rel);
+  }
+  while (k < count) {
+    uint32_t nk = k, nstart = start, nlen = len, nb0 = b0 + G * U;
+    if (nb0 >= len) {
+      nk = k + kGroups, nb0 = 0;
+      if (nk < count) nstart = s_start[nk], nlen = s_len[nk];
+    }
+    uint32_t nrel[U];
+    if (nk < count) load_rel(nstart, nb0, nlen, nrel);
+    if (HETER) {
+      F w[U];
+#pragma unroll
+      for (uint32_t u = 0; u < U; ++u) {
+        w[u] = F(0);
+        if (rel[u] < width) w[u] = data[start + b0 + u * G + gl];
+      }
+#pragma unroll
+      for (uint32_t u = 0; u < U; ++u)
+        if (rel[u] < width) atomicAdd(&window[rel[u]], w[u]);
+    } else {
+#pragma unroll
+      for (uint32_t u = 0; u < U; ++u)
+        if (rel[u] < width) atomicAdd(&cwindow[rel[u]], 1u);
+    }
+    k = nk, start = nstart, len = nlen, b0 = nb0;
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) rel[u] = nrel[u];
+  }
+  __syncthreads();
+  for (uint32_t i = tid; i < width; i += kWinThreads) {
+    if (HETER) {
+      y[c0 + i] = window[i];
+    } else {
+      // n synapses of weight w: n * w rounded once (nothing, not 0 * w, where no synapse arrived)
+      const uint32_t n = cwindow[i];
+      y[c0 + i] = n ? static_cast<F>(static_cast<double>(w_homo) * static_cast<double>(n)) : F(0);
+    }
+  }
+}
+
 template <typename F, typename VT, bool HETER, int MODE>
-void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, const uint32_t *indptr,
+void launch_scatter(const ScratchSource &src, const F *data, const uint32_t *indices, const uint32_t *indptr,
                     const VT *x, F *y, uint32_t n_row, uint32_t n_col) {
+  hipStream_t stream = src.stream;
   if (n_col == 0) return;
   if (n_row == 0) {
     fill_zero(stream, y, n_col);
@@ -851,19 +979,34 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
   // nonzero (about 21 G/s) for a few windows; a wave walks its rows one after the other.
   using A = typename std::conditional<MODE == kDense, double, F>::type;  // window accumulators
   const size_t list_bytes = kWinMaxRows * (8 + (MODE == kDense ? sizeof(F) : 0));
+  if constexpr (MODE == kEvent) {
+    if (n_row <= kSmallRows && n_col <= kSmallCols) {
+      uint32_t n_win = div_up(n_col, 256);
+      if (n_win > kSmallMaxWindows) n_win = kSmallMaxWindows;
+      const uint32_t win = div_up(n_col, n_win);
+      n_win = div_up(n_col, win);
+      hipLaunchKernelGGL((csr_scatter_small_kernel<F, VT, HETER>), dim3(n_win), dim3(kWinThreads),
+                         static_cast<size_t>(win) * sizeof(F), stream, data, indices, indptr, x, y, n_row, n_col, win);
+      return;
+    }
+  }
   const uint32_t win_cap = static_cast<uint32_t>((static_cast<size_t>(128) * 1024) / sizeof(A));
   const uint32_t n_win = div_up(n_col, win_cap);
   NnzGate direct_gate = kAlways;
+  auto round_up = [](size_t v) { return (v + 255) / 256 * 256; };
   // Event input and more than 8,192 outputs: the active rows' nonzeros are flattened and sorted
   // coarsely by output window instead (csr_bin_scatter.hip), at a cost that neither grows with the
   // number of windows nor with the number of rows a wave would have to walk in turn.
   if (MODE == kEvent && n_col > 8192 && bin_event_scatter_usable<F>(n_col)) {
-    const size_t list_sz = (static_cast<size_t>(n_row) * sizeof(uint2) + 255) / 256 * 256;
-    unsigned char *ws =
-        static_cast<unsigned char *>(stream_workspace(stream, list_sz + bin_event_scatter_bytes<F>(n_row, n_col)));
-    uint32_t *counters = ws ? stream_counters(stream) : nullptr;
+    const size_t list_sz = round_up(static_cast<size_t>(n_row) * sizeof(uint2));
+    size_t got = 0;
+    unsigned char *ws = static_cast<unsigned char *>(src.request(list_sz + bin_event_scatter_bytes<F>(n_row, n_col),
+                                                                 list_sz + bin_event_scatter_min_bytes<F>(n_col), &got));
+    uint32_t *counters = ws ? src.counters() : nullptr;
     if (ws != nullptr && counters != nullptr) {
       uint2 *active_list = reinterpret_cast<uint2 *>(ws);
+      // (a fixed arena is shared by every call on the device and keeps the last call's contents)
+      if (src.fixed()) fill_zero(stream, counters, 2u);
       // the kernel that lists the active rows also zeroes the windows' fill counters and, unless
       // the output is much longer than the input, y
       const unsigned collectors = collect_workgroups<F, VT, MODE>(n_row);
@@ -873,11 +1016,12 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
                                   reinterpret_cast<uint32_t *>(ws + list_sz),
                                   static_cast<uint32_t>(kBinEventFillBytes / sizeof(uint32_t)), y,
                                   fold_zero ? n_col : 0u);
-      if (bin_event_scatter<F>(stream, data, HETER, indices, indptr, y, n_row, n_col, counters, active_list,
-                               ws + list_sz))
+      if (bin_event_scatter<F>(stream, data, HETER, indices, indptr, y, n_row, n_col, counters, active_list, n_row,
+                               ws + list_sz, got - list_sz))
         return;
       fill_zero(stream, counters, 1u);  // (the sort could not run: the list is not used)
     } else {
+      if (src.failure_is_final()) return;  // beyond a fixed arena, or during a capture: the error stands
       bpl_clear_error();  // no scratch memory: the paths below need less or none
     }
   }
@@ -924,16 +1068,18 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
       // Per-row-group partial outputs in scratch memory, summed by a second kernel (no global
       // atomics, no zero fill), as long as they stay small; else atomics into the zeroed y.
       const size_t partial_bytes = static_cast<size_t>(groups) * n_col * sizeof(F);
-      const bool want_partial = groups > 1 && partial_bytes <= (static_cast<size_t>(64) << 20);
+      bool want_partial = groups > 1 && partial_bytes <= (static_cast<size_t>(64) << 20);
       // workspace: [active-row list][dense mode: their input values][partial outputs]
-      auto round_up = [](size_t v) { return (v + 255) / 256 * 256; };
       const size_t list_off = 0, list_sz = use_list ? round_up(static_cast<size_t>(n_row) * sizeof(uint2)) : 0;
       const size_t scale_sz = (use_list && MODE == kDense) ? round_up(static_cast<size_t>(n_row) * sizeof(F)) : 0;
       const size_t partial_off = list_sz + scale_sz;
       const size_t ws_bytes = partial_off + (want_partial ? partial_bytes : 0);
-      unsigned char *ws = ws_bytes ? static_cast<unsigned char *>(stream_workspace(stream, ws_bytes)) : nullptr;
-      uint32_t *counters = use_list ? stream_counters(stream) : nullptr;
+      size_t got = 0;
+      unsigned char *ws = ws_bytes ? static_cast<unsigned char *>(src.request(ws_bytes, partial_off, &got)) : nullptr;
+      if (ws != nullptr && got < ws_bytes) want_partial = false;  // (a fixed arena too small for the partial outputs)
+      uint32_t *counters = (use_list && (ws != nullptr || ws_bytes == 0)) ? src.counters() : nullptr;
       if (ws_bytes != 0 && (ws == nullptr || (use_list && counters == nullptr))) {
+        if (src.failure_is_final()) return;  // beyond a fixed arena, or during a capture: the error stands
         // no scratch memory: the direct kernel needs none
         bpl_clear_error();
         fill_zero(stream, y, n_col);
@@ -946,6 +1092,7 @@ void launch_scatter(hipStream_t stream, const F *data, const uint32_t *indices, 
       F *active_scales = scale_sz ? reinterpret_cast<F *>(ws + list_sz) : nullptr;
       uint32_t *active_count = use_list ? counters : nullptr;
       const bool gated = n_win > 4;
+      if (use_list && src.fixed()) fill_zero(stream, counters, 2u);
       if (partial == nullptr || gated) fill_zero(stream, y, n_col);
       if (use_list)
         launch_collect<F, VT, MODE>(stream, indptr, x, n_row, active_count, active_list, active_scales, window_gate,
@@ -1012,8 +1159,9 @@ bool launch_gather_impl(const char *target, hipStream_t stream, const F *data, c
 }
 
 template <typename F, typename VT, bool HETER, int MODE>
-void launch_gather(const char *target, hipStream_t stream, const F *data, const uint32_t *indices,
+void launch_gather(const char *target, const ScratchSource &src, const F *data, const uint32_t *indices,
                    const uint32_t *indptr, const VT *x, F *y, uint32_t n_row, uint32_t n_col) {
+  hipStream_t stream = src.stream;
   if (n_row == 0) return;
   if constexpr (MODE == kEvent && !std::is_same<VT, PackedBits>::value) {
     // A bitmap that does not fit LDS (more than 1.3 million columns): two levels, the exact one in
@@ -1022,8 +1170,7 @@ void launch_gather(const char *target, hipStream_t stream, const F *data, const 
       const uint32_t g = coarse_shift(n_col);
       const uint32_t n_words = (n_col + 31u) / 32u, off = coarse_offset_words(n_col);
       const uint32_t c_words = (coarse_bits(n_col, g) + 31u) / 32u;
-      uint32_t *bits = static_cast<uint32_t *>(
-          stream_workspace(stream, (static_cast<size_t>(off) + c_words + 1) * sizeof(uint32_t)));
+      uint32_t *bits = static_cast<uint32_t *>(src.request((static_cast<size_t>(off) + c_words + 1) * sizeof(uint32_t)));
       if (bits != nullptr) {
         pack_event_bitmap<VT>(stream, x, n_col, bits);
         hipLaunchKernelGGL(coarsen_bitmap_kernel, dim3(div_up(c_words, 256)), dim3(256), 0, stream, bits, n_words, g,
@@ -1033,6 +1180,7 @@ void launch_gather(const char *target, hipStream_t stream, const F *data, const 
                                                               n_col, static_cast<size_t>(c_words) * 4))
           return;
       }
+      if (src.failure_is_final()) return;  // beyond a fixed arena, or during a capture: the error stands
       bpl_clear_error();
     }
   }
@@ -1040,13 +1188,14 @@ void launch_gather(const char *target, hipStream_t stream, const F *data, const 
     // Wide event types: every persistent workgroup would read the whole vector (4 or 8 bytes per
     // element) to build its bitmap; pack it once instead and hand the words to the kernels.
     const size_t words = (static_cast<size_t>(n_col) + 31) / 32;
-    uint32_t *bits = static_cast<uint32_t *>(stream_workspace(stream, (words + 1) * sizeof(uint32_t)));
+    uint32_t *bits = static_cast<uint32_t *>(src.request((words + 1) * sizeof(uint32_t)));
     if (bits != nullptr) {
       pack_event_bitmap<VT>(stream, x, n_col, bits);
-      launch_gather<F, PackedBits, HETER, MODE>(target, stream, data, indices, indptr,
+      launch_gather<F, PackedBits, HETER, MODE>(target, src, data, indices, indptr,
                                                 reinterpret_cast<const PackedBits *>(bits), y, n_row, n_col);
       return;
     }
+    if (src.failure_is_final()) return;  // beyond a fixed arena, or during a capture: the error stands
     bpl_clear_error();
   }
   if (MODE == kEvent) {
@@ -1086,7 +1235,7 @@ void launch_gather(const char *target, hipStream_t stream, const F *data, const 
 
 // event_csr_matvec: buffers = [data, indices, indptr, events, out]
 template <typename F, typename VT, bool HETER>
-void event_csr_matvec_entry(const char *target, hipStream_t stream, void **buffers, const char *opaque,
+void event_csr_matvec_entry(const char *target, const ScratchSource &src, void **buffers, const char *opaque,
                             size_t opaque_len) {
   bpl_twouint_onebool_descriptor d;
   if (!unpack(target, opaque, opaque_len, &d)) return;
@@ -1100,10 +1249,10 @@ void event_csr_matvec_entry(const char *target, hipStream_t stream, void **buffe
   const VT *events = static_cast<const VT *>(buffers[3]);
   F *out = static_cast<F *>(buffers[4]);
   if (d.transpose) {
-    launch_scatter<F, VT, HETER, kEvent>(stream, data, indices, indptr, events, out, d.n_row, d.n_col);
+    launch_scatter<F, VT, HETER, kEvent>(src, data, indices, indptr, events, out, d.n_row, d.n_col);
     check_launch(target);
   } else {
-    launch_gather<F, VT, HETER, kEvent>(target, stream, data, indices, indptr, events, out, d.n_row, d.n_col);
+    launch_gather<F, VT, HETER, kEvent>(target, src, data, indices, indptr, events, out, d.n_row, d.n_col);
   }
 }
 
@@ -1134,13 +1283,14 @@ void csr_matvec_entry(const char *target, hipStream_t stream, void **buffers, co
     // further window means another pass over the whole matrix; the windows remain for matrices too
     // small to sort or of unknown size, direct atomics beyond four windows.)
     const uint32_t plain_windows = div_up(d.n_col, static_cast<uint32_t>((128u * 1024u) / sizeof(double)));
-    if (plain_windows > 1 && d.n_row > 0 && bin_scatter_usable<F>(d.n_col, nnz) &&
-        bin_scatter<F>(target, stream, data, HETER, indices, indptr, vec, out, d.n_row, d.n_col, nnz))
-      return;
-    launch_scatter<F, F, HETER, kDense>(stream, data, indices, indptr, vec, out, d.n_row, d.n_col);
+    if (plain_windows > 1 && d.n_row > 0 && bin_scatter_usable<F>(d.n_col, nnz)) {
+      if (bin_scatter<F>(target, stream, data, HETER, indices, indptr, vec, out, d.n_row, d.n_col, nnz)) return;
+      if (scratch_refused_by_capture()) return;  // (the error stands)
+    }
+    launch_scatter<F, F, HETER, kDense>(ScratchSource{stream}, data, indices, indptr, vec, out, d.n_row, d.n_col);
     check_launch(target);
   } else {
-    launch_gather<F, F, HETER, kDense>(target, stream, data, indices, indptr, vec, out, d.n_row, d.n_col);
+    launch_gather<F, F, HETER, kDense>(target, ScratchSource{stream}, data, indices, indptr, vec, out, d.n_row, d.n_col);
   }
 }
 
@@ -1416,8 +1566,8 @@ void event_csr_batching_entry(const char *target, hipStream_t stream, void **buf
       const size_t vrows = static_cast<size_t>(group) * d.n_row;
       const size_t list_sz = round_up(vrows * sizeof(uint2));
       const size_t base_sz = round_up(vrows * sizeof(uint32_t));
-      unsigned char *ws = static_cast<unsigned char *>(
-          stream_workspace(stream, list_sz + base_sz + bin_event_scatter_bytes<F>(d.n_row, vcols)));
+      const size_t scratch_bytes = bin_event_scatter_bytes<F>(d.n_row, vcols);
+      unsigned char *ws = static_cast<unsigned char *>(stream_workspace(stream, list_sz + base_sz + scratch_bytes));
       uint32_t *counters = ws ? stream_counters(stream) : nullptr;
       if (ws != nullptr && counters != nullptr) {
         uint2 *list = reinterpret_cast<uint2 *>(ws);
@@ -1434,7 +1584,7 @@ void event_csr_batching_entry(const char *target, hipStream_t stream, void **buf
                              static_cast<uint32_t>(kBinEventFillBytes / sizeof(uint32_t)), o,
                              static_cast<uint64_t>(g) * d.n_col);
           if (!bin_event_scatter<F>(stream, values, HETER, indices, indptr, o, d.n_row, g * d.n_col, counters, list,
-                                    scratch, colbase)) {
+                                    static_cast<uint32_t>(vrows), scratch, scratch_bytes, colbase)) {
             set_error("%s: the sorted scatter could not be enqueued", target);
             return;
           }
@@ -1442,6 +1592,7 @@ void event_csr_batching_entry(const char *target, hipStream_t stream, void **buf
         check_launch(target);
         return;
       }
+      if (scratch_refused_by_capture()) return;
       bpl_clear_error();
     }
   }
@@ -1452,10 +1603,10 @@ void event_csr_batching_entry(const char *target, hipStream_t stream, void **buf
     const VT *ev = events + static_cast<size_t>(bi % d.events_batch) * n_in;
     F *o = out + static_cast<size_t>(bi) * n_out;
     if (d.transpose) {
-      launch_scatter<F, VT, HETER, kEvent>(stream, v, ix, ip, ev, o, d.n_row, d.n_col);
+      launch_scatter<F, VT, HETER, kEvent>(ScratchSource{stream}, v, ix, ip, ev, o, d.n_row, d.n_col);
       if (!check_launch(target)) return;
     } else {
-      launch_gather<F, VT, HETER, kEvent>(target, stream, v, ix, ip, ev, o, d.n_row, d.n_col);
+      launch_gather<F, VT, HETER, kEvent>(target, ScratchSource{stream}, v, ix, ip, ev, o, d.n_row, d.n_col);
     }
   }
 }
@@ -1471,7 +1622,7 @@ void csr_event_sum_i32_entry(const char *target, hipStream_t stream, void **buff
     set_error("%s: null buffer table", target);
     return;
   }
-  launch_scatter<F, uint8_t, HETER, kEvent>(stream, static_cast<const F *>(buffers[3]),
+  launch_scatter<F, uint8_t, HETER, kEvent>(ScratchSource{stream}, static_cast<const F *>(buffers[3]),
                                             static_cast<const uint32_t *>(buffers[1]),
                                             static_cast<const uint32_t *>(buffers[2]),
                                             static_cast<const uint8_t *>(buffers[0]), static_cast<F *>(buffers[4]),
@@ -1494,14 +1645,14 @@ using bpl::event_csr_matvec_entry;
   }
 
 // bool events are read as bytes: any nonzero byte is an event
-BPL_DEFINE(event_csr_matvec_heter_float_bool, (event_csr_matvec_entry<float, uint8_t, true>(__func__, s, buffers, opaque, opaque_len)))
-BPL_DEFINE(event_csr_matvec_heter_float_float, (event_csr_matvec_entry<float, float, true>(__func__, s, buffers, opaque, opaque_len)))
-BPL_DEFINE(event_csr_matvec_heter_double_bool, (event_csr_matvec_entry<double, uint8_t, true>(__func__, s, buffers, opaque, opaque_len)))
-BPL_DEFINE(event_csr_matvec_heter_double_double, (event_csr_matvec_entry<double, double, true>(__func__, s, buffers, opaque, opaque_len)))
-BPL_DEFINE(event_csr_matvec_homo_float_bool, (event_csr_matvec_entry<float, uint8_t, false>(__func__, s, buffers, opaque, opaque_len)))
-BPL_DEFINE(event_csr_matvec_homo_float_float, (event_csr_matvec_entry<float, float, false>(__func__, s, buffers, opaque, opaque_len)))
-BPL_DEFINE(event_csr_matvec_homo_double_bool, (event_csr_matvec_entry<double, uint8_t, false>(__func__, s, buffers, opaque, opaque_len)))
-BPL_DEFINE(event_csr_matvec_homo_double_double, (event_csr_matvec_entry<double, double, false>(__func__, s, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_heter_float_bool, (event_csr_matvec_entry<float, uint8_t, true>(__func__, bpl::ScratchSource{s}, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_heter_float_float, (event_csr_matvec_entry<float, float, true>(__func__, bpl::ScratchSource{s}, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_heter_double_bool, (event_csr_matvec_entry<double, uint8_t, true>(__func__, bpl::ScratchSource{s}, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_heter_double_double, (event_csr_matvec_entry<double, double, true>(__func__, bpl::ScratchSource{s}, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_homo_float_bool, (event_csr_matvec_entry<float, uint8_t, false>(__func__, bpl::ScratchSource{s}, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_homo_float_float, (event_csr_matvec_entry<float, float, false>(__func__, bpl::ScratchSource{s}, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_homo_double_bool, (event_csr_matvec_entry<double, uint8_t, false>(__func__, bpl::ScratchSource{s}, buffers, opaque, opaque_len)))
+BPL_DEFINE(event_csr_matvec_homo_double_double, (event_csr_matvec_entry<double, double, false>(__func__, bpl::ScratchSource{s}, buffers, opaque, opaque_len)))
 
 BPL_DEFINE(csr_matvec_heter_scalar_float, (csr_matvec_entry<float, true, false>(__func__, s, buffers, opaque, opaque_len, 3)))
 BPL_DEFINE(csr_matvec_heter_scalar_double, (csr_matvec_entry<double, true, false>(__func__, s, buffers, opaque, opaque_len, 3)))

@@ -376,7 +376,10 @@ void launch_rowwalk_impl(hipStream_t stream, const VT *in, T1 *out, uint32_t n_o
   uint32_t *states = nullptr;
   if (n_out >= kSeedAheadMin)
     states = static_cast<uint32_t *>(stream_workspace(stream, static_cast<size_t>(kSeedChunk) * kMtN * 4));
-  if (states == nullptr) bpl_clear_error();
+  if (states == nullptr) {
+    if (n_out >= kSeedAheadMin && scratch_refused_by_capture()) return;
+    bpl_clear_error();
+  }
   const uint32_t chunk = states ? kSeedChunk : n_out;
   for (uint32_t first = 0; first < n_out; first += chunk) {
     const uint32_t count = (n_out - first < chunk) ? n_out - first : chunk;
@@ -413,6 +416,7 @@ void launch_rowwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
                                                       static_cast<size_t>(c_words) * 4 + 16 * state_bytes);
         return;
       }
+      if (scratch_refused_by_capture()) return;
       bpl_clear_error();
     }
   }
@@ -429,6 +433,7 @@ void launch_rowwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
                                             log_p, wa, wb);
       return;
     }
+    if (scratch_refused_by_capture()) return;
     bpl_clear_error();
   }
   const size_t state_bytes = StreamLds<T1, W>::words * 4;
@@ -520,6 +525,7 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
         if (list_count != nullptr) fill_zero(stream, list_count, 1u);
         fill_zero(stream, out, n_out);
       } else {
+        if (scratch_refused_by_capture()) return;
         bpl_clear_error();
       }
     }

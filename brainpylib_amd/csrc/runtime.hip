@@ -1,6 +1,7 @@
 // Host-side runtime of libbrainpylib_amd.so: error channel, device properties, descriptor
 // builders and the target registry.  Replaces the reference's lib/kernel_helpers.h,
 // lib/kernel_helper_descriptor.cu and the Registrations() table of lib/gpu_ops.cc.
+#include <atomic>
 #include <cstdarg>
 #include <cstddef>
 #include <cstdio>
@@ -15,6 +16,11 @@ namespace bpl {
 
 namespace {
 thread_local std::string t_error;
+thread_local bool t_refused_by_capture = false;
+// Set per device when a launch has failed: a pipeline that failed half way may have left the
+// stream counters of that device nonzero (its last kernel, which resets them, never ran).
+constexpr int kMaxDev = 64;
+std::atomic<bool> g_counters_suspect[kMaxDev];
 }
 
 void set_error(const char *fmt, ...) {
@@ -31,13 +37,15 @@ bool check_launch(const char *target) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     set_error("%s: launch failed: %s", target, hipGetErrorString(e));
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if (dev >= 0 && dev < kMaxDev) g_counters_suspect[dev].store(true);
     return false;
   }
   return true;
 }
 
 const DeviceInfo &device_info() {
-  constexpr int kMaxDev = 64;
   static DeviceInfo infos[kMaxDev];
   static bool known[kMaxDev] = {};
   static std::mutex mu;
@@ -59,42 +67,68 @@ const DeviceInfo &device_info() {
   return infos[dev];
 }
 
+namespace {
+struct WorkspaceEntry {
+  int dev;
+  hipStream_t stream;
+  void *ptr;
+  size_t bytes;
+};
+std::vector<WorkspaceEntry> g_workspaces;
+// Buffers that were handed out and then outgrown.  They stay allocated until the process ends:
+// kernels enqueued earlier and HIP graphs captured earlier may still read and write them.
+std::vector<WorkspaceEntry> g_retired;
+std::mutex g_workspace_mu;
+
+bool capturing(hipStream_t stream) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return st != hipStreamCaptureStatusNone;
+}
+}  // namespace
+
+bool scratch_refused_by_capture() { return t_refused_by_capture; }
+
 void *stream_workspace(hipStream_t stream, size_t bytes) {
-  struct Entry {
-    int dev;
-    hipStream_t stream;
-    void *ptr;
-    size_t bytes;
-  };
-  static std::vector<Entry> entries;
-  static std::mutex mu;
+  t_refused_by_capture = false;
   int dev = 0;
   (void)hipGetDevice(&dev);
-  std::lock_guard<std::mutex> lock(mu);
-  Entry *e = nullptr;
-  for (auto &x : entries)
+  std::lock_guard<std::mutex> lock(g_workspace_mu);
+  WorkspaceEntry *e = nullptr;
+  for (auto &x : g_workspaces)
     if (x.dev == dev && x.stream == stream) e = &x;
-  if (e == nullptr) {
-    entries.push_back(Entry{dev, stream, nullptr, 0});
-    e = &entries.back();
+  if (e != nullptr && e->bytes >= bytes) return e->ptr;
+  if (capturing(stream)) {
+    set_error("scratch memory of %zu bytes is needed while the stream is being captured (it holds %zu): run the "
+              "call once on this stream before capturing it", bytes, e ? e->bytes : size_t(0));
+    t_refused_by_capture = true;
+    return nullptr;
   }
-  if (e->bytes < bytes) {
-    // the old buffer may still be read by work already enqueued on this stream
-    if (e->ptr != nullptr) {
-      (void)hipStreamSynchronize(stream);
-      (void)hipFree(e->ptr);
-      e->ptr = nullptr;
-      e->bytes = 0;
-    }
-    const size_t want = bytes + bytes / 4;
-    if (hipMalloc(&e->ptr, want) != hipSuccess) {
+  // A quarter of head room, and at least twice the buffer it replaces, so that the retired
+  // buffers of a stream together stay below the size of its current one.
+  size_t got = bytes + bytes / 4;
+  if (e != nullptr && got < 2 * e->bytes) got = 2 * e->bytes;
+  void *fresh = nullptr;
+  if (hipMalloc(&fresh, got) != hipSuccess) {
+    (void)hipGetLastError();
+    fresh = nullptr;
+    got = bytes;  // (once more without the head room)
+    if (hipMalloc(&fresh, got) != hipSuccess) {
       (void)hipGetLastError();
-      e->ptr = nullptr;
-      set_error("workspace allocation of %zu bytes failed", want);
+      set_error("workspace allocation of %zu bytes failed", bytes);
       return nullptr;
     }
-    e->bytes = want;
   }
+  if (e == nullptr) {
+    g_workspaces.push_back(WorkspaceEntry{dev, stream, nullptr, 0});
+    e = &g_workspaces.back();
+  }
+  if (e->ptr != nullptr) g_retired.push_back(*e);
+  e->ptr = fresh;
+  e->bytes = got;
   return e->ptr;
 }
 
@@ -106,19 +140,49 @@ uint32_t *stream_counters(hipStream_t stream) {
   };
   static std::vector<Entry> entries;
   static std::mutex mu;
+  t_refused_by_capture = false;
   int dev = 0;
   (void)hipGetDevice(&dev);
   std::lock_guard<std::mutex> lock(mu);
+  if (dev >= 0 && dev < kMaxDev && g_counters_suspect[dev].exchange(false)) {
+    // a launch failed on this device since the counters were last handed out: zero them all, each
+    // on its own stream, before anything reads them again
+    for (auto &x : entries)
+      if (x.dev == dev) fill_zero(x.stream, x.ptr, static_cast<uint32_t>(kStreamCounterBytes / sizeof(uint32_t)));
+  }
   for (auto &x : entries)
     if (x.dev == dev && x.stream == stream) return x.ptr;
+  if (capturing(stream)) {
+    set_error("the stream's counters would be allocated while it is being captured: run the call once on this "
+              "stream before capturing it");
+    t_refused_by_capture = true;
+    return nullptr;
+  }
   uint32_t *p = nullptr;
-  constexpr size_t kBytes = 256;
-  if (hipMalloc(reinterpret_cast<void **>(&p), kBytes) != hipSuccess || hipMemset(p, 0, kBytes) != hipSuccess) {
+  if (hipMalloc(reinterpret_cast<void **>(&p), kStreamCounterBytes) != hipSuccess ||
+      hipMemset(p, 0, kStreamCounterBytes) != hipSuccess) {
     (void)hipGetLastError();
     return nullptr;
   }
   entries.push_back(Entry{dev, stream, p});
   return p;
+}
+
+void *ScratchSource::request(size_t want, size_t need, size_t *got) const {
+  if (need > want) want = need;
+  if (!fixed()) {
+    void *p = stream_workspace(stream, want);
+    *got = p ? want : 0;
+    return p;
+  }
+  if (need > arena_bytes) {
+    set_error("the call needs %zu bytes of scratch memory and the allocation-free entry point holds %zu", need,
+              arena_bytes);
+    *got = 0;
+    return nullptr;
+  }
+  *got = want < arena_bytes ? want : arena_bytes;
+  return arena;
 }
 
 }  // namespace bpl
@@ -285,6 +349,22 @@ bpl_target_fn bpl_find_target(const char *name) {
   for (int i = 0; i < kNumTargets; ++i)
     if (std::strcmp(kTargets[i].name, name) == 0) return kTargets[i].fn;
   return nullptr;
+}
+
+int bpl_stream_workspace_query(bpl_stream_t stream, void **ptr, size_t *bytes, size_t *retired_bytes) {
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  std::lock_guard<std::mutex> lock(bpl::g_workspace_mu);
+  void *p = nullptr;
+  size_t n = 0, r = 0;
+  for (const auto &x : bpl::g_workspaces)
+    if (x.dev == dev && x.stream == static_cast<hipStream_t>(stream)) p = x.ptr, n = x.bytes;
+  for (const auto &x : bpl::g_retired)
+    if (x.dev == dev && x.stream == static_cast<hipStream_t>(stream)) r += x.bytes;
+  if (ptr != nullptr) *ptr = p;
+  if (bytes != nullptr) *bytes = n;
+  if (retired_bytes != nullptr) *retired_bytes = r;
+  return p != nullptr;
 }
 
 const char *bpl_last_error(void) { return bpl::t_error.c_str(); }

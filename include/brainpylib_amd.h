@@ -188,6 +188,19 @@ void bpl_clear_error(void);
 /* Library version string. */
 const char *bpl_version(void);
 
+/* Scratch memory.  The custom-call ABI carries no workspace operand, so operators that need
+ * staging memory (lists of active rows, sorted (column, weight) pairs, packed event bitmaps,
+ * seeded generator states) take it from one allocation per (device, stream) that the library
+ * makes with hipMalloc on first use and keeps until the process ends.  When a call needs more
+ * than the stream's buffer holds, a larger buffer is allocated and the old one is retired but
+ * never freed (earlier work and HIP graphs captured earlier may still use it).  While a stream is
+ * being captured into a HIP graph nothing can be allocated: a call that would have to fails with
+ * an error and enqueues nothing, so run every shape once on the stream before capturing it.
+ * This query reports the current buffer of `stream` on the current device (its address and size)
+ * and the bytes of retired buffers; it returns 0 if the stream has no buffer yet.  Any of the
+ * three pointers may be NULL. */
+int bpl_stream_workspace_query(bpl_stream_t stream, void **ptr, size_t *bytes, size_t *retired_bytes);
+
 /* ------------------------------------------------------------------------------------------
  * event_csr_matvec  (lib/gpu_event_csr_matvec.cu:222-260; launchers :148-217)
  *   buffers = [data, indices, indptr, events, out]

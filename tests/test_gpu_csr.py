@@ -595,3 +595,36 @@ def test_csr_matvec_with_the_vector_staged_in_lds(cuda, oracle_mod, dtype):
       got = bpl.csr_matvec(d, indices, indptr, v, shape=shape).cpu().numpy()
       assert got.dtype == dtype
       assert_close(got, want, what="csr_matvec %s" % (shape,))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_small_event_scatter_in_one_launch(cuda, oracle_mod, dtype):
+  # up to 4,096 rows and 8,192 columns one launch does the whole transposed product (every output
+  # window's workgroup tests all events and walks all active rows); sizes on both sides of that
+  # limit, windows of 1 .. 512 columns, every row active, empty rows, rows of several steps
+  rng = np.random.default_rng(31)
+  for n_row, n_col, mean, rate in ((4000, 4000, 80, 0.02), (4096, 8192, 20, 1.0), (4097, 8192, 20, 0.3),
+                                   (4096, 8193, 20, 0.3), (300, 7, 5, 0.5), (3000, 257, 3, 0.9), (1, 1, 1, 1.0),
+                                   (4000, 4097, 700, 0.01), (17, 8000, 3000, 0.5)):
+    counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_row + n_col)
+    data = rng.standard_normal(indices.shape[0]).astype(dtype)
+    ev = rng.random(n_row) < rate
+    shape = (n_row, n_col)
+    print("shape", shape, dtype.__name__, flush=True)
+    want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True)
+    mag = oracle_mod.event_csr_matvec(np.abs(data), indices, indptr, ev, shape=shape, transpose=True)
+    got = bpl.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+    assert_close_reordered(got, want, mag, dtype, what="small scatter heter")
+    evf = (ev * rng.uniform(0.5, 2.0, n_row)).astype(dtype)
+    got = bpl.event_csr_matvec(data, indices, indptr, evf, shape=shape, transpose=True).cpu().numpy()
+    assert_close_reordered(got, want, mag, dtype, what="small scatter heter, float events")
+    # unit weight: counts, exact; integer weights: exact in any order
+    ones = np.ones(1, dtype=dtype)
+    want = oracle_mod.event_csr_matvec(ones, indices, indptr, ev, shape=shape, transpose=True)
+    got = bpl.event_csr_matvec(ones, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+    assert np.array_equal(got, want)
+    di = rng.integers(-2, 3, size=indices.shape[0]).astype(dtype)
+    want = oracle_mod.event_csr_matvec(di, indices, indptr, ev, shape=shape, transpose=True)
+    got = bpl.event_csr_matvec(di, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+    assert np.array_equal(got, want)
