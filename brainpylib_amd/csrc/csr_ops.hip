@@ -21,6 +21,7 @@
 //
 // Reference boundary: lib/gpu_event_csr_matvec.cu:148-260, lib/gpu_csr_matvec.cu:84-135,195-246,
 // 505-621 (buffer order, descriptor, target names).
+#include <mutex>
 #include <type_traits>
 
 #include "common.h"
@@ -1632,6 +1633,76 @@ void csr_event_sum_i32_entry(const char *target, hipStream_t stream, void **buff
 
 }  // namespace
 }  // namespace bpl
+
+// ------------------------------------------------------------------------------------------------
+// Allocation-free entry point
+// ------------------------------------------------------------------------------------------------
+// event_csr_matvec_heter_float_bool for callers that cannot allocate device memory (code under HIP
+// graph capture, serving loops, harnesses that forbid hipMalloc): the scratch memory of the call
+// (stream counters, the list of active rows, fill counters and runs of the sorted scatter, partial
+// outputs of the window scatter, packed event bitmaps) lives in this file-scope device array
+// instead of the cached allocation.  Every GPU the library runs on holds its own copy of the array,
+// at its own address, until the process ends; all calls on a GPU share it, so calls that overlap
+// on one GPU (different streams) race.  It keeps the last call's contents: the launchers zero the
+// counters they use before the first kernel that reads them.
+namespace bpl {
+namespace {
+constexpr size_t kStaticScratchBytes = static_cast<size_t>(64) << 20;  // 64 MiB of arena behind the counters
+}  // namespace
+}  // namespace bpl
+
+static __device__ __align__(256) unsigned char scratch[bpl::kStreamCounterBytes + bpl::kStaticScratchBytes];
+
+namespace bpl {
+namespace {
+// Device address of `scratch` on the current device, looked up once per device.  (In host code the
+// array's name is a stand-in for the symbol, not a device address: only this pointer may be handed to
+// kernels.)
+unsigned char *static_scratch(const char *target) {
+  constexpr int kMaxDev = 64;
+  static unsigned char *ptrs[kMaxDev] = {};
+  static std::mutex mu;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) {
+    (void)hipGetLastError();
+    set_error("%s: no current device", target);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptrs[dev] == nullptr) {
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      (void)hipGetLastError();
+      set_error("%s: hipGetSymbolAddress of the static scratch array failed on device %d: %s", target, dev,
+                hipGetErrorString(e));
+      return nullptr;
+    }
+    ptrs[dev] = static_cast<unsigned char *>(p);
+  }
+  return ptrs[dev];
+}
+}  // namespace
+}  // namespace bpl
+
+extern "C" void event_csr_matvec_heter_float_bool_noalloc(bpl_stream_t stream, void **buffers, const char *opaque,
+                                                          size_t opaque_len) {
+  // (a malformed call is refused before the device is touched)
+  bpl_twouint_onebool_descriptor d;
+  if (!bpl::unpack(__func__, opaque, opaque_len, &d)) return;
+  if (buffers == nullptr) {
+    bpl::set_error("%s: null buffer table", __func__);
+    return;
+  }
+  unsigned char *base = bpl::static_scratch(__func__);
+  if (base == nullptr) return;
+  bpl::ScratchSource src;
+  src.stream = static_cast<hipStream_t>(stream);
+  src.arena_counters = reinterpret_cast<uint32_t *>(base);
+  src.arena = base + bpl::kStreamCounterBytes;
+  src.arena_bytes = bpl::kStaticScratchBytes;
+  bpl::event_csr_matvec_entry<float, uint8_t, true>(__func__, src, buffers, opaque, opaque_len);
+}
 
 using bpl::csr_event_sum_i32_entry;
 using bpl::csr_matvec_entry;

@@ -10,7 +10,8 @@
   X(event_csr_matvec_homo_float_bool)       \
   X(event_csr_matvec_homo_float_float)      \
   X(event_csr_matvec_homo_double_bool)      \
-  X(event_csr_matvec_homo_double_double)
+  X(event_csr_matvec_homo_double_double)    \
+  X(event_csr_matvec_heter_float_bool_noalloc)
 
 #define BPL_CSR_TARGETS(X)                  \
   X(csr_matvec_heter_scalar_float)          \

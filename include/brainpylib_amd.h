@@ -222,6 +222,24 @@ BPL_TARGET(event_csr_matvec_homo_float_float);
 BPL_TARGET(event_csr_matvec_homo_double_bool);
 BPL_TARGET(event_csr_matvec_homo_double_double);
 
+/* event_csr_matvec_heter_float_bool that allocates nothing.  No counterpart in the reference: it
+ * is for callers that cannot allocate device memory inside the call -- code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  Same buffers, same descriptor,
+ * same result as event_csr_matvec_heter_float_bool; the scratch memory that target takes from the
+ * cached per-stream allocation (active-row list, counters, sorted runs, partial outputs, packed
+ * bitmaps) lives in a static device array of 64 MiB (+ 256 bytes of counters) that every GPU
+ * the library runs on holds until the process ends.  The call makes no hipMalloc / hipFree.
+ *   Limits: a call whose scratch memory does not fit is rejected with an error and enqueues
+ *   nothing.  transpose, more than 8,192 columns: 8 bytes per row + 128 KiB + 64 KiB per output
+ *   window (at most 128 windows) must fit, i.e. any n_col with n_row <= 7,000,000; runs that
+ *   overflow the rest of the array (about 7 million active nonzeros per call when n_row is
+ *   100,000) are added with direct atomics, more slowly but correctly.  transpose, up to 8,192
+ *   columns: 8 bytes per row.  no transpose: nothing up to 1,302,528 columns, n_col / 8 bytes +
+ *   160 KiB beyond.
+ *   All calls on one GPU share the array: calls that overlap on one GPU (different streams)
+ *   race; calls on one stream, or ordered by events, are safe. */
+BPL_TARGET(event_csr_matvec_heter_float_bool_noalloc);
+
 /* ------------------------------------------------------------------------------------------
  * event_csr_matvec_batching  (the batching rule's primitive,
  * brainpylib/_src/event_ops/event_csr_matvec.py:112-193, which the reference runs on the CPU
