@@ -176,7 +176,7 @@ def main():
 
   import torch
   import brainpylib_amd as bpl
-  from brainpylib_amd import synth
+  import benchdata as synth
   import oracle  # checker and CPU baseline only
 
   assert torch.cuda.is_available(), "bench.py needs a HIP device"

@@ -127,8 +127,8 @@ class _JitconnMatvec(torch.autograd.Function):
 
 
 def _run(fn_prefix, w_kind, inp, out_dtype, suffix, **kw):
-  if inp.is_floating_point() and (inp.requires_grad or (torch.autograd.forward_ad._current_level >= 0 and
-                                                        torch.autograd.forward_ad.unpack_dual(inp).tangent is not None)):
+  if inp.is_floating_point() and (inp.requires_grad or
+                                  torch.autograd.forward_ad.unpack_dual(inp).tangent is not None):
     # move first (differentiably), so that the gradient comes back on the caller's device
     return _JitconnMatvec.apply(to_device(inp, device_of(inp)), fn_prefix, w_kind, out_dtype, suffix, kw)
   return _launch(fn_prefix, w_kind, inp, out_dtype, suffix, **kw)

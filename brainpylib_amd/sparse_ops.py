@@ -110,11 +110,11 @@ def _launch(data, indices, indptr, vector, shape, transpose, method='vector'):
 
 def _wants_grad(*tensors):
   """True if a floating-point argument takes part in reverse- or forward-mode differentiation."""
-  forward = torch.autograd.forward_ad._current_level >= 0  # a dual level is open
   for t in tensors:
     if t.requires_grad:
       return True
-    if forward and t.is_floating_point() and torch.autograd.forward_ad.unpack_dual(t).tangent is not None:
+    # (outside a dual level unpack_dual returns at once with no tangent)
+    if t.is_floating_point() and torch.autograd.forward_ad.unpack_dual(t).tangent is not None:
       return True
   return False
 

@@ -35,7 +35,7 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
 import oracle  # noqa: E402
 from oracle import ref  # noqa: E402
-from brainpylib_amd import synth  # noqa: E402
+import benchdata as synth  # noqa: E402
 
 JIT_SHAPES = [(100, 200), (10, 1000), (2, 1000), (1000, 10), (1000, 2)]
 PROBS = [0.01, 0.1, 0.5]

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import brainpylib_amd as bpl
-from brainpylib_amd import synth
+import benchdata as synth
 from util import assert_close_reordered
 
 pytestmark = pytest.mark.gpu

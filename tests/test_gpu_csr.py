@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import brainpylib_amd as bpl
-from brainpylib_amd import synth
+import benchdata as synth
 from util import CSR_SHAPES, assert_close, assert_close_reordered, random_csr
 
 pytestmark = pytest.mark.gpu

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 import brainpylib_amd as bpl
-from brainpylib_amd import synth
+import benchdata as synth
 from util import assert_close, assert_close_reordered, batched_csr
 
 pytestmark = pytest.mark.gpu

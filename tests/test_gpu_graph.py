@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import brainpylib_amd as bpl
-from brainpylib_amd import synth
+import benchdata as synth
 
 pytestmark = pytest.mark.gpu
 

@@ -13,7 +13,8 @@ import pytest
 import torch
 
 import brainpylib_amd as bpl
-from brainpylib_amd import _lib, synth
+from brainpylib_amd import _lib
+import benchdata as synth
 from util import JIT_SHAPES, assert_close, assert_close_reordered
 
 pytestmark = pytest.mark.gpu

@@ -8,7 +8,8 @@ import pytest
 import torch
 
 import brainpylib_amd as bpl
-from brainpylib_amd import _lib, synth
+from brainpylib_amd import _lib
+import benchdata as synth
 
 pytestmark = pytest.mark.gpu
 

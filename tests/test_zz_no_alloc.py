@@ -10,7 +10,8 @@ import numpy as np
 import pytest
 import torch
 
-from brainpylib_amd import _lib, synth
+from brainpylib_amd import _lib
+import benchdata as synth
 from util import assert_close_reordered
 
 pytestmark = pytest.mark.gpu

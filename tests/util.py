@@ -1,7 +1,7 @@
 """Helpers shared by the tests: seeded inputs, dense brute force, tolerance check."""
 import numpy as np
 
-from brainpylib_amd import synth
+import benchdata as synth
 
 # north_star tolerance for fp32 outputs (atomics may reorder additions)
 RTOL, ATOL = 1e-5, 1e-6
