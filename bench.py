@@ -24,11 +24,60 @@ if ROOT not in sys.path:
   sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
-GATHER_TRAFFIC_BYTES = 740.1e6  # measured HBM traffic of one launch of the headline kernel (see main())
+# Counter readings cannot be taken in-process: the figures that come from rocprofv3 --pmc runs are kept in
+# this file together with the kernel name, the workload, the kernel duration and the git revision they were
+# taken at, and are only emitted while the run's own timing still agrees with them.
+RECORDED_COUNTERS = os.path.join(ROOT, "profiles", "recorded_counters.json")
+BENCH_SRC = os.path.join(ROOT, "bench_kernels.hip")
+BENCH_LIB = os.path.join(ROOT, "libbench_kernels.so")
 
 
 def log(*a):
   print(*a, file=sys.stderr, flush=True)
+
+
+def build_kernels(force=False):
+  """Compiles bench_kernels.hip (the measurement kernels: flat gather, plain stream) for gfx950."""
+  from brainpylib_amd import build as b
+  if force or b._newer(BENCH_LIB, [BENCH_SRC]):
+    b._run([b.HIPCC] + b.HIP_FLAGS + ["-shared", BENCH_SRC, "-o", BENCH_LIB])
+  return BENCH_LIB
+
+
+def load_kernels():
+  import ctypes
+  if not os.path.exists(BENCH_LIB):
+    build_kernels()
+  lib = ctypes.CDLL(BENCH_LIB)
+  vp, u64, i = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int
+  lib.bench_gather_fma.argtypes = [vp, vp, vp, vp, vp, u64, i, i, i]
+  lib.bench_gather_fma.restype = i
+  lib.bench_gather_fma4.argtypes = [vp, vp, vp, vp, vp, u64, i, i, i, i, i]
+  lib.bench_gather_fma4.restype = i
+  lib.bench_stream.argtypes = [vp, vp, vp, u64, i, i]
+  lib.bench_stream.restype = i
+  return lib
+
+
+def recorded_counters(key, kernel_us, tolerance=0.05, **must_match):
+  """The entry `key` of profiles/recorded_counters.json if it still describes this run: the fields in
+  `must_match` are equal and the kernel's duration measured now is within `tolerance` of the one at
+  which the counters were read.  Else None (and the reason on stderr)."""
+  try:
+    with open(RECORDED_COUNTERS) as f:
+      entry = json.load(f)[key]
+  except (OSError, KeyError, ValueError) as e:
+    log("recorded counters: no usable entry %r (%s)" % (key, e))
+    return None
+  for k, v in must_match.items():
+    if entry.get(k) != v:
+      log("recorded counters %r: %s is %r there, %r here: not used" % (key, k, entry.get(k), v))
+      return None
+  if abs(kernel_us - entry["kernel_us"]) > tolerance * entry["kernel_us"]:
+    log("recorded counters %r: kernel took %.1f us when they were read, %.1f us now: not used" % (
+      key, entry["kernel_us"], kernel_us))
+    return None
+  return entry
 
 
 def time_calls(fn, steps, warmup):
@@ -76,6 +125,67 @@ def copy_bandwidth_gb_per_s(dev, n_bytes=1 << 30):
   b = torch.empty_like(a)
   dur, _ = time_calls(lambda: b.copy_(a), 20, 3)
   return 2.0 * n_bytes / (float(np.median(dur)) * 1e-3) / 1e9
+
+
+def gather_ceiling(lib, dev, x, idx, w, steps):
+  """What a kernel that does csr_matvec's work per nonzero WITHOUT the row structure reaches on this
+  device: acc += x[idx[j]] * w[j] over the flat index and weight streams (two coalesced streams, one
+  random 4-byte read of the vector per nonzero), at the occupancies and numbers of loads in flight a CSR
+  product can run with, the streams read 4 bytes per lane or 16 bytes per lane with the nontemporal hint.
+  The best rate is the ceiling of any product that gathers the vector from L2."""
+  import ctypes
+  import torch
+  n = int(idx.numel())
+  cu = torch.cuda.get_device_properties(dev).multi_processor_count
+  stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+  rows = []
+  for per_cu, threads, inflight in ((2, 1024, 4), (2, 1024, 8), (1, 1024, 8), (4, 512, 8), (8, 256, 8)):
+    blocks = cu * per_cu
+    out = torch.zeros(blocks * threads, dtype=torch.float32, device=dev)
+    fn = lambda: lib.bench_gather_fma(stream, x.data_ptr(), idx.data_ptr(), w.data_ptr(), out.data_ptr(), n, blocks,
+                                      threads, inflight)
+    if fn() != 0:
+      raise SystemExit("bench_gather_fma failed to launch")
+    d, _ = time_calls(fn, steps, 2)
+    rows.append(dict(stream_loads="4 bytes", workgroups_per_cu=per_cu, threads=threads, loads_in_flight=inflight,
+                     us=float(d.mean() * 1e3), g_gathers_per_s=n / (d.mean() * 1e-3) / 1e9,
+                     checksum=float(out.double().sum().item())))
+  n4 = n - n % 4
+  for per_cu, threads, quads, pieces in ((2, 1024, 4, 1), (1, 1024, 4, 1), (2, 512, 4, 1), (2, 512, 4, 8), (4, 512, 2, 1)):
+    blocks = cu * per_cu
+    out = torch.zeros(blocks * threads, dtype=torch.float32, device=dev)
+    fn = lambda: lib.bench_gather_fma4(stream, x.data_ptr(), idx.data_ptr(), w.data_ptr(), out.data_ptr(), n4, blocks,
+                                       threads, quads, 1, pieces)
+    if fn() != 0:
+      raise SystemExit("bench_gather_fma4 failed to launch")
+    d, _ = time_calls(fn, steps, 2)
+    tail = float((x[idx[n4:].long()].double() * w[n4:].double()).sum().item())
+    rows.append(dict(stream_loads="16 bytes, nontemporal, %d piece(s) per instruction" % pieces, workgroups_per_cu=per_cu,
+                     threads=threads, loads_in_flight=4 * quads, us=float(d.mean() * 1e3),
+                     g_gathers_per_s=n4 / (d.mean() * 1e-3) / 1e9, checksum=float(out.double().sum().item()) + tail))
+  return rows
+
+
+def stream_ceiling(lib, dev, n_bytes, steps):
+  """GB/s of plain 16-byte loads over `n_bytes` of HBM at a persistent kernel's occupancies: the read rate a
+  streaming kernel reaches on this device (the published peak is not reachable by any kernel)."""
+  import ctypes
+  import torch
+  n16 = n_bytes // 16
+  buf = torch.empty(n16 * 4, dtype=torch.int32, device=dev).random_()
+  cu = torch.cuda.get_device_properties(dev).multi_processor_count
+  stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+  rows = []
+  for per_cu, threads in ((2, 1024), (1, 1024), (4, 512), (8, 256)):
+    blocks = cu * per_cu
+    out = torch.zeros(blocks * threads, dtype=torch.int32, device=dev)
+    fn = lambda: lib.bench_stream(stream, buf.data_ptr(), out.data_ptr(), n16, blocks, threads)
+    if fn() != 0:
+      raise SystemExit("bench_stream failed to launch")
+    d, _ = time_calls(fn, steps, 2)
+    rows.append(dict(workgroups_per_cu=per_cu, threads=threads, us=float(d.mean() * 1e3),
+                     gb_per_s=n16 * 16 / (d.mean() * 1e-3) / 1e9))
+  return rows
 
 
 def back_to_back_us(fn, calls):
@@ -159,12 +269,16 @@ def main():
   ap.add_argument("--warmup", type=int, default=20)
   ap.add_argument("--skip-extra", action="store_true", help="only the headline workload")
   ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU baseline")
-  ap.add_argument("--pmc", choices=["gather", "scatter", "jitconn", "jitconn-normal"], default=None,
+  ap.add_argument("--pmc", choices=["gather", "scatter", "csr", "jitconn", "jitconn-normal", "jitconn-dense", "matmat"],
+                  default=None,
                   help="counter-collection mode for rocprofv3 --pmc.  gather: three plain copies of 400 MB "
-                       "(the calibration kernel) and three calls of the headline kernel.  scatter: three calls of "
-                       "the same matrix with transpose=True.  jitconn: three calls "
+                       "(the calibration kernel), three calls of the headline kernel and three plain streams over "
+                       "740 MB.  scatter: three calls of the same matrix with transpose=True.  csr: three calls of "
+                       "csr_matvec on the 1,000,000 x 1,000,000 matrix in each orientation and three flat gathers over "
+                       "the same index and weight streams.  jitconn: three calls "
                        "of jitconn event matvec (1e6 x 1e6, p=0.001) in both walks.  jitconn-normal: three "
-                       "row walks of the same matrix with normal weights.  Nothing else runs.")
+                       "row walks of the same matrix with normal weights.  jitconn-dense: three row walks over a "
+                       "dense vector.  matmat: three calls of jitconn matmat 10,000 x 10,000 x 128.  Nothing else runs.")
   ap.add_argument("--reference-shapes", action="store_true",
                   help="instead of the headline run: the shapes of the reference's own benchmark scripts "
                        "(event_matvec_jitconn_performance.py, csr_matvec_VS_cusparse_csr_matvec.py), with the "
@@ -195,6 +309,45 @@ def main():
       for _ in range(3):
         bpl.event_matvec_prob_conn_homo_weight(ev, j["weight"], conn_prob=j["conn_prob"], shape=j["shape"],
                                                seed=j["seed"], outdim_parallel=odp)
+    torch.cuda.synchronize()
+    log("pmc mode done")
+    return
+
+  if args.pmc == "jitconn-dense":
+    j = synth.config_jitconn_event()
+    vec = torch.randn(j["shape"][0], dtype=torch.float32, device=dev)
+    for _ in range(3):
+      bpl.matvec_prob_conn_homo_weight(vec, j["weight"], conn_prob=j["conn_prob"], shape=j["shape"], seed=j["seed"],
+                                       outdim_parallel=True)
+    torch.cuda.synchronize()
+    log("pmc mode done")
+    return
+
+  if args.pmc == "matmat":
+    mm = synth.config_jitconn_matmat()
+    X = torch.from_numpy(np.ascontiguousarray(mm["B"].T)).to(dev)
+    for _ in range(3):
+      bpl.matmat_prob_conn_normal_weight(X, w_mu=mm["w_mu"], w_sigma=mm["w_sigma"], conn_prob=mm["conn_prob"],
+                                         shape=mm["shape"], seed=mm["seed"])
+    torch.cuda.synchronize()
+    log("pmc mode done")
+    return
+
+  if args.pmc == "csr":
+    import ctypes
+    m = synth.config_csr_matvec()
+    md = {k: torch.from_numpy(v).to(dev) for k, v in m.items() if isinstance(v, np.ndarray)}
+    for _ in range(3):
+      bpl.csr_matvec(md["data"], md["indices"], md["indptr"], md["vector"], shape=m["shape"])
+    for _ in range(3):
+      bpl.cusparse_csr_matvec(md["data"], md["indices"], md["indptr"], md["vector"], shape=m["shape"], transpose=True)
+    lib = load_kernels()
+    cu = torch.cuda.get_device_properties(dev).multi_processor_count
+    out = torch.zeros(cu * 2 * 1024, dtype=torch.float32, device=dev)
+    for _ in range(3):
+      lib.bench_gather_fma(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), md["vector"].data_ptr(),
+                           md["indices"].data_ptr(), md["data"].data_ptr(), out.data_ptr(), md["indices"].numel(),
+                           cu * 2, 1024, 8)
     torch.cuda.synchronize()
     log("pmc mode done")
     return
@@ -255,6 +408,15 @@ def main():
     for _ in range(3):
       bpl.event_csr_matvec(data, indices, indptr, events, shape=c["shape"])
     torch.cuda.synchronize()
+    import ctypes
+    lib = load_kernels()
+    cu = torch.cuda.get_device_properties(dev).multi_processor_count
+    buf = torch.empty(740_000_000 // 4, dtype=torch.int32, device=dev).random_()
+    out = torch.zeros(cu * 2 * 1024, dtype=torch.int32, device=dev)
+    for _ in range(3):
+      lib.bench_stream(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), buf.data_ptr(), out.data_ptr(),
+                       740_000_000 // 16, cu * 2, 1024)
+    torch.cuda.synchronize()
     log("pmc mode done")
     return
 
@@ -280,10 +442,18 @@ def main():
   one = single_call_us(gather)
   copy_rate = copy_bandwidth_gb_per_s(dev)
   extra["hbm_copy_gb_per_s"] = copy_rate  # 1 GiB device-to-device copy, read + write
-  if nnz == 100014049:
-    extra["gather_hbm_traffic_gb_per_s"] = GATHER_TRAFFIC_BYTES / (kernel_ms * 1e-3) / 1e9
-    extra["gather_traffic_over_copy_rate"] = extra["gather_hbm_traffic_gb_per_s"] / copy_rate
   log("device-to-device copy of 1 GiB: %.0f GB/s (read + write)" % copy_rate)
+  # what plain 16-byte loads over the same number of bytes reach at this kernel's occupancy
+  bench_lib = load_kernels()
+  rec = recorded_counters("event_csr_gather_1e8", kernel_ms * 1e3, nnz=nnz)
+  traffic = float(rec["hbm_bytes_per_launch"]) if rec else None
+  streams = stream_ceiling(bench_lib, dev, int(traffic) if traffic else bytes_gather, 20)
+  stream_rate = max(r["gb_per_s"] for r in streams)
+  extra["hbm_stream_read"] = dict(best_gb_per_s=stream_rate, runs=streams)
+  log("plain 16-byte loads: %s" % streams)
+  if traffic:
+    extra["gather_hbm_traffic_gb_per_s"] = traffic / (kernel_ms * 1e-3) / 1e9
+    extra["gather_traffic_over_copy_rate"] = extra["gather_hbm_traffic_gb_per_s"] / copy_rate
   extra["gather_single_call_wall_us"] = dict(cold_first_in_process=cold_gather_us, warm_median=one["median"])
 
   # ---------------------------------------------------------------------------------------------
@@ -450,6 +620,18 @@ def main():
     extra["csr_matvec_1e8"] = dict(stats(dur3), nnz=nnz3, gsop_per_s=nnz3 / (dur3.mean() * 1e-3) / 1e9,
                                    algorithmic_gb_per_s=bytes3 / (dur3.mean() * 1e-3) / 1e9,
                                    cpu_port_allcores_ms=t_cpu3 * 1e3, cpu_cores=cores)
+    # Its bound: the rate at which 4-byte elements of a 4 MB vector can be gathered from L2 at all, measured
+    # here by a flat kernel over the same index and weight streams (no rows, no reduction, no output).
+    ceil_rows = gather_ceiling(bench_lib, dev, md["vector"], md["indices"], md["data"], 10)
+    want_sum = float(np.dot(m["vector"][m["indices"]].astype(np.float64), m["data"].astype(np.float64)))
+    for r in ceil_rows:
+      if abs(r["checksum"] - want_sum) > 1e-4 * abs(want_sum) + 1.0:
+        raise SystemExit("flat gather kernel computed %r, expected %r" % (r["checksum"], want_sum))
+    ceiling = max(r["g_gathers_per_s"] for r in ceil_rows)
+    extra["csr_matvec_1e8"]["roofline"] = dict(
+      bound="l2-gather", unit="G gathers/s", achieved=extra["csr_matvec_1e8"]["gsop_per_s"], peak=ceiling,
+      frac=extra["csr_matvec_1e8"]["gsop_per_s"] / ceiling, peak_measured_by="bench_gather_fma, best of runs",
+      runs=ceil_rows, hbm_frac=bytes3 / (dur3.mean() * 1e-3) / 1e9 / HBM_PEAK_GBS)
     log("csr_matvec 1e8: %s" % extra["csr_matvec_1e8"])
     want = oracle.csr_matvec(m["data"], m["indices"], m["indptr"], m["vector"], shape=m["shape"], transpose=True)
     mag = oracle.csr_matvec(m["data"], m["indices"], m["indptr"], np.abs(m["vector"]), shape=m["shape"], transpose=True)
@@ -460,6 +642,11 @@ def main():
                                                           shape=m["shape"], transpose=True), max(20, args.steps // 4), 5)
     extra["csr_matvec_transposed_1e8"] = dict(stats(dur3t), gsop_per_s=nnz3 / (dur3t.mean() * 1e-3) / 1e9,
                                               algorithmic_gb_per_s=bytes3 / (dur3t.mean() * 1e-3) / 1e9)
+    # the sorted scatter writes and reads every (column, product) pair once more: 8 + 16 bytes per nonzero
+    extra["csr_matvec_transposed_1e8"]["roofline"] = dict(
+      bound="hbm", unit="GB/s", achieved=bytes3 / (dur3t.mean() * 1e-3) / 1e9, peak=HBM_PEAK_GBS,
+      frac=bytes3 / (dur3t.mean() * 1e-3) / 1e9 / HBM_PEAK_GBS,
+      bytes_moved_by_design_gb_per_s=(bytes3 + 16.0 * nnz3) / (dur3t.mean() * 1e-3) / 1e9)
     log("csr_matvec transposed 1e8: %s" % extra["csr_matvec_transposed_1e8"])
     # a dense vector short enough for LDS (up to 159 KB): 200,000 x 19,000, 100 per row, 2.0e7 nnz
     rng_s = np.random.default_rng(23)
@@ -517,8 +704,7 @@ def main():
     props = torch.cuda.get_device_properties(dev)
     clock_hz = float(getattr(props, "clock_rate", 2400000)) * 1e3
     jit["valu_roofline"] = {"bound": "valu", "peak_lane_instr_per_s": props.multi_processor_count * 64 * clock_hz,
-                            "compute_units": props.multi_processor_count, "clock_ghz": clock_hz / 1e9,
-                            "busy_frac_recorded": 0.897}
+                            "compute_units": props.multi_processor_count, "clock_ghz": clock_hz / 1e9}
     for transpose in (False, True):
       for odp in (True, False):
         fn = lambda: bpl.event_matvec_prob_conn_homo_weight(ev, j["weight"], conn_prob=j["conn_prob"], shape=j["shape"],
@@ -526,6 +712,13 @@ def main():
         d, _ = time_calls(fn, max(10, args.steps // 10), 3)
         key = "transpose=%s,outdim_parallel=%s" % (transpose, odp)
         jit[key] = dict(stats(d), implicit_gsyn_per_s=generated / (d.mean() * 1e-3) / 1e9)
+    call_us = jit["transpose=False,outdim_parallel=True"]["mean_us"]
+    rec_j = recorded_counters("jitconn_rowwalk_1e9", call_us, generated_synapses=generated)
+    jit["valu_roofline"]["busy_frac_recorded"] = rec_j["valu_busy_frac"] if rec_j else None
+    jit["valu_roofline"]["valu_instr_per_64_synapses_recorded"] = rec_j["valu_instr_per_64_synapses"] if rec_j else None
+    jit["valu_roofline"]["recorded_in"] = rec_j["profile"] if rec_j else None
+    jit["valu_roofline"]["recorded_at"] = dict(git_rev=rec_j["git_rev"], kernel=rec_j["kernel"],
+                                               call_us=rec_j["kernel_us"]) if rec_j else None
     if not args.skip_cpu:
       # reference CPU algorithm (one sequential mt19937) on the first 4,000 rows of the same matrix
       rows = 4000
@@ -603,11 +796,18 @@ def main():
                            "weights N(0,0.1^2), events Bernoulli(0.05), transpose=False, seed 1" % nnz},
     # traffic: HBM bytes per launch of this kernel on this workload, from two rocprofv3 --pmc runs (FETCH_SIZE,
     # WRITE_SIZE; `--pmc gather` mode above) scaled by what a 400 MB copy reads on the same counters; counters
-    # cannot be read in-process, so the figure is a recorded constant for exactly this workload
+    # cannot be read in-process, so the figure is the one recorded in profiles/recorded_counters.json, emitted
+    # only while this run's kernel time agrees with the time at which it was recorded (else null)
     "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                 "frac": achieved / HBM_PEAK_GBS, "traffic": GATHER_TRAFFIC_BYTES if nnz == 100014049 else None,
+                 "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                 "traffic_recorded_in": rec["profile"] if rec else None,
+                 "traffic_recorded_at": dict(git_rev=rec["git_rev"], kernel=rec["kernel"],
+                                             kernel_us=rec["kernel_us"]) if rec else None,
                  "kernel": "csr_gather_kernel<float,bool,heter,event,lds-bitmap>",
-                 "algorithmic_bytes_per_launch": bytes_gather, "kernel_us": kernel_ms * 1e3},
+                 "algorithmic_bytes_per_launch": bytes_gather, "kernel_us": kernel_ms * 1e3,
+                 # the same launch against what plain loads of its real traffic reach in this run
+                 "streaming_ceiling_gb_per_s": stream_rate,
+                 "frac_of_streaming_ceiling": (traffic / (kernel_ms * 1e-3) / 1e9 / stream_rate) if traffic else None},
     "cpu_baseline": cpu_baseline,
     "extra": extra,
   }

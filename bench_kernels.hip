@@ -5,6 +5,10 @@
 //                      what csr_matvec does per nonzero (two coalesced streams and one random
 //                      4-byte read of the vector), at the same occupancy.  Its rate is the ceiling
 //                      of any CSR product that gathers the vector from L2.
+//   bench_gather_fma4  the same with the two streams read 16 bytes per lane (four consecutive nonzeros per
+//                      request), optionally with the nontemporal hint, and with the lanes of an
+//                      instruction reading either one contiguous kilobyte or eight pieces of 128 bytes
+//                      (what groups of 8 lanes per CSR row read).
 //   bench_stream       plain 16-byte loads over a buffer, at the same occupancy: the HBM read
 //                      rate a streaming kernel reaches on this device.
 #include <hip/hip_runtime.h>
@@ -31,6 +35,55 @@ __global__ __launch_bounds__(1024) void gather_fma_kernel(const float *__restric
   }
   for (; base < n; base += total) acc += static_cast<double>(x[idx[base]] * w[base]);
   out[gtid] = static_cast<float>(acc);
+}
+
+// A wave takes blocks of U * 64 consecutive quads.  SEG lanes read consecutive quads in one instruction:
+// SEG = 64: an instruction reads 1 KB in one piece; SEG = 8: it reads 8 pieces of 128 bytes that lie
+// U * 128 bytes apart.
+template <int U, bool NT, int SEG>
+__global__ __launch_bounds__(1024) void gather_fma4_kernel(const float *__restrict__ x, const uint4 *__restrict__ idx,
+                                                           const float4 *__restrict__ w, float *__restrict__ out,
+                                                           uint64_t n4) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  const uint32_t lane = threadIdx.x % 64;
+  const uint64_t waves = static_cast<uint64_t>(gridDim.x) * (blockDim.x / 64);
+  const uint64_t wave = static_cast<uint64_t>(blockIdx.x) * (blockDim.x / 64) + threadIdx.x / 64;
+  double acc = 0.0;
+  for (uint64_t b = wave; (b + 1) * (U * 64) <= n4; b += waves) {
+    u32x4 c[U];
+    f32x4 d[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint64_t at = b * (U * 64) + (lane / SEG) * (U * SEG) + u * SEG + lane % SEG;
+      if (NT) {
+        c[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(idx) + at);
+        d[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(w) + at);
+      } else {
+        c[u] = reinterpret_cast<const u32x4 *>(idx)[at];
+        d[u] = reinterpret_cast<const f32x4 *>(w)[at];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float a0 = x[c[u].x] * d[u].x, a1 = x[c[u].y] * d[u].y, a2 = x[c[u].z] * d[u].z, a3 = x[c[u].w] * d[u].w;
+      acc += static_cast<double>(a0);
+      acc += static_cast<double>(a1);
+      acc += static_cast<double>(a2);
+      acc += static_cast<double>(a3);
+    }
+  }
+  // the quads that do not fill a block
+  const uint64_t done = n4 / (U * 64) * (U * 64);
+  for (uint64_t at = done + wave * 64 + lane; at < n4; at += waves * 64) {
+    const uint4 c = idx[at];
+    const float4 d = w[at];
+    acc += static_cast<double>(x[c.x] * d.x);
+    acc += static_cast<double>(x[c.y] * d.y);
+    acc += static_cast<double>(x[c.z] * d.z);
+    acc += static_cast<double>(x[c.w] * d.w);
+  }
+  out[static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x] = static_cast<float>(acc);
 }
 
 __global__ __launch_bounds__(1024) void stream_kernel(const uint4 *__restrict__ p, uint32_t *__restrict__ out,
@@ -67,6 +120,33 @@ int bench_gather_fma(void *stream, const float *x, const uint32_t *idx, const fl
   else if (loads_in_flight == 4) hipLaunchKernelGGL(gather_fma_kernel<4>, dim3(blocks), dim3(threads), 0, s, x, idx, w, out, n);
   else if (loads_in_flight == 8) hipLaunchKernelGGL(gather_fma_kernel<8>, dim3(blocks), dim3(threads), 0, s, x, idx, w, out, n);
   else return 1;
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+
+// The same over n (a multiple of 4) nonzeros with 16-byte stream loads.  quads_in_flight 1, 2 or 4;
+// nontemporal != 0: the two streams are read with the nontemporal hint; pieces: 1 or 8 (see the kernel).
+int bench_gather_fma4(void *stream, const float *x, const uint32_t *idx, const float *w, float *out, uint64_t n,
+                      int blocks, int threads, int quads_in_flight, int nontemporal, int pieces) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (blocks <= 0 || threads <= 0 || threads > 1024 || threads % 64 != 0 || n % 4 != 0) return 1;
+  if (pieces != 1 && pieces != 8) return 1;
+  const uint4 *i4 = reinterpret_cast<const uint4 *>(idx);
+  const float4 *w4 = reinterpret_cast<const float4 *>(w);
+#define BPL_LAUNCH4(U, NT, SEG) \
+  hipLaunchKernelGGL((gather_fma4_kernel<U, NT, SEG>), dim3(blocks), dim3(threads), 0, s, x, i4, w4, out, n / 4)
+#define BPL_PICK(U)                                   \
+  do {                                                \
+    if (nontemporal && pieces == 1) BPL_LAUNCH4(U, true, 64);  \
+    else if (nontemporal) BPL_LAUNCH4(U, true, 8);    \
+    else if (pieces == 1) BPL_LAUNCH4(U, false, 64);  \
+    else BPL_LAUNCH4(U, false, 8);                    \
+  } while (0)
+  if (quads_in_flight == 1) BPL_PICK(1);
+  else if (quads_in_flight == 2) BPL_PICK(2);
+  else if (quads_in_flight == 4) BPL_PICK(4);
+  else return 1;
+#undef BPL_PICK
+#undef BPL_LAUNCH4
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 

@@ -25,6 +25,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "csr_quad_gather.h"
 #include "targets.h"
 
 namespace bpl {
@@ -769,7 +770,7 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
                                                           const uint32_t *__restrict__ indices,
                                                           const uint32_t *__restrict__ indptr,
                                                           const VT *__restrict__ x, F *__restrict__ y,
-                                                          uint32_t n_row, uint32_t n_col) {
+                                                          uint32_t n_row, uint32_t n_col, uint32_t skip_mean) {
   extern __shared__ __attribute__((aligned(16))) uint32_t s_bits[];
   uint32_t coarse_g = 0;
   if constexpr (MODE == kDense) {
@@ -803,6 +804,10 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
   }
   // lanes per row from the mean row length
   const uint32_t mean = nnz / n_row;
+  if constexpr (MODE == kDense && BITS == 0) {
+    // (rows of `skip_mean` nonzeros or more on average: the launcher's other kernel has taken this matrix)
+    if (skip_mean != 0 && mean >= skip_mean) return;
+  }
   if constexpr (MODE == kDense && BITS == 1) {
     // (nothing left to hide but the index and weight streams: the walks of the event gather)
     const VT *xs = reinterpret_cast<const VT *>(s_bits);
@@ -1122,7 +1127,7 @@ void launch_scatter(const ScratchSource &src, const F *data, const uint32_t *ind
 template <typename F, typename VT, bool HETER, int MODE, int BITS>
 bool launch_gather_impl(const char *target, hipStream_t stream, const F *data, const uint32_t *indices,
                         const uint32_t *indptr, const VT *x, F *y, uint32_t n_row, uint32_t n_col,
-                        size_t lds_bytes) {
+                        size_t lds_bytes, uint32_t skip_mean = 0) {
   auto kernel = csr_gather_kernel<F, VT, HETER, MODE, BITS>;
   // Small problems: 256-thread workgroups, one wave per row at most.  Large ones: 1024-thread
   // persistent workgroups so that few copies of the event bitmap are built.
@@ -1155,7 +1160,7 @@ bool launch_gather_impl(const char *target, hipStream_t stream, const F *data, c
   const unsigned needed = div_up(n_row, block / kWave);  // one wave per row
   const unsigned grid = needed < resident ? (needed ? needed : 1u) : resident;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), lds_bytes, stream, data, indices, indptr, x, y, n_row,
-                     n_col);
+                     n_col, skip_mean);
   return check_launch(target);
 }
 
@@ -1229,6 +1234,20 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
                                                     kLdsBitmapCap))
         return;
       bpl_clear_error();
+    }
+    if constexpr (std::is_same<F, VT>::value) {
+      // A longer vector is gathered from L2.  Rows of 24 nonzeros or more on average: the walk that reads the
+      // index and weight streams 16 bytes per lane (csr_quad_gather.hip); shorter ones: the walks below.
+      // The mean is known on the device only, so both kernels are enqueued and one of them returns at once.
+      constexpr uint32_t kQuadMinMean = 24;
+      if (n_row >= 16384 && n_col > 0) {
+        if (csr_quad_gather<F>(target, stream, data, HETER, indices, indptr, x, y, n_row, kQuadMinMean)) {
+          launch_gather_impl<F, VT, HETER, MODE, 0>(target, stream, data, indices, indptr, x, y, n_row, n_col, 0,
+                                                    kQuadMinMean);
+          return;
+        }
+        bpl_clear_error();
+      }
     }
   }
   launch_gather_impl<F, VT, HETER, MODE, 0>(target, stream, data, indices, indptr, x, y, n_row, n_col, 0);

@@ -628,3 +628,69 @@ def test_small_event_scatter_in_one_launch(cuda, oracle_mod, dtype):
     want = oracle_mod.event_csr_matvec(di, indices, indptr, ev, shape=shape, transpose=True)
     got = bpl.event_csr_matvec(di, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_csr_matvec_with_16_byte_stream_loads(cuda, oracle_mod, dtype):
+  # at least 16,384 rows, a vector too long for LDS and 24 nonzeros or more per row on average: the walk
+  # that reads four consecutive nonzeros per lane and request.  Every lanes-per-row choice of that walk
+  # (means 30 .. 900), a mean just below its limit (the other kernel runs), nnz not a multiple of 4, empty
+  # rows, rows of one nonzero, hub rows that go to the whole workgroup, both weight kinds.
+  rng = np.random.default_rng(71)
+  limit = 4 * (160 * 1024 - 1024) // np.dtype(dtype).itemsize + 1  # first length that is not staged at all
+  for n_row, n_col, mean, hubs in ((20_000, limit, 30, 0), (16_384, limit + 3, 60, 2), (17_001, 400_000, 100, 3),
+                                   (16_400, 300_000, 250, 1), (16_390, 200_000, 500, 0), (16_385, 170_000, 900, 1),
+                                   (40_000, 1_000_000, 23, 0), (30_000, 250_000, 24, 40)):
+    counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
+    counts[rng.integers(0, n_row, 50)] = 0
+    counts[rng.integers(0, n_row, 50)] = 1
+    for h in range(hubs):
+      counts[rng.integers(0, n_row)] = min(n_col, (5_000, 70_000, 150_000)[h % 3])
+    if counts.sum() % 4 == 0:
+      counts[0] += 1
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_row)
+    data = rng.standard_normal(indices.shape[0]).astype(dtype)
+    v = rng.standard_normal(n_col).astype(dtype)
+    shape = (n_row, n_col)
+    print("shape", shape, "nnz", indices.shape[0], flush=True)
+    for d in (data, np.array([0.75], dtype=dtype)):
+      want = oracle_mod.csr_matvec(d, indices, indptr, v, shape=shape)
+      got = bpl.csr_matvec(d, indices, indptr, v, shape=shape).cpu().numpy()
+      assert got.dtype == dtype
+      assert_close(got, want, what="csr_matvec %s" % (shape,))
+  # operands that do not start on a 16-byte boundary: the 4-byte walks take the call
+  dev = torch.device("cuda:0")
+  big_i = torch.from_numpy(np.concatenate([[0], indices]).astype(np.int32)).to(dev)[1:]
+  big_d = torch.from_numpy(np.concatenate([[0], data]).astype(dtype)).to(dev)[1:]
+  assert big_i.data_ptr() % 16 != 0
+  got = bpl.csr_matvec(big_d, big_i, indptr, v, shape=shape).cpu().numpy()
+  assert_close(got, oracle_mod.csr_matvec(data, indices, indptr, v, shape=shape), what="unaligned operands")
+
+
+def test_csr_matvec_hub_row_time(cuda):
+  # one row with a million nonzeros among 20,000 ordinary ones must not serialise the call: the whole
+  # workgroup walks it (a single wave took milliseconds)
+  rng = np.random.default_rng(5)
+  n_row, n_col = 20_000, 2_000_000
+  counts = np.full(n_row, 50)
+  counts[777] = 1_000_000
+  indices, indptr = synth.counted_csr(counts, n_col, seed=9)
+  data = rng.integers(-2, 3, size=indices.shape[0]).astype(np.float32)
+  v = rng.integers(-3, 4, size=n_col).astype(np.float32)
+  dev = torch.device("cuda:0")
+  args = [torch.from_numpy(a).to(dev) for a in (data, indices, indptr, v)]
+  got = bpl.csr_matvec(*args, shape=(n_row, n_col))
+  # small integers: exact in any order
+  rows = np.repeat(np.arange(n_row), counts)
+  want = np.bincount(rows, weights=data.astype(np.float64) * v[indices], minlength=n_row)
+  assert np.array_equal(got.cpu().numpy().astype(np.float64), want)
+  torch.cuda.synchronize()
+  e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+  e0.record()
+  for _ in range(5):
+    bpl.csr_matvec(*args, shape=(n_row, n_col))
+  e1.record()
+  torch.cuda.synchronize()
+  per_call_us = e0.elapsed_time(e1) * 1e3 / 5
+  print("hub row of 1e6 nonzeros: %.1f us per call" % per_call_us, flush=True)
+  assert per_call_us < 500.0
