@@ -534,8 +534,10 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
                      stream, in, out, n_out, n_in, seed, log_p, wa, wb);
 }
 
-// buffers = [input, out]
-template <typename T1, typename VT, int IN, int W, bool COLWALK>
+// buffers = [input, out].  RAW_PROB: the descriptor's probability field holds conn_prob itself, as the
+// reference packs it for its first-generation dense-vector targets (matvec.py:338-343); the walk then uses
+// the log_p its CPU path derives from it (matvec.py:298), so that both versions give one matrix.
+template <typename T1, typename VT, int IN, int W, bool COLWALK, bool RAW_PROB = false>
 void jitconn_entry(const char *target, hipStream_t stream, void **buffers, const char *opaque, size_t opaque_len) {
   uint32_t n_row, n_col, seed;
   double log_p, a = 0, b = 0;
@@ -547,6 +549,14 @@ void jitconn_entry(const char *target, hipStream_t stream, void **buffers, const
     bpl_jitconn_prob_weight_descriptor d;
     if (!unpack(target, opaque, opaque_len, &d)) return;
     n_row = d.n_row, n_col = d.n_col, seed = d.seed, log_p = d.log_p, a = d.w_a, b = d.w_b;
+  }
+  if (RAW_PROB) {
+    const double p = log_p;
+    if (!(p > 0.0) || std::isinf(p)) {
+      set_error("%s: conn_prob must be in (0, 1], got %g", target, p);
+      return;
+    }
+    log_p = std::log(p < 1.0 ? 1.0 - p : 1e-40);
   }
   if (!valid_log_p(target, log_p)) return;
   if (buffers == nullptr) {
@@ -587,9 +597,17 @@ using namespace bpl;
   BPL_DEFINE(gpu_matvec_atomic_prob_##wname##_v2_float, float, float, kInDense, W, true)      \
   BPL_DEFINE(gpu_matvec_atomic_prob_##wname##_v2_double, double, double, kInDense, W, true)
 
+// the reference's first-generation names (lib/gpu_ops.cc:143-148): row walk only, conn_prob in the descriptor
+#define BPL_DENSE_V1_FAMILY(wname, W)                                                        \
+  BPL_DEFINE(gpu_matvec_prob_##wname##_v1_float, float, float, kInDense, W, false, true)      \
+  BPL_DEFINE(gpu_matvec_prob_##wname##_v1_double, double, double, kInDense, W, false, true)
+
 BPL_EVENT_FAMILY(homo, kHomo)
 BPL_EVENT_FAMILY(uniform, kUniform)
 BPL_DENSE_FAMILY(homo, kHomo)
 BPL_DENSE_FAMILY(uniform, kUniform)
 BPL_EVENT_FAMILY(normal, kNormal)
 BPL_DENSE_FAMILY(normal, kNormal)
+BPL_DENSE_V1_FAMILY(homo, kHomo)
+BPL_DENSE_V1_FAMILY(uniform, kUniform)
+BPL_DENSE_V1_FAMILY(normal, kNormal)

@@ -67,7 +67,13 @@
   X(gpu_matvec_prob_normal_v2_float) \
   X(gpu_matvec_prob_normal_v2_double) \
   X(gpu_matvec_atomic_prob_normal_v2_float) \
-  X(gpu_matvec_atomic_prob_normal_v2_double)
+  X(gpu_matvec_atomic_prob_normal_v2_double) \
+  X(gpu_matvec_prob_homo_v1_float) \
+  X(gpu_matvec_prob_homo_v1_double) \
+  X(gpu_matvec_prob_uniform_v1_float) \
+  X(gpu_matvec_prob_uniform_v1_double) \
+  X(gpu_matvec_prob_normal_v1_float) \
+  X(gpu_matvec_prob_normal_v1_double)
 
 #define BPL_JITCONN_HASH_TARGETS(X) \
   X(gpu_event_matvec_prob_homo_float) \

@@ -75,20 +75,24 @@ def _type_name(dt):
 
 
 def _launch(fn_prefix, w_kind, inp, out_dtype, suffix, *, conn_prob, shape, seed, transpose, outdim_parallel,
-            w_a=0.0, w_b=0.0):
+            w_a=0.0, w_b=0.0, version='v2'):
   n_row, n_col = (shape[1], shape[0]) if transpose else (shape[0], shape[1])
   if not (conn_prob > 0):
     raise ValueError(f'conn_prob should be in (0, 1], got {conn_prob}.')
+  name = fn_prefix + ('' if outdim_parallel else '_atomic') + '_prob_' + w_kind + '_' + version + suffix
+  if version == 'v1' and not outdim_parallel:
+    # matvec.py:355-358 builds this name, lib/gpu_ops.cc registers no such target
+    raise _lib.GPUOperatorNotFound(name)
   device = device_of(inp)
   inp = to_device(inp, device)
-  log_p = _log_p(conn_prob)
+  # version 1 descriptors carry conn_prob itself (matvec.py:338-343), version 2 log(1 - conn_prob)
+  log_p = float(conn_prob) if version == 'v1' else _log_p(conn_prob)
   if w_kind == 'homo':
     opaque = _lib.build_jitconn_prob_homo_descriptor(n_row, n_col, seed, log_p)
   elif w_kind == 'uniform':
     opaque = _lib.build_jitconn_prob_uniform_descriptor(n_row, n_col, seed, log_p, w_a, w_b)
   else:
     opaque = _lib.build_jitconn_prob_normal_descriptor(n_row, n_col, seed, log_p, w_a, w_b)
-  name = fn_prefix + ('' if outdim_parallel else '_atomic') + '_prob_' + w_kind + '_v2' + suffix
   out = torch.empty(n_row, dtype=out_dtype, device=device)
   _lib.custom_call(name, [inp, out], opaque)
   return out
@@ -114,7 +118,7 @@ class _JitconnMatvec(torch.autograd.Function):
   def backward(ctx, ct):
     if ct is None or not ctx.needs_input_grad[0]:
       return None, None, None, None, None, None
-    kw = dict(ctx.kw, transpose=not ctx.kw['transpose'], outdim_parallel=not ctx.kw['outdim_parallel'])
+    kw = dict(ctx.kw, transpose=not ctx.kw['transpose'], outdim_parallel=not ctx.kw['outdim_parallel'], version='v2')
     g = _launch('gpu_matvec', ctx.w_kind, ct.contiguous(), ct.dtype, _type_name(ct.dtype), **kw)
     return g, None, None, None, None, None
 
@@ -224,17 +228,21 @@ def event_matvec_prob_conn_hashed(events, *, w_kind: str = 'homo', weight=1.0, w
   return _apply_weight(out, weight) if w_kind == 'homo' else out
 
 
+def _check_version(version):
+  """matvec.py:102.  Both versions give the matrix of the reference's CPU path, which has one kernel for
+  either (matvec.py:296-308)."""
+  assert version in ['v1', 'v2']
+
+
 def matvec_prob_conn_homo_weight(vector, weight, *, conn_prob: float, shape: Tuple[int, int],
                                  seed: Optional[int] = None, transpose: bool = False, outdim_parallel: bool = True,
                                  version: str = 'v2'):
   """``y = M @ vector`` with ``M`` drawn just in time with the scalar ``weight`` at each connection."""
   vector = _dense(vector)
   _check_vector(vector, shape, transpose, 'vector')
-  assert version in ['v1', 'v2']
-  if version != 'v2':
-    raise _lib.GPUOperatorNotFound('matvec_prob_homo version v1 (superseded Bernoulli-per-entry kernel)')
+  _check_version(version)
   r = _run('gpu_matvec', 'homo', vector, vector.dtype, _type_name(vector.dtype), conn_prob=conn_prob, shape=shape,
-           seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel)
+           seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, version=version)
   return _apply_weight(r, weight)
 
 
@@ -245,11 +253,11 @@ def matvec_prob_conn_uniform_weight(vector, *, w_low: float, w_high: float, conn
   vector = _dense(vector)
   assert w_high > w_low
   _check_vector(vector, shape, transpose, 'vector')
-  if version != 'v2':
-    raise _lib.GPUOperatorNotFound('matvec_prob_uniform version v1 (superseded Bernoulli-per-entry kernel)')
+  _check_version(version)
   w_min, w_range = _uniform_range(w_low, w_high, vector.dtype)
   return _run('gpu_matvec', 'uniform', vector, vector.dtype, _type_name(vector.dtype), conn_prob=conn_prob, shape=shape,
-              seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, w_a=w_min, w_b=w_range)
+              seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, w_a=w_min, w_b=w_range,
+              version=version)
 
 
 def matvec_prob_conn_normal_weight(vector, *, w_mu: float, w_sigma: float, conn_prob: float, shape: Tuple[int, int],
@@ -258,10 +266,10 @@ def matvec_prob_conn_normal_weight(vector, *, w_mu: float, w_sigma: float, conn_
   """``y = M @ vector`` with each connection's weight drawn from N(w_mu, w_sigma^2)."""
   vector = _dense(vector)
   _check_vector(vector, shape, transpose, 'vector')
-  if version != 'v2':
-    raise _lib.GPUOperatorNotFound('matvec_prob_normal version v1 (superseded Bernoulli-per-entry kernel)')
+  _check_version(version)
   return _run('gpu_matvec', 'normal', vector, vector.dtype, _type_name(vector.dtype), conn_prob=conn_prob, shape=shape,
-              seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, w_a=w_mu, w_b=w_sigma)
+              seed=_seed(seed), transpose=transpose, outdim_parallel=outdim_parallel, w_a=w_mu, w_b=w_sigma,
+              version=version)
 
 
 def _matmat(w_kind, matrix, w_a, w_b, conn_prob, shape, seed, version):

@@ -433,6 +433,24 @@ BPL_TARGET(gpu_matvec_atomic_prob_normal_v2_float);
 BPL_TARGET(gpu_matvec_atomic_prob_normal_v2_double);
 
 /* ------------------------------------------------------------------------------------------
+ * jitconn dense matvec under the reference's first-generation names (lib/gpu_ops.cc:143-148,
+ * built by matvec.py:338-343,475-482,623-630 for version='v1', outdim_parallel=True only).
+ *   buffers and descriptors as for the version 2 row walk, except that the descriptor's
+ *   probability field holds conn_prob itself (lib/kernel_helper_descriptor.cuh:49-54); the
+ *   library derives log_p = log(1 - conn_prob) (log(1e-40) at conn_prob >= 1) from it, as the
+ *   reference's CPU path does for either version (matvec.py:296-308, one cpu_matvec_prob_* name
+ *   for both).  The matrix therefore is the version 2 matrix: on the reference's CPU path the
+ *   version does not change the result, and its own first-generation GPU kernels
+ *   (a cuRAND Bernoulli test per entry, lib/gpu_jitconn_matvec.cu) are not followed.
+ * ---------------------------------------------------------------------------------------- */
+BPL_TARGET(gpu_matvec_prob_homo_v1_float);
+BPL_TARGET(gpu_matvec_prob_homo_v1_double);
+BPL_TARGET(gpu_matvec_prob_uniform_v1_float);
+BPL_TARGET(gpu_matvec_prob_uniform_v1_double);
+BPL_TARGET(gpu_matvec_prob_normal_v1_float);
+BPL_TARGET(gpu_matvec_prob_normal_v1_double);
+
+/* ------------------------------------------------------------------------------------------
  * jitconn event matvec, first kernel generation ("hash" connectivity)
  *   (lib/gpu_jitconn_event_matvec.cu:10-79,138-215,281-362; names lib/gpu_ops.cc:107-112;
  *   generators lib/kernel_helpers_random.cuh:12-71)

@@ -60,7 +60,8 @@ def test_reference_registry_keys_of_the_other_operators_present():
       want += ["gpu_event_matvec_prob_%s_v2_%s" % (w, t), "gpu_event_matvec_atomic_prob_%s_v2_%s" % (w, t)]
     for t in ("float", "double"):
       want += ["gpu_matvec_prob_%s_v2_%s" % (w, t), "gpu_matvec_atomic_prob_%s_v2_%s" % (w, t),
-               "gpu_event_matvec_prob_%s_%s" % (w, t)]  # (the last: first-generation event kernels)
+               "gpu_event_matvec_prob_%s_%s" % (w, t),  # first-generation event kernels
+               "gpu_matvec_prob_%s_v1_%s" % (w, t)]  # first-generation dense names (lib/gpu_ops.cc:143-148)
   for w in ("normal", "uniform"):
     for t in ("float", "double"):
       want.append("gpu_matmat_prob_prob_%s_%s_v1" % (w, t))
@@ -72,7 +73,7 @@ def test_reference_registry_keys_of_the_other_operators_present():
           want.append("%s_%s_%s_%s" % (op, data, f, i))
   missing = [n for n in want if n not in names]
   assert not missing, missing
-  assert len(want) == 36 + 6 + 4 + 5 + 32
+  assert len(want) == 36 + 6 + 6 + 4 + 5 + 32  # + the 20 csr keys above: 109 of the reference's 113
 
 
 @pytest.mark.parametrize("name", sorted(_lib.target_names()))

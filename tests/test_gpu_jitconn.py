@@ -434,3 +434,65 @@ def test_random_shapes_walks_weights_and_inputs_against_oracle(cuda, oracle_mod,
       mag = np.full(n_out, 3.0 * (abs(a) + 5 * abs(b)) * (syn * 3 + 20))
       assert_close_reordered(got, want, mag, np.float32 if kind == "bool" else dtype, what="case %d" % case)
 
+
+
+@pytest.mark.parametrize("w_kind,a,b", [("homo", 0.0, 0.0), ("uniform", 0.25, 1.75), ("normal", 0.5, 2.0)])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_first_generation_dense_targets_give_the_cpu_paths_matrix(cuda, oracle_mod, w_kind, a, b, dtype):
+  # gpu_matvec_prob_*_v1_*: the descriptor carries conn_prob itself; on the reference's CPU path the
+  # version does not change the result (matvec.py:296-308), so the oracle is the same row walk.
+  n_row, n_col, seed = 70, 3000, 21
+  rng = np.random.default_rng(3)
+  tn = "_float" if dtype == np.float32 else "_double"
+  np_dt = dtype
+  for p, vec in ((0.07, rng.integers(-3, 4, n_col).astype(dtype)), (0.5, np.arange(n_col).astype(dtype)),
+                 (1.0, np.ones(n_col, dtype=dtype))):
+    lp = oracle_mod.log_p_of(p)
+    want = oracle_mod.jitconn_matvec(vec, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=seed, n_row=n_row, n_col=n_col,
+                                     dense=True, per_stream_seed=True)
+    if w_kind == "homo":
+      opaque = _lib.build_jitconn_prob_homo_descriptor(n_row, n_col, seed, p)
+    elif w_kind == "uniform":
+      opaque = _lib.build_jitconn_prob_uniform_descriptor(n_row, n_col, seed, p, float(np_dt(a)),
+                                                          float(np_dt(np_dt(b) - np_dt(a))))
+    else:
+      opaque = _lib.build_jitconn_prob_normal_descriptor(n_row, n_col, seed, p, a, b)
+    t = torch.from_numpy(vec).to("cuda:0")
+    out = torch.full((n_row,), 123.0, dtype=t.dtype, device="cuda:0")
+    _lib.custom_call("gpu_matvec_prob_" + w_kind + "_v1" + tn, [t, out], opaque)
+    got = out.cpu().numpy()
+    v2 = kernel_call(vec, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=seed, n_row=n_row, n_col=n_col, col_walk=False,
+                     dense=True)
+    assert np.array_equal(got, v2), (w_kind, p)  # one kernel behind both names
+    if w_kind == "homo":
+      assert np.array_equal(got.astype(np.float64), want.astype(np.float64)), p  # integer data: exact sums
+      if p >= 1.0:
+        assert np.all(got == n_col - 1)  # closed form: every index from 1 on
+    else:
+      meta = dict(dense=True, conn_prob=p, col_walk=False, n_row=n_row, n_col=n_col, seed=seed, w_kind=w_kind,
+                  w_a=a, w_b=b)
+      assert_close_reordered(got, want, _abs_bound(oracle_mod, vec, meta, dtype), dtype, what="v1 " + w_kind)
+
+
+def test_version_argument_of_the_dense_wrappers(cuda):
+  rng = np.random.default_rng(8)
+  shape = (200, 300)
+  kw = dict(conn_prob=0.1, shape=shape, seed=77)
+  for transpose in (False, True):
+    v = rng.standard_normal(shape[0] if transpose else shape[1]).astype(np.float32)
+    calls = ((bpl.matvec_prob_conn_homo_weight, (v, 0.3), {}),
+             (bpl.matvec_prob_conn_uniform_weight, (v,), dict(w_low=-1.0, w_high=2.0)),
+             (bpl.matvec_prob_conn_normal_weight, (v,), dict(w_mu=0.1, w_sigma=0.5)))
+    for fn, args, extra in calls:
+      y1 = fn(*args, transpose=transpose, version='v1', **extra, **kw)
+      y2 = fn(*args, transpose=transpose, version='v2', **extra, **kw)
+      assert torch.equal(y1, y2), fn.__name__
+      with pytest.raises(_lib.GPUOperatorNotFound):  # the reference registers no atomic v1 target either
+        fn(*args, transpose=transpose, outdim_parallel=False, version='v1', **extra, **kw)
+      with pytest.raises(AssertionError):
+        fn(*args, transpose=transpose, version='v3', **extra, **kw)
+  # the raw probability is validated where it is converted
+  t = torch.zeros(10, dtype=torch.float32, device="cuda:0")
+  out = torch.zeros(10, dtype=torch.float32, device="cuda:0")
+  with pytest.raises(RuntimeError):
+    _lib.custom_call("gpu_matvec_prob_homo_v1_float", [t, out], _lib.build_jitconn_prob_homo_descriptor(10, 10, 1, -0.5))
