@@ -210,16 +210,23 @@ def stats(dur_ms):
 
 
 def check(got, want, what, mag=None):
+  """Parity gate.  The bound is rel 1e-5 / abs 1e-6; sums accumulated in another order than the oracle's
+  sequential loop (`mag` = sum of |addends| per element) may additionally differ by the reordering bound
+  4 eps sum|addends|.  Both counts are printed: elements outside the plain bound, and violations of the gate."""
   got = np.asarray(got, dtype=np.float64)
   want = np.asarray(want, dtype=np.float64)
-  bound = 1e-6 + 1e-5 * np.abs(want)
-  if mag is not None:  # sums accumulated in another order (atomics): reordering bound
-    bound = bound + 4 * np.finfo(np.float32).eps * np.asarray(mag, dtype=np.float64)
+  plain = 1e-6 + 1e-5 * np.abs(want)
+  bound = plain
+  if mag is not None:
+    bound = plain + 4 * np.finfo(np.float32).eps * np.asarray(mag, dtype=np.float64)
   err = np.abs(got - want)
   bad = int((err > bound).sum())
-  log("parity %-34s max abs err %.3e  violations %d / %d" % (what, float(err.max(initial=0)), bad, got.size))
+  outside_plain = int((err > plain).sum())
+  log("parity %-34s max abs err %.3e  outside rel 1e-5/abs 1e-6: %d  violations%s: %d / %d" % (
+    what, float(err.max(initial=0)), outside_plain, " (with reordering term)" if mag is not None else "", bad, got.size))
   if bad:
     raise SystemExit("parity gate failed for " + what)
+  return outside_plain
 
 
 def reference_shapes(bpl, synth, torch, dev):

@@ -26,6 +26,7 @@
 
 #include "common.h"
 #include "csr_quad_gather.h"
+#include "repeated_sum.h"
 #include "targets.h"
 
 namespace bpl {
@@ -48,6 +49,44 @@ constexpr NnzGate kAlways = {0u, 0xffffffffu};
 constexpr int kScatterThreads = 256;
 
 enum : int { kEvent = 0, kDense = 1 };
+
+// A homogeneous weight delivered by n synapses.  The reference adds the weight once per synapse:
+// in place in the precision of the output when it scatters (event_csr_matvec.py:313-331), into a
+// float64 accumulator that is rounded once when it gathers (event_csr_matvec.py:334-357).  Every
+// addend being the same, the result depends on the count alone, so kernels that count in integers
+// reproduce the reference's bits whatever order the synapses arrive in.
+template <typename F>
+__device__ __forceinline__ F scattered_sum(F w, uint64_t n) {
+  return repeated_sum<F>(w, n);
+}
+__device__ __forceinline__ float gathered_sum(float w, uint32_t n) {
+  // up to 2^29 additions of a 24-bit weight are exact in float64: the product, rounded once
+  return static_cast<float>(static_cast<double>(w) * static_cast<double>(n));
+}
+__device__ __forceinline__ double gathered_sum(double w, uint32_t n) { return repeated_sum<double>(w, n); }
+
+// A synapse count kept in the storage of an output element until the last kernel of a call turns
+// it into the sum (float: the 32 bits hold the integer; double: the count as a number, exact).
+__device__ __forceinline__ float count_as_element(uint32_t n, float) { return __uint_as_float(n); }
+__device__ __forceinline__ double count_as_element(uint32_t n, double) { return static_cast<double>(n); }
+__device__ __forceinline__ uint64_t element_as_count(float v) { return __float_as_uint(v); }
+__device__ __forceinline__ uint64_t element_as_count(double v) { return static_cast<uint64_t>(v); }
+// adds n to the count held in *y (y zeroed before)
+__device__ __forceinline__ void add_count(float *y, uint32_t n) { atomicAdd(reinterpret_cast<uint32_t *>(y), n); }
+__device__ __forceinline__ void add_count(double *y, uint32_t n) {
+  // (the count as a number: float64 atomic adds of integers are exact and commute)
+  atomic_add(y, static_cast<double>(n));
+}
+
+// y[i] = the sum of y[i]'s count of synapses of weight data[0] (see above), in place
+template <typename F>
+__global__ __launch_bounds__(256) void counts_to_sums_kernel(F *__restrict__ y, uint32_t n, const F *__restrict__ data,
+                                                             const uint32_t *__restrict__ indptr, uint32_t n_row,
+                                                             NnzGate gate) {
+  if (!gate.open(indptr, n_row)) return;
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  if (i < n) y[i] = scattered_sum<F>(data[0], element_as_count(y[i]));
+}
 
 // ------------------------------------------------------------------------------------------------
 // scatter
@@ -186,7 +225,7 @@ __global__ __launch_bounds__(kWinThreads) void collect_active_rows_kernel(
         on[e] = is_event(x[r]);
       } else {
         scale[e] = static_cast<F>(x[r]);
-        on[e] = scale[e] != F(0);  // a zero input adds nothing
+        on[e] = true;  // also a zero input: 0 * inf and 0 * NaN must reach the output (cusparse_matvec.py:204-211)
       }
     }
   }
@@ -363,10 +402,6 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
   const uint32_t width = (c0 + win <= n_col) ? win : n_col - c0;
 
   const F w_homo = HETER ? F(0) : data[0];
-  // n synapses of weight w: n * w rounded once (nothing, not 0 * w, where no synapse arrived)
-  auto counted = [&](uint32_t n) {
-    return n ? static_cast<F>(static_cast<double>(w_homo) * static_cast<double>(n)) : F(0);
-  };
   for (uint32_t i = tid; i < width; i += kWinThreads) {
     if (kCount) cwindow[i] = 0u;
     else window[i] = A(0);
@@ -406,7 +441,7 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
         on = is_event(x[r]);
       } else {
         scale = static_cast<F>(x[r]);
-        on = scale != F(0);  // a zero input adds nothing
+        on = true;  // also a zero input, whose products with inf and NaN weights are NaN
       }
       if (on) {
         start = indptr[r];
@@ -495,23 +530,32 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_window_kernel(
   if (partial != nullptr) {
     // plain contiguous stores of the whole window into this row group's slice; a second
     // kernel sums the slices
+    // (counting windows leave their counts: the summing kernel adds the integers and forms the sum once)
     F *dst = partial + static_cast<size_t>(g) * n_col + c0;
+    for (uint32_t i = tid; i < width; i += kWinThreads) {
+      if constexpr (kCount) dst[i] = count_as_element(cwindow[i], F(0));
+      else dst[i] = static_cast<F>(window[i]);
+    }
+  } else if constexpr (kCount) {
+    // counts into the zeroed y; counts_to_sums_kernel follows
     for (uint32_t i = tid; i < width; i += kWinThreads)
-      dst[i] = kCount ? counted(cwindow[i]) : static_cast<F>(window[i]);
+      if (cwindow[i] != 0u) add_count(&y[c0 + i], cwindow[i]);
   } else {
     for (uint32_t i = tid; i < width; i += kWinThreads) {
-      const F v = kCount ? counted(cwindow[i]) : static_cast<F>(window[i]);
+      const F v = static_cast<F>(window[i]);
       if (v != F(0)) atomic_add(&y[c0 + i], v);
     }
   }
 }
 
 // y[c] = sum over row groups of partial[g][c]
-template <typename F>
+// (COUNT: the slices hold synapse counts of the homogeneous weight data[0])
+template <typename F, bool COUNT>
 __global__ __launch_bounds__(256) void sum_partials_kernel(const F *__restrict__ partial, F *__restrict__ y,
                                                            uint32_t n_col, uint32_t groups,
                                                            const uint32_t *__restrict__ indptr, uint32_t n_row,
-                                                           NnzGate gate, uint32_t *__restrict__ reset) {
+                                                           NnzGate gate, uint32_t *__restrict__ reset,
+                                                           const F *__restrict__ data) {
   if (!gate.open(indptr, n_row)) return;
   // with a device list of active rows: the groups that took part, as the window kernel left them
   // in the second counter; the active-row counter itself goes back to zero for the next call
@@ -521,6 +565,12 @@ __global__ __launch_bounds__(256) void sum_partials_kernel(const F *__restrict__
   }
   const uint32_t c = blockIdx.x * 256u + threadIdx.x;
   if (c >= n_col) return;
+  if constexpr (COUNT) {
+    uint64_t n = 0;
+    for (uint32_t g = 0; g < groups; ++g) n += element_as_count(partial[static_cast<size_t>(g) * n_col + c]);
+    y[c] = scattered_sum<F>(data[0], n);
+    return;
+  }
   F acc = F(0);
   uint32_t g = 0;
   for (; g + 4 <= groups; g += 4) {
@@ -667,7 +717,7 @@ __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const ui
       if (MODE == kEvent && !HETER) {
         hits = group_sum<G>(hits);
         // n additions of the same fp32 value into a float64 accumulator are exact: n * w
-        if (gl == 0) y[row] = static_cast<F>(static_cast<double>(w_homo) * static_cast<double>(hits));
+        if (gl == 0) y[row] = gathered_sum(w_homo, hits);
         hits = 0;
       } else {
         acc = group_sum<G>(acc);
@@ -754,7 +804,7 @@ __device__ __forceinline__ void gather_rows_wave(const F *__restrict__ data, con
     if (MODE == kEvent && !HETER) {
       hits = wave_sum(hits);
       // n additions of the same fp32 value into a float64 accumulator are exact: n * w
-      if (lane == 0) y[urow] = static_cast<F>(static_cast<double>(w_homo) * static_cast<double>(hits));
+      if (lane == 0) y[urow] = gathered_sum(w_homo, hits);
     } else {
       acc = wave_sum(acc);
       if (lane == 0) y[urow] = static_cast<F>(acc);
@@ -963,9 +1013,7 @@ __global__ __launch_bounds__(kWinThreads) void csr_scatter_small_kernel(
     if (HETER) {
       y[c0 + i] = window[i];
     } else {
-      // n synapses of weight w: n * w rounded once (nothing, not 0 * w, where no synapse arrived)
-      const uint32_t n = cwindow[i];
-      y[c0 + i] = n ? static_cast<F>(static_cast<double>(w_homo) * static_cast<double>(n)) : F(0);
+      y[c0 + i] = scattered_sum<F>(w_homo, cwindow[i]);  // the weight added once per synapse, as the reference adds it
     }
   }
 }
@@ -1107,11 +1155,17 @@ void launch_scatter(const ScratchSource &src, const F *data, const uint32_t *ind
                          n_row, n_col, rows_per_wg, win, n_win, partial, window_gate, active_count,
                          active_list, active_scales);
       // the list's counter goes back to zero: by the summing kernel, else by a fill of its own
-      if (partial != nullptr)
-        hipLaunchKernelGGL(sum_partials_kernel<F>, dim3(div_up(n_col, 256)), dim3(256), 0, stream, partial, y, n_col,
-                           groups, indptr, n_row, window_gate, active_count);
-      else if (use_list)
-        fill_zero(stream, active_count, 1u);
+      constexpr bool kCount = !HETER && MODE == kEvent;  // the windows count synapses of the homogeneous weight
+      if (partial != nullptr) {
+        hipLaunchKernelGGL((sum_partials_kernel<F, kCount>), dim3(div_up(n_col, 256)), dim3(256), 0, stream,
+                           static_cast<const F *>(partial), y, n_col, groups, indptr, n_row, window_gate, active_count,
+                           data);
+      } else {
+        if (use_list) fill_zero(stream, active_count, 1u);
+        if (kCount)  // y holds the counts the windows added
+          hipLaunchKernelGGL(counts_to_sums_kernel<F>, dim3(div_up(n_col, 256)), dim3(256), 0, stream, y, n_col, data,
+                             indptr, n_row, window_gate);
+      }
       if (!gated) return;
     } else {
       direct_gate = kAlways;
@@ -1455,9 +1509,8 @@ __device__ __forceinline__ void gather_rows_batched(const F *__restrict__ data,
     if (HETER) {
       result = static_cast<F>(group_sum8<G>(acc, gl, &k));
     } else {
-      // n additions of the same value into a float64 accumulator are exact: n * w
       const uint32_t n = group_sum8<G>(cnt, gl, &k);
-      result = static_cast<F>(static_cast<double>(w_homo) * static_cast<double>(n));
+      result = gathered_sum(w_homo, n);
     }
     const uint32_t bi = tile * kBatchTile + k;
     if ((gl & (G / 8 - 1)) == 0 && bi < batch) y[static_cast<size_t>(bi) * n_row + row] = result;

@@ -42,9 +42,10 @@ def test_batching_broadcast_combinations(cuda, oracle_mod, shape, transpose, dty
     fev = (events * rng.uniform(0.5, 2.0, events.shape)).astype(dtype)
     _check(oracle_mod, data[:vb], indices[:ib], indptr[:pb], fev, batch, shape, transpose, "heter float")
     w = rng.standard_normal((vb, 1)).astype(dtype)
-    _check(oracle_mod, w, indices[:ib], indptr[:pb], events, batch, shape, transpose, "homo bool")
-    # unit weight: counts, exact whatever the order
-    one = np.ones((1, 1), dtype=dtype)
+    # homogeneous weights are added once per synapse, as the reference adds them: its bits, whatever the order
+    got, want = _check(oracle_mod, w, indices[:ib], indptr[:pb], events, batch, shape, transpose, "homo bool")
+    assert np.array_equal(got, want)
+    one = np.full((1, 1), 0.6, dtype=dtype)
     got, want = _check(oracle_mod, one, indices[:ib], indptr[:pb], events, batch, shape, transpose, "counts")
     assert np.array_equal(got, want)
 
@@ -80,7 +81,7 @@ def test_batching_transposed_through_one_sorted_scatter(cuda, oracle_mod):
     print("shape", shape, "batch", batch, flush=True)
     events = rng.random((eb, n_row)) < rate
     _check(oracle_mod, data[None], indices[None], indptr[None], events, batch, shape, True, "heter")
-    one = np.ones((1, 1), dtype=np.float32)
+    one = np.full((1, 1), 0.6, dtype=np.float32)
     got, want = _check(oracle_mod, one, indices[None], indptr[None], events, batch, shape, True, "counts")
     assert np.array_equal(got, want)
     # twice in a row (the list's counter is back at zero), float events
