@@ -42,14 +42,22 @@ constexpr uint32_t kRowwalkCoarseBytes = 38912;
 // the register allocation has to leave room for; the normal-weight walk needs 66 otherwise.)
 // Register budget: eight waves per SIMD need at most 64 vector AND at most 80 scalar registers per
 // wave here (with 81..96 scalar registers only seven fit, so a second 16-wave workgroup does not).
-template <typename T1, typename VT, int IN, int W, int BITS>
+constexpr uint32_t kFuseBatch = 64;   // streams seeded together, one per lane
+constexpr uint32_t kFuseSlots = 3;    // batches of seeded states in a workgroup's ring
+constexpr uint32_t kFuseSpin = 1u << 22;           // polls of a flag in LDS before a wave stops waiting
+constexpr uint32_t kFuseNotSeeded = 0x80000000u;   // flag bit: the batch's rows seed their own generators
+constexpr size_t kFuseRingBytes = static_cast<size_t>(kFuseSlots) * kFuseBatch * kMtN * sizeof(uint32_t);  // per workgroup
+static_assert(kMtSeedTileWords <= kMtStateWords, "the seeding wave transposes through its own state buffer");
+
+template <typename T1, typename VT, int IN, int W, int BITS, bool FUSED>
 __global__ __launch_bounds__(1024, (BITS == 2 || (W == kNormal && sizeof(T1) == 4)) ? 8 : 4)
     __attribute__((amdgpu_num_sgpr(80))) void jitconn_rowwalk_kernel(const VT *__restrict__ in, T1 *__restrict__ out,
                                                                uint32_t n_out, uint32_t n_in, uint32_t seed,
                                                                double log_p, T1 wa, T1 wb, uint32_t first,
-                                                               const uint32_t *__restrict__ states) {
+                                                               uint32_t *states) {
   // Handles the n_out outputs first .. first + n_out - 1; `states` (optional) holds their
-  // generators' seeded states.
+  // generators' seeded states.  FUSED: all outputs from 0, `states` is the workgroups' rings
+  // (kFuseRingBytes each).
   extern __shared__ __attribute__((aligned(8))) uint32_t smem[];
   const int lane = lane_id();
   const uint32_t wave = threadIdx.x / kWave;
@@ -71,9 +79,8 @@ __global__ __launch_bounds__(1024, (BITS == 2 || (W == kNormal && sizeof(T1) == 
     for (uint32_t i = threadIdx.x; i < words; i += blockDim.x) wbits[i] = pack_events32<VT>(in, i << 5, n_in);
     __syncthreads();
   }
-  for (uint32_t i = blockIdx.x * nwaves + wave; i < n_out; i += gridDim.x * nwaves) {
-    const uint32_t o = first + i;
-    const uint32_t *pre = states ? states + static_cast<size_t>(i) * kMtN : nullptr;
+  // output o from stream seed + o, whose seeded state is at `pre` (or nullptr: the wave seeds it itself)
+  auto walk_row = [&](uint32_t o, const uint32_t *pre, auto &&loaded) {
     double acc = 0.0;
     uint32_t cnt = 0;
     // two-level bitmap: the exact word of a batch is requested when the batch is drawn and looked
@@ -115,13 +122,80 @@ __global__ __launch_bounds__(1024, (BITS == 2 || (W == kNormal && sizeof(T1) == 
         if (W == kHomo) cnt += static_cast<uint32_t>(__popcll(__ballot(hit)));
         else if (hit) acc += static_cast<double>(w);
       }
-    });
+    }, loaded);
     if constexpr (IN == kInEvent && BITS == 2) settle();
     if (IN == kInEvent && W == kHomo) {
       if (lane == 0) out[o] = static_cast<T1>(cnt);
     } else {
       acc = wave_sum(acc);
       if (lane == 0) out[o] = static_cast<T1>(acc);
+    }
+  };
+
+  if constexpr (!FUSED) {
+    for (uint32_t i = blockIdx.x * nwaves + wave; i < n_out; i += gridDim.x * nwaves)
+      walk_row(first + i, states ? states + static_cast<size_t>(i) * kMtN : nullptr, NoLoadHook());
+  } else {
+    // The generators are seeded inside the kernel, 64 streams at a time on the vector unit (the scalar
+    // unit, one per CU, cannot seed a stream per wave fast enough), while the other waves walk: the
+    // workgroup takes batches of 64 consecutive outputs (batch blockIdx.x + j * gridDim.x is its j-th),
+    // its waves take (batch, row) tasks from a counter in LDS, and the wave that takes the first row of
+    // batch j first seeds batch j + 1 into slot (j + 1) % 3 of the workgroup's ring of seeded states in
+    // device memory (`states`), which stays in the L2.  A slot is written again only after all 64 rows
+    // of its previous batch have copied their state to LDS, and read only after its flag says which
+    // batch it holds; every wait is bounded, and a wave that gives up seeds its own generator instead.
+    __shared__ uint32_t s_task, s_ready[kFuseSlots], s_loaded[kFuseSlots];
+    const uint32_t n_batches = (n_out + kFuseBatch - 1u) / kFuseBatch;
+    const uint32_t mine = n_batches > blockIdx.x ? (n_batches - blockIdx.x + gridDim.x - 1u) / gridDim.x : 0u;
+    // (`states` is neither const nor restrict: other waves write what this one reads behind a flag)
+    uint32_t *ring = states + static_cast<size_t>(blockIdx.x) * kFuseSlots * kFuseBatch * kMtN;
+    if (threadIdx.x == 0) {
+      s_task = 0;
+      for (uint32_t k = 0; k < kFuseSlots; ++k) s_ready[k] = 0, s_loaded[k] = 0;
+    }
+    __syncthreads();
+    if (mine == 0) return;
+    auto seed_batch = [&](uint32_t j) {
+      const uint32_t slot = j % kFuseSlots;
+      mt_seed_batch(st, lane, seed + (blockIdx.x + j * gridDim.x) * kFuseBatch,
+                    ring + static_cast<size_t>(slot) * kFuseBatch * kMtN);
+      __hip_atomic_store(&s_ready[slot], j + 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
+    if (wave == 0) seed_batch(0);
+    for (;;) {
+      // Every lane adds one, so the counter advances by 64 per task and any lane's old value / 64 is the
+      // task.  (With the add under `if (lane == 0)` the compiler split the loop by lane: lane 0 went back
+      // to the add alone and the other lanes stayed behind with task 0 for ever.)
+      const uint32_t t = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(
+                             static_cast<int>(atomicAdd(&s_task, 1u)))) / kWave;
+      const uint32_t j = t / kFuseBatch, r = t % kFuseBatch;
+      if (j >= mine) break;
+      if (r == 0 && j + 1 < mine) {
+        // slot (j + 1) % 3 last held batch j - 2: (j + 1) / 3 batches have used it, 64 loads each
+        const uint32_t slot = (j + 1u) % kFuseSlots, need = ((j + 1u) / kFuseSlots) * kFuseBatch;
+        bool free_ = false;
+        for (uint32_t spin = 0; spin < kFuseSpin && !free_; ++spin) {
+          free_ = __hip_atomic_load(&s_loaded[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) >= need;
+          if (!free_) __builtin_amdgcn_s_sleep(2);
+        }
+        if (free_) seed_batch(j + 1u);
+        else __hip_atomic_store(&s_ready[slot], kFuseNotSeeded | (j + 2u), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+      const uint32_t slot = j % kFuseSlots;
+      uint32_t flag = 0;
+      for (uint32_t spin = 0; spin < kFuseSpin; ++spin) {
+        flag = __hip_atomic_load(&s_ready[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if ((flag & ~kFuseNotSeeded) >= j + 1u) break;
+        flag = kFuseNotSeeded;
+        __builtin_amdgcn_s_sleep(2);
+      }
+      const uint32_t *pre = (flag & kFuseNotSeeded) ? nullptr : ring + (static_cast<size_t>(slot) * kFuseBatch + r) * kMtN;
+      auto loaded = [&]() {
+        if (lane == 0) __hip_atomic_fetch_add(&s_loaded[slot], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      };
+      const uint32_t o = (blockIdx.x + j * gridDim.x) * kFuseBatch + r;
+      if (o < n_out) walk_row(o, pre, loaded);
+      else loaded();
     }
   }
 }
@@ -347,17 +421,58 @@ bool valid_log_p(const char *target, double log_p) {
   return true;
 }
 
+// Scratch memory of one row-walk call, taken with ONE request so that its parts cannot move apart:
+//   [packed event bitmap, the coarse bitmap behind it (only where the launcher packs one)]
+//   [rings of seeded generator states, kFuseRingBytes per workgroup (only from kSeedAheadMin outputs)]
+struct RowwalkScratch {
+  unsigned char *base = nullptr;
+  size_t bitmap_bytes = 0;   // a multiple of 256
+  uint32_t ring_groups = 0;  // workgroups that have a ring
+  bool refused = false;      // the stream is being captured and the memory is not there yet: the call fails
+  uint32_t *bitmap() const { return bitmap_bytes && base ? reinterpret_cast<uint32_t *>(base) : nullptr; }
+  uint32_t *rings() const { return ring_groups && base ? reinterpret_cast<uint32_t *>(base + bitmap_bytes) : nullptr; }
+};
+
+// At most four row-walk workgroups share a CU (eight waves each; sixteen-wave ones two).
+inline uint32_t rowwalk_max_groups() { return 4u * static_cast<uint32_t>(device_info().num_cu); }
+
+inline RowwalkScratch rowwalk_scratch(hipStream_t stream, uint32_t n_out, size_t bitmap_bytes) {
+  RowwalkScratch sc;
+  sc.bitmap_bytes = (bitmap_bytes + 255) / 256 * 256;
+  if (n_out >= kSeedAheadMin) {
+    const uint32_t batches = div_up(n_out, kFuseBatch);
+    sc.ring_groups = batches < rowwalk_max_groups() ? batches : rowwalk_max_groups();
+  }
+  const size_t want = sc.bitmap_bytes + sc.ring_groups * kFuseRingBytes;
+  if (want == 0) return sc;
+  sc.base = static_cast<unsigned char *>(stream_workspace(stream, want));
+  if (sc.base == nullptr && !scratch_refused_by_capture() && sc.ring_groups != 0 && sc.bitmap_bytes != 0) {
+    // no room for the rings: the bitmap alone (the waves then seed their own generators)
+    bpl_clear_error();
+    sc.ring_groups = 0;
+    sc.base = static_cast<unsigned char *>(stream_workspace(stream, sc.bitmap_bytes));
+  }
+  if (sc.base == nullptr) {
+    sc.refused = scratch_refused_by_capture();
+    if (!sc.refused) bpl_clear_error();  // (an allocation failed: paths that need no scratch memory remain)
+    sc.ring_groups = 0;
+  }
+  return sc;
+}
+
 template <typename T1, typename VT, int IN, int W, int BITS>
 void launch_rowwalk_impl(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, uint32_t n_in, uint32_t seed,
-                         double log_p, T1 wa, T1 wb, int nwaves, size_t lds_bytes) {
-  auto kernel = jitconn_rowwalk_kernel<T1, VT, IN, W, BITS>;
+                         double log_p, T1 wa, T1 wb, int nwaves, size_t lds_bytes, const RowwalkScratch &sc) {
+  const bool fused = sc.rings() != nullptr;
+  auto kernel = fused ? jitconn_rowwalk_kernel<T1, VT, IN, W, BITS, true> : jitconn_rowwalk_kernel<T1, VT, IN, W, BITS, false>;
   const int block = nwaves * kWave;
   struct Cached {
     size_t lds_bytes;
     int block;
     int per_cu;
   };
-  static thread_local Cached cached = {~size_t(0), 0, 0};
+  static thread_local Cached cached_for[2] = {{~size_t(0), 0, 0}, {~size_t(0), 0, 0}};
+  Cached &cached = cached_for[fused];
   if (cached.lds_bytes != lds_bytes || cached.block != block) {
     if (lds_bytes > 64 * 1024)
       (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -371,90 +486,85 @@ void launch_rowwalk_impl(hipStream_t stream, const VT *in, T1 *out, uint32_t n_o
     cached = {lds_bytes, block, q};
   }
   const unsigned resident = static_cast<unsigned>(device_info().num_cu) * static_cast<unsigned>(cached.per_cu);
-  // Large outputs: the generators are seeded ahead, a chunk of streams at a time, by a kernel that
-  // runs the recurrence on the vector unit; small ones seed in place.
-  uint32_t *states = nullptr;
-  if (n_out >= kSeedAheadMin)
-    states = static_cast<uint32_t *>(stream_workspace(stream, static_cast<size_t>(kSeedChunk) * kMtN * 4));
-  if (states == nullptr) {
-    if (n_out >= kSeedAheadMin && scratch_refused_by_capture()) return;
-    bpl_clear_error();
-  }
-  const uint32_t chunk = states ? kSeedChunk : n_out;
-  for (uint32_t first = 0; first < n_out; first += chunk) {
-    const uint32_t count = (n_out - first < chunk) ? n_out - first : chunk;
-    if (states) launch_seed_streams(stream, seed, first, count, states);
-    const unsigned needed = div_up(count, nwaves);
-    const unsigned grid = needed < resident ? needed : resident;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), lds_bytes, stream, in, out, count, n_in, seed, log_p, wa, wb,
-                       first, static_cast<const uint32_t *>(states));
-  }
+  // From kSeedAheadMin outputs the generators are seeded inside the kernel, 64 at a time on the vector
+  // unit, into the workgroups' rings (one launch for the whole walk); smaller walks seed in place.
+  unsigned needed = fused ? div_up(n_out, kFuseBatch) : div_up(n_out, nwaves);
+  if (fused && needed > sc.ring_groups) needed = sc.ring_groups;
+  const unsigned grid = needed < resident ? needed : resident;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), lds_bytes, stream, in, out, n_out, n_in, seed, log_p, wa, wb, 0u,
+                     sc.rings());
 }
 
+// Event probes from an LDS bitmap when it fits beside the generator states, else from global memory.
 template <typename T1, typename VT, int IN, int W>
-void launch_rowwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, uint32_t n_in, uint32_t seed,
-                    double log_p, T1 wa, T1 wb) {
-  if (n_out == 0) return;
-  if constexpr (IN == kInEvent && !std::is_same<VT, PackedBits>::value) {
-    // An event bitmap that would leave room for fewer than two 16-wave workgroups per CU: two
-    // levels instead, the exact bitmap packed into global memory and a coarse one made for LDS.
-    if ((static_cast<size_t>(n_in) + 31) / 32 * 4 > kRowwalkCoarseBytes) {
-      const size_t state_ws = (n_out >= kSeedAheadMin) ? static_cast<size_t>(kSeedChunk) * kMtN * 4 : 0;
-      const uint32_t g = coarse_shift(n_in, kRowwalkCoarseBytes);
-      const uint32_t n_words = (n_in + 31u) / 32u, off = coarse_offset_words(n_in);
-      const uint32_t c_words = (coarse_bits(n_in, g) + 31u) / 32u;
-      unsigned char *ws = static_cast<unsigned char *>(
-          stream_workspace(stream, state_ws + (static_cast<size_t>(off) + c_words + 1) * sizeof(uint32_t)));
-      if (ws != nullptr) {
-        uint32_t *bits = reinterpret_cast<uint32_t *>(ws + state_ws);
-        pack_event_bitmap<VT>(stream, in, n_in, bits);
-        hipLaunchKernelGGL(coarsen_bitmap_kernel, dim3(div_up(c_words, 256)), dim3(256), 0, stream, bits, n_words, g,
-                           bits + off, c_words);
-        const size_t state_bytes = StreamLds<T1, W>::words * 4;
-        launch_rowwalk_impl<T1, PackedBits, IN, W, 2>(stream, reinterpret_cast<const PackedBits *>(bits), out, n_out, n_in,
-                                                      seed, log_p, wa, wb, 16,
-                                                      static_cast<size_t>(c_words) * 4 + 16 * state_bytes);
-        return;
-      }
-      if (scratch_refused_by_capture()) return;
-      bpl_clear_error();
-    }
-  }
-  if constexpr (IN == kInEvent && sizeof(VT) > 1 && !std::is_same<VT, PackedBits>::value) {
-    // Wide event types: pack the vector to one bit per element once, instead of once per workgroup.
-    // (The seeded generator states of large walks share the scratch buffer: the bitmap lies behind them.)
-    const size_t state_ws = (n_out >= kSeedAheadMin) ? static_cast<size_t>(kSeedChunk) * kMtN * 4 : 0;
-    const size_t words = (static_cast<size_t>(n_in) + 31) / 32;
-    unsigned char *ws = static_cast<unsigned char *>(stream_workspace(stream, state_ws + (words + 1) * 4));
-    if (ws != nullptr) {
-      uint32_t *bits = reinterpret_cast<uint32_t *>(ws + state_ws);
-      pack_event_bitmap<VT>(stream, in, n_in, bits);
-      launch_rowwalk<T1, PackedBits, IN, W>(stream, reinterpret_cast<const PackedBits *>(bits), out, n_out, n_in, seed,
-                                            log_p, wa, wb);
-      return;
-    }
-    if (scratch_refused_by_capture()) return;
-    bpl_clear_error();
-  }
+void launch_rowwalk_plain(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, uint32_t n_in, uint32_t seed,
+                          double log_p, T1 wa, T1 wb, const RowwalkScratch &sc) {
   const size_t state_bytes = StreamLds<T1, W>::words * 4;
   const size_t cap = static_cast<size_t>(160) * 1024 - 512;
+  // With the generators seeded inside the kernel every workgroup has a ring of seeded states in device
+  // memory: 16-wave workgroups, so that the rings in use together are half as many and stay in the L2
+  // and the memory-side cache.
+  const int fused_waves = sc.rings() != nullptr ? 16 : 8;
   if (IN == kInEvent) {
     const size_t bitmap = (static_cast<size_t>(n_in) + 31) / 32 * 4;
     if (bitmap + 4 * state_bytes <= cap) {
       // Small bitmaps: 8-wave workgroups, several per CU.  Large ones: one workgroup per CU with
       // as many waves as fit beside the bitmap (each wave can issue one instruction every four
       // cycles, so the number of resident waves bounds the VALU utilisation).
-      int nw = 8;
+      int nw = fused_waves;
       if (bitmap > 16 * 1024) {
         nw = static_cast<int>((cap - bitmap) / state_bytes);
         if (nw > 16) nw = 16;
       }
       launch_rowwalk_impl<T1, VT, IN, W, 1>(stream, in, out, n_out, n_in, seed, log_p, wa, wb, nw,
-                                            bitmap + nw * state_bytes);
+                                            bitmap + nw * state_bytes, sc);
       return;
     }
   }
-  launch_rowwalk_impl<T1, VT, IN, W, 0>(stream, in, out, n_out, n_in, seed, log_p, wa, wb, 8, 8 * state_bytes);
+  launch_rowwalk_impl<T1, VT, IN, W, 0>(stream, in, out, n_out, n_in, seed, log_p, wa, wb, fused_waves,
+                                        fused_waves * state_bytes, sc);
+}
+
+template <typename T1, typename VT, int IN, int W>
+void launch_rowwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, uint32_t n_in, uint32_t seed,
+                    double log_p, T1 wa, T1 wb) {
+  if (n_out == 0) return;
+  constexpr bool kEvents = IN == kInEvent;
+  const size_t words = (static_cast<size_t>(n_in) + 31) / 32;
+  // An event bitmap that would leave room for fewer than two 16-wave workgroups per CU: two levels
+  // instead, the exact bitmap packed into global memory and a coarse one made for LDS.  Wide event
+  // types: the vector is packed to one bit per element once, instead of once per workgroup.
+  const bool two_level = kEvents && words * 4 > kRowwalkCoarseBytes;
+  const bool packed = kEvents && (two_level || sizeof(VT) > 1);
+  uint32_t g = 0, off = 0, c_words = 0;
+  size_t bitmap_ws = 0;
+  if (two_level) {
+    g = coarse_shift(n_in, kRowwalkCoarseBytes);
+    off = coarse_offset_words(n_in);
+    c_words = (coarse_bits(n_in, g) + 31u) / 32u;
+    bitmap_ws = (static_cast<size_t>(off) + c_words + 1) * sizeof(uint32_t);
+  } else if (packed) {
+    bitmap_ws = (words + 1) * sizeof(uint32_t);
+  }
+  const RowwalkScratch sc = rowwalk_scratch(stream, n_out, bitmap_ws);
+  if (sc.refused) return;  // (the error stands: a graph must not record a slower path)
+  if constexpr (kEvents) {
+    if (uint32_t *bits = sc.bitmap()) {
+      pack_event_bitmap<VT>(stream, in, n_in, bits);
+      const PackedBits *pin = reinterpret_cast<const PackedBits *>(bits);
+      if (two_level) {
+        hipLaunchKernelGGL(coarsen_bitmap_kernel, dim3(div_up(c_words, 256)), dim3(256), 0, stream, bits,
+                           static_cast<uint32_t>(words), g, bits + off, c_words);
+        const size_t state_bytes = StreamLds<T1, W>::words * 4;
+        launch_rowwalk_impl<T1, PackedBits, IN, W, 2>(stream, pin, out, n_out, n_in, seed, log_p, wa, wb, 16,
+                                                      static_cast<size_t>(c_words) * 4 + 16 * state_bytes, sc);
+      } else {
+        launch_rowwalk_plain<T1, PackedBits, IN, W>(stream, pin, out, n_out, n_in, seed, log_p, wa, wb, sc);
+      }
+      return;
+    }
+  }
+  launch_rowwalk_plain<T1, VT, IN, W>(stream, in, out, n_out, n_in, seed, log_p, wa, wb, sc);
 }
 
 template <typename T1, typename VT, int IN, int W>

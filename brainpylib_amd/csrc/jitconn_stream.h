@@ -124,12 +124,18 @@ __device__ __forceinline__ uint64_t accepted_units(const RoleTable &tab, uint64_
 //
 // `pre` points at the stream's 624 seeded state words when they were prepared by
 // launch_seed_streams(); with nullptr the wave seeds the generator itself on the scalar unit.
-template <typename T1, int W, typename F>
+//
+// `loaded()` is called once, when the generator state is in LDS and `pre` is no longer read.
+struct NoLoadHook {
+  __device__ __forceinline__ void operator()() const {}
+};
+template <typename T1, int W, typename F, typename L = NoLoadHook>
 __device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t stream_seed, const uint32_t *pre,
-                                            uint32_t n, double log_p_, T1 wa, T1 wb, F &&f) {
+                                            uint32_t n, double log_p_, T1 wa, T1 wb, F &&f, L &&loaded = L()) {
   const SkipParams log_p = make_skip_params(log_p_);
   if (pre != nullptr) mt_load(st, pre, lane);
   else mt_seed(st, stream_seed, lane);
+  loaded();
   uint32_t pos = 0;
   // With every skip >= 1 a row ends within n/64 + 1 batches; the cap only guards against a
   // generator state that yields zero skips forever (log_p is validated on the host).

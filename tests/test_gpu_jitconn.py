@@ -496,3 +496,32 @@ def test_version_argument_of_the_dense_wrappers(cuda):
   out = torch.zeros(10, dtype=torch.float32, device="cuda:0")
   with pytest.raises(RuntimeError):
     _lib.custom_call("gpu_matvec_prob_homo_v1_float", [t, out], _lib.build_jitconn_prob_homo_descriptor(10, 10, 1, -0.5))
+
+
+@pytest.mark.parametrize("n_out,n_in", [(8192, 3000), (10_007, 200_000), (20_000, 400_000), (70_001, 5000)])
+def test_row_walk_with_generators_seeded_inside_the_kernel(cuda, oracle_mod, n_out, n_in):
+  # from 8,192 outputs the row walk seeds its generators itself, 64 streams at a time, into rings of
+  # seeded states that its workgroups keep in device memory: whole outputs against the per-stream
+  # oracle for every weight kind, event (LDS bitmap / two-level bitmap / packed float events) and
+  # dense input, output counts that are and are not multiples of 64, fewer batches than workgroups,
+  # twice in a row (the second call finds the rings of the first).
+  rng = np.random.default_rng(n_out)
+  lp = oracle_mod.log_p_of(200.0 / n_in)
+  ev = rng.random(n_in) < 0.1
+  fev = (ev * rng.uniform(0.5, 2.0, n_in)).astype(np.float32)
+  vec = rng.integers(-3, 4, n_in).astype(np.float64)
+  print("case", n_out, n_in, flush=True)
+  for _ in range(2):
+    for inp, dense in ((ev, False), (fev, False), (vec, True)):
+      want = oracle_mod.jitconn_matvec(inp, log_p=lp, seed=5, n_row=n_out, n_col=n_in, dense=dense, per_stream_seed=True)
+      got = kernel_call(inp, w_kind="homo", log_p=lp, seed=5, n_row=n_out, n_col=n_in, col_walk=False, dense=dense)
+      assert want.any() and np.array_equal(got.astype(np.float64), want.astype(np.float64)), (inp.dtype, dense)
+  for w_kind, a, b in (("uniform", 0.25, 1.75), ("normal", 0.5, 2.0)):
+    for inp, dense, dt in ((ev, False, np.float32), (vec.astype(np.float32), True, np.float32), (vec, True, np.float64)):
+      want = oracle_mod.jitconn_matvec(inp, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=5, n_row=n_out, n_col=n_in,
+                                       dense=dense, per_stream_seed=True)
+      got = kernel_call(inp, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=5, n_row=n_out, n_col=n_in, col_walk=False,
+                        dense=dense)
+      # about 200 synapses per row (20 of them active for events), inputs up to 3 in magnitude
+      mag = np.full(n_out, (abs(a) + 5 * abs(b)) * (3 * 260 if dense else 60))
+      assert_close_reordered(got, want, mag, dt, what="fused row walk %s" % w_kind)

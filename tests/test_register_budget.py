@@ -24,8 +24,8 @@ TWO_PER_CU = [
   (r"csr_gather_kernel<float, float, (true|false), 1, 1>", "csr_matvec with the vector staged in LDS, float"),
   (r"csr_scatter_window_kernel<", "event scatter into LDS windows"),
   (r"bin_active_rows_kernel<", "producer of the sorted event scatter"),
-  (r"jitconn_rowwalk_kernel<\w+, bpl::PackedBits, 0, \d, 2>", "jitconn row walk with the two-level bitmap"),
-  (r"jitconn_rowwalk_kernel<float, [\w: ]+, \d, 2, \d>", "jitconn row walk, float normal weights"),
+  (r"jitconn_rowwalk_kernel<\w+, bpl::PackedBits, 0, \d, 2, (true|false)>", "jitconn row walk with the two-level bitmap"),
+  (r"jitconn_rowwalk_kernel<float, [\w: ]+, \d, 2, \d, (true|false)>", "jitconn row walk, float normal weights"),
   (r"jitconn_colwalk_bins_kernel<float,", "jitconn column walk into bins, float"),
 ]
 
@@ -72,7 +72,10 @@ def test_kernels_meant_to_share_a_cu_fit_twice(kernels):
 
 def test_no_kernel_spills_vector_registers_unexpectedly(kernels):
   # scratch-memory spills are tolerated only where the eight-wave budget was chosen knowingly
-  allowed = (r"jitconn_rowwalk_kernel<double, bpl::PackedBits, 0, 2, 2>",)
+  # (double normal weights behind the two-level bitmap: 6-7 registers; float normal weights with the
+  # generators seeded inside the kernel: 2-4 registers, and still 13 % faster than seeding ahead)
+  allowed = (r"jitconn_rowwalk_kernel<double, bpl::PackedBits, 0, 2, 2, (true|false)>",
+             r"jitconn_rowwalk_kernel<float, [\w: ]+, \d, 2, \d, true>")
   spilled = [k.split("(")[0] for k, (_, _, spill) in kernels.items()
              if spill and not any(re.search(a, k) for a in allowed)]
   assert not spilled, spilled
