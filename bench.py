@@ -705,9 +705,10 @@ def main():
       if out_row[r] != np.float32(j["events"][idx].sum()) * np.float32(0.1):
         raise SystemExit("parity gate failed for jitconn event matvec row %d" % r)
     jit = {"generated_synapses": generated}
-    # the row walk is bound by VALU issue: peak = CUs x 64 lanes x clock lane-instructions per second; the
-    # busy fraction is a counter reading (SQ_ACTIVE_INST_VALU x 4 / SQ_BUSY_CYCLES per SIMD) recorded from the
-    # rocprofv3 --pmc run of this workload (`--pmc jitconn`), since counters cannot be read in-process
+    # the row walk is bound by VALU issue: peak = CUs x 64 lanes x clock lane-instructions per second (one
+    # wave64 instruction per SIMD every four cycles).  The number of vector instructions a call executes is a
+    # counter reading (SQ_INSTS_VALU, rocprofv3 --pmc run of this workload, `--pmc jitconn`), since counters
+    # cannot be read in-process; the time it is divided by is measured here.
     props = torch.cuda.get_device_properties(dev)
     clock_hz = float(getattr(props, "clock_rate", 2400000)) * 1e3
     jit["valu_roofline"] = {"bound": "valu", "peak_lane_instr_per_s": props.multi_processor_count * 64 * clock_hz,
@@ -721,11 +722,17 @@ def main():
         jit[key] = dict(stats(d), implicit_gsyn_per_s=generated / (d.mean() * 1e-3) / 1e9)
     call_us = jit["transpose=False,outdim_parallel=True"]["mean_us"]
     rec_j = recorded_counters("jitconn_rowwalk_1e9", call_us, generated_synapses=generated)
-    jit["valu_roofline"]["busy_frac_recorded"] = rec_j["valu_busy_frac"] if rec_j else None
-    jit["valu_roofline"]["valu_instr_per_64_synapses_recorded"] = rec_j["valu_instr_per_64_synapses"] if rec_j else None
-    jit["valu_roofline"]["recorded_in"] = rec_j["profile"] if rec_j else None
-    jit["valu_roofline"]["recorded_at"] = dict(git_rev=rec_j["git_rev"], kernel=rec_j["kernel"],
-                                               call_us=rec_j["kernel_us"]) if rec_j else None
+    vr = jit["valu_roofline"]
+    if rec_j:
+      lane_instr = rec_j["valu_wave_instr_per_call"] * 64.0
+      vr.update(achieved_lane_instr_per_s=lane_instr / (call_us * 1e-6),
+                frac=lane_instr / (call_us * 1e-6) / vr["peak_lane_instr_per_s"],
+                valu_instr_per_64_synapses_recorded=rec_j["valu_instr_per_64_synapses"],
+                valu_active_over_simd_cycles_recorded=rec_j["valu_active_over_simd_cycles"],
+                recorded_in=rec_j["profile"],
+                recorded_at=dict(git_rev=rec_j["git_rev"], kernel=rec_j["kernel"], call_us=rec_j["kernel_us"]))
+    else:
+      vr.update(achieved_lane_instr_per_s=None, frac=None, recorded_in=None)
     if not args.skip_cpu:
       # reference CPU algorithm (one sequential mt19937) on the first 4,000 rows of the same matrix
       rows = 4000
