@@ -316,6 +316,7 @@ __global__ __launch_bounds__(1024) void collect_active_columns_kernel(const VT *
 // first launch of a call), so that a call may be split into several launches; a pair that finds
 // its bin full is added to `out` directly.  add_uniform_bins() then adds the bins window by window.
 constexpr int kColBinThreads = 1024;  // 16 waves share one set of bins: 4 times fewer, 4 times larger bins
+constexpr size_t kColBinBytesMax = static_cast<size_t>(3) << 30;  // bins of the dense column walk (scratch memory)
 
 template <typename T1, typename VT, int IN, int W>
 __global__ __launch_bounds__(kColBinThreads, sizeof(T1) == 4 ? 8 : 4) void jitconn_colwalk_bins_kernel(
@@ -583,12 +584,23 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
   if (n_win <= kBinMaxWindows && full >= (IN == kInDense ? 1048576.0 : 5.0e7)) {
     uint32_t producers = 2u * static_cast<uint32_t>(device_info().num_cu);
     if (producers > div_up(n_in, kColBinThreads / kWave)) producers = div_up(n_in, kColBinThreads / kWave);
-    const double per_bin = full / (static_cast<double>(producers) * n_win);  // every column active
-    double cap_d = 1.25 * per_bin + 6.0 * std::sqrt(per_bin) + 128.0;
-    if (IN == kInEvent) cap_d = cap_d / 8.0 < 512.0 ? 512.0 : cap_d / 8.0;
     auto round_up = [](size_t v) { return (v + 255) / 256 * 256; };
-    const size_t total_pairs = static_cast<size_t>(producers) * n_win * static_cast<size_t>(cap_d);
-    const size_t pair_bytes = round_up(total_pairs * sizeof(BinPair<T1>));
+    // Dense input: the bins are emptied (added to `out`) after every `group` chunks of kSeedChunk columns,
+    // the largest number of chunks whose pairs fit kColBinBytesMax of scratch memory (every column of a
+    // 1,000,000 x 1,000,000 matrix with conn_prob 0.001 at once would take 10.7 GB).
+    const uint32_t chunks = div_up(n_in, kSeedChunk);
+    uint32_t group = chunks;
+    double cap_d = 0.0;
+    size_t pair_bytes = 0;
+    for (;;) {
+      const double share = (group >= chunks) ? 1.0 : static_cast<double>(group) * kSeedChunk / static_cast<double>(n_in);
+      const double per_bin = full * share / (static_cast<double>(producers) * n_win);  // every column active
+      cap_d = 1.25 * per_bin + 6.0 * std::sqrt(per_bin) + 128.0;
+      if (IN == kInEvent) cap_d = cap_d / 8.0 < 512.0 ? 512.0 : cap_d / 8.0;
+      pair_bytes = round_up(static_cast<size_t>(producers) * n_win * static_cast<size_t>(cap_d) * sizeof(BinPair<T1>));
+      if (IN == kInEvent || group == 1 || pair_bytes <= kColBinBytesMax) break;
+      group = (group + 1u) / 2u;
+    }
     const size_t count_bytes = round_up(static_cast<size_t>(n_win) * producers * sizeof(uint32_t));
     const uint32_t seeded_max = n_in < kSeedChunk ? n_in : kSeedChunk;
     const size_t state_bytes = round_up(static_cast<size_t>(seeded_max) * kMtN * 4);
@@ -619,7 +631,8 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
                              static_cast<const T1 *>(list_val), static_cast<const uint32_t *>(states), seeded_max,
                              n_win, shift, cap, pairs, counts);
         } else {
-          // every column, a chunk of seeded generators at a time
+          // every column, a chunk of seeded generators at a time; the bins are emptied after every `group` chunks
+          uint32_t in_bins = 0;
           for (uint32_t first = 0; first < n_in; first += kSeedChunk) {
             const uint32_t count = (n_in - first < kSeedChunk) ? n_in - first : kSeedChunk;
             launch_seed_streams(stream, seed, first, count, states);
@@ -627,6 +640,13 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
                                wb, first, count, static_cast<const uint32_t *>(nullptr),
                                static_cast<const uint32_t *>(nullptr), static_cast<const T1 *>(nullptr),
                                static_cast<const uint32_t *>(states), count, n_win, shift, cap, pairs, counts);
+            if (++in_bins == group && first + kSeedChunk < n_in) {
+              if (!add_uniform_bins<T1>("jitconn column walk", stream, out, n_out, shift, producers, cap, pairs, counts,
+                                        static_cast<uint32_t *>(nullptr)))
+                return;  // (the error stands: part of the pairs is in `out` already)
+              fill_zero(stream, counts, n_win * producers);
+              in_bins = 0;
+            }
           }
         }
         if (add_uniform_bins<T1>("jitconn column walk", stream, out, n_out, shift, producers, cap, pairs, counts, list_count))
