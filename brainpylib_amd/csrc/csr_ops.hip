@@ -588,6 +588,8 @@ __global__ __launch_bounds__(256) void sum_partials_kernel(const F *__restrict__
 // gather
 // ------------------------------------------------------------------------------------------------
 
+constexpr uint32_t kHubSteps = 64;  // a row of more steps than this is left to the whole workgroup (gather_hub_rows)
+
 // G lanes walk the rows assigned to their group as ONE sequence of steps of U*G nonzeros: the
 // column indices of the next step (which may belong to the group's next row) are requested
 // before the loads that depend on the current step's indices are consumed, so a row change
@@ -649,12 +651,19 @@ __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const ui
   const uint32_t gl = threadIdx.x % G;
   const uint32_t total_groups = gridDim.x * groups_per_block;
   const F w_homo = HETER ? F(0) : data[0];
+  // A row of more than kHubSteps steps looks empty here: gather_hub_rows() gives it to the whole workgroup.
+  constexpr uint32_t hub_len = kHubSteps * U * G;
+  auto bounds = [&](uint32_t r, uint32_t &s, uint32_t &e) {
+    s = indptr[r], e = indptr[r + 1];
+    if (e - s > hub_len) e = s;
+  };
 
   uint32_t row = blockIdx.x * groups_per_block + threadIdx.x / G;
   if (row >= n_row) return;
-  uint32_t base = indptr[row], end = indptr[row + 1];        // current step: [base, base + U*G) of this row
+  uint32_t base, end;                                         // current step: [base, base + U*G) of this row
+  bounds(row, base, end);
   uint32_t nrow_start = 0, nrow_end = 0;                      // bounds of the group's next row
-  if (row + total_groups < n_row) nrow_start = indptr[row + total_groups], nrow_end = indptr[row + total_groups + 1];
+  if (row + total_groups < n_row) bounds(row + total_groups, nrow_start, nrow_end);
 
   auto load_cols = [&](uint32_t b, uint32_t e, uint32_t (&c)[U]) {
     const uint32_t safe = e ? e - 1 : 0u;  // any valid element (the matrix has at least one)
@@ -705,8 +714,7 @@ __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const ui
     uint32_t coln[U];
     if (more) {
       load_cols(next_base, next_end, coln);
-      if (last_of_row && next_row + total_groups < n_row)
-        nrow_start = indptr[next_row + total_groups], nrow_end = indptr[next_row + total_groups + 1];
+      if (last_of_row && next_row + total_groups < n_row) bounds(next_row + total_groups, nrow_start, nrow_end);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -793,7 +801,8 @@ __device__ __forceinline__ void gather_rows_wave(const F *__restrict__ data, con
   for (uint32_t row = blockIdx.x * waves_per_block + threadIdx.x / kWave; row < n_row; row += total_waves) {
     const uint32_t urow = __builtin_amdgcn_readfirstlane(row);
     const uint32_t start = indptr[urow];
-    const uint32_t len = indptr[urow + 1] - start;
+    uint32_t len = indptr[urow + 1] - start;
+    if (len > kHubSteps * U * kWave) len = 0;  // (the whole workgroup takes it: gather_hub_rows())
     const uint32_t *ip = indices + start;
     const F *dp = data + (HETER ? start : 0u);
     double acc = 0.0;
@@ -812,11 +821,93 @@ __device__ __forceinline__ void gather_rows_wave(const F *__restrict__ data, con
   }
 }
 
+// Hub rows.  The walks above give a row to G lanes (or one wave), so one row that holds a large share
+// of the nonzeros would be walked by a handful of lanes while the rest of the device is done (a row of
+// 1e6 nonzeros among 20,000 of 50: 19 ms).  They treat a row of more than kHubSteps of their steps as
+// empty, and after its walk every workgroup looks through the bounds of the rows it was dealt again
+// (workgroup b: rows b * gpb + g + k * total_groups, g < gpb) and walks each such row with all its
+// threads: partial sums per lane, a wave sum, one float64 (or integer) LDS atomic per wave.
+template <typename F, typename VT, bool HETER, int MODE, int BITS>
+__device__ __forceinline__ void gather_hub_rows(const F *__restrict__ data, const uint32_t *__restrict__ indices,
+                                                const uint32_t *__restrict__ indptr, const VT *__restrict__ x,
+                                                F *__restrict__ y, uint32_t n_row, const uint32_t *s_bits,
+                                                uint32_t coarse_g, uint32_t gpb, uint32_t hub_len) {
+  __shared__ unsigned long long s_mask[1024 / kWave];
+  __shared__ double s_acc;
+  __shared__ uint32_t s_hits;
+  const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave, nwaves = blockDim.x / kWave;
+  const uint32_t total_groups = gridDim.x * gpb;
+  const uint32_t first = blockIdx.x * gpb;
+  if (first >= n_row) return;
+  const uint32_t count = ((n_row - first + total_groups - 1u) / total_groups) * gpb;  // rows dealt to this workgroup
+  const F w_homo = HETER ? F(0) : data[0];
+  auto row_of = [&](uint32_t i) { return (i / gpb) * total_groups + first + (i % gpb); };
+  for (uint32_t i0 = 0; i0 < count; i0 += blockDim.x) {
+    bool hub = false;
+    if (i0 + tid < count) {
+      const uint32_t r = row_of(i0 + tid);
+      if (r < n_row) hub = indptr[r + 1] - indptr[r] > hub_len;
+    }
+    const unsigned long long mine = __ballot(hub);
+    if (!__syncthreads_or(hub)) continue;  // (the usual case: none)
+    if (lane == 0) s_mask[wave] = mine;
+    __syncthreads();
+    for (uint32_t w = 0; w < nwaves; ++w) {
+      unsigned long long m = s_mask[w];
+      while (m != 0) {
+        const uint32_t r = row_of(i0 + w * kWave + static_cast<uint32_t>(__ffsll(m) - 1));
+        m &= m - 1ull;
+        if (tid == 0) s_acc = 0.0, s_hits = 0u;
+        __syncthreads();
+        const uint32_t start = indptr[r], len = indptr[r + 1] - start;
+        double acc = 0.0;
+        uint32_t hits = 0;
+        constexpr uint32_t U = 4;  // loads in flight per lane
+        for (uint32_t j0 = tid; j0 < len; j0 += U * blockDim.x) {
+          uint32_t col[U];
+#pragma unroll
+          for (uint32_t u = 0; u < U; ++u) {
+            const uint32_t j = j0 + u * blockDim.x;
+            col[u] = indices[start + (j < len ? j : len - 1u)];
+          }
+#pragma unroll
+          for (uint32_t u = 0; u < U; ++u) {
+            const uint32_t j = j0 + u * blockDim.x;
+            if (j >= len) continue;
+            if (MODE == kEvent) {
+              if (event_hit<BITS>(s_bits, x, col[u], coarse_g)) {
+                if (HETER) acc += static_cast<double>(data[start + j]);
+                else ++hits;
+              }
+            } else {
+              const F d = HETER ? data[start + j] : w_homo;
+              acc += static_cast<double>(static_cast<F>(static_cast<F>(dense_element<VT, BITS>(x, s_bits, coarse_g, col[u])) * d));
+            }
+          }
+        }
+        if (MODE == kEvent && !HETER) {
+          hits = wave_sum(hits);
+          if (lane == 0 && hits != 0u) atomicAdd(&s_hits, hits);
+        } else {
+          acc = wave_sum(acc);
+          if (lane == 0) atomicAdd(&s_acc, acc);
+        }
+        __syncthreads();
+        if (tid == 0) y[r] = (MODE == kEvent && !HETER) ? gathered_sum(w_homo, s_hits) : static_cast<F>(s_acc);
+        __syncthreads();
+      }
+    }
+  }
+}
+
+// (Event input with the bitmap in LDS is meant to run two workgroups per CU: eight waves per SIMD, asked
+// for here because the homogeneous-weight walks sit at exactly 64 registers and the hub-row pass behind
+// them would otherwise raise the kernel's allocation to 66.)
 // BITS: where the event probes go.  0: the event vector in global memory; 1: a bitmap in LDS;
 // 2: a bitmap in LDS of more than 80 KB (one workgroup per CU; a kernel of its own, because its
 // variants need more than the 64 registers that let two workgroups of the other cases share a CU).
 template <typename F, typename VT, bool HETER, int MODE, int BITS>
-__global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ data,
+__global__ __launch_bounds__(1024, (MODE == kEvent && BITS == 1) ? 8 : 4) void csr_gather_kernel(const F *__restrict__ data,
                                                           const uint32_t *__restrict__ indices,
                                                           const uint32_t *__restrict__ indptr,
                                                           const VT *__restrict__ x, F *__restrict__ y,
@@ -854,6 +945,7 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
   }
   // lanes per row from the mean row length
   const uint32_t mean = nnz / n_row;
+  uint32_t gpb = 0, hub_len = 0;  // rows per workgroup and round of the walk chosen below, its longest row
   if constexpr (MODE == kDense && BITS == 0) {
     // (rows of `skip_mean` nonzeros or more on average: the launcher's other kernel has taken this matrix)
     if (skip_mean != 0 && mean >= skip_mean) return;
@@ -861,35 +953,41 @@ __global__ __launch_bounds__(1024) void csr_gather_kernel(const F *__restrict__ 
   if constexpr (MODE == kDense && BITS == 1) {
     // (nothing left to hide but the index and weight streams: the walks of the event gather)
     const VT *xs = reinterpret_cast<const VT *>(s_bits);
-    if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g);
-    else if (mean >= 24) gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g);
-    else if (mean >= 12) gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g);
-    else gather_rows<F, VT, HETER, MODE, BITS, 4, 4>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g);
+    if (mean >= 384) { gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g); gpb = blockDim.x / kWave; hub_len = kHubSteps * 8 * kWave; }
+    else if (mean >= 24) { gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 8; hub_len = kHubSteps * 8 * 8; }
+    else if (mean >= 12) { gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 4; hub_len = kHubSteps * 8 * 4; }
+    else { gather_rows<F, VT, HETER, MODE, BITS, 4, 4>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 4; hub_len = kHubSteps * 4 * 4; }
   } else if constexpr (MODE == kDense && BITS == 2) {
-    if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
-    else if (mean >= 24) gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
-    else gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    if (mean >= 384) { gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / kWave; hub_len = kHubSteps * 8 * kWave; }
+    else if (mean >= 24) { gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 8; hub_len = kHubSteps * 8 * 8; }
+    else { gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 4; hub_len = kHubSteps * 8 * 4; }
   } else if constexpr (MODE == kEvent && (BITS == 2 || BITS == 3)) {
     // An event bitmap above 80 KB leaves room for one workgroup (16 waves) per CU only: every lane
     // then keeps 16 (rows under 48 nonzeros: 8) loads in flight instead of 2 to 8, in groups of
     // 8 or 4 lanes per row, or HBM sees too few requests (1e6 columns, 100 per row: 424 -> 164 us).
-    if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
-    else if (mean >= 48) gather_rows<F, VT, HETER, MODE, BITS, 8, 16>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
-    else gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    if (mean >= 384) { gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / kWave; hub_len = kHubSteps * 8 * kWave; }
+    else if (mean >= 48) { gather_rows<F, VT, HETER, MODE, BITS, 8, 16>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 8; hub_len = kHubSteps * 16 * 8; }
+    else { gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 4; hub_len = kHubSteps * 8 * 4; }
   } else {
-    if (mean >= 384) gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    if (mean >= 384) { gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / kWave; hub_len = kHubSteps * 8 * kWave; }
     // (a dense vector is gathered from L2: for rows of 48 .. 191 nonzeros the pipelined 32-lane walk keeps more
     // of those gathers in flight than a wave per row does)
-    else if (MODE == kEvent && mean >= 48u) gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
-    else if (MODE == kDense && mean >= 192u) gather_rows_wave<F, VT, HETER, MODE, BITS, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
-    else if (mean >= 48) gather_rows<F, VT, HETER, MODE, BITS, 32, 4>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
-    else if (MODE == kEvent && mean >= 24) gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
-    else if (MODE == kEvent && mean >= 12) gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
-    else if (MODE == kEvent) gather_rows<F, VT, HETER, MODE, BITS, 4, 4>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
-    else if (mean >= 24) gather_rows<F, VT, HETER, MODE, BITS, 32, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
-    else if (mean >= 12) gather_rows<F, VT, HETER, MODE, BITS, 16, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
-    else gather_rows<F, VT, HETER, MODE, BITS, 8, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g);
+    else if (MODE == kEvent && mean >= 48u) { gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 8; hub_len = kHubSteps * 8 * 8; }
+    else if (MODE == kDense && mean >= 192u) { gather_rows_wave<F, VT, HETER, MODE, BITS, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / kWave; hub_len = kHubSteps * 2 * kWave; }
+    else if (mean >= 48) { gather_rows<F, VT, HETER, MODE, BITS, 32, 4>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 32; hub_len = kHubSteps * 4 * 32; }
+    else if (MODE == kEvent && mean >= 24) { gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 8; hub_len = kHubSteps * 8 * 8; }
+    else if (MODE == kEvent && mean >= 12) { gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 4; hub_len = kHubSteps * 8 * 4; }
+    else if (MODE == kEvent) { gather_rows<F, VT, HETER, MODE, BITS, 4, 4>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 4; hub_len = kHubSteps * 4 * 4; }
+    else if (mean >= 24) { gather_rows<F, VT, HETER, MODE, BITS, 32, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 32; hub_len = kHubSteps * 2 * 32; }
+    else if (mean >= 12) { gather_rows<F, VT, HETER, MODE, BITS, 16, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 16; hub_len = kHubSteps * 2 * 16; }
+    else { gather_rows<F, VT, HETER, MODE, BITS, 8, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 8; hub_len = kHubSteps * 2 * 8; }
   }
+  // the rows the walk left to the whole workgroup
+  if constexpr (MODE == kDense && BITS == 1)
+    gather_hub_rows<F, VT, HETER, MODE, BITS>(data, indices, indptr, reinterpret_cast<const VT *>(s_bits), y, n_row, s_bits,
+                                              coarse_g, gpb, hub_len);
+  else
+    gather_hub_rows<F, VT, HETER, MODE, BITS>(data, indices, indptr, x, y, n_row, s_bits, coarse_g, gpb, hub_len);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1262,7 +1360,7 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
     const size_t lds_bytes = (static_cast<size_t>(n_col) + 31) / 32 * 4;
     const size_t lds_cap = kLdsBitmapCap;
     if (lds_bytes <= lds_cap) {
-      const bool ok = lds_bytes > 80 * 1024
+      const bool ok = lds_bytes > 80 * 1024 - 512  // (two workgroups per CU below: 80 KB each, less their static LDS)
                           ? launch_gather_impl<F, VT, HETER, MODE, 2>(target, stream, data, indices, indptr, x, y, n_row,
                                                                       n_col, lds_bytes)
                           : launch_gather_impl<F, VT, HETER, MODE, 1>(target, stream, data, indices, indptr, x, y, n_row,

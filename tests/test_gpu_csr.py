@@ -690,3 +690,49 @@ def test_csr_matvec_hub_row_time(cuda):
   per_call_us = e0.elapsed_time(e1) * 1e3 / 5
   print("hub row of 1e6 nonzeros: %.1f us per call" % per_call_us, flush=True)
   assert per_call_us < 500.0
+
+
+def test_gather_hub_rows(cuda, oracle_mod):
+  # rows that hold a large share of the nonzeros are left to the whole workgroup by every walk of the
+  # gather (groups of 4, 8 or 32 lanes per row, a wave per row; LDS bitmap and two-level bitmap; the
+  # dense product of matrices too small for its 16-byte walk): exact results on integer data, several
+  # hub rows per workgroup, and a bound on the time of a row of a million nonzeros (one wave: 19 ms)
+  rng = np.random.default_rng(8)
+  cases = [  # n_row, n_col, ordinary rows, {row: nonzeros}
+    (100_000, 100_000, 12, {777: 90_000, 778: 5000, 99_999: 2000, 0: 1025}),
+    (30_000, 60_000, 30, {5: 50_000, 29_000: 4097}),
+    (2000, 50_000, 500, {3: 40_000, 1999: 33_000}),
+    (20_000, 2_000_000, 50, {777: 1_000_000}),
+  ]
+  dev = torch.device("cuda:0")
+  for n_row, n_col, base, hubs in cases:
+    counts = np.full(n_row, base)
+    for r, c in hubs.items():
+      counts[r] = c
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_row)
+    print("case", n_row, n_col, base, hubs, flush=True)
+    ev = rng.random(n_col) < 0.3
+    for dtype in (np.float32, np.float64):
+      data = rng.integers(-2, 3, size=indices.shape[0]).astype(dtype)
+      for d in (data, np.array([0.6], dtype=dtype)):
+        want = oracle_mod.event_csr_matvec(d, indices, indptr, ev, shape=(n_row, n_col))
+        got = bpl.event_csr_matvec(d, indices, indptr, ev, shape=(n_row, n_col)).cpu().numpy()
+        assert np.array_equal(got, want), (n_row, dtype.__name__, d.shape, np.flatnonzero(got != want)[:5])
+      if n_row <= 30_000 and n_col <= 60_000:  # (dense product through the same kernel)
+        v = rng.integers(-3, 4, size=n_col).astype(dtype)
+        want = oracle_mod.csr_matvec(data, indices, indptr, v, shape=(n_row, n_col))
+        got = bpl.csr_matvec(data, indices, indptr, v, shape=(n_row, n_col)).cpu().numpy()
+        assert np.array_equal(got, want), (n_row, dtype.__name__)
+  # time of the last case (float32, heterogeneous weights)
+  args = [torch.from_numpy(a).to(dev) for a in (data.astype(np.float32), indices, indptr, ev)]
+  bpl.event_csr_matvec(*args, shape=(n_row, n_col))
+  torch.cuda.synchronize()
+  e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+  e0.record()
+  for _ in range(5):
+    bpl.event_csr_matvec(*args, shape=(n_row, n_col))
+  e1.record()
+  torch.cuda.synchronize()
+  per_call_us = e0.elapsed_time(e1) * 1e3 / 5
+  print("event gather with a hub row of 1e6 nonzeros: %.1f us per call" % per_call_us, flush=True)
+  assert per_call_us < 3000.0
