@@ -159,11 +159,14 @@ uint32_t *stream_counters(hipStream_t stream) {
     return nullptr;
   }
   uint32_t *p = nullptr;
-  if (hipMalloc(reinterpret_cast<void **>(&p), kStreamCounterBytes) != hipSuccess ||
-      hipMemset(p, 0, kStreamCounterBytes) != hipSuccess) {
+  if (hipMalloc(reinterpret_cast<void **>(&p), kStreamCounterBytes) != hipSuccess) {
     (void)hipGetLastError();
     return nullptr;
   }
+  // Zeroed by a kernel on the stream that will use them.  (hipMemset works on the null stream and does not
+  // wait for the host; a non-blocking stream does not wait for the null stream either, so the first call on
+  // such a stream could count its active rows before the zeros arrived and then lose the count to them.)
+  fill_zero(stream, p, static_cast<uint32_t>(kStreamCounterBytes / sizeof(uint32_t)));
   entries.push_back(Entry{dev, stream, p});
   return p;
 }

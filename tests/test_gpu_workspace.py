@@ -60,7 +60,7 @@ def test_outgrown_buffer_is_retired_not_freed(cuda):
   del b
 
 
-def test_growth_is_refused_during_capture_and_works_after_a_warm_up(cuda):
+def test_growth_is_refused_during_capture_and_works_after_a_warm_up(cuda, oracle_mod):
   s = torch.cuda.Stream()
   args = _scatter_inputs(cuda, 30_000, 30_000, 3)
   torch.cuda.synchronize()
@@ -78,6 +78,10 @@ def test_growth_is_refused_during_capture_and_works_after_a_warm_up(cuda):
   with torch.cuda.stream(s):
     want = bpl.event_csr_matvec(*args, shape=(30_000, 30_000), transpose=True).clone()
   s.synchronize()
+  # (the stream's first call: its counters and scratch memory were allocated inside it)
+  host = [a.cpu().numpy() for a in args]
+  ref = oracle_mod.event_csr_matvec(*host, shape=(30_000, 30_000), transpose=True)
+  assert np.allclose(want.cpu().numpy(), ref, rtol=1e-5, atol=1e-5)
   before = _query(s.cuda_stream)
   g2 = torch.cuda.CUDAGraph()
   with torch.cuda.graph(g2, stream=s):
