@@ -65,6 +65,11 @@ BPL_HOST_DEVICE inline F repeated_sum(F w, uint64_t n) {
   if (n == 0) return F(0);
   const F first = F(0) + w;  // 0 + (-0) is +0; NaN and the infinities stay what they are
   if (!(w == w) || w == F(0) || biased_exponent(w) == FloatFormat<F>::kExpMask) return first;
+  if (n <= 16) {  // few addends (the usual count of a spiking network's time step): the loop itself
+    F s = first;
+    for (uint32_t k = 1; k < static_cast<uint32_t>(n); ++k) s = s + w;
+    return s;
+  }
   const F a = w < F(0) ? -w : w;  // rounding to nearest is symmetric: sum |w|, restore the sign
   F s = a;
   uint64_t left = n - 1;
