@@ -59,6 +59,17 @@ def counted_csr(counts, n_col, seed):
   assert total < 2 ** 31 and counts.max(initial=0) <= n_col
   rows = np.repeat(np.arange(n_row, dtype=np.int64), counts)
   key = rows * n_col + rng.integers(0, n_col, size=total, dtype=np.int64)
+  # rows that want more than half of the columns take the head of a shuffle of all columns: drawing
+  # again until nothing repeats would need ~n_col * ln(n_col) rounds for a full row
+  crowded = np.flatnonzero(counts * 2 > n_col)
+  if crowded.size:
+    shuffle = np.random.default_rng([int(seed), 0x5eed])
+    r = np.repeat(crowded, n_col)
+    c = np.tile(np.arange(n_col, dtype=np.int64), crowded.size)
+    order = np.lexsort((shuffle.random(r.size), r))
+    keep = (np.arange(r.size) % n_col) < counts[r]
+    crowded_key = (r * n_col + c[order])[keep]  # r is already grouped by row, in rising order
+    key[np.isin(rows, crowded)] = crowded_key
   key.sort()
   # re-draw the few duplicates until every row's columns are distinct
   while True:
