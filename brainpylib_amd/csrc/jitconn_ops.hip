@@ -65,10 +65,11 @@ __global__ __launch_bounds__(1024, (BITS == 2 || (W == kNormal && sizeof(T1) == 
   constexpr int kWords = StreamLds<T1, W>::words;
   uint32_t *st = smem + wave * kWords;
   const uint32_t *bits = smem + nwaves * kWords;
-  uint32_t coarse_g = 0;
+  uint32_t coarse_g = 0, coarse_g5 = 5;
   if constexpr (BITS == 2) {
     uint32_t *wbits = smem + nwaves * kWords;
     coarse_g = coarse_shift(n_in, kRowwalkCoarseBytes);
+    coarse_g5 = coarse_g + 5u;
     const uint32_t words = (coarse_bits(n_in, coarse_g) + 31u) >> 5;
     const uint32_t *coarse = reinterpret_cast<const uint32_t *>(in) + coarse_offset_words(n_in);
     for (uint32_t i = threadIdx.x; i < words; i += blockDim.x) wbits[i] = coarse[i];
@@ -85,26 +86,28 @@ __global__ __launch_bounds__(1024, (BITS == 2 || (W == kNormal && sizeof(T1) == 
     uint32_t cnt = 0;
     // two-level bitmap: the exact word of a batch is requested when the batch is drawn and looked
     // at when the next one is, so that no wave waits for it
-    uint32_t late_word = 0, late_bit = 0;
-    bool late_coarse = false;
+    uint32_t late_word = 0, late_idx = 0;
+    uint64_t late_coarse = 0;  // lanes whose coarse bit was set (wave uniform, so the scalar unit combines the masks)
+    bool late_lane = false;    // this lane's bit of it
     T1 late_w = T1(0);
     auto settle = [&]() {
-      const bool hit = late_coarse && ((late_word >> late_bit) & 1u);
-      if (W == kHomo) cnt += static_cast<uint32_t>(__popcll(__ballot(hit)));
-      else if (hit) acc += static_cast<double>(late_w);
+      const bool bit = __builtin_amdgcn_ubfe(late_word, late_idx, 1u) != 0u;
+      if (W == kHomo) cnt += static_cast<uint32_t>(__popcll(late_coarse & __builtin_amdgcn_ballot_w64(bit)));
+      else if (bit && late_lane) acc += static_cast<double>(late_w);
     };
     walk_stream<T1, W>(st, lane, seed + o, pre, n_in, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
       if constexpr (IN == kInEvent && BITS == 2) {
         settle();
-        bool coarse = false;
-        if (valid) {
-          const uint32_t c = idx >> coarse_g;
-          coarse = (bits[c >> 5] >> (c & 31u)) & 1u;
-        }
+        // bit c = idx >> g of the coarse bitmap: word c >> 5, bit c & 31 (the bit-field extract takes the
+        // low five bits); lanes past the end of the row look at word 0 and drop what they see
+        const uint32_t c = idx >> coarse_g;
+        const uint32_t cword = bits[valid ? idx >> coarse_g5 : 0u];
+        const bool coarse = static_cast<int>(valid) & static_cast<int>(__builtin_amdgcn_ubfe(cword, c, 1u) != 0u);
         // (lanes without a coarse hit read word 0 and ignore it: a plain load for the whole wave)
         late_word = reinterpret_cast<const uint32_t *>(in)[coarse ? idx >> 5 : 0u];
-        late_bit = idx & 31u;
-        late_coarse = coarse;
+        late_idx = idx;
+        late_coarse = __builtin_amdgcn_ballot_w64(coarse);
+        late_lane = coarse;
         late_w = w;
         return;
       }
@@ -700,10 +703,70 @@ void jitconn_entry(const char *target, hipStream_t stream, void **buffers, const
   check_launch(target);
 }
 
+// ---- self-check of the skip computation -------------------------------------------------------------
+// Draw t of the check: mode 0, two hashed words; mode 1, the canonical value next to a ceil() boundary:
+// U * 2^64 = exp(k * log_p) * 2^64 + j * 2^11 for k = t / 64 + 1, j = t % 64 - 32 (2^11: one unit in the
+// last place of a double in [0.5, 1)).
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {
+  z += 0x9e3779b97f4a7c15ull;
+  z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+  z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+  return z ^ (z >> 31);
+}
+
+__global__ __launch_bounds__(256) void check_skips_kernel(uint32_t seed, uint64_t n, int mode, double log_p,
+                                                          unsigned long long *__restrict__ counts) {
+  const SkipParams sp = make_skip_params(log_p);
+  unsigned long long differ = 0, untrusted = 0;
+  for (uint64_t t = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x; t < n;
+       t += static_cast<uint64_t>(gridDim.x) * 256u) {
+    uint64_t bits;
+    if (mode == 0) {
+      bits = mix64(t + (static_cast<uint64_t>(seed) << 32));
+    } else {
+      const double edge = exp(static_cast<double>(t / 64u + 1u) * log_p) * 0x1p64;
+      bits = (edge < 0x1p64 ? static_cast<uint64_t>(edge) : ~0ull) +
+             static_cast<uint64_t>((static_cast<int64_t>(t % 64u) - 32) * 2048);
+    }
+    const uint32_t lo = static_cast<uint32_t>(bits), hi = static_cast<uint32_t>(bits >> 32);
+    bool safe;
+    const uint32_t fast = skip_fast(lo, hi, sp, safe);
+    const uint32_t exact = skip_exact(lo, hi, sp);
+    if (!safe) ++untrusted;
+    else if (fast != exact) ++differ;
+  }
+  if (differ) atomicAdd(&counts[0], differ);
+  if (untrusted) atomicAdd(&counts[1], untrusted);
+}
+
+// |hardware log2 - log2| over every fp32 in [0.5, 1): the largest, as the bits of a double
+__global__ __launch_bounds__(256) void check_log2_kernel(unsigned long long *__restrict__ worst) {
+  const uint32_t t = blockIdx.x * 256u + threadIdx.x;  // < 2^23
+  const float m = __uint_as_float(0x3f000000u | t);
+  const double err = fabs(static_cast<double>(__log2f(m)) - log2(static_cast<double>(m)));
+  double wave_worst = err;
+  for (int d = kWave / 2; d > 0; d >>= 1) wave_worst = fmax(wave_worst, __shfl_xor(wave_worst, d, kWave));
+  if (lane_id() == 0) atomicMax(worst, static_cast<unsigned long long>(__double_as_longlong(wave_worst)));
+  if (t == 0) worst[1] = static_cast<unsigned long long>(__double_as_longlong(kSkipLog2Error));
+}
+
 }  // namespace
 }  // namespace bpl
 
 using namespace bpl;
+
+extern "C" int bpl_selfcheck_jitconn_skips(bpl_stream_t stream, uint32_t seed, uint64_t n_draws, int near_boundaries,
+                                           double log_p, uint64_t *counts) {
+  if (counts == nullptr || !(log_p < 0.0)) {
+    set_error("bpl_selfcheck_jitconn_skips: counts must be device memory for four words and log_p negative");
+    return 1;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  unsigned long long *c = reinterpret_cast<unsigned long long *>(counts);
+  hipLaunchKernelGGL(check_skips_kernel, dim3(2048), dim3(256), 0, s, seed, n_draws, near_boundaries ? 1 : 0, log_p, c);
+  hipLaunchKernelGGL(check_log2_kernel, dim3((1u << 23) / 256u), dim3(256), 0, s, c + 2);
+  return check_launch("bpl_selfcheck_jitconn_skips") ? 0 : 1;
+}
 
 #define BPL_DEFINE(name, ...)                                                                      \
   extern "C" void name(bpl_stream_t stream, void **buffers, const char *opaque, size_t opaque_len) { \

@@ -8,7 +8,8 @@
 //
 // MT19937 produces word t from words t-624, t-623 and t-227, so up to 227 consecutive words can
 // be produced at once from the previous 624: each lane computes K consecutive words
-// (64*K <= 227) of the next batch and the 624-word state is a circular buffer in LDS.
+// (64*K <= 227) of the next batch and the 624-word state is a circular buffer in LDS, followed by
+// a copy of its first kMtMirror words so that a lane's run of consecutive words never wraps.
 // Seeding is a serial 623-step recurrence; it runs on the scalar unit (the seed is wave
 // uniform) and the values are packed 64 at a time into a vector register with v_writelane.
 #pragma once
@@ -19,7 +20,8 @@ namespace bpl {
 
 constexpr int kMtN = 624;
 constexpr int kMtM = 397;
-constexpr int kMtStateWords = 624;  // LDS words reserved per wave
+constexpr int kMtMirror = 4;        // st[624 + i] repeats st[i]: runs of up to 5 words from any slot are contiguous
+constexpr int kMtStateWords = kMtN + kMtMirror;  // LDS words reserved per wave
 
 __device__ __forceinline__ void mt_seed(uint32_t *st, uint32_t seed, int lane) {
   uint32_t x = __builtin_amdgcn_readfirstlane(seed);
@@ -33,6 +35,7 @@ __device__ __forceinline__ void mt_seed(uint32_t *st, uint32_t seed, int lane) {
       x = 1812433253u * (x ^ (x >> 30)) + static_cast<uint32_t>(base + i + 1);
     }
     if (base + lane < kMtN) st[base + lane] = v;
+    if (base == 0 && lane < kMtMirror) st[kMtN + lane] = v;
   }
 }
 
@@ -41,6 +44,7 @@ __device__ __forceinline__ void mt_load(uint32_t *st, const uint32_t *__restrict
 #pragma unroll
   for (int base = 0; base < kMtN; base += kWave)
     if (base + lane < kMtN) st[base + lane] = src[base + lane];
+  if (lane < kMtMirror) st[kMtN + lane] = src[lane];
 }
 
 // Seeds 64 generators at once, lane l the stream std::mt19937{first_seed + l}, and stores their
@@ -75,15 +79,24 @@ __device__ __forceinline__ void mt_seed_batch(uint32_t *tile, int lane, uint32_t
   }
 }
 
+// gfx950 evaluates any function of three words bit by bit in one instruction; 0x6c is (a & c) ^ b,
+// 0x96 is a ^ b ^ c (the compiler finds the first only now and then).
+__device__ __forceinline__ uint32_t and_xor(uint32_t a, uint32_t c, uint32_t b) {
+  return __builtin_amdgcn_bitop3_b32(a, b, c, 0x6c);
+}
+
 __device__ __forceinline__ uint32_t mt_twist(uint32_t a, uint32_t b, uint32_t c) {
-  const uint32_t y = (a & 0x80000000u) | (b & 0x7fffffffu);
-  return c ^ (y >> 1) ^ ((y & 1u) ? 0x9908b0dfu : 0u);
+  // y = (a & 0x80000000) | (b & 0x7fffffff) in one bit-field insert (the compiler makes two instructions of it)
+  uint32_t y;
+  asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(y) : "s"(0x7fffffffu), "v"(b), "v"(a));
+  const uint32_t odd = static_cast<uint32_t>(-static_cast<int32_t>(b & 1u));  // all ones when y is odd
+  return and_xor(odd, 0x9908b0dfu, c) ^ (y >> 1);
 }
 
 __device__ __forceinline__ uint32_t mt_temper(uint32_t y) {
   y ^= y >> 11;
-  y ^= (y << 7) & 0x9d2c5680u;
-  y ^= (y << 15) & 0xefc60000u;
+  y = and_xor(y << 7, 0x9d2c5680u, y);
+  y = and_xor(y << 15, 0xefc60000u, y);
   y ^= y >> 18;
   return y;
 }
@@ -91,34 +104,41 @@ __device__ __forceinline__ uint32_t mt_temper(uint32_t y) {
 // Produces the next K * nlanes words of the stream; lane l < nlanes receives words
 // K*l .. K*l + K-1 of them (tempered) in w[].  `pos` is the state slot of the first new word
 // (wave uniform, < 624) and is advanced.  Requires K * nlanes <= 227.
+//
+// A lane reads the K + 1 old words from its first slot s on and the K words from slot
+// (s + 397) mod 624 on, and writes K new words from s on: with the first kMtMirror words repeated
+// behind the 624th, all three runs are contiguous (s + K <= 627), and only a batch that touches
+// the first words or runs past the 624th (a wave-uniform test on `pos`) has copies to keep equal.
 template <int K>
 __device__ __forceinline__ void mt_generate(uint32_t *st, uint32_t &pos, int lane, int nlanes, uint32_t (&w)[K]) {
-  static_assert(K >= 1 && K <= 4, "words per lane");
+  static_assert(K >= 1 && K <= kMtMirror, "words per lane");
+  const uint32_t span = static_cast<uint32_t>(K * nlanes);
   if (lane < nlanes) {
     uint32_t s = pos + static_cast<uint32_t>(K * lane);
-    if (s >= kMtN) s -= kMtN;
-    uint32_t near_[K + 1], far_[K], slot[K];
+    s = min(s, s - kMtN);  // (unsigned: s - 624 wraps to a huge value while s < 624)
+    uint32_t f = s + kMtM;
+    f = min(f, f - kMtN);
+    uint32_t near_[K + 1], far_[K], fresh[K];
 #pragma unroll
-    for (int i = 0; i <= K; ++i) {
-      uint32_t a = s + i;
-      if (a >= kMtN) a -= kMtN;
-      if (i < K) slot[i] = a;
-      near_[i] = st[a];
-    }
+    for (int i = 0; i <= K; ++i) near_[i] = st[s + i];
 #pragma unroll
-    for (int i = 0; i < K; ++i) {
-      uint32_t a = s + i + kMtM;
-      if (a >= kMtN) a -= kMtN;
-      far_[i] = st[a];
-    }
+    for (int i = 0; i < K; ++i) far_[i] = st[f + i];
 #pragma unroll
     for (int i = 0; i < K; ++i) {
-      const uint32_t n = mt_twist(near_[i], near_[i + 1], far_[i]);
-      st[slot[i]] = n;
-      w[i] = mt_temper(n);
+      fresh[i] = mt_twist(near_[i], near_[i + 1], far_[i]);
+      st[s + i] = fresh[i];
+      w[i] = mt_temper(fresh[i]);
+    }
+    if (pos < static_cast<uint32_t>(kMtMirror) || pos + span > static_cast<uint32_t>(kMtN)) {
+#pragma unroll
+      for (int i = 0; i < K; ++i) {
+        const uint32_t a = s + i;
+        if (a >= kMtN) st[a - kMtN] = fresh[i];
+        else if (a < static_cast<uint32_t>(kMtMirror)) st[a + kMtN] = fresh[i];
+      }
     }
   }
-  pos += static_cast<uint32_t>(K * nlanes);
+  pos += span;
   if (pos >= kMtN) pos -= kMtN;
 }
 
@@ -148,41 +168,59 @@ __device__ __forceinline__ uint32_t f64_to_u32_x86(double x) {
 struct SkipParams {
   double log_p;      // log(1 - p)
   double inv_log2;   // ln(2) / log_p: skip = ceil(log2(U) * inv_log2)
-  double guard;      // half-width of the band around integers in which the fast path is not trusted
+  double offset;     // 1 - 32 * inv_log2: the fast path works on log2(U * 2^32) and truncates instead of ceil()
+  double safe_half;  // the fast path is trusted while |frac(q) - 1/2| < safe_half = 1/2 - guard
 };
+
+// Error of the fast path's log2(U): U * 2^32 is formed in fp32 from the two words (two roundings,
+// 2^-23 relative, 1.72e-7 on the logarithm) and the hardware fp32 log2 of its mantissa in [0.5, 1) is
+// documented to 1 ulp, 2^-24 = 5.96e-8 on a result in [-1, 0] (bpl_selfcheck_jitconn_skips measures
+// it over all 2^23 mantissas): 2.32e-7 together, the rest is margin.
+constexpr double kSkipLog2Error = 3e-7;
 
 __device__ __forceinline__ SkipParams make_skip_params(double log_p) {
   SkipParams sp;
   sp.log_p = log_p;
   sp.inv_log2 = 0.6931471805599453094 / log_p;
-  // The fast path takes log2 of the mantissa from the hardware fp32 log (documented to 1 ulp; 4e-7
-  // absolute on log2(U) is assumed here, which also covers rounding the mantissa to fp32), so the
-  // quotient is off by at most 4e-7 * |inv_log2| plus fp64 rounding.
-  sp.guard = 4e-7 * fabs(sp.inv_log2) + 1e-9;
+  sp.offset = 1.0 - 32.0 * sp.inv_log2;
+  // The quotient is off by at most kSkipLog2Error * |inv_log2| plus fp64 rounding; inside that band
+  // around an integer the exact path decides.  Quotients that could leave the range of uint32
+  // (log2(U) >= -64): always the exact path, which converts as x86-64 does.
+  const double guard = kSkipLog2Error * fabs(sp.inv_log2) + 1e-9;
+  sp.safe_half = (fabs(sp.inv_log2) * 64.0 + 2.0 < 4.0e9) ? 0.5 - guard : -1.0;
   return sp;
 }
 
 // One geometric skip: (unsigned) ceil(log(U) / log_p)  (lib/cpu_jitconn_event_matvec.cpp:24),
-// U = canonical double of two generator words.
+// U = canonical double of two generator words (low word first).
 //
-// Exact path: fp64 log and IEEE division, as the CPU code.  Fast path: log2(U) = exponent +
-// v_log_f32(mantissa) and one multiply; its result is used only when it is further than
-// `guard` from an integer, i.e. when no rounding of the exact path could land on another
-// ceil().  If any lane of the wave is inside the band, the whole wave takes the exact path
-// (a wave-uniform branch); for conn_prob around 1e-3 that happens in a few per cent of the
-// batches, for very sparse matrices (guard >= 0.5) always.
-__device__ __forceinline__ uint32_t skip_from_words(uint32_t lo, uint32_t hi, const SkipParams &sp) {
-  const double u = canonical_f64(lo, hi);
+// Exact path: fp64 log and IEEE division, as the CPU code.
+__device__ __forceinline__ uint32_t skip_exact(uint32_t lo, uint32_t hi, const SkipParams &sp) {
+  return f64_to_u32_x86(ceil(log(canonical_f64(lo, hi)) / sp.log_p));
+}
+
+// Fast path: log2(U * 2^32) = exponent + v_log_f32(mantissa) of the fp32 value of the two words, one
+// fused multiply-add to q + 1 = log2(U) * inv_log2 + 1, truncation.  `safe` says that q is further
+// than the guard from an integer, i.e. that no rounding of the exact path could land on another
+// ceil() (not so for q = inf or NaN, U = 0).
+__device__ __forceinline__ uint32_t skip_fast(uint32_t lo, uint32_t hi, const SkipParams &sp, bool &safe) {
+  const float f = fmaf(static_cast<float>(lo), 0x1p-32f, static_cast<float>(hi));
   int e;
-  const double m = frexp(u, &e);  // u = m * 2^e, m in [0.5, 1)
-  const double l2 = static_cast<double>(e) + static_cast<double>(__log2f(static_cast<float>(m)));
-  const double q = l2 * sp.inv_log2;
-  const double c = ceil(q);
-  // distance of q to the nearest integer: c - q or q - (c - 1)
-  const double d = fmin(c - q, q - (c - 1.0));
-  const bool risky = !(d > sp.guard) || !(q < 4.0e9);
-  if (__ballot(risky) == 0) return static_cast<uint32_t>(c);
-  return f64_to_u32_x86(ceil(log(u) / sp.log_p));
+  const float m = frexpf(f, &e);  // f = m * 2^e, m in [0.5, 1)
+  const double l2 = static_cast<double>(e) + static_cast<double>(__log2f(m));
+  const double q1 = fma(l2, sp.inv_log2, sp.offset);
+  safe = fabs(__builtin_amdgcn_fract(q1) - 0.5) < sp.safe_half;
+  return static_cast<uint32_t>(q1);
+}
+
+// If any lane of the wave is inside the band, the whole wave takes the exact path (a wave-uniform
+// branch); for conn_prob around 1e-3 that happens in a few per cent of the batches, for very sparse
+// matrices (guard >= 0.5) always.
+__device__ __forceinline__ uint32_t skip_from_words(uint32_t lo, uint32_t hi, const SkipParams &sp) {
+  bool safe;
+  const uint32_t fast = skip_fast(lo, hi, sp, safe);
+  if (__ballot(!safe) == 0) return fast;
+  return skip_exact(lo, hi, sp);
 }
 
 }  // namespace bpl

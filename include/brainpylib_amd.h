@@ -201,6 +201,20 @@ const char *bpl_version(void);
  * three pointers may be NULL. */
 int bpl_stream_workspace_query(bpl_stream_t stream, void **ptr, size_t *bytes, size_t *retired_bytes);
 
+/* Self-check of the jitconn operators' skip computation (no counterpart in the reference, whose
+ * kernels call log() per synapse, lib/gpu_jitconn_event_matvec.cu:94-110).  The kernels compute
+ * ceil(log(U) / log_p) on a fast path (hardware fp32 log2) wherever the quotient is further from an
+ * integer than a guard band, and as the CPU code does (lib/cpu_jitconn_event_matvec.cpp:24)
+ * elsewhere.  This call evaluates both paths for n_draws values of U on the device: hashed ones, or
+ * (near_boundaries != 0) values within 32 units in the last place of exp(k * log_p), k = 1, 2, ...
+ * `counts` is device memory for four 64-bit words which the CALLER has zeroed: [0] += draws where
+ * the fast path was trusted and differs from the exact one (must stay 0), [1] += draws inside the
+ * guard band, [2] = max(old, bits of the largest |hardware log2(m) - log2(m)| over every fp32 m in
+ * [0.5, 1) as a double), [3] = bits of the error of log2(U) that the guard band is built for, as a
+ * double.  Returns 0 when the kernels were enqueued on `stream`. */
+int bpl_selfcheck_jitconn_skips(bpl_stream_t stream, uint32_t seed, uint64_t n_draws, int near_boundaries,
+                                double log_p, uint64_t *counts);
+
 /* ------------------------------------------------------------------------------------------
  * event_csr_matvec  (lib/gpu_event_csr_matvec.cu:222-260; launchers :148-217)
  *   buffers = [data, indices, indptr, events, out]
