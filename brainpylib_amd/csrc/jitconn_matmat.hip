@@ -70,7 +70,9 @@ __global__ __launch_bounds__(256) void jitconn_matmat_kernel(const T1 *__restric
   const uint32_t row_base = blockIdx.y * (MT * kWave);  // first row of Y of this pass
   // byte offsets into XT fit 32 bits (checked by the host): one add per synapse instead of a 64-bit product
   const uint32_t row_bytes = m_pad * static_cast<uint32_t>(sizeof(T1));
-  const char *xt_lane = reinterpret_cast<const char *>(XT + row_base + lane);
+  // (a wave-uniform base and a 32-bit offset per lane: one address add per synapse and the base in scalar registers)
+  const char *xt_base = reinterpret_cast<const char *>(XT + row_base);
+  const uint32_t lane_bytes = static_cast<uint32_t>(lane) * static_cast<uint32_t>(sizeof(T1));
 
   for (uint32_t j = blockIdx.x * kWaves + wave; j < n; j += gridDim.x * kWaves) {
     T1 acc[MT];
@@ -100,7 +102,7 @@ __global__ __launch_bounds__(256) void jitconn_matmat_kernel(const T1 *__restric
         for (int u = 0; u < U; ++u) {
           const Synapse<T1> e = syn[i + u];
           ws[u] = e.w;
-          const T1 *row = reinterpret_cast<const T1 *>(xt_lane + e.off);
+          const T1 *row = reinterpret_cast<const T1 *>(xt_base + (e.off + lane_bytes));
 #pragma unroll
           for (int t = 0; t < MT; ++t) x[u][t] = row[t * kWave];
         }
@@ -112,7 +114,7 @@ __global__ __launch_bounds__(256) void jitconn_matmat_kernel(const T1 *__restric
       }
       for (; i < count; ++i) {
         const Synapse<T1> e = syn[i];
-        const T1 *row = reinterpret_cast<const T1 *>(xt_lane + e.off);
+        const T1 *row = reinterpret_cast<const T1 *>(xt_base + (e.off + lane_bytes));
 #pragma unroll
         for (int t = 0; t < MT; ++t) acc[t] = add_rn(acc[t], mul_rn(e.w, row[t * kWave]));
       }
