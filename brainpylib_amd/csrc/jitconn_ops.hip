@@ -160,7 +160,7 @@ __global__ __launch_bounds__(1024, (BITS == 2 || (W == kNormal && sizeof(T1) == 
     if (mine == 0) return;
     auto seed_batch = [&](uint32_t j) {
       const uint32_t slot = j % kFuseSlots;
-      mt_seed_batch(st, lane, seed + (blockIdx.x + j * gridDim.x) * kFuseBatch,
+      mt_seed_batch(st, lane, seed + (blockIdx.x + j * gridDim.x) * kFuseBatch + static_cast<uint32_t>(lane),
                     ring + static_cast<size_t>(slot) * kFuseBatch * kMtN);
       __hip_atomic_store(&s_ready[slot], j + 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     };
@@ -385,24 +385,17 @@ __global__ __launch_bounds__(kSeedThreads) void mt_seed_streams_kernel(uint32_t 
                                                                       uint32_t *__restrict__ states,
                                                                       const uint32_t *__restrict__ ids,
                                                                       const uint32_t *__restrict__ count_dev) {
-  __shared__ uint32_t s_tile[kSeedThreads / kWave][kWave][kWave + 1];
-  const uint32_t lane = static_cast<uint32_t>(lane_id()), wave = threadIdx.x / kWave;
+  __shared__ uint32_t s_tile[kSeedThreads / kWave][kMtSeedTileWords];
+  const int lane = lane_id();
+  const uint32_t wave = threadIdx.x / kWave;
   const uint32_t base = (blockIdx.x * (kSeedThreads / kWave) + wave) * kWave;  // first stream of this wave
   if (count_dev != nullptr && *count_dev < count) count = *count_dev;
   if (base >= count) return;
-  uint32_t (*tile)[kWave + 1] = s_tile[wave];
-  uint32_t x = seed + first + base + lane;  // lane l seeds stream base + l
-  if (ids != nullptr) x = seed + ((base + lane < count) ? ids[base + lane] : 0u);
-  for (uint32_t w0 = 0; w0 < kMtN; w0 += kWave) {
-    const uint32_t nw = (kMtN - w0 < kWave) ? kMtN - w0 : kWave;
-    for (uint32_t i = 0; i < nw; ++i) {
-      tile[i][lane] = x;  // word w0 + i of stream base + lane
-      x = 1812433253u * (x ^ (x >> 30)) + (w0 + i + 1);
-    }
-    // transposed: one contiguous run of words per stream
-    for (uint32_t r = 0; r < kWave && base + r < count; ++r)
-      if (lane < nw) states[static_cast<size_t>(base + r) * kMtN + w0 + lane] = tile[lane][r];
-  }
+  const uint32_t mine = base + static_cast<uint32_t>(lane);  // lane l seeds stream base + l
+  uint32_t x = seed + first + mine;
+  if (ids != nullptr) x = seed + (mine < count ? ids[mine] : 0u);
+  mt_seed_batch(s_tile[wave], lane, x, states + static_cast<size_t>(base) * kMtN,
+                count - base < static_cast<uint32_t>(kWave) ? count - base : static_cast<uint32_t>(kWave));
 }
 
 }  // namespace

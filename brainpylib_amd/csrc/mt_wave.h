@@ -47,16 +47,18 @@ __device__ __forceinline__ void mt_load(uint32_t *st, const uint32_t *__restrict
   if (lane < kMtMirror) st[kMtN + lane] = src[lane];
 }
 
-// Seeds 64 generators at once, lane l the stream std::mt19937{first_seed + l}, and stores their
-// states at dst[l * 624 .. + 624).  The 623-step recurrence of the 64 streams advances in lock step
-// on the vector unit (a few dozen instructions per stream instead of the scalar unit's 3,100 for
-// one); every eight steps the words pass through `tile` (LDS of the calling wave, 8 x 65 words) so
-// that they leave as 32-byte runs per stream instead of 4-byte words 2,496 bytes apart.  (Plain
-// stores: the states are read back soon, by waves of the same workgroup, and do best when they stay
-// in the L2; with nontemporal stores and loads the 1e6-row walk took 3.6 instead of 3.1 ms.)
+// Seeds 64 generators at once, lane l the stream std::mt19937{lane_seed}, and stores the states of
+// the first n_streams of them at dst[l * 624 .. + 624).  The 623-step recurrence of the 64 streams
+// advances in lock step on the vector unit (a few dozen instructions per stream instead of the
+// scalar unit's 3,100 for one); every eight steps the words pass through `tile` (LDS of the calling
+// wave, 8 x 65 words) so that they leave as 32-byte runs per stream instead of 4-byte words 2,496
+// bytes apart.  (Plain stores: the states are read back soon, by waves of the same workgroup, and do
+// best when they stay in the L2; with nontemporal stores and loads the 1e6-row walk took 3.6 instead
+// of 3.1 ms.)
 constexpr int kMtSeedTileWords = 8 * (kWave + 1);
-__device__ __forceinline__ void mt_seed_batch(uint32_t *tile, int lane, uint32_t first_seed, uint32_t *__restrict__ dst) {
-  uint32_t x = first_seed + static_cast<uint32_t>(lane);
+__device__ __forceinline__ void mt_seed_batch(uint32_t *tile, int lane, uint32_t lane_seed, uint32_t *__restrict__ dst,
+                                              uint32_t n_streams = kWave) {
+  uint32_t x = lane_seed;
   const uint32_t sub = static_cast<uint32_t>(lane) >> 2, pair = static_cast<uint32_t>(lane) & 3u;  // stream within 16, word pair
   uint2 *out = reinterpret_cast<uint2 *>(dst + static_cast<size_t>(sub) * kMtN) + pair;
 #pragma unroll 1
@@ -73,7 +75,7 @@ __device__ __forceinline__ void mt_seed_batch(uint32_t *tile, int lane, uint32_t
       uint2 v;
       v.x = tile[(2u * pair) * (kWave + 1) + s];
       v.y = tile[(2u * pair + 1u) * (kWave + 1) + s];
-      out[(static_cast<size_t>(16u * q) * kMtN + w0) / 2u] = v;
+      if (s < n_streams) out[(static_cast<size_t>(16u * q) * kMtN + w0) / 2u] = v;
     }
     __builtin_amdgcn_wave_barrier();
   }
