@@ -41,6 +41,21 @@ __device__ __forceinline__ double read_lane_f64(double v, int l) {
   return __longlong_as_double(static_cast<long long>((static_cast<unsigned long long>(hi) << 32) | lo));
 }
 
+// Lane l receives lane l - 1's value, across the whole wave, in one data-parallel move (lane 0
+// keeps its own); the general shuffle goes through the LDS crossbar and a dozen index instructions.
+__device__ __forceinline__ uint32_t wave_shift_up1(uint32_t v) {
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(static_cast<int>(v), static_cast<int>(v), 0x138 /* wave_shr:1 */,
+                                                           0xf, 0xf, false));
+}
+__device__ __forceinline__ float wave_shift_up1(float v) {
+  return __builtin_bit_cast(float, wave_shift_up1(__builtin_bit_cast(uint32_t, v)));
+}
+__device__ __forceinline__ double wave_shift_up1(double v) {
+  const unsigned long long b = static_cast<unsigned long long>(__double_as_longlong(v));
+  const uint32_t lo = wave_shift_up1(static_cast<uint32_t>(b)), hi = wave_shift_up1(static_cast<uint32_t>(b >> 32));
+  return __longlong_as_double(static_cast<long long>((static_cast<unsigned long long>(hi) << 32) | lo));
+}
+
 // std::normal_distribution<float> (libstdc++, Marsaglia polar): candidate pair from two words
 struct PolarF32 {
   float x, y, r2;
@@ -208,8 +223,8 @@ __device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t str
         xw = __fmul_rn(a.x, mult);
         yw = __fmul_rn(a.y, mult);
       }
-      float y_m1 = __shfl_up(yw, 1, kWave);
-      float x_m2 = __shfl_up(xw, 2, kWave);
+      float y_m1 = wave_shift_up1(yw);
+      float x_m2 = wave_shift_up1(wave_shift_up1(xw));
       if (lane == 0) y_m1 = prev_y63, x_m2 = prev_x62;
       if (lane == 1) x_m2 = prev_x63;
       const float raw = is_k1 ? y_m1 : x_m2;
@@ -243,7 +258,7 @@ __device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t str
       uint32_t w[2] = {1u, 1u};
       mt_generate<2>(st, pos, lane, kWave, w);
       const double v = __dsub_rn(__dmul_rn(2.0, canonical_f64(w[0], w[1])), 1.0);
-      double v_m1 = __shfl_up(v, 1, kWave);
+      double v_m1 = wave_shift_up1(v);
       if (lane == 0) v_m1 = prev_v63;
       const double r2 = __dadd_rn(__dmul_rn(v_m1, v_m1), __dmul_rn(v, v));
       const bool ok = !(r2 > 1.0 || r2 == 0.0);  // an attempt (lane - 1, lane) would be accepted
@@ -262,8 +277,8 @@ __device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t str
         xw = __dmul_rn(v_m1, mult);
         yw = __dmul_rn(v, mult);
       }
-      double y_m1 = __shfl_up(yw, 1, kWave);
-      double x_m2 = __shfl_up(xw, 2, kWave);
+      double y_m1 = wave_shift_up1(yw);
+      double x_m2 = wave_shift_up1(wave_shift_up1(xw));
       if (lane == 0) y_m1 = prev_y63, x_m2 = prev_x62;
       if (lane == 1) x_m2 = prev_x63;
       const double raw = is_k1 ? y_m1 : x_m2;
