@@ -163,9 +163,10 @@ __device__ __forceinline__ void walk_stream(uint32_t *st, int lane, uint32_t str
       mt_generate<2>(st, pos, lane, kWave, w);
       const uint32_t skip = skip_from_words(w[0], w[1], log_p);
       const uint32_t idx = carry + wave_inclusive_scan_u32(skip);
-      const uint64_t done = __ballot(idx >= n);
-      const int nvalid = done ? (__ffsll(static_cast<unsigned long long>(done)) - 1) : kWave;
-      f(idx, T1(1), lane < nvalid);
+      // (the positions rise from lane to lane: the lanes of the row are exactly those below n)
+      const bool over = idx >= n;
+      const uint64_t done = __ballot(over);
+      f(idx, T1(1), !over);
       if (done) break;
       carry = __builtin_amdgcn_readlane(idx, kWave - 1);
     }
