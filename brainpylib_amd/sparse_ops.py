@@ -13,7 +13,7 @@ import torch
 from . import _lib
 from ._tensors import FLOAT_DTYPES, as_tensor, device_of, is_index_dtype, to_device
 
-__all__ = ["csr_matvec", "cusparse_csr_matvec", "csr_to_coo", "coo_to_csr", "csr_to_dense"]
+__all__ = ["csr_matvec", "cusparse_csr_matvec", "csr_to_coo", "coo_to_csr", "csr_to_dense", "check_csr"]
 
 
 def _prepare(data, indices, indptr, vector):
@@ -47,6 +47,34 @@ def _check(data, indices, indptr, vector, shape):
 
 def _int64(t):
   return t.view(torch.int32).to(torch.int64) if t.dtype == torch.uint32 else t.to(torch.int64)
+
+
+def check_csr(indices, indptr, *, shape: Tuple[int, int]):
+  """Raises ValueError unless (indices, indptr) describe a CSR matrix of `shape`: indptr starts at 0,
+  never decreases and ends at len(indices); every column index lies in [0, shape[1]).
+
+  The operators trust their index arrays, as the reference's kernels do (an index beyond the
+  matrix is read or written where it points: lib/gpu_event_csr_matvec.cu:47-70 has no check
+  either), so that no call pays for a pass over them.  This check is that pass, for callers who
+  build the arrays themselves; it runs where the arrays live and synchronises once."""
+  indices, indptr = as_tensor(indices), as_tensor(indptr)
+  if not (is_index_dtype(indices.dtype) and is_index_dtype(indptr.dtype)):
+    raise ValueError('indices and indptr should be 1D vectors with int32 or uint32 type.')
+  if indices.ndim != 1 or indptr.ndim != 1 or len(shape) != 2:
+    raise ValueError('indices and indptr should be 1D vectors and shape a length-2 tuple.')
+  if indptr.shape[0] != shape[0] + 1:
+    raise ValueError(f'indptr should have shape[0] + 1 = {shape[0] + 1} entries, got {indptr.shape[0]}.')
+  # (uint32 arrays are looked at as int32: an entry of 2^31 or more then reads as negative and fails below)
+  ptr = indptr.view(torch.int32) if indptr.dtype == torch.uint32 else indptr
+  idx = indices.view(torch.int32) if indices.dtype == torch.uint32 else indices
+  nnz = indices.shape[0]
+  bad_ptr = (ptr[0] != 0) | (ptr[-1] != nnz) | (ptr[1:] < ptr[:-1]).any()
+  bad_idx = ((idx < 0) | (idx >= shape[1])).any() if nnz else torch.zeros((), dtype=torch.bool, device=idx.device)
+  bad_ptr, bad_idx = bool(bad_ptr), bool(bad_idx)
+  if bad_ptr:
+    raise ValueError(f'indptr should start at 0, never decrease and end at len(indices) = {nnz}.')
+  if bad_idx:
+    raise ValueError(f'indices should lie in [0, {shape[1]}).')
 
 
 def csr_to_coo(indices, indptr):

@@ -52,3 +52,28 @@ def test_no_cpu_fallback():
     bpl.event_csr_matvec(1.0, IDX, PTR, np.zeros(7, bool), shape=(4, 7))
   with pytest.raises(RuntimeError, match="no CPU path"):
     bpl.csr_matvec(1.0, IDX, PTR, np.zeros(7, np.float32), shape=(4, 7))
+
+
+def test_check_csr_accepts_a_matrix_and_names_what_is_wrong_with_the_others():
+  # the operators trust their index arrays as the reference's kernels do; this is the opt-in pass over them
+  idx = np.array([0, 6, 2, 2, 5, 1], dtype=np.int32)
+  ptr = np.array([0, 2, 2, 5, 6], dtype=np.int32)
+  bpl.check_csr(idx, ptr, shape=(4, 7))
+  bpl.check_csr(idx.astype(np.uint32), ptr.astype(np.uint32), shape=(4, 7))
+  bpl.check_csr(np.zeros(0, np.int32), np.zeros(5, np.int32), shape=(4, 7))
+  with pytest.raises(ValueError, match=r"indices should lie in \[0, 6\)"):
+    bpl.check_csr(idx, ptr, shape=(4, 6))
+  with pytest.raises(ValueError, match="indices should lie"):
+    bpl.check_csr(np.array([0, -1, 2, 2, 5, 1], dtype=np.int32), ptr, shape=(4, 7))
+  with pytest.raises(ValueError, match="indices should lie"):
+    bpl.check_csr(np.array([0, 2 ** 31 + 3, 2, 2, 5, 1], dtype=np.uint32), ptr, shape=(4, 7))
+  with pytest.raises(ValueError, match="never decrease"):
+    bpl.check_csr(idx, np.array([0, 3, 2, 5, 6], dtype=np.int32), shape=(4, 7))
+  with pytest.raises(ValueError, match="end at len"):
+    bpl.check_csr(idx, np.array([0, 2, 2, 5, 7], dtype=np.int32), shape=(4, 7))
+  with pytest.raises(ValueError, match="start at 0"):
+    bpl.check_csr(idx, np.array([1, 2, 2, 5, 6], dtype=np.int32), shape=(4, 7))
+  with pytest.raises(ValueError, match="shape\\[0\\] \\+ 1 = 4 entries"):
+    bpl.check_csr(idx, ptr, shape=(3, 7))
+  with pytest.raises(ValueError, match="int32 or uint32"):
+    bpl.check_csr(idx.astype(np.int64), ptr, shape=(4, 7))
