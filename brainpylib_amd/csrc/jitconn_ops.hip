@@ -269,12 +269,17 @@ template <typename T1, typename VT>
 __global__ __launch_bounds__(1024) void collect_active_columns_kernel(const VT *__restrict__ in, uint32_t n_in,
                                                                       uint32_t *__restrict__ counter,
                                                                       uint32_t *__restrict__ list_col,
-                                                                      T1 *__restrict__ list_val) {
+                                                                      T1 *__restrict__ list_val,
+                                                                      uint32_t *__restrict__ clear, uint32_t n_clear,
+                                                                      T1 *__restrict__ zero, uint32_t n_zero) {
+  // (also clears the bins' counters and the output, which the kernels behind this one add to: two launches less)
   __shared__ uint32_t s_col[kCollectCols];
   __shared__ T1 s_val[kCollectCols];
   __shared__ uint32_t s_count, s_base;
   const uint32_t tid = threadIdx.x, lane = tid % kWave;
   if (tid == 0) s_count = 0;
+  for (uint32_t i = blockIdx.x * 1024u + tid; i < n_clear; i += gridDim.x * 1024u) clear[i] = 0u;
+  for (uint32_t i = blockIdx.x * 1024u + tid; i < n_zero; i += gridDim.x * 1024u) zero[i] = T1(0);
   __syncthreads();
   const uint32_t c0 = blockIdx.x * kCollectCols;
   for (uint32_t t = 0; t < kCollectCols; t += 1024) {
@@ -567,8 +572,11 @@ void launch_rowwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
 template <typename T1, typename VT, int IN, int W>
 void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, uint32_t n_in, uint32_t seed,
                     double log_p, T1 wa, T1 wb) {
-  fill_zero(stream, out, n_out);
-  if (n_in == 0 || n_out == 0) return;
+  if (n_in == 0 || n_out == 0) {
+    fill_zero(stream, out, n_out);
+    return;
+  }
+  bool out_cleared = false;  // (with event input and bins, the kernel that lists the active columns clears it)
   // Many pairs: bins (also for a narrow output: seeding ahead and the even spread of the streams pay).  The number of pairs is n_in * n_out * p for a
   // dense input; for events it depends on the activity, which the host does not know: bins are sized
   // for one column in eight being active (fuller bins overflow into direct atomics) and used when
@@ -613,12 +621,12 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
         uint32_t *states = reinterpret_cast<uint32_t *>(ws + pair_bytes + count_bytes);
         uint32_t *list_col = list_bytes ? reinterpret_cast<uint32_t *>(ws + pair_bytes + count_bytes + state_bytes) : nullptr;
         T1 *list_val = val_bytes ? reinterpret_cast<T1 *>(ws + pair_bytes + count_bytes + state_bytes + list_bytes) : nullptr;
-        fill_zero(stream, counts, n_win * producers);
         auto walk = jitconn_colwalk_bins_kernel<T1, VT, IN, W>;
+        out_cleared = true;
         if (IN == kInEvent) {
           // the active columns, their generators seeded ahead (those beyond kSeedChunk seed themselves), one walk
           hipLaunchKernelGGL((collect_active_columns_kernel<T1, VT>), dim3(div_up(n_in, kCollectCols)), dim3(1024), 0, stream,
-                             in, n_in, list_count, list_col, list_val);
+                             in, n_in, list_count, list_col, list_val, counts, n_win * producers, out, n_out);
           hipLaunchKernelGGL(mt_seed_streams_kernel, dim3(div_up(seeded_max, kSeedThreads)), dim3(kSeedThreads), 0,
                              stream, seed, 0u, seeded_max, states, static_cast<const uint32_t *>(list_col),
                              static_cast<const uint32_t *>(list_count));
@@ -628,6 +636,8 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
                              n_win, shift, cap, pairs, counts);
         } else {
           // every column, a chunk of seeded generators at a time; the bins are emptied after every `group` chunks
+          fill_zero(stream, out, n_out);
+          fill_zero(stream, counts, n_win * producers);
           uint32_t in_bins = 0;
           for (uint32_t first = 0; first < n_in; first += kSeedChunk) {
             const uint32_t count = (n_in - first < kSeedChunk) ? n_in - first : kSeedChunk;
@@ -649,13 +659,14 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
           return;
         // (the bins could not be added: nothing reached `out` yet except overflow pairs; start over)
         if (list_count != nullptr) fill_zero(stream, list_count, 1u);
-        fill_zero(stream, out, n_out);
+        out_cleared = false;
       } else {
         if (scratch_refused_by_capture()) return;
         bpl_clear_error();
       }
     }
   }
+  if (!out_cleared) fill_zero(stream, out, n_out);
   hipLaunchKernelGGL((jitconn_colwalk_kernel<T1, VT, IN, W>), dim3(div_up(n_in, kColThreads)), dim3(kColThreads), 0,
                      stream, in, out, n_out, n_in, seed, log_p, wa, wb);
 }

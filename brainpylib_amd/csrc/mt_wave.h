@@ -61,6 +61,10 @@ __device__ __forceinline__ void mt_seed_batch(uint32_t *tile, int lane, uint32_t
   uint32_t x = lane_seed;
   const uint32_t sub = static_cast<uint32_t>(lane) >> 2, pair = static_cast<uint32_t>(lane) & 3u;  // stream within 16, word pair
   uint2 *out = reinterpret_cast<uint2 *>(dst + static_cast<size_t>(sub) * kMtN) + pair;
+  // The words of a tile are read back from LDS at the end of a round and stored at the start of the next
+  // one, behind its eight steps of the recurrence, so that the chain of multiplications does not wait for
+  // the LDS (a wave's LDS operations complete in order: the next round's writes cannot overtake the reads).
+  uint2 v[4];
 #pragma unroll 1
   for (uint32_t w0 = 0; w0 < kMtN; w0 += 8) {
 #pragma unroll
@@ -69,16 +73,22 @@ __device__ __forceinline__ void mt_seed_batch(uint32_t *tile, int lane, uint32_t
       x = 1812433253u * (x ^ (x >> 30)) + (w0 + i + 1);
     }
     __builtin_amdgcn_wave_barrier();
+    if (w0 != 0) {
 #pragma unroll
-    for (uint32_t q = 0; q < 4; ++q) {  // streams 16 q + sub: words w0 + 2 pair, + 1
+      for (uint32_t q = 0; q < 4; ++q)  // streams 16 q + sub: words w0 - 8 + 2 pair, + 1
+        if (16u * q + sub < n_streams) out[(static_cast<size_t>(16u * q) * kMtN + (w0 - 8u)) / 2u] = v[q];
+    }
+#pragma unroll
+    for (uint32_t q = 0; q < 4; ++q) {
       const uint32_t s = 16u * q + sub;
-      uint2 v;
-      v.x = tile[(2u * pair) * (kWave + 1) + s];
-      v.y = tile[(2u * pair + 1u) * (kWave + 1) + s];
-      if (s < n_streams) out[(static_cast<size_t>(16u * q) * kMtN + w0) / 2u] = v;
+      v[q].x = tile[(2u * pair) * (kWave + 1) + s];
+      v[q].y = tile[(2u * pair + 1u) * (kWave + 1) + s];
     }
     __builtin_amdgcn_wave_barrier();
   }
+#pragma unroll
+  for (uint32_t q = 0; q < 4; ++q)
+    if (16u * q + sub < n_streams) out[(static_cast<size_t>(16u * q) * kMtN + (kMtN - 8u)) / 2u] = v[q];
 }
 
 // gfx950 evaluates any function of three words bit by bit in one instruction; 0x6c is (a & c) ^ b,
