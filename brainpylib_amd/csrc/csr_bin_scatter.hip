@@ -203,59 +203,94 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
   __syncthreads();
   const uint32_t p_lo = static_cast<uint32_t>(static_cast<uint64_t>(s) * producers / parts);
   const uint32_t p_hi = static_cast<uint32_t>(static_cast<uint64_t>(s + 1) * producers / parts);
-  // One producer's bin per wave at a time, 8 pairs per lane in flight.  Where the bins are and how
-  // many pairs they hold is fetched for 64 bins at once (one per lane), so that the walk over the
-  // bins waits for pairs only.
-  for (uint32_t g0 = p_lo + wave; g0 < p_hi; g0 += kWaves * kWave) {
-    uint64_t my_off = 0;
-    uint32_t my_n = 0;
-    {
-      const uint64_t p64 = static_cast<uint64_t>(g0) + static_cast<uint64_t>(lane) * kWaves;
-      if (p64 < p_hi) {
-        const uint32_t p = static_cast<uint32_t>(p64);
-        if (indptr != nullptr) {
-          uint32_t r0, r1;
-          producer_rows(p, rows_per, n_row, &r0, &r1);
-          const uint32_t a0 = indptr[r0], a1 = indptr[r1];
-          my_off = region_base(a0, p, n_win) + static_cast<uint64_t>(b) * region_cap(a0, a1, n_win);
-        } else {
-          my_off = (static_cast<uint64_t>(p) * n_win + b) * uniform_cap;
-        }
-        my_n = counts[static_cast<size_t>(b) * producers + p];
-        if (indptr == nullptr && my_n > uniform_cap) my_n = uniform_cap;  // the producer counts what it could not store too
-        if (my_off >= n_pairs) my_n = 0;  // (only if the caller's nonzero count was too small)
-        else if (my_n > n_pairs - my_off) my_n = static_cast<uint32_t>(n_pairs - my_off);
+  // A wave takes the bins of the producers p_lo + wave, + kWaves, ... one after the other, in steps of
+  // 8 pairs per lane; where the bins are and how many pairs they hold is fetched for 64 bins at once
+  // (one per lane).  The steps of consecutive bins form ONE sequence, and a step's pairs are requested
+  // before the step before it is added: two steps (16 pairs per lane) are in flight, and a wave that
+  // walks many small bins (a jitconn column walk leaves a few hundred pairs in each) does not pay a
+  // round trip per bin.
+  constexpr int kAddU = 8;
+  uint32_t g0 = p_lo + wave;  // producer of lane 0's bin in the current block of 64 bins
+  uint32_t j = kWave;         // bin of the block the sequence is in (kWave: fetch a block first)
+  bool first_block = true;
+  uint64_t my_off = 0;
+  uint32_t my_n = 0;
+  const BinPair<F> *bin = nullptr;
+  uint32_t n = 0, i0 = 0, i_next = 0;
+  auto next_step = [&]() -> bool {  // moves (bin, n, i0) on; false at the end of the wave's share (wave uniform)
+    for (;;) {
+      if (i_next < n) {
+        i0 = i_next;
+        i_next += kAddU * kWave;
+        return true;
       }
-    }
-    for (uint32_t j = 0; j < kWave && static_cast<uint64_t>(g0) + static_cast<uint64_t>(j) * kWaves < p_hi; ++j) {
-      const uint32_t n = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(my_n), j));
-      if (n == 0) continue;
+      ++j;
+      if (j >= static_cast<uint32_t>(kWave) || static_cast<uint64_t>(g0) + static_cast<uint64_t>(j) * kWaves >= p_hi) {
+        if (!first_block) {
+          if (static_cast<uint64_t>(g0) + static_cast<uint64_t>(kWaves) * kWave >= p_hi) return false;
+          g0 += kWaves * kWave;
+        } else if (g0 >= p_hi) {
+          return false;
+        }
+        first_block = false;
+        my_off = 0;
+        my_n = 0;
+        const uint64_t p64 = static_cast<uint64_t>(g0) + static_cast<uint64_t>(lane) * kWaves;
+        if (p64 < p_hi) {
+          const uint32_t p = static_cast<uint32_t>(p64);
+          if (indptr != nullptr) {
+            uint32_t r0, r1;
+            producer_rows(p, rows_per, n_row, &r0, &r1);
+            const uint32_t a0 = indptr[r0], a1 = indptr[r1];
+            my_off = region_base(a0, p, n_win) + static_cast<uint64_t>(b) * region_cap(a0, a1, n_win);
+          } else {
+            my_off = (static_cast<uint64_t>(p) * n_win + b) * uniform_cap;
+          }
+          my_n = counts[static_cast<size_t>(b) * producers + p];
+          if (indptr == nullptr && my_n > uniform_cap) my_n = uniform_cap;  // the producer counts what it could not store too
+          if (my_off >= n_pairs) my_n = 0;  // (only if the caller's nonzero count was too small)
+          else if (my_n > n_pairs - my_off) my_n = static_cast<uint32_t>(n_pairs - my_off);
+        }
+        j = 0;
+      }
+      n = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(my_n), j));
       const uint32_t off_lo = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(my_off), j));
       const uint32_t off_hi = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(my_off >> 32), j));
-      const BinPair<F> *bin = pairs + ((static_cast<uint64_t>(off_hi) << 32) | off_lo);
-      constexpr int U = 8;
-      uint32_t i0 = 0;
-      for (; i0 + U * kWave <= n; i0 += U * kWave) {  // full steps: plain loads, all in flight
-        BinPair<F> e[U];
+      bin = pairs + ((static_cast<uint64_t>(off_hi) << 32) | off_lo);
+      i_next = 0;
+    }
+  };
+  auto load_step = [&](BinPair<F> (&e)[kAddU]) {
+    if (i0 + kAddU * kWave <= n) {  // a full step: plain loads
 #pragma unroll
-        for (int u = 0; u < U; ++u) e[u] = bin[i0 + u * kWave + lane];
+      for (int u = 0; u < kAddU; ++u) e[u] = bin[i0 + u * kWave + lane];
+    } else {
 #pragma unroll
-        for (int u = 0; u < U; ++u)
-          if (e[u].rel - r0 < width) atomicAdd(&window[e[u].rel - r0], static_cast<double>(e[u].val));  // (wraps below r0)
+      for (int u = 0; u < kAddU; ++u) {
+        const uint32_t i = i0 + u * kWave + lane;
+        e[u].rel = 0xffffffffu;
+        e[u].val = F(0);
+        if (i < n) e[u] = bin[i];
       }
-      if (i0 < n) {
-        BinPair<F> e[U];
+    }
+  };
+  auto add_step = [&](const BinPair<F> (&e)[kAddU]) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const uint32_t i = i0 + u * kWave + lane;
-          e[u].rel = 0xffffffffu;
-          e[u].val = F(0);
-          if (i < n) e[u] = bin[i];
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-          if (e[u].rel - r0 < width) atomicAdd(&window[e[u].rel - r0], static_cast<double>(e[u].val));  // (wraps below r0)
-      }
+    for (int u = 0; u < kAddU; ++u)
+      if (e[u].rel - r0 < width) atomicAdd(&window[e[u].rel - r0], static_cast<double>(e[u].val));  // (wraps below r0)
+  };
+  {
+    BinPair<F> ea[kAddU], eb[kAddU];
+    bool more = next_step();
+    if (more) load_step(ea);
+    while (more) {
+      more = next_step();
+      if (more) load_step(eb);
+      add_step(ea);
+      if (!more) break;
+      more = next_step();
+      if (more) load_step(ea);
+      add_step(eb);
     }
   }
   __syncthreads();
