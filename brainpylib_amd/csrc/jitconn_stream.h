@@ -63,8 +63,10 @@ struct PolarF32 {
 };
 __device__ __forceinline__ PolarF32 polar_attempt(uint32_t w0, uint32_t w1) {
   PolarF32 a;
-  a.x = __fsub_rn(__fmul_rn(2.0f, canonical_f32(w0)), 1.0f);
-  a.y = __fsub_rn(__fmul_rn(2.0f, canonical_f32(w1)), 1.0f);
+  // 2 * canonical - 1: the scalings by powers of two are exact, so one fused multiply-add rounds where
+  // the subtraction of the CPU code rounds
+  a.x = fmaf(canonical_f32_scaled(w0), 0x1p-31f, -1.0f);
+  a.y = fmaf(canonical_f32_scaled(w1), 0x1p-31f, -1.0f);
   a.r2 = __fadd_rn(__fmul_rn(a.x, a.x), __fmul_rn(a.y, a.y));
   a.ok = !(a.r2 > 1.0f || a.r2 == 0.0f);
   return a;

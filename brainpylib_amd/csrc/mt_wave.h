@@ -162,11 +162,14 @@ __device__ __forceinline__ double canonical_f64(uint32_t lo, uint32_t hi) {
   return r >= 1.0 ? 0x1.fffffffffffffp-1 : r;  // nextafter(1, 0)
 }
 
-// libstdc++ generate_canonical<float,24>(mt19937): one word rounded to float, scaled by 2^-32.
-__device__ __forceinline__ float canonical_f32(uint32_t word) {
-  const float r = static_cast<float>(word) * 0x1p-32f;
-  return r >= 1.0f ? 0x1.fffffep-1f : r;  // nextafterf(1, 0)
+// libstdc++ generate_canonical<float,24>(mt19937): one word rounded to float, scaled by 2^-32, and a
+// result of 1 replaced by nextafterf(1, 0).  The word rounds up to 2^32 from 0xffffff80 on, and every
+// word from 0xffffff00 to 0xffffff7f rounds to 0xffffff00 = nextafterf(1, 0) * 2^32: capping the WORD
+// at 0xffffff7f gives the same floats with one integer minimum instead of a compare and a select.
+__device__ __forceinline__ float canonical_f32_scaled(uint32_t word) {  // canonical * 2^32
+  return static_cast<float>(min(word, 0xffffff7fu));
 }
+__device__ __forceinline__ float canonical_f32(uint32_t word) { return canonical_f32_scaled(word) * 0x1p-32f; }
 
 // (unsigned int) of a double as x86-64 compiles it: truncate to int64, keep the low 32 bits;
 // out of range and NaN give 0.
