@@ -25,7 +25,7 @@
 #include <type_traits>
 
 #include "common.h"
-#include "csr_quad_gather.h"
+#include "csr_flat_gather.h"
 #include "repeated_sum.h"
 #include "targets.h"
 
@@ -1388,17 +1388,22 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
       bpl_clear_error();
     }
     if constexpr (std::is_same<F, VT>::value) {
-      // A longer vector is gathered from L2.  Rows of 24 nonzeros or more on average: the walk that reads the
-      // index and weight streams 16 bytes per lane (csr_quad_gather.hip); shorter ones: the walks below.
-      // The mean is known on the device only, so both kernels are enqueued and one of them returns at once.
-      constexpr uint32_t kQuadMinMean = 24;
+      // A longer vector is gathered from L2.  Rows of 24 nonzeros or more on average: the flat walk over the
+      // nonzeros with 16-byte loads of the index and weight streams (csr_flat_gather.hip); shorter ones: the
+      // walks below.  The mean is known on the device only, so both are enqueued and one returns at once.
+      constexpr uint32_t kFlatMinMean = 24;
       if (n_row >= 16384 && n_col > 0) {
-        if (csr_quad_gather<F>(target, stream, data, HETER, indices, indptr, x, y, n_row, kQuadMinMean)) {
+        const FlatGather flat =
+          csr_flat_gather<F>(target, stream, data, HETER, indices, indptr, x, y, n_row, kFlatMinMean, 0xffffffffu);
+        if (flat == FlatGather::kEnqueued) {
           launch_gather_impl<F, VT, HETER, MODE, 0>(target, stream, data, indices, indptr, x, y, n_row, n_col, 0,
-                                                    kQuadMinMean);
+                                                    kFlatMinMean);
           return;
         }
-        bpl_clear_error();
+        if (flat == FlatGather::kFailed) {
+          if (scratch_refused_by_capture()) return;  // (the error stands: a graph must not record a slower path)
+          bpl_clear_error();
+        }
       }
     }
   }

@@ -738,3 +738,59 @@ def test_gather_hub_rows(cuda, oracle_mod):
   per_call_us = e0.elapsed_time(e1) * 1e3 / 5
   print("event gather with a hub row of 1e6 nonzeros: %.1f us per call" % per_call_us, flush=True)
   assert per_call_us < 3000.0
+
+
+def _flat_walk_counts(kind, n_row, rng):
+  """Row lengths that exercise the flat walk of csr_matvec (mean of 24 or more, 16,384 rows or more)."""
+  if kind == "poisson":
+    return np.maximum(1, rng.poisson(100, n_row))
+  if kind == "even":
+    return np.full(n_row, 64)
+  if kind == "ragged":  # two thirds of the rows empty, the others long: steps that meet several hundred rows
+    c = np.zeros(n_row, dtype=np.int64)
+    some = rng.random(n_row) < 0.33
+    c[some] = rng.integers(1, 400, size=int(some.sum()))
+    return c
+  if kind == "empty ends":  # empty rows at both ends and in runs of more than a window of 64
+    c = np.maximum(1, rng.poisson(60, n_row))
+    c[:300] = 0
+    c[-500:] = 0
+    c[5000:5200] = 0
+    return c
+  if kind == "hubs":  # rows across many waves' ranges, next to rows of one nonzero
+    c = np.full(n_row, 30)
+    c[7] = 150_000
+    c[8] = 1
+    c[n_row // 2] = 70_000
+    c[n_row - 1] = 40_000
+    return c
+  if kind == "steps":  # rows of exactly one step and of one quad, so that rows end where steps and ranges end
+    c = np.full(n_row, 4)
+    c[::3] = 1024
+    return c
+  raise ValueError(kind)
+
+
+@pytest.mark.parametrize("kind", ["poisson", "even", "ragged", "empty ends", "hubs", "steps"])
+def test_csr_matvec_flat_walk_over_the_nonzeros(cuda, oracle_mod, kind):
+  # vectors too long for LDS (more than 162,816 elements) and rows of 24 nonzeros or more on average: every wave
+  # owns a contiguous range of the nonzeros and tells the rows apart through windows of indptr
+  # (csr_flat_gather.hip).  Integer data: every sum is exact in float64, so the result is the oracle's bit for bit.
+  rng = np.random.default_rng(len(kind))
+  n_row, n_col = 20_011, 170_003
+  counts = np.minimum(_flat_walk_counts(kind, n_row, rng), n_col)
+  indices, indptr = synth.counted_csr(counts, n_col, seed=3)
+  assert indices.shape[0] // n_row >= 24
+  for dtype in (np.float32, np.float64):
+    data = rng.integers(-3, 4, size=indices.shape[0]).astype(dtype)
+    v = rng.integers(-4, 5, size=n_col).astype(dtype)
+    for d in (data, np.array([0.75], dtype=dtype)):
+      want = oracle_mod.csr_matvec(d, indices, indptr, v, shape=(n_row, n_col))
+      got = bpl.csr_matvec(d, indices, indptr, v, shape=(n_row, n_col)).cpu().numpy()
+      assert np.array_equal(got, want), (kind, dtype.__name__, d.shape, np.flatnonzero(got != want)[:8])
+  # real-valued data: within the tolerance of the gather paths
+  data = rng.standard_normal(indices.shape[0]).astype(np.float32)
+  v = rng.standard_normal(n_col).astype(np.float32)
+  want = oracle_mod.csr_matvec(data, indices, indptr, v, shape=(n_row, n_col))
+  got = bpl.csr_matvec(data, indices, indptr, v, shape=(n_row, n_col)).cpu().numpy()
+  assert_close(got, want, what="flat walk " + kind)
