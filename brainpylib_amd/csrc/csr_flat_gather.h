@@ -7,8 +7,12 @@
 
 namespace bpl {
 
+// The flat walk computes positions of nonzeros one step beyond the end of a wave's range in 32 bits: matrices
+// with more nonzeros than this are left to the caller's other kernel, whatever their mean.
+constexpr uint32_t kFlatMaxNnz = 0xffffffffu - 8192u;
+
 // y = A x, walked flat: every wave owns a contiguous range of the nonzeros and tells the rows apart through
-// windows of indptr in LDS.  For matrices with min_mean <= nnz / n_row < max_mean; for others the kernels
+// windows of indptr in LDS.  For matrices with min_mean <= nnz / n_row < max_mean and nnz <= kFlatMaxNnz; for others the kernels
 // return at once and write nothing (the mean is known on the device only, so the caller enqueues its kernel
 // for short rows behind this one).  x must have at least one element.  Takes 20 bytes of the stream's scratch
 // memory per wave of its launch.

@@ -110,7 +110,7 @@ __global__ __launch_bounds__(kFlatThreads, 4) void csr_flat_gather_kernel(
   __shared__ double s_sum_all[kFlatWaves][kFlatRows];
   const uint32_t nnz = indptr[n_row];
   const uint32_t mean = nnz / n_row;
-  if (mean < min_mean || mean >= max_mean) return;  // (the launcher's other kernels take those matrices)
+  if (mean < min_mean || mean >= max_mean || nnz > kFlatMaxNnz) return;  // (the launcher's other kernel takes those matrices)
   const uint32_t lane = static_cast<uint32_t>(lane_id()), wv = threadIdx.x / kWave;
   uint32_t *s_ptr = s_ptr_all[wv];
   double *s_sum = s_sum_all[wv];
@@ -291,7 +291,7 @@ __global__ __launch_bounds__(kWave) void csr_flat_finish_kernel(const uint32_t *
   constexpr uint32_t kStepQuads = FlatQuads<F>::value * kWave;
   const uint32_t nnz = indptr[n_row];
   const uint32_t mean = nnz / n_row;
-  if (mean < min_mean || mean >= max_mean) return;
+  if (mean < min_mean || mean >= max_mean || nnz > kFlatMaxNnz) return;
   const uint32_t w = blockIdx.x, lane = threadIdx.x;
   const uint32_t row = tail_row[w];
   if (row == kNoRow) return;

@@ -948,7 +948,7 @@ __global__ __launch_bounds__(1024, (MODE == kEvent && BITS == 1) ? 8 : 4) void c
   uint32_t gpb = 0, hub_len = 0;  // rows per workgroup and round of the walk chosen below, its longest row
   if constexpr (MODE == kDense && BITS == 0) {
     // (rows of `skip_mean` nonzeros or more on average: the launcher's other kernel has taken this matrix)
-    if (skip_mean != 0 && mean >= skip_mean) return;
+    if (skip_mean != 0 && mean >= skip_mean && nnz <= kFlatMaxNnz) return;
   }
   if constexpr (MODE == kDense && BITS == 1) {
     // (nothing left to hide but the index and weight streams: the walks of the event gather)
