@@ -196,11 +196,7 @@ __global__ __launch_bounds__(kFlatThreads, 4) void csr_flat_gather_kernel(
       // quads that lie in one row or in two; a loop only for quads that meet three rows or more.
       uint32_t kq[U], e1[U], e2[U];
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const uint32_t p0 = 4u * (s0 / 4u + static_cast<uint32_t>(u) * kWave + lane);
-        const uint32_t pe = p0 > lo ? p0 : lo;
-        kq[u] = 0;  // the last k < 64 with s_ptr[k] <= pe (s_ptr[0] = lo <= pe)
-      }
+      for (int u = 0; u < U; ++u) kq[u] = 0;  // the last k < 64 with s_ptr[k] <= max(p0, lo) (s_ptr[0] = lo)
 #pragma unroll
       for (uint32_t step = kFlatRows / 2; step != 0; step >>= 1) {
 #pragma unroll
