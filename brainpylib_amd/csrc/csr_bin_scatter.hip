@@ -27,16 +27,42 @@ constexpr int kBinThreads = 1024;
 constexpr uint32_t kTileRows = 1024;      // rows staged in LDS at a time by a producer
 constexpr uint32_t kMaxWindows = kBinMaxWindows;
 constexpr uint32_t kRegionSlack = 128;    // pairs a region holds beyond 5/4 of its even share
+constexpr uint32_t kRegionSpacing = kRegionSlack + 8;  // (regions begin and end at multiples of 4 pairs)
 
-// Where producer `p`, whose rows hold nonzeros [a0, a1), keeps the pairs of window b:
-// region_base + b * cap.  Both kernels evaluate the same expressions.
+// Where producer `p`, whose rows hold nonzeros [a0, a1) counted from the first row of the launch, keeps
+// the pairs of window b: region_base + b * cap, both multiples of 4 pairs (16-byte loads of the products).
+// Both kernels evaluate the same expressions.
 __device__ __forceinline__ uint32_t region_cap(uint32_t a0, uint32_t a1, uint32_t n_win) {
   const uint32_t share = (a1 - a0) / n_win;
-  return share + share / 4u + kRegionSlack;
+  return (share + share / 4u + kRegionSlack + 3u) & ~3u;
 }
 __device__ __forceinline__ uint64_t region_base(uint32_t a0, uint32_t p, uint32_t n_win) {
-  return static_cast<uint64_t>(a0) + a0 / 4u + static_cast<uint64_t>(p) * n_win * kRegionSlack;
+  return ((static_cast<uint64_t>(a0) + a0 / 4u) & ~3ull) + static_cast<uint64_t>(p) * n_win * kRegionSpacing;
 }
+
+// A bin's pairs in memory.  Unpacked: an array of BinPair<F>.  PACKED (windows of at most 2^16 outputs): the
+// products in one array of F and the positions within the window in an array of 16-bit words behind it,
+// 6 bytes a pair instead of 8 (float) or 10 instead of 16 (double): the pairs are written once and read
+// once, which is two thirds of the memory traffic of the transposed product.
+typedef float bin_f32x4 __attribute__((ext_vector_type(4)));
+typedef double bin_f64x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void load_quad(const float *p, float (&v)[4]) {  // (p: 16-byte aligned)
+  const bin_f32x4 t = *reinterpret_cast<const bin_f32x4 *>(p);
+  v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+}
+__device__ __forceinline__ void load_quad(const double *p, double (&v)[4]) {
+  const bin_f64x2 a = *reinterpret_cast<const bin_f64x2 *>(p), b = *reinterpret_cast<const bin_f64x2 *>(p + 2);
+  v[0] = a.x, v[1] = a.y, v[2] = b.x, v[3] = b.y;
+}
+template <typename F>
+struct PackedBins {
+  F *val;
+  uint16_t *rel;
+  __device__ __forceinline__ PackedBins(void *pairs, uint64_t n_pairs)
+      : val(static_cast<F *>(pairs)), rel(reinterpret_cast<uint16_t *>(static_cast<F *>(pairs) + n_pairs)) {}
+};
+template <typename F>
+constexpr size_t bin_pair_bytes(bool packed) { return packed ? sizeof(F) + 2 : sizeof(BinPair<F>); }
 __device__ __forceinline__ void producer_rows(uint32_t p, uint32_t rows_per, uint32_t n_row, uint32_t *r0,
                                               uint32_t *r1) {
   const uint64_t lo = static_cast<uint64_t>(p) * rows_per, hi = lo + rows_per;
@@ -44,14 +70,18 @@ __device__ __forceinline__ void producer_rows(uint32_t p, uint32_t rows_per, uin
   *r1 = hi < n_row ? static_cast<uint32_t>(hi) : n_row;
 }
 
+constexpr uint32_t kWindowIdShift = 24;  // (positions within a window take kBinMaxShift = 17 bits, window numbers 7)
+static_assert(kBinMaxShift <= kWindowIdShift && kBinMaxWindows <= (1u << (32 - kWindowIdShift)), "window id above the position");
 constexpr uint32_t kHintShift = 8;                       // one row hint per 256 nonzeros
 constexpr uint32_t kSegment = kBinThreads << kHintShift;  // nonzeros covered by one set of hints
 
-template <typename F, bool HETER>
+template <typename F, bool HETER, bool PACKED>
 __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
     const F *__restrict__ vec, F *__restrict__ y, uint32_t n_row, uint32_t rows_per, uint32_t n_win, uint32_t shift,
-    BinPair<F> *__restrict__ pairs, uint64_t n_pairs, uint32_t *__restrict__ counts) {
+    void *__restrict__ pairs_raw, uint64_t n_pairs, uint32_t *__restrict__ counts) {
+  BinPair<F> *__restrict__ pairs = static_cast<BinPair<F> *>(pairs_raw);
+  const PackedBins<F> packed(pairs_raw, n_pairs);
   __shared__ uint32_t s_ptr[kTileRows + 1];
   __shared__ F s_v[kTileRows];
   __shared__ uint32_t s_hint[kBinThreads + 1];  // row (within the tile) of every 256th nonzero of the segment
@@ -60,8 +90,8 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
   __shared__ uint32_t s_total[kMaxWindows];     // pairs already in this producer's bin, per window
   constexpr int U = (sizeof(F) == 4) ? 4 : 2;
   constexpr uint32_t kRound = U * kBinThreads;
-  __shared__ BinPair<F> s_sorted[kRound];
-  __shared__ uint8_t s_window[kRound];
+  __shared__ uint32_t s_base[kMaxWindows];
+  __shared__ BinPair<F> s_sorted[kRound];  // (rel: the window's number above the position, from bit kWindowIdShift)
   const uint32_t tid = threadIdx.x;
   const uint32_t p = blockIdx.x;
   uint32_t r0, r1;
@@ -69,7 +99,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
   if (tid < kMaxWindows) s_cnt[tid] = 0, s_total[tid] = 0;
   const uint32_t a0 = indptr[r0], a1 = indptr[r1];
   const uint32_t cap = region_cap(a0, a1, n_win);
-  const uint64_t region_off = region_base(a0, p, n_win);
+  const uint64_t region_off = region_base(a0 - indptr[0], p, n_win);
   const F w_homo = HETER ? F(0) : data[0];
 
   // largest k < rows with s_ptr[k] <= j, searched in [lo, hi]
@@ -92,6 +122,21 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
     const uint32_t j0 = s_ptr[0], j1 = s_ptr[rows];
     for (uint32_t seg = j0; seg < j1; seg += kSegment) {
       const uint32_t seg_end = (j1 - seg < kSegment) ? j1 : seg + kSegment;
+      // The columns and weights of a round are requested a round ahead, all of a lane's loads at once and
+      // without a branch around them (beyond the segment: its last nonzero again), before the stores of
+      // the round before: a wave that asks for them where it needs them waits for memory twice a round.
+      uint32_t col[U];
+      F dat[U];
+      auto load_round = [&](uint32_t jb) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t j = jb + u * kBinThreads;
+          const uint32_t jc = j < seg_end ? j : seg_end - 1u;
+          col[u] = indices[jc];
+          dat[u] = HETER ? data[jc] : F(0);
+        }
+      };
+      load_round(seg + tid);
       // hints: the row of nonzero seg + 256 q, for every q up to the end of the segment
       __syncthreads();  // the previous segment is done with s_hint
       {
@@ -107,22 +152,22 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
       for (uint32_t jb = seg + tid; jb - tid < seg_end; jb += kRound) {
         uint32_t rank[U], win[U], rel[U];
         F val[U];
+        uint32_t k[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {  // (LDS only: the round's columns and weights are on their way)
+          const uint32_t j = jb + u * kBinThreads;
+          const uint32_t jc = j < seg_end ? j : seg_end - 1u;
+          const uint32_t q = (jc - seg) >> kHintShift;
+          k[u] = row_of(jc, s_hint[q], s_hint[q + 1]);
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const uint32_t j = jb + u * kBinThreads;
-          win[u] = 0xffffffffu;  // no pair
-          rel[u] = 0;
-          val[u] = F(0);
+          // v * values[j] (heter) or values * v (homo), as the reference's CPU loop multiplies
+          val[u] = HETER ? static_cast<F>(s_v[k[u]] * dat[u]) : static_cast<F>(w_homo * s_v[k[u]]);
+          win[u] = j < seg_end ? col[u] >> shift : 0xffffffffu;  // (0xffffffff: no pair)
+          rel[u] = col[u] & ((1u << shift) - 1u);
           rank[u] = 0;
-          if (j < seg_end) {
-            const uint32_t q = (j - seg) >> kHintShift;
-            const uint32_t k = row_of(j, s_hint[q], s_hint[q + 1]);
-            const uint32_t col = indices[j];
-            // v * values[j] (heter) or values * v (homo), as the reference's CPU loop multiplies
-            val[u] = HETER ? static_cast<F>(s_v[k] * data[j]) : static_cast<F>(w_homo * s_v[k]);
-            win[u] = col >> shift;
-            rel[u] = col & ((1u << shift) - 1u);
-          }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
@@ -131,9 +176,18 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
         if (tid < kWave) {  // offsets of the windows within the round: two counters per lane
           const uint32_t c0 = s_cnt[2 * tid], c1 = s_cnt[2 * tid + 1];
           const uint32_t incl = wave_inclusive_scan_u32(c0 + c1);
-          s_off[2 * tid] = incl - (c0 + c1);
-          s_off[2 * tid + 1] = incl - c1;
+          const uint32_t o0 = incl - (c0 + c1), o1 = incl - c1;
+          s_off[2 * tid] = o0;
+          s_off[2 * tid + 1] = o1;
           if (tid == kWave - 1) s_off[kMaxWindows] = incl;
+          // slot in the bin of the pair at position i of the sorted round: s_base[window] + i (modulo 2^32)
+          const uint32_t t0w = s_total[2 * tid], t1w = s_total[2 * tid + 1];
+          s_base[2 * tid] = t0w - o0;
+          s_base[2 * tid + 1] = t1w - o1;
+          s_total[2 * tid] = t0w + c0;
+          s_total[2 * tid + 1] = t1w + c1;
+          s_cnt[2 * tid] = 0;
+          s_cnt[2 * tid + 1] = 0;
         }
         __syncthreads();
 #pragma unroll
@@ -141,28 +195,29 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
           if (win[u] != 0xffffffffu) {
             const uint32_t pos = s_off[win[u]] + rank[u];
             BinPair<F> e;
-            e.rel = rel[u];
+            e.rel = rel[u] | (win[u] << kWindowIdShift);
             e.val = val[u];
             s_sorted[pos] = e;
-            s_window[pos] = static_cast<uint8_t>(win[u]);
           }
         }
         __syncthreads();
+        // (No barrier behind the stores: the next round's loads and counting follow at once; what the stores
+        // read is written again only behind the next round's barriers.)
+        if (jb - tid + kRound < seg_end) load_round(jb + kRound);
         const uint32_t round_total = s_off[kMaxWindows];
         for (uint32_t i = tid; i < round_total; i += kBinThreads) {
-          const uint32_t w = s_window[i];
-          const BinPair<F> e = s_sorted[i];
-          const uint32_t slot = s_total[w] + (i - s_off[w]);
+          BinPair<F> e = s_sorted[i];
+          const uint32_t w = e.rel >> kWindowIdShift;
+          e.rel &= (1u << kWindowIdShift) - 1u;
+          const uint32_t slot = s_base[w] + i;
           const uint64_t at = region_off + static_cast<uint64_t>(w) * cap + slot;
-          if (slot < cap && at < n_pairs) pairs[at] = e;
-          else atomic_add(y + ((w << shift) | e.rel), e.val);
+          if (slot < cap && at < n_pairs) {
+            if (PACKED) packed.val[at] = e.val, packed.rel[at] = static_cast<uint16_t>(e.rel);
+            else pairs[at] = e;
+          } else {
+            atomic_add(y + ((w << shift) | e.rel), e.val);
+          }
         }
-        __syncthreads();
-        if (tid < kMaxWindows) {
-          s_total[tid] += s_cnt[tid];
-          s_cnt[tid] = 0;
-        }
-        __syncthreads();
       }
     }
   }
@@ -177,16 +232,18 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
 // wider than the 2^lds_shift accumulators in LDS is added slice by slice, every slice reading the pairs).
 // Bin of (producer p, window b): derived from indptr as in bin_products_kernel, or, with
 // indptr == nullptr, the uniform layout pairs + (p * n_win + b) * uniform_cap.
-template <typename F>
+template <typename F, bool PACKED>
 __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *__restrict__ indptr,
                                                                F *__restrict__ y, uint32_t n_row, uint32_t n_col,
                                                                uint32_t rows_per, uint32_t n_win, uint32_t shift,
                                                                uint32_t lds_shift, uint32_t parts,
                                                                uint32_t producers,
-                                                               const BinPair<F> *__restrict__ pairs,
+                                                               const void *__restrict__ pairs_raw,
                                                                uint64_t n_pairs,
                                                                const uint32_t *__restrict__ counts,
                                                                uint32_t uniform_cap, uint32_t *__restrict__ reset) {
+  const BinPair<F> *__restrict__ pairs = static_cast<const BinPair<F> *>(pairs_raw);
+  const PackedBins<F> packed(const_cast<void *>(pairs_raw), n_pairs);
   extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
   // (a counter of the producer's, left at zero for the next call)
   if (reset != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *reset = 0u;
@@ -216,6 +273,7 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
   uint64_t my_off = 0;
   uint32_t my_n = 0;
   const BinPair<F> *bin = nullptr;
+  uint64_t bin_off = 0;  // (in pairs)
   uint32_t n = 0, i0 = 0, i_next = 0;
   auto next_step = [&]() -> bool {  // moves (bin, n, i0) on; false at the end of the wave's share (wave uniform)
     for (;;) {
@@ -242,7 +300,7 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
             uint32_t r0, r1;
             producer_rows(p, rows_per, n_row, &r0, &r1);
             const uint32_t a0 = indptr[r0], a1 = indptr[r1];
-            my_off = region_base(a0, p, n_win) + static_cast<uint64_t>(b) * region_cap(a0, a1, n_win);
+            my_off = region_base(a0 - indptr[0], p, n_win) + static_cast<uint64_t>(b) * region_cap(a0, a1, n_win);
           } else {
             my_off = (static_cast<uint64_t>(p) * n_win + b) * uniform_cap;
           }
@@ -256,7 +314,8 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
       n = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(my_n), j));
       const uint32_t off_lo = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(my_off), j));
       const uint32_t off_hi = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(my_off >> 32), j));
-      bin = pairs + ((static_cast<uint64_t>(off_hi) << 32) | off_lo);
+      bin_off = (static_cast<uint64_t>(off_hi) << 32) | off_lo;
+      bin = pairs + bin_off;
       i_next = 0;
     }
   };
@@ -279,7 +338,54 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
     for (int u = 0; u < kAddU; ++u)
       if (e[u].rel - r0 < width) atomicAdd(&window[e[u].rel - r0], static_cast<double>(e[u].val));  // (wraps below r0)
   };
-  {
+  // Packed bins: a lane takes two quads of a step, each 16 or 32 bytes of products and 8 bytes of positions
+  // (bins begin at multiples of 4 pairs and their regions end at one: a bin's last quad is read whole and
+  // its elements beyond the count are left out by their number).
+  struct PackedStep {
+    F v[2][4];
+    uint32_t r[2][2];  // four 16-bit positions
+    uint32_t valid[2];
+  };
+  auto load_packed = [&](PackedStep &e) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const uint32_t i = i0 + 4u * (static_cast<uint32_t>(u) * kWave + lane);
+      e.valid[u] = i < n ? n - i : 0u;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) e.v[u][t] = F(0);
+      e.r[u][0] = e.r[u][1] = 0u;
+      if (i < n) {
+        const uint2 r = *reinterpret_cast<const uint2 *>(packed.rel + bin_off + i);
+        e.r[u][0] = r.x, e.r[u][1] = r.y;
+        load_quad(packed.val + bin_off + i, e.v[u]);
+      }
+    }
+  };
+  auto add_packed = [&](const PackedStep &e) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const uint32_t rel = (e.r[u][t / 2] >> (16 * (t % 2))) & 0xffffu;
+        if (static_cast<uint32_t>(t) < e.valid[u] && rel - r0 < width)
+          atomicAdd(&window[rel - r0], static_cast<double>(e.v[u][t]));  // (wraps below r0)
+      }
+    }
+  };
+  if (PACKED) {
+    PackedStep ea, eb;
+    bool more = next_step();
+    if (more) load_packed(ea);
+    while (more) {
+      more = next_step();
+      if (more) load_packed(eb);
+      add_packed(ea);
+      if (!more) break;
+      more = next_step();
+      if (more) load_packed(ea);
+      add_packed(eb);
+    }
+  } else {
     BinPair<F> ea[kAddU], eb[kAddU];
     bool more = next_step();
     if (more) load_step(ea);
@@ -727,6 +833,9 @@ bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint
   return true;
 }
 
+constexpr uint64_t kChunkPairBytes = 200ull << 20;
+constexpr uint32_t kMaxChunks = 6;
+
 template <typename F>
 bool bin_scatter_usable(uint32_t n_col, uint32_t nnz) {
   const uint32_t n_win = div_up(n_col, 1u << bin_window_shift(n_col));
@@ -750,39 +859,55 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
   if (parts == 0) parts = 1;
   if (parts > producers) parts = producers;
 
-  // the last region ends at or before nnz + nnz / 4 + producers * n_win * kRegionSlack
-  const size_t n_pairs = static_cast<size_t>(nnz) + nnz / 4u + static_cast<size_t>(producers) * n_win * kRegionSlack + 64u;
-  const size_t pair_bytes = (n_pairs * sizeof(BinPair<F>) + 255) / 256 * 256;
+  // the last region ends at or before nnz + nnz / 4 + producers * n_win * kRegionSpacing
+  const bool packed = shift <= 16;
+  const size_t n_pairs =
+      (static_cast<size_t>(nnz) + nnz / 4u + static_cast<size_t>(producers) * n_win * kRegionSpacing + 127u) / 64u * 64u;
+  const size_t pair_bytes = (n_pairs * bin_pair_bytes<F>(packed) + 255) / 256 * 256;
   const size_t count_bytes = static_cast<size_t>(n_win) * producers * sizeof(uint32_t);
   unsigned char *ws = static_cast<unsigned char *>(stream_workspace(stream, pair_bytes + count_bytes));
   if (ws == nullptr) {
     if (!scratch_refused_by_capture()) bpl_clear_error();  // (an allocation failed: the caller has other paths)
     return false;
   }
-  BinPair<F> *pairs = reinterpret_cast<BinPair<F> *>(ws);
+  void *pairs = ws;
   uint32_t *counts = reinterpret_cast<uint32_t *>(ws + pair_bytes);
 
-  auto add_kernel = add_bins_kernel<F>;
+  auto add_kernel = packed ? add_bins_kernel<F, true> : add_bins_kernel<F, false>;
   const size_t lds = sizeof(double) << lds_shift;
-  static thread_local bool attr_set = false;
-  if (!attr_set && lds > 64 * 1024) {
+  static thread_local bool attr_set[2] = {false, false};
+  if (!attr_set[packed] && lds > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(add_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             static_cast<int>(lds)) != hipSuccess) {
       (void)hipGetLastError();
       return false;
     }
-    attr_set = true;
+    attr_set[packed] = true;
   }
   fill_zero(stream, y, n_col);
-  if (heter)
-    hipLaunchKernelGGL((bin_products_kernel<F, true>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
-                       indptr, vec, y, n_row, rows_per, n_win, shift, pairs, static_cast<uint64_t>(n_pairs), counts);
-  else
-    hipLaunchKernelGGL((bin_products_kernel<F, false>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
-                       indptr, vec, y, n_row, rows_per, n_win, shift, pairs, static_cast<uint64_t>(n_pairs), counts);
-  hipLaunchKernelGGL(add_kernel, dim3(n_win * slices * parts), dim3(kBinThreads), lds, stream, indptr, y, n_row, n_col,
-                     rows_per, n_win, shift, lds_shift, parts, producers, pairs, static_cast<uint64_t>(n_pairs), counts, 0u,
-                     static_cast<uint32_t *>(nullptr));
+  auto bin_kernel = heter ? (packed ? bin_products_kernel<F, true, true> : bin_products_kernel<F, true, false>)
+                          : (packed ? bin_products_kernel<F, false, true> : bin_products_kernel<F, false, false>);
+  // The rows are taken in chunks whose pairs (about kChunkPairBytes) stay in the 256 MB cache in front of the
+  // memory between the kernel that writes them and the kernel that reads them: at 1e8 nonzeros three chunks
+  // take 535 us, one 590, six 630 (every chunk is a pair of launches that start and drain on their own, and
+  // one more float32 addition per output element).
+  uint32_t chunks = div_up(static_cast<uint64_t>(nnz) * bin_pair_bytes<F>(packed), kChunkPairBytes);
+  if (chunks > kMaxChunks) chunks = kMaxChunks;
+  if (chunks == 0) chunks = 1;
+  const uint32_t chunk_rows = div_up(n_row, chunks);
+  for (uint32_t rb = 0; rb < n_row; rb += chunk_rows) {
+    const uint32_t rows = n_row - rb < chunk_rows ? n_row - rb : chunk_rows;
+    uint32_t prods = 2u * num_cu;
+    if (prods > div_up(rows, 64)) prods = div_up(rows, 64);
+    const uint32_t rper = div_up(rows, prods);
+    prods = div_up(rows, rper);
+    uint32_t pts = parts > prods ? prods : parts;
+    hipLaunchKernelGGL(bin_kernel, dim3(prods), dim3(kBinThreads), 0, stream, data, indices, indptr + rb, vec + rb, y, rows,
+                       rper, n_win, shift, pairs, static_cast<uint64_t>(n_pairs), counts);
+    hipLaunchKernelGGL(add_kernel, dim3(n_win * slices * pts), dim3(kBinThreads), lds, stream, indptr + rb, y, rows, n_col,
+                       rper, n_win, shift, lds_shift, pts, prods, static_cast<const void *>(pairs),
+                       static_cast<uint64_t>(n_pairs), counts, 0u, static_cast<uint32_t *>(nullptr));
+  }
   return check_launch(target);
 }
 
@@ -792,7 +917,7 @@ template <typename F>
 bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_out, uint32_t shift, uint32_t producers,
                       uint32_t cap, const void *pairs, const uint32_t *counts, uint32_t *reset) {
   const uint32_t n_win = div_up(n_out, 1u << shift);
-  auto add_kernel = add_bins_kernel<F>;
+  auto add_kernel = add_bins_kernel<F, false>;
   const uint32_t lds_shift = bin_lds_shift(shift);
   const uint32_t slices = 1u << (shift - lds_shift);
   const size_t lds = sizeof(double) << lds_shift;
@@ -811,7 +936,7 @@ bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_o
   const uint64_t n_pairs = static_cast<uint64_t>(producers) * n_win * cap;
   hipLaunchKernelGGL(add_kernel, dim3(n_win * slices * parts), dim3(kBinThreads), lds, stream,
                      static_cast<const uint32_t *>(nullptr), y, 0u, n_out, 0u, n_win, shift, lds_shift, parts, producers,
-                     static_cast<const BinPair<F> *>(pairs), n_pairs, counts, cap, reset);
+                     pairs, n_pairs, counts, cap, reset);
   return check_launch(target);
 }
 

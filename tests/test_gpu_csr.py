@@ -432,7 +432,9 @@ def test_transposed_csr_matvec_wide_output_sorted_scatter(cuda, oracle_mod, dtyp
   for n_row, n_col, mean, long_row in ((30_000, 300_000, 50, 0), (50_000, 400_000, 25, 250_000),
                                        (1500, 2_000_000, 1000, 0), (200_000, 140_000, 8, 0),
                                        # (above 2^21 columns: windows wider than their LDS accumulators, added in slices)
-                                       (4000, 5_000_001, 300, 0)):
+                                       (4000, 5_000_001, 300, 0),
+                                       # (above 2^23 columns: positions within a window beyond 16 bits, whole pairs)
+                                       (3000, 9_000_000, 400, 0)):
     counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
     if long_row:
       counts[7] = long_row
@@ -452,6 +454,31 @@ def test_transposed_csr_matvec_wide_output_sorted_scatter(cuda, oracle_mod, dtyp
     want = oracle_mod.csr_matvec(w, indices, indptr, vi, shape=shape, transpose=True)
     got = bpl.cusparse_csr_matvec(w, indices, indptr, vi, shape=shape, transpose=True).cpu().numpy()
     assert np.array_equal(got, want)  # multiples of 0.5: exact in any order
+
+
+def test_transposed_csr_matvec_rows_taken_in_chunks(cuda, oracle_mod):
+  # float64 pairs of 10 bytes: from 21 million nonzeros on the rows are binned and added in two or more
+  # chunks, one after the other over the same scratch memory; uneven rows, so that the chunks differ
+  rng = np.random.default_rng(43)
+  n_row, n_col = 260_000, 300_000
+  counts = rng.poisson(60, size=n_row)
+  counts[n_row // 2:] *= 2
+  counts[5] = 200_000
+  indices, indptr = synth.counted_csr(counts, n_col, seed=3)
+  assert indices.shape[0] * 10 > 200 << 20
+  data = rng.random(indices.shape[0])
+  v = rng.standard_normal(n_row)
+  shape = (n_row, n_col)
+  want = oracle_mod.csr_matvec(data, indices, indptr, v, shape=shape, transpose=True)
+  mag = oracle_mod.csr_matvec(data, indices, indptr, np.abs(v), shape=shape, transpose=True)
+  for _ in range(2):
+    got = bpl.cusparse_csr_matvec(data, indices, indptr, v, shape=shape, transpose=True).cpu().numpy()
+    assert_close_reordered(got, want, mag, np.float64, what="sorted scatter in chunks %s" % (shape,))
+  vi = rng.integers(-2, 3, size=n_row).astype(np.float64)
+  w = np.array([0.5])
+  want = oracle_mod.csr_matvec(w, indices, indptr, vi, shape=shape, transpose=True)
+  got = bpl.cusparse_csr_matvec(w, indices, indptr, vi, shape=shape, transpose=True).cpu().numpy()
+  assert np.array_equal(got, want)  # multiples of 0.5: exact in any order
 
 
 def test_full_size_csr_matvec_both_orientations(cuda, oracle_mod):
