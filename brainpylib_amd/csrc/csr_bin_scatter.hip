@@ -54,6 +54,27 @@ __device__ __forceinline__ void load_quad(const double *p, double (&v)[4]) {
   const bin_f64x2 a = *reinterpret_cast<const bin_f64x2 *>(p), b = *reinterpret_cast<const bin_f64x2 *>(p + 2);
   v[0] = a.x, v[1] = a.y, v[2] = b.x, v[3] = b.y;
 }
+// U consecutive columns or weights for a lane, from an address that is a multiple of the element's size only
+typedef uint32_t bin_u32x4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t bin_u32x2_unaligned __attribute__((ext_vector_type(2), aligned(4)));
+typedef float bin_f32x4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
+typedef double bin_f64x2_unaligned __attribute__((ext_vector_type(2), aligned(8)));
+__device__ __forceinline__ void load_consecutive(const uint32_t *p, uint32_t (&c)[4]) {
+  const bin_u32x4_unaligned t = *reinterpret_cast<const bin_u32x4_unaligned *>(p);
+  c[0] = t.x, c[1] = t.y, c[2] = t.z, c[3] = t.w;
+}
+__device__ __forceinline__ void load_consecutive(const uint32_t *p, uint32_t (&c)[2]) {
+  const bin_u32x2_unaligned t = *reinterpret_cast<const bin_u32x2_unaligned *>(p);
+  c[0] = t.x, c[1] = t.y;
+}
+__device__ __forceinline__ void load_consecutive(const float *p, float (&v)[4]) {
+  const bin_f32x4_unaligned t = *reinterpret_cast<const bin_f32x4_unaligned *>(p);
+  v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+}
+__device__ __forceinline__ void load_consecutive(const double *p, double (&v)[2]) {
+  const bin_f64x2_unaligned t = *reinterpret_cast<const bin_f64x2_unaligned *>(p);
+  v[0] = t.x, v[1] = t.y;
+}
 template <typename F>
 struct PackedBins {
   F *val;
@@ -85,18 +106,19 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
   __shared__ uint32_t s_ptr[kTileRows + 1];
   __shared__ F s_v[kTileRows];
   __shared__ uint32_t s_hint[kBinThreads + 1];  // row (within the tile) of every 256th nonzero of the segment
-  __shared__ uint32_t s_cnt[kMaxWindows];       // pairs of the current round, per window
+  __shared__ uint32_t s_cnt[kMaxWindows + 1];   // pairs of the current round, per window (and a spare counter)
   __shared__ uint32_t s_off[kMaxWindows + 1];   // their offsets in the sorted round
   __shared__ uint32_t s_total[kMaxWindows];     // pairs already in this producer's bin, per window
   constexpr int U = (sizeof(F) == 4) ? 4 : 2;
   constexpr uint32_t kRound = U * kBinThreads;
   __shared__ uint32_t s_base[kMaxWindows];
-  __shared__ BinPair<F> s_sorted[kRound];  // (rel: the window's number above the position, from bit kWindowIdShift)
+  __shared__ BinPair<F> s_sorted[kRound + 1];  // (and a spare slot; rel: the window's number above the position, from bit kWindowIdShift)
   const uint32_t tid = threadIdx.x;
   const uint32_t p = blockIdx.x;
   uint32_t r0, r1;
   producer_rows(p, rows_per, n_row, &r0, &r1);
   if (tid < kMaxWindows) s_cnt[tid] = 0, s_total[tid] = 0;
+  if (tid == 0) s_cnt[kMaxWindows] = 0;
   const uint32_t a0 = indptr[r0], a1 = indptr[r1];
   const uint32_t cap = region_cap(a0, a1, n_win);
   const uint64_t region_off = region_base(a0 - indptr[0], p, n_win);
@@ -122,21 +144,28 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
     const uint32_t j0 = s_ptr[0], j1 = s_ptr[rows];
     for (uint32_t seg = j0; seg < j1; seg += kSegment) {
       const uint32_t seg_end = (j1 - seg < kSegment) ? j1 : seg + kSegment;
-      // The columns and weights of a round are requested a round ahead, all of a lane's loads at once and
-      // without a branch around them (beyond the segment: its last nonzero again), before the stores of
-      // the round before: a wave that asks for them where it needs them waits for memory twice a round.
+      // A lane takes U consecutive nonzeros of a round: one request for their columns and one for their
+      // weights, made a round ahead (before the stores of the round before), one search for the row of the
+      // first of them.  The LDS reads and writes of a phase are issued together, without branches around them
+      // (a nonzero beyond the segment counts in a spare counter and is sorted into a spare slot): between two
+      // barriers a wave waits for LDS two or three times, not once per nonzero.
       uint32_t col[U];
       F dat[U];
-      auto load_round = [&](uint32_t jb) {
+      auto load_round = [&](uint32_t base) {
+        const uint32_t j = base + U * tid;
+        if (j + U <= seg_end) {
+          load_consecutive(indices + j, col);
+          if (HETER) load_consecutive(data + j, dat);
+        } else {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const uint32_t j = jb + u * kBinThreads;
-          const uint32_t jc = j < seg_end ? j : seg_end - 1u;
-          col[u] = indices[jc];
-          dat[u] = HETER ? data[jc] : F(0);
+          for (int t = 0; t < U; ++t) {
+            const uint32_t jc = j + t < seg_end ? j + t : seg_end - 1u;
+            col[t] = indices[jc];
+            if (HETER) dat[t] = data[jc];
+          }
         }
       };
-      load_round(seg + tid);
+      load_round(seg);
       // hints: the row of nonzero seg + 256 q, for every q up to the end of the segment
       __syncthreads();  // the previous segment is done with s_hint
       {
@@ -149,29 +178,33 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
       // the window from an LDS counter, window offsets from a scan of the counters), then written
       // out in that order: pairs of one window go to consecutive addresses of its bin, so the
       // stores of neighbouring lanes merge instead of arriving as single 8-byte requests.
-      for (uint32_t jb = seg + tid; jb - tid < seg_end; jb += kRound) {
-        uint32_t rank[U], win[U], rel[U];
-        F val[U];
-        uint32_t k[U];
+      for (uint32_t base = seg; base < seg_end; base += kRound) {
+        const uint32_t j = base + U * tid;
+        uint32_t rank[U], win[U], rel[U], krow[U];
+        F val[U], v[U];
+        {
+          const uint32_t jf = j < seg_end ? j : seg_end - 1u;
+          const uint32_t q = (jf - seg) >> kHintShift;
+          uint32_t kk = row_of(jf, s_hint[q], s_hint[q + 1]);
+          uint32_t e = s_ptr[kk + 1u];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {  // (LDS only: the round's columns and weights are on their way)
-          const uint32_t j = jb + u * kBinThreads;
-          const uint32_t jc = j < seg_end ? j : seg_end - 1u;
-          const uint32_t q = (jc - seg) >> kHintShift;
-          k[u] = row_of(jc, s_hint[q], s_hint[q + 1]);
+          for (int t = 0; t < U; ++t) {
+            const uint32_t jt = j + t < seg_end ? j + t : seg_end - 1u;
+            while (e <= jt) e = s_ptr[++kk + 1u];  // (ends: jt < seg_end <= s_ptr[rows])
+            krow[t] = kk;
+          }
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const uint32_t j = jb + u * kBinThreads;
+        for (int t = 0; t < U; ++t) v[t] = s_v[krow[t]];
+#pragma unroll
+        for (int t = 0; t < U; ++t) {
           // v * values[j] (heter) or values * v (homo), as the reference's CPU loop multiplies
-          val[u] = HETER ? static_cast<F>(s_v[k[u]] * dat[u]) : static_cast<F>(w_homo * s_v[k[u]]);
-          win[u] = j < seg_end ? col[u] >> shift : 0xffffffffu;  // (0xffffffff: no pair)
-          rel[u] = col[u] & ((1u << shift) - 1u);
-          rank[u] = 0;
+          val[t] = HETER ? static_cast<F>(v[t] * dat[t]) : static_cast<F>(w_homo * v[t]);
+          win[t] = j + t < seg_end ? col[t] >> shift : kMaxWindows;  // (kMaxWindows: no pair)
+          rel[t] = col[t] & ((1u << shift) - 1u);
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u)
-          if (win[u] != 0xffffffffu) rank[u] = atomicAdd(&s_cnt[win[u]], 1u);
+        for (int t = 0; t < U; ++t) rank[t] = atomicAdd(&s_cnt[win[t]], 1u);
         __syncthreads();
         if (tid < kWave) {  // offsets of the windows within the round: two counters per lane
           const uint32_t c0 = s_cnt[2 * tid], c1 = s_cnt[2 * tid + 1];
@@ -190,32 +223,46 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
           s_cnt[2 * tid + 1] = 0;
         }
         __syncthreads();
+        uint32_t pos[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          if (win[u] != 0xffffffffu) {
-            const uint32_t pos = s_off[win[u]] + rank[u];
-            BinPair<F> e;
-            e.rel = rel[u] | (win[u] << kWindowIdShift);
-            e.val = val[u];
-            s_sorted[pos] = e;
-          }
+        for (int t = 0; t < U; ++t) pos[t] = s_off[win[t]];
+#pragma unroll
+        for (int t = 0; t < U; ++t) {
+          BinPair<F> e;
+          e.rel = rel[t] | (win[t] << kWindowIdShift);
+          e.val = val[t];
+          s_sorted[win[t] != kMaxWindows ? pos[t] + rank[t] : kRound] = e;
         }
         __syncthreads();
-        // (No barrier behind the stores: the next round's loads and counting follow at once; what the stores
-        // read is written again only behind the next round's barriers.)
-        if (jb - tid + kRound < seg_end) load_round(jb + kRound);
+        // (No barrier behind the stores: the next round's counting follows at once; what the stores read is
+        // written again only behind the next round's barriers.)
+        if (base + kRound < seg_end) load_round(base + kRound);
         const uint32_t round_total = s_off[kMaxWindows];
-        for (uint32_t i = tid; i < round_total; i += kBinThreads) {
-          BinPair<F> e = s_sorted[i];
-          const uint32_t w = e.rel >> kWindowIdShift;
-          e.rel &= (1u << kWindowIdShift) - 1u;
-          const uint32_t slot = s_base[w] + i;
-          const uint64_t at = region_off + static_cast<uint64_t>(w) * cap + slot;
-          if (slot < cap && at < n_pairs) {
-            if (PACKED) packed.val[at] = e.val, packed.rel[at] = static_cast<uint16_t>(e.rel);
-            else pairs[at] = e;
-          } else {
-            atomic_add(y + ((w << shift) | e.rel), e.val);
+        BinPair<F> out[U];
+        uint32_t slot0[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) out[u] = s_sorted[tid + u * kBinThreads];  // (beyond the round's total: stale, unused)
+#pragma unroll
+        for (int u = 0; u < U; ++u) slot0[u] = s_base[(out[u].rel >> kWindowIdShift) % kMaxWindows];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t i = tid + u * kBinThreads;
+          if (i < round_total) {
+            const uint32_t w = out[u].rel >> kWindowIdShift;
+            const uint32_t r = out[u].rel & ((1u << kWindowIdShift) - 1u);
+            const uint32_t slot = slot0[u] + i;
+            const uint64_t at = region_off + static_cast<uint64_t>(w) * cap + slot;
+            if (slot < cap && at < n_pairs) {
+              if (PACKED) {
+                packed.val[at] = out[u].val, packed.rel[at] = static_cast<uint16_t>(r);
+              } else {
+                BinPair<F> e;
+                e.rel = r, e.val = out[u].val;
+                pairs[at] = e;
+              }
+            } else {
+              atomic_add(y + ((w << shift) | r), out[u].val);
+            }
           }
         }
       }
@@ -319,24 +366,27 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
       i_next = 0;
     }
   };
-  auto load_step = [&](BinPair<F> (&e)[kAddU]) {
-    if (i0 + kAddU * kWave <= n) {  // a full step: plain loads
+  // Every step issues the same loads whatever it holds (a lane beyond the bin's count reads the bin's first
+  // pairs again and leaves them out by their number; behind the last step come empty ones): the compiler can
+  // then count the loads in flight and wait for one step's while the next ones' are on their way.  With loads
+  // inside branches it waits for all of them before it issues more.
+  struct PairStep {
+    BinPair<F> p[kAddU];
+    uint32_t left;  // pairs from the step's first one to the end of the bin
+  };
+  auto load_pairs = [&](PairStep &e) {
+    e.left = i0 < n ? n - i0 : 0u;
 #pragma unroll
-      for (int u = 0; u < kAddU; ++u) e[u] = bin[i0 + u * kWave + lane];
-    } else {
-#pragma unroll
-      for (int u = 0; u < kAddU; ++u) {
-        const uint32_t i = i0 + u * kWave + lane;
-        e[u].rel = 0xffffffffu;
-        e[u].val = F(0);
-        if (i < n) e[u] = bin[i];
-      }
+    for (int u = 0; u < kAddU; ++u) {
+      const uint32_t i = i0 + u * kWave + lane;
+      e.p[u] = bin[i < n ? i : 0u];
     }
   };
-  auto add_step = [&](const BinPair<F> (&e)[kAddU]) {
+  auto add_pairs = [&](const PairStep &e) {
 #pragma unroll
     for (int u = 0; u < kAddU; ++u)
-      if (e[u].rel - r0 < width) atomicAdd(&window[e[u].rel - r0], static_cast<double>(e[u].val));  // (wraps below r0)
+      if (u * kWave + lane < e.left && e.p[u].rel - r0 < width)
+        atomicAdd(&window[e.p[u].rel - r0], static_cast<double>(e.p[u].val));  // (wraps below r0)
   };
   // Packed bins: a lane takes two quads of a step, each 16 or 32 bytes of products and 8 bytes of positions
   // (bins begin at multiples of 4 pairs and their regions end at one: a bin's last quad is read whole and
@@ -351,14 +401,10 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
     for (int u = 0; u < 2; ++u) {
       const uint32_t i = i0 + 4u * (static_cast<uint32_t>(u) * kWave + lane);
       e.valid[u] = i < n ? n - i : 0u;
-#pragma unroll
-      for (int t = 0; t < 4; ++t) e.v[u][t] = F(0);
-      e.r[u][0] = e.r[u][1] = 0u;
-      if (i < n) {
-        const uint2 r = *reinterpret_cast<const uint2 *>(packed.rel + bin_off + i);
-        e.r[u][0] = r.x, e.r[u][1] = r.y;
-        load_quad(packed.val + bin_off + i, e.v[u]);
-      }
+      const uint64_t at = bin_off + (i < n ? i : 0u);
+      const uint2 r = *reinterpret_cast<const uint2 *>(packed.rel + at);
+      e.r[u][0] = r.x, e.r[u][1] = r.y;
+      load_quad(packed.val + at, e.v[u]);
     }
   };
   auto add_packed = [&](const PackedStep &e) {
@@ -372,32 +418,44 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
       }
     }
   };
+  // D steps are under way at a time; step k is added when step k + D - 1 has been requested.
+  auto run = [&](auto &e, auto load, auto add) {
+    constexpr int D = static_cast<int>(sizeof(e) / sizeof(e[0]));
+    bool live = next_step();
+    if (!live) return;
+    uint64_t last_off = bin_off;  // a bin that holds pairs: what an empty step reads
+    auto advance = [&]() {
+      live = live && next_step();
+      if (live) last_off = bin_off;
+      else n = 0, bin_off = last_off, bin = pairs + last_off;
+    };
+    bool has[D];
+    load(e[0]);
+    has[0] = true;
+#pragma unroll
+    for (int d = 1; d < D - 1; ++d) {
+      advance();
+      load(e[d]);
+      has[d] = live;
+    }
+    for (;;) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        const int nx = (d + D - 1) % D;
+        advance();
+        load(e[nx]);
+        has[nx] = live;
+        add(e[d]);
+        if (!has[(d + 1) % D]) return;
+      }
+    }
+  };
   if (PACKED) {
-    PackedStep ea, eb;
-    bool more = next_step();
-    if (more) load_packed(ea);
-    while (more) {
-      more = next_step();
-      if (more) load_packed(eb);
-      add_packed(ea);
-      if (!more) break;
-      more = next_step();
-      if (more) load_packed(ea);
-      add_packed(eb);
-    }
+    PackedStep e[4];
+    run(e, load_packed, add_packed);
   } else {
-    BinPair<F> ea[kAddU], eb[kAddU];
-    bool more = next_step();
-    if (more) load_step(ea);
-    while (more) {
-      more = next_step();
-      if (more) load_step(eb);
-      add_step(ea);
-      if (!more) break;
-      more = next_step();
-      if (more) load_step(ea);
-      add_step(eb);
-    }
+    PairStep e[2];
+    run(e, load_pairs, add_pairs);
   }
   __syncthreads();
   for (uint32_t i = tid; i < width; i += kBinThreads) {
