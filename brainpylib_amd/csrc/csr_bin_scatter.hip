@@ -580,18 +580,27 @@ __global__ __launch_bounds__(kBinThreads) __attribute__((amdgpu_num_sgpr(80))) v
       // One round's column indices and weights are requested a round ahead, so that their latency
       // overlaps the sort, the reservation and the stores of the round before.
       auto fetch = [&](uint32_t jb, uint32_t (&col)[U], F (&val)[U]) {
+        // first where every nonzero of the lane lies (LDS only), then all the loads together, without a
+        // branch around them (beyond the segment: its last nonzero again)
+        uint32_t at[U], cb[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const uint32_t j = jb + u * kBinThreads;
-          col[u] = 0xffffffffu;  // no pair
-          val[u] = F(0);
-          if (j < seg_end) {
-            const uint32_t q = (j - seg) >> kHintShift;
-            const uint32_t k = row_of(j, s_hint[q], s_hint[q + 1]);
-            const uint32_t at = s_start[k] + (j - s_ptr[k]);
-            col[u] = indices[at] + s_colbase[k];
-            val[u] = HETER ? data[at] : w_homo;
-          }
+          const uint32_t jc = j < seg_end ? j : seg_end - 1u;
+          const uint32_t q = (jc - seg) >> kHintShift;
+          const uint32_t k = row_of(jc, s_hint[q], s_hint[q + 1]);
+          at[u] = s_start[k] + (jc - s_ptr[k]);
+          cb[u] = s_colbase[k];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          col[u] = indices[at[u]];
+          val[u] = HETER ? data[at[u]] : w_homo;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t j = jb + u * kBinThreads;
+          col[u] = j < seg_end ? col[u] + cb[u] : 0xffffffffu;  // (0xffffffff: no pair)
         }
       };
       uint32_t col[U];
@@ -624,8 +633,11 @@ __global__ __launch_bounds__(kBinThreads) __attribute__((amdgpu_num_sgpr(80))) v
           s_off[2 * tid] = sum - (c0 + c1);
           s_off[2 * tid + 1] = sum - c1;
           if (tid == kWave - 1) s_off[kMaxWindows] = sum;
-          s_base[2 * tid] = c0 ? atomicAdd(&fill[(2 * tid * kSubRuns + sub) * kFillStride], c0) : 0u;
-          s_base[2 * tid + 1] = c1 ? atomicAdd(&fill[((2 * tid + 1) * kSubRuns + sub) * kFillStride], c1) : 0u;
+          // (both reservations under way together; a window without pairs adds nothing to its counter)
+          const uint32_t b0 = atomicAdd(&fill[(2 * tid * kSubRuns + sub) * kFillStride], c0);
+          const uint32_t b1 = atomicAdd(&fill[((2 * tid + 1) * kSubRuns + sub) * kFillStride], c1);
+          s_base[2 * tid] = b0;
+          s_base[2 * tid + 1] = b1;
         }
         __syncthreads();
 #pragma unroll
