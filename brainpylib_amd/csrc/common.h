@@ -95,6 +95,15 @@ template <typename F>
 bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool heter, const uint32_t *indices,
                  const uint32_t *indptr, const F *vec, F *y, uint32_t n_row, uint32_t n_col, uint32_t nnz);
 
+// Transposed CSR times dense vector for outputs of at most kFlatWindowMaxSlices windows of kFlatWindowMaxCols
+// columns (a float64 window in LDS per workgroup, the workgroups of a window equal shares of the nonzeros;
+// csr_bin_scatter.hip).  false, having enqueued nothing, if it cannot run (wider output, no scratch memory).
+constexpr uint32_t kFlatWindowMaxCols = 16384;
+constexpr uint32_t kFlatWindowMaxSlices = 2;  // (a third window costs a third pass over the matrix: sorting wins)
+template <typename F>
+bool flat_window_scatter(const char *target, hipStream_t stream, const F *data, bool heter, const uint32_t *indices,
+                         const uint32_t *indptr, const F *vec, F *y, uint32_t n_row, uint32_t n_col);
+
 // The same for event input (event_csr_matvec, transposed, wide outputs): the caller lists the
 // active rows on the device, (first nonzero, length) each in `active_list`, their number in
 // active_count[0] (the list has room for `list_cap` rows); `scratch` is device memory of `scratch_bytes` bytes whose first

@@ -276,6 +276,147 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
   }
 }
 
+// ---- one output window ------------------------------------------------------------------------
+// Transposed product whose output fits ONE float64 window in LDS (up to 16,384 columns): no sorting.
+// Every workgroup takes a contiguous range of the NONZEROS (whatever rows they belong to, so that
+// uneven rows and hub rows cost nothing), walks it like the producer above (a lane takes U consecutive
+// nonzeros with one 16-byte request each for columns and weights, one search for the row of the first)
+// and adds the products to its window with float64 LDS atomics; there is no barrier inside a tile of
+// 1,024 rows.  The windows go to scratch memory as float64 and a second kernel adds them in a fixed
+// order and rounds once.  (A wave per row, as the window kernel of the event operators walks, leaves
+// most lanes idle on short rows: 1,000,000 x 16,000 with 100 per row 616 us, 4,000,000 x 8,000 with
+// 20 per row 1,510 us.)
+template <typename F, bool HETER>
+__global__ __launch_bounds__(kBinThreads) void flat_window_kernel(
+    const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
+    const F *__restrict__ vec, uint32_t n_row, uint32_t n_col, uint32_t slices, double *__restrict__ partial) {
+  extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
+  double *window = reinterpret_cast<double *>(smem_raw);
+  // workgroup (share, slice): the share's nonzeros whose columns lie in slice `slice` of the output (one slice
+  // unless the output is wider than a window: every slice's workgroups then read the share again)
+  const uint32_t shares = gridDim.x / slices, share = blockIdx.x / slices, slice = blockIdx.x % slices;
+  const uint32_t c_lo = slice * kFlatWindowMaxCols;
+  const uint32_t width = n_col - c_lo < kFlatWindowMaxCols ? n_col - c_lo : kFlatWindowMaxCols;
+  __shared__ uint32_t s_ptr[kTileRows + 1];
+  __shared__ F s_v[kTileRows];
+  __shared__ uint32_t s_hint[kBinThreads + 1];  // row (within the tile) of every 256th nonzero of the segment
+  constexpr int U = (sizeof(F) == 4) ? 4 : 2;
+  constexpr uint32_t kRound = U * kBinThreads;
+  const uint32_t tid = threadIdx.x;
+  for (uint32_t i = tid; i < width; i += kBinThreads) window[i] = 0.0;
+  const uint32_t nnz = indptr[n_row];
+  // the share's nonzeros [a, b): equal shares, multiples of 4
+  const uint32_t per = (static_cast<uint32_t>((static_cast<uint64_t>(nnz) + shares - 1u) / shares) + 3u) & ~3u;
+  const uint64_t a64 = static_cast<uint64_t>(share) * per;
+  const uint32_t a = a64 < nnz ? static_cast<uint32_t>(a64) : nnz;
+  const uint32_t b = a64 + per < nnz ? static_cast<uint32_t>(a64 + per) : nnz;
+  const F w_homo = HETER ? F(0) : data[0];
+
+  // largest k in [lo, hi] with s_ptr[k] <= j
+  auto row_of = [&](uint32_t j, uint32_t lo, uint32_t hi) {
+    while (lo < hi) {
+      const uint32_t mid = (lo + hi + 1u) >> 1;
+      if (s_ptr[mid] <= j) lo = mid;
+      else hi = mid - 1u;
+    }
+    return lo;
+  };
+
+  if (a < b) {
+    // the row that holds nonzero a: the last r with indptr[r] <= a (every thread searches: uniform)
+    uint32_t t0 = 0;
+    {
+      uint32_t lo = 0, hi = n_row - 1u;
+      while (lo < hi) {
+        const uint32_t mid = lo + ((hi - lo + 1u) >> 1);
+        if (indptr[mid] <= a) lo = mid;
+        else hi = mid - 1u;
+      }
+      t0 = lo;
+    }
+    for (;;) {
+      const uint32_t rows = (n_row - t0 < kTileRows) ? n_row - t0 : kTileRows;
+      __syncthreads();  // the previous tile is done with s_ptr / s_v (and the window is cleared)
+      if (tid < rows) s_v[tid] = vec[t0 + tid];
+      if (tid <= rows) s_ptr[tid] = indptr[t0 + tid];
+      if (tid == 0 && rows == kTileRows) s_ptr[kTileRows] = indptr[t0 + kTileRows];
+      __syncthreads();
+      const uint32_t tile_end = s_ptr[rows];
+      const uint32_t j0 = s_ptr[0] > a ? s_ptr[0] : a, j1 = tile_end < b ? tile_end : b;
+      for (uint32_t seg = j0; seg < j1; seg += kSegment) {
+        const uint32_t seg_end = (j1 - seg < kSegment) ? j1 : seg + kSegment;
+        __syncthreads();  // the previous segment is done with s_hint
+        {
+          const uint32_t j = seg + (tid << kHintShift);
+          s_hint[tid] = (j < seg_end) ? row_of(j, 0u, rows - 1u) : rows - 1u;
+          if (tid == 0) s_hint[kBinThreads] = rows - 1u;
+        }
+        __syncthreads();
+        for (uint32_t base = seg; base < seg_end; base += kRound) {
+          const uint32_t j = base + U * tid;
+          if (j >= seg_end) continue;
+          uint32_t col[U];
+          F dat[U];
+          if (j + U <= seg_end) {
+            load_consecutive(indices + j, col);
+            if (HETER) load_consecutive(data + j, dat);
+          } else {
+#pragma unroll
+            for (int t = 0; t < U; ++t) {
+              const uint32_t jc = j + t < seg_end ? j + t : seg_end - 1u;
+              col[t] = indices[jc];
+              if (HETER) dat[t] = data[jc];
+            }
+          }
+          const uint32_t q = (j - seg) >> kHintShift;
+          uint32_t kk = row_of(j, s_hint[q], s_hint[q + 1]);
+          uint32_t e = s_ptr[kk + 1u];
+          uint32_t krow[U];
+#pragma unroll
+          for (int t = 0; t < U; ++t) {
+            const uint32_t jt = j + t < seg_end ? j + t : seg_end - 1u;
+            while (e <= jt) e = s_ptr[++kk + 1u];  // (ends: jt < seg_end <= s_ptr[rows])
+            krow[t] = kk;
+          }
+          F v[U];
+#pragma unroll
+          for (int t = 0; t < U; ++t) v[t] = s_v[krow[t]];
+#pragma unroll
+          for (int t = 0; t < U; ++t) {
+            // v * values[j] (heter) or values * v (homo), as the reference's CPU loop multiplies
+            const F prod = HETER ? static_cast<F>(v[t] * dat[t]) : static_cast<F>(w_homo * v[t]);
+            if (j + t < seg_end && col[t] - c_lo < width) atomicAdd(&window[col[t] - c_lo], static_cast<double>(prod));  // (wraps below c_lo)
+          }
+        }
+      }
+      if (tile_end >= b || t0 + rows >= n_row) break;
+      t0 += rows;
+    }
+  }
+  __syncthreads();
+  double *mine = partial + static_cast<size_t>(share) * n_col + c_lo;
+  for (uint32_t i = tid; i < width; i += kBinThreads) mine[i] = window[i];
+}
+
+// y[c] = the workgroups' windows added in the order of the workgroups, in float64, rounded once
+template <typename F>
+__global__ __launch_bounds__(256) void sum_windows_kernel(const double *__restrict__ partial, F *__restrict__ y,
+                                                          uint32_t n_col, uint32_t groups) {
+  const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+  if (c >= n_col) return;
+  double acc = 0.0;
+  uint32_t g = 0;
+  for (; g + 4 <= groups; g += 4) {  // (four loads in flight; the additions stay in order)
+    const double a0 = partial[static_cast<size_t>(g) * n_col + c];
+    const double a1 = partial[static_cast<size_t>(g + 1) * n_col + c];
+    const double a2 = partial[static_cast<size_t>(g + 2) * n_col + c];
+    const double a3 = partial[static_cast<size_t>(g + 3) * n_col + c];
+    acc = (((acc + a0) + a1) + a2) + a3;
+  }
+  for (; g < groups; ++g) acc += partial[static_cast<size_t>(g) * n_col + c];
+  y[c] = static_cast<F>(acc);
+}
+
 // grid = n_win * slices * parts; workgroup (b, q, s) adds window b's pairs of producers
 // [s * P / parts, ...) that fall into slice q of the window (slices = 2^(shift - lds_shift): a window
 // wider than the 2^lds_shift accumulators in LDS is added slice by slice, every slice reading the pairs).
@@ -905,6 +1046,40 @@ bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint
   return true;
 }
 
+template <typename F>
+bool flat_window_scatter(const char *target, hipStream_t stream, const F *data, bool heter, const uint32_t *indices,
+                         const uint32_t *indptr, const F *vec, F *y, uint32_t n_row, uint32_t n_col) {
+  if (n_row == 0 || n_col == 0 || n_col > kFlatWindowMaxSlices * kFlatWindowMaxCols) return false;
+  const uint32_t slices = div_up(n_col, kFlatWindowMaxCols);
+  const size_t lds = static_cast<size_t>(slices > 1 ? kFlatWindowMaxCols : n_col) * sizeof(double);
+  auto kernel = heter ? flat_window_kernel<F, true> : flat_window_kernel<F, false>;
+  static thread_local bool attr_set[2] = {false, false};
+  if (!attr_set[heter]) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(kFlatWindowMaxCols * sizeof(double))) != hipSuccess) {
+      (void)hipGetLastError();
+      return false;
+    }
+    attr_set[heter] = true;
+  }
+  // two workgroups per CU where their windows and 12 KB of row tables each fit the CU's 160 KB
+  const unsigned num_cu = static_cast<unsigned>(device_info().num_cu);
+  const size_t static_lds = 2 * (kBinThreads + 1) * sizeof(uint32_t) + kTileRows * sizeof(F) + 256;  // (row tables)
+  unsigned shares = (lds + static_lds <= 80 * 1024 ? 2u : 1u) * num_cu / slices;
+  if (shares > div_up(n_row, 64)) shares = div_up(n_row, 64);
+  const size_t partial_bytes = static_cast<size_t>(shares) * n_col * sizeof(double);
+  double *partial = static_cast<double *>(stream_workspace(stream, partial_bytes));
+  if (partial == nullptr) {
+    if (!scratch_refused_by_capture()) bpl_clear_error();  // (an allocation failed: the caller has other paths)
+    return false;
+  }
+  hipLaunchKernelGGL(kernel, dim3(shares * slices), dim3(kBinThreads), lds, stream, data, indices, indptr, vec, n_row,
+                     n_col, slices, partial);
+  hipLaunchKernelGGL(sum_windows_kernel<F>, dim3(div_up(n_col, 256)), dim3(256), 0, stream,
+                     static_cast<const double *>(partial), y, n_col, shares);
+  return check_launch(target);
+}
+
 constexpr uint64_t kChunkPairBytes = 200ull << 20;
 constexpr uint32_t kMaxChunks = 6;
 
@@ -1028,6 +1203,10 @@ template bool bin_event_scatter<float>(hipStream_t, const float *, bool, const u
 template bool bin_event_scatter<double>(hipStream_t, const double *, bool, const uint32_t *, const uint32_t *, double *,
                                         uint32_t, uint32_t, uint32_t *, const uint2 *, uint32_t, void *, size_t,
                                         const uint32_t *);
+template bool flat_window_scatter<float>(const char *, hipStream_t, const float *, bool, const uint32_t *, const uint32_t *,
+                                         const float *, float *, uint32_t, uint32_t);
+template bool flat_window_scatter<double>(const char *, hipStream_t, const double *, bool, const uint32_t *,
+                                          const uint32_t *, const double *, double *, uint32_t, uint32_t);
 template bool bin_scatter_usable<float>(uint32_t, uint32_t);
 template bool bin_scatter_usable<double>(uint32_t, uint32_t);
 template bool bin_scatter<float>(const char *, hipStream_t, const float *, bool, const uint32_t *, const uint32_t *,

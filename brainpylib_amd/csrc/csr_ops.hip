@@ -1460,8 +1460,15 @@ void csr_matvec_entry(const char *target, hipStream_t stream, void **buffers, co
     // further window means another pass over the whole matrix; the windows remain for matrices too
     // small to sort or of unknown size, direct atomics beyond four windows.)
     const uint32_t plain_windows = div_up(d.n_col, static_cast<uint32_t>((128u * 1024u) / sizeof(double)));
-    if (plain_windows > 1 && d.n_row > 0 && bin_scatter_usable<F>(d.n_col, nnz)) {
+    if (plain_windows > kFlatWindowMaxSlices && d.n_row > 0 && bin_scatter_usable<F>(d.n_col, nnz)) {
       if (bin_scatter<F>(target, stream, data, HETER, indices, indptr, vec, out, d.n_row, d.n_col, nnz)) return;
+      if (scratch_refused_by_capture()) return;  // (the error stands)
+    }
+    // One or two windows and a matrix worth a chip full of workgroups: the flat walk over the nonzeros, once per
+    // window (167 and 330 us at 1e8 nonzeros; the sort takes 420).  (Smaller ones, and callers whose descriptor
+    // does not say how many nonzeros there are, keep the walk that hands rows to waves.)
+    if (plain_windows <= kFlatWindowMaxSlices && nnz >= (1u << 20)) {
+      if (flat_window_scatter<F>(target, stream, data, HETER, indices, indptr, vec, out, d.n_row, d.n_col)) return;
       if (scratch_refused_by_capture()) return;  // (the error stands)
     }
     launch_scatter<F, F, HETER, kDense>(ScratchSource{stream}, data, indices, indptr, vec, out, d.n_row, d.n_col);

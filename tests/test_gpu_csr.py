@@ -456,6 +456,44 @@ def test_transposed_csr_matvec_wide_output_sorted_scatter(cuda, oracle_mod, dtyp
     assert np.array_equal(got, want)  # multiples of 0.5: exact in any order
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_transposed_csr_matvec_one_output_window_flat_walk(cuda, oracle_mod, dtype):
+  # outputs of at most 32,768 columns with at least 2^20 nonzeros: every workgroup walks an equal share of the
+  # nonzeros into one float64 window of up to 16,384 columns.  Short rows, empty rows (also first and last), one row that holds a
+  # third of the nonzeros, more than 1,024 rows per workgroup, the widest and a narrow window, twice in a row.
+  rng = np.random.default_rng(47)
+  for n_row, n_col, mean, hub in ((400_000, 16_384, 4, 0), (30_000, 16_000, 60, 600_000), (900_000, 700, 2, 0),
+                                  (2000, 9000, 800, 0),
+                                  # (two windows: every share of the nonzeros is walked once per window)
+                                  (150_000, 32_768, 9, 0), (60_000, 16_385, 25, 0)):
+    counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
+    counts[0] = counts[-1] = 0
+    counts[rng.integers(0, n_row, size=n_row // 7)] = 0
+    if hub:
+      counts = counts.astype(np.int64)
+      counts[n_row // 3] = min(hub, n_col)
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_row)
+    assert indices.shape[0] >= 1 << 20
+    data = rng.standard_normal(indices.shape[0]).astype(dtype)
+    shape = (n_row, n_col)
+    print("shape", shape, dtype.__name__, flush=True)
+    v = rng.standard_normal(n_row).astype(dtype)
+    want = oracle_mod.csr_matvec(data, indices, indptr, v, shape=shape, transpose=True)
+    mag = oracle_mod.csr_matvec(np.abs(data), indices, indptr, np.abs(v), shape=shape, transpose=True)
+    for _ in range(2):
+      got = bpl.cusparse_csr_matvec(data, indices, indptr, v, shape=shape, transpose=True).cpu().numpy()
+      assert_close_reordered(got, want, mag, dtype, what="one-window flat walk %s" % (shape,))
+    vi = rng.integers(-2, 3, size=n_row).astype(dtype)
+    di = rng.integers(-3, 4, size=indices.shape[0]).astype(dtype)
+    want = oracle_mod.csr_matvec(di, indices, indptr, vi, shape=shape, transpose=True)
+    got = bpl.cusparse_csr_matvec(di, indices, indptr, vi, shape=shape, transpose=True).cpu().numpy()
+    assert np.array_equal(got, want)  # small integers: exact in any order
+    w = np.array([0.5], dtype=dtype)
+    want = oracle_mod.csr_matvec(w, indices, indptr, vi, shape=shape, transpose=True)
+    got = bpl.cusparse_csr_matvec(w, indices, indptr, vi, shape=shape, transpose=True).cpu().numpy()
+    assert np.array_equal(got, want)  # multiples of 0.5
+
+
 def test_transposed_csr_matvec_rows_taken_in_chunks(cuda, oracle_mod):
   # float64 pairs of 10 bytes: from 21 million nonzeros on the rows are binned and added in two or more
   # chunks, one after the other over the same scratch memory; uneven rows, so that the chunks differ
