@@ -338,13 +338,16 @@ __global__ __launch_bounds__(kWinThreads) void collect_active_rows_batched_kerne
 }
 
 // Row groups that take part in a launch whose active rows are listed in device memory: one per
-// 32,768 active nonzeros (estimated from the mean row length), at least one, at most the launched
-// number.  Every group writes a slice of partial outputs that the summing kernel reads again, so
-// with little activity a few groups finish sooner than a chip full of them.
+// 32,768 active nonzeros (estimated from the mean row length) or per 128 active rows (a wave walks
+// its rows one after the other, a memory round trip or two each: short rows are bound by their
+// number), at least one, at most the launched number.  Every group writes a slice of partial outputs
+// that the summing kernel reads again, so with little activity a few groups finish sooner than a
+// chip full of them.
 __device__ __forceinline__ uint32_t groups_in_use(uint32_t active_rows, uint32_t nnz, uint32_t n_row,
                                                  uint32_t launched) {
   const uint64_t work = static_cast<uint64_t>(active_rows) * (nnz / n_row + 1u);
-  const uint64_t want = (work + 32767u) / 32768u;
+  const uint64_t by_work = (work + 32767u) / 32768u, by_rows = (active_rows + 127u) / 128u;
+  const uint64_t want = by_work > by_rows ? by_work : by_rows;
   return want < 1u ? 1u : want > launched ? launched : static_cast<uint32_t>(want);
 }
 
@@ -573,6 +576,13 @@ __global__ __launch_bounds__(256) void sum_partials_kernel(const F *__restrict__
   }
   F acc = F(0);
   uint32_t g = 0;
+  for (; g + 16 <= groups; g += 16) {  // (sixteen loads in flight: with hundreds of groups a column is a chain of round trips)
+    F a[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) a[k] = partial[static_cast<size_t>(g + k) * n_col + c];
+#pragma unroll
+    for (int k = 0; k < 16; k += 4) acc += (a[k] + a[k + 1]) + (a[k + 2] + a[k + 3]);
+  }
   for (; g + 4 <= groups; g += 4) {
     const F a0 = partial[static_cast<size_t>(g) * n_col + c];
     const F a1 = partial[static_cast<size_t>(g + 1) * n_col + c];
