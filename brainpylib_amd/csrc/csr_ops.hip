@@ -1398,10 +1398,14 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
       bpl_clear_error();
     }
     if constexpr (std::is_same<F, VT>::value) {
-      // A longer vector is gathered from L2.  Rows of 24 nonzeros or more on average: the flat walk over the
-      // nonzeros with 16-byte loads of the index and weight streams (csr_flat_gather.hip); shorter ones: the
-      // walks below.  The mean is known on the device only, so both are enqueued and one returns at once.
-      constexpr uint32_t kFlatMinMean = 24;
+      // A longer vector is gathered from L2.  Rows of 4 nonzeros or more on average: the flat walk over the
+      // nonzeros with 16-byte loads of the index and weight streams (csr_flat_gather.hip; 4,000,000 rows of 8:
+      // 224 against 304 us, 2,000,000 rows of 20: 255 against 348 us); shorter ones: the walks below.  The
+      // mean is known on the device only, so both are enqueued and one returns at once.  (Under 16,384 rows
+      // the walks below stay: with 2,000 rows of 40,000 and a vector of 12 MB the walk that keeps a row's
+      // gathers together takes 507 us, the flat one 835; only matrices of a few hundred rows that are
+      // nearly dense would gain, and small ones would pay for a launch that returns at once.)
+      constexpr uint32_t kFlatMinMean = 4;
       if (n_row >= 16384 && n_col > 0) {
         const FlatGather flat =
           csr_flat_gather<F>(target, stream, data, HETER, indices, indptr, x, y, n_row, kFlatMinMean, 0xffffffffu);

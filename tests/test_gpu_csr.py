@@ -695,15 +695,16 @@ def test_small_event_scatter_in_one_launch(cuda, oracle_mod, dtype):
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_csr_matvec_with_16_byte_stream_loads(cuda, oracle_mod, dtype):
-  # at least 16,384 rows, a vector too long for LDS and 24 nonzeros or more per row on average: the walk
-  # that reads four consecutive nonzeros per lane and request.  Every lanes-per-row choice of that walk
-  # (means 30 .. 900), a mean just below its limit (the other kernel runs), nnz not a multiple of 4, empty
+  # at least 16,384 rows, a vector too long for LDS and 4 nonzeros or more per row on average: the walk
+  # that reads four consecutive nonzeros per lane and request.  Means from 30 to 900, means on both sides of
+  # its limit (3: the other kernel runs; 4), nnz not a multiple of 4, empty
   # rows, rows of one nonzero, hub rows that go to the whole workgroup, both weight kinds.
   rng = np.random.default_rng(71)
   limit = 4 * (160 * 1024 - 1024) // np.dtype(dtype).itemsize + 1  # first length that is not staged at all
   for n_row, n_col, mean, hubs in ((20_000, limit, 30, 0), (16_384, limit + 3, 60, 2), (17_001, 400_000, 100, 3),
                                    (16_400, 300_000, 250, 1), (16_390, 200_000, 500, 0), (16_385, 170_000, 900, 1),
-                                   (40_000, 1_000_000, 23, 0), (30_000, 250_000, 24, 40)):
+                                   (40_000, 1_000_000, 23, 0), (30_000, 250_000, 24, 40),
+                                   (300_000, 170_000, 3, 0), (280_000, 170_000, 4, 2)):
     counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
     counts[rng.integers(0, n_row, 50)] = 0
     counts[rng.integers(0, n_row, 50)] = 1
@@ -806,7 +807,7 @@ def test_gather_hub_rows(cuda, oracle_mod):
 
 
 def _flat_walk_counts(kind, n_row, rng):
-  """Row lengths that exercise the flat walk of csr_matvec (mean of 24 or more, 16,384 rows or more)."""
+  """Row lengths that exercise the flat walk of csr_matvec (mean of 4 or more, 16,384 rows or more)."""
   if kind == "poisson":
     return np.maximum(1, rng.poisson(100, n_row))
   if kind == "even":
@@ -833,19 +834,25 @@ def _flat_walk_counts(kind, n_row, rng):
     c = np.full(n_row, 4)
     c[::3] = 1024
     return c
+  if kind == "short":  # a mean just above the limit: a step of 1,024 nonzeros meets some 200 rows, four windows of indptr
+    return rng.poisson(5, n_row)
+  if kind == "ones":  # rows of one nonzero among rows of twelve: quads that meet four rows
+    c = np.ones(n_row, dtype=np.int64)
+    c[::3] = 12
+    return c
   raise ValueError(kind)
 
 
-@pytest.mark.parametrize("kind", ["poisson", "even", "ragged", "empty ends", "hubs", "steps"])
+@pytest.mark.parametrize("kind", ["poisson", "even", "ragged", "empty ends", "hubs", "steps", "short", "ones"])
 def test_csr_matvec_flat_walk_over_the_nonzeros(cuda, oracle_mod, kind):
-  # vectors too long for LDS (more than 162,816 elements) and rows of 24 nonzeros or more on average: every wave
+  # vectors too long for LDS (more than 162,816 elements) and rows of 4 nonzeros or more on average: every wave
   # owns a contiguous range of the nonzeros and tells the rows apart through windows of indptr
   # (csr_flat_gather.hip).  Integer data: every sum is exact in float64, so the result is the oracle's bit for bit.
   rng = np.random.default_rng(len(kind))
   n_row, n_col = 20_011, 170_003
   counts = np.minimum(_flat_walk_counts(kind, n_row, rng), n_col)
   indices, indptr = synth.counted_csr(counts, n_col, seed=3)
-  assert indices.shape[0] // n_row >= 24
+  assert indices.shape[0] // n_row >= 4
   for dtype in (np.float32, np.float64):
     data = rng.integers(-3, 4, size=indices.shape[0]).astype(dtype)
     v = rng.integers(-4, 5, size=n_col).astype(dtype)
