@@ -86,11 +86,41 @@ struct PackedBins {
 };
 template <typename F>
 constexpr size_t bin_pair_bytes(bool packed) { return packed ? sizeof(F) + 2 : sizeof(BinPair<F>); }
-__device__ __forceinline__ void producer_rows(uint32_t p, uint32_t rows_per, uint32_t n_row, uint32_t *r0,
-                                              uint32_t *r1) {
-  const uint64_t lo = static_cast<uint64_t>(p) * rows_per, hi = lo + rows_per;
-  *r0 = lo < n_row ? static_cast<uint32_t>(lo) : n_row;
-  *r1 = hi < n_row ? static_cast<uint32_t>(hi) : n_row;
+// The nonzeros [a, b) of producer p: equal shares (multiples of 4) of the launch's nonzeros [lo, hi), whatever
+// rows they belong to, so that neither uneven rows nor a matrix of a few long rows leave producers idle.
+// lo = chunk_lo; hi = the end of the chunk, or of the matrix for the last chunk (the matrix's nonzero count
+// is read on the device: a caller's count that is too small costs speed, not nonzeros).
+struct NonzeroShare {
+  uint32_t a, b;
+};
+__device__ __forceinline__ NonzeroShare producer_share(uint32_t nnz, uint32_t chunk_lo, uint32_t chunk_nnz, bool last,
+                                                       uint32_t producers, uint32_t p, uint32_t *lo_out) {
+  const uint32_t lo = chunk_lo < nnz ? chunk_lo : nnz;
+  const uint32_t hi = (last || nnz - lo < chunk_nnz) ? nnz : lo + chunk_nnz;
+  const uint32_t per = (static_cast<uint32_t>((static_cast<uint64_t>(hi - lo) + producers - 1u) / producers) + 3u) & ~3u;
+  const uint64_t a = static_cast<uint64_t>(lo) + static_cast<uint64_t>(p) * per;
+  NonzeroShare s;
+  s.a = a < hi ? static_cast<uint32_t>(a) : hi;
+  s.b = a + per < hi ? static_cast<uint32_t>(a + per) : hi;
+  *lo_out = lo;
+  return s;
+}
+
+// The last row r in [0, n_row) with indptr[r] <= pos, for pos < indptr[n_row]: the wave searches together,
+// 64 probes a round (four rounds for a million rows).
+__device__ __forceinline__ uint32_t row_of_nonzero(const uint32_t *__restrict__ indptr, uint32_t n_row, uint32_t pos) {
+  const uint32_t lane = static_cast<uint32_t>(lane_id());
+  uint32_t lo = 0, hi = n_row;  // indptr[lo] <= pos < indptr[hi]
+  while (hi - lo > 1u) {
+    const uint32_t span = hi - lo;
+    const uint32_t stride = span / kWave + (span % kWave ? 1u : 0u);
+    const uint64_t probe = static_cast<uint64_t>(lo) + static_cast<uint64_t>(lane) * stride;
+    const bool below = probe < hi && indptr[probe] <= pos;  // (true for lane 0; true lanes form a prefix)
+    const uint32_t cnt = static_cast<uint32_t>(__popcll(__ballot(below)));
+    lo += (cnt - 1u) * stride;
+    hi = (hi - lo > stride) ? lo + stride : hi;
+  }
+  return lo;
 }
 
 constexpr uint32_t kWindowIdShift = 24;  // (positions within a window take kBinMaxShift = 17 bits, window numbers 7)
@@ -101,8 +131,8 @@ constexpr uint32_t kSegment = kBinThreads << kHintShift;  // nonzeros covered by
 template <typename F, bool HETER, bool PACKED>
 __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
-    const F *__restrict__ vec, F *__restrict__ y, uint32_t n_row, uint32_t rows_per, uint32_t n_win, uint32_t shift,
-    void *__restrict__ pairs_raw, uint64_t n_pairs, uint32_t *__restrict__ counts) {
+    const F *__restrict__ vec, F *__restrict__ y, uint32_t n_row, uint32_t chunk_lo, uint32_t chunk_nnz, uint32_t last,
+    uint32_t n_win, uint32_t shift, void *__restrict__ pairs_raw, uint64_t n_pairs, uint32_t *__restrict__ counts) {
   BinPair<F> *__restrict__ pairs = static_cast<BinPair<F> *>(pairs_raw);
   const PackedBins<F> packed(pairs_raw, n_pairs);
   __shared__ uint32_t s_ptr[kTileRows + 1];
@@ -117,13 +147,13 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
   __shared__ BinPair<F> s_sorted[kRound + 1];  // (and a spare slot; rel: the window's number above the position, from bit kWindowIdShift)
   const uint32_t tid = threadIdx.x;
   const uint32_t p = blockIdx.x;
-  uint32_t r0, r1;
-  producer_rows(p, rows_per, n_row, &r0, &r1);
   if (tid < kMaxWindows) s_cnt[tid] = 0, s_total[tid] = 0;
   if (tid == 0) s_cnt[kMaxWindows] = 0;
-  const uint32_t a0 = indptr[r0], a1 = indptr[r1];
+  uint32_t chunk_first;
+  const NonzeroShare share = producer_share(indptr[n_row], chunk_lo, chunk_nnz, last != 0, gridDim.x, p, &chunk_first);
+  const uint32_t a0 = share.a, a1 = share.b;
   const uint32_t cap = region_cap(a0, a1, n_win);
-  const uint64_t region_off = region_base(a0 - indptr[0], p, n_win);
+  const uint64_t region_off = region_base(a0 - chunk_first, p, n_win);
   const F w_homo = HETER ? F(0) : data[0];
 
   // largest k < rows with s_ptr[k] <= j, searched in [lo, hi]
@@ -136,14 +166,16 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
     return lo;
   };
 
-  for (uint32_t t0 = r0; t0 < r1; t0 += kTileRows) {
-    const uint32_t rows = (r1 - t0 < kTileRows) ? r1 - t0 : kTileRows;
+  // tiles of 1,024 rows from the row that holds nonzero a0 on, until one reaches the end of the share
+  for (uint32_t t0 = a0 < a1 ? row_of_nonzero(indptr, n_row, a0) : n_row; t0 < n_row; t0 += kTileRows) {
+    const uint32_t rows = (n_row - t0 < kTileRows) ? n_row - t0 : kTileRows;
     __syncthreads();  // the previous tile is done with s_ptr / s_v (and s_cnt is cleared)
     if (tid < rows) s_v[tid] = vec[t0 + tid];
     if (tid <= rows) s_ptr[tid] = indptr[t0 + tid];
     if (tid == 0 && rows == kTileRows) s_ptr[kTileRows] = indptr[t0 + kTileRows];
     __syncthreads();
-    const uint32_t j0 = s_ptr[0], j1 = s_ptr[rows];
+    const uint32_t tile_end = s_ptr[rows];
+    const uint32_t j0 = s_ptr[0] > a0 ? s_ptr[0] : a0, j1 = tile_end < a1 ? tile_end : a1;
     for (uint32_t seg = j0; seg < j1; seg += kSegment) {
       const uint32_t seg_end = (j1 - seg < kSegment) ? j1 : seg + kSegment;
       // A lane takes U consecutive nonzeros of a round: one request for their columns and one for their
@@ -269,6 +301,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
         }
       }
     }
+    if (tile_end >= a1) break;
   }
   if (tid < n_win) {
     const uint32_t c = s_total[tid];
@@ -323,17 +356,7 @@ __global__ __launch_bounds__(kBinThreads) void flat_window_kernel(
   };
 
   if (a < b) {
-    // the row that holds nonzero a: the last r with indptr[r] <= a (every thread searches: uniform)
-    uint32_t t0 = 0;
-    {
-      uint32_t lo = 0, hi = n_row - 1u;
-      while (lo < hi) {
-        const uint32_t mid = lo + ((hi - lo + 1u) >> 1);
-        if (indptr[mid] <= a) lo = mid;
-        else hi = mid - 1u;
-      }
-      t0 = lo;
-    }
+    uint32_t t0 = row_of_nonzero(indptr, n_row, a);  // the row that holds nonzero a
     for (;;) {
       const uint32_t rows = (n_row - t0 < kTileRows) ? n_row - t0 : kTileRows;
       __syncthreads();  // the previous tile is done with s_ptr / s_v (and the window is cleared)
@@ -420,12 +443,13 @@ __global__ __launch_bounds__(256) void sum_windows_kernel(const double *__restri
 // grid = n_win * slices * parts; workgroup (b, q, s) adds window b's pairs of producers
 // [s * P / parts, ...) that fall into slice q of the window (slices = 2^(shift - lds_shift): a window
 // wider than the 2^lds_shift accumulators in LDS is added slice by slice, every slice reading the pairs).
-// Bin of (producer p, window b): derived from indptr as in bin_products_kernel, or, with
-// indptr == nullptr, the uniform layout pairs + (p * n_win + b) * uniform_cap.
+// Bin of (producer p, window b): derived from the producers' shares of the nonzeros as in bin_products_kernel,
+// or, with indptr == nullptr, the uniform layout pairs + (p * n_win + b) * uniform_cap.
 template <typename F, bool PACKED>
 __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *__restrict__ indptr,
                                                                F *__restrict__ y, uint32_t n_row, uint32_t n_col,
-                                                               uint32_t rows_per, uint32_t n_win, uint32_t shift,
+                                                               uint32_t chunk_lo, uint32_t chunk_nnz, uint32_t last,
+                                                               uint32_t n_win, uint32_t shift,
                                                                uint32_t lds_shift, uint32_t parts,
                                                                uint32_t producers,
                                                                const void *__restrict__ pairs_raw,
@@ -448,6 +472,7 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
   const uint32_t width = (n_col - c0 < (1u << lds_shift)) ? n_col - c0 : (1u << lds_shift);
   for (uint32_t i = tid; i < width; i += kBinThreads) window[i] = 0.0;
   __syncthreads();
+  const uint32_t nnz_all = indptr != nullptr ? indptr[n_row] : 0u;
   const uint32_t p_lo = static_cast<uint32_t>(static_cast<uint64_t>(s) * producers / parts);
   const uint32_t p_hi = static_cast<uint32_t>(static_cast<uint64_t>(s + 1) * producers / parts);
   // A wave takes the bins of the producers p_lo + wave, + kWaves, ... one after the other, in steps of
@@ -487,10 +512,9 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
         if (p64 < p_hi) {
           const uint32_t p = static_cast<uint32_t>(p64);
           if (indptr != nullptr) {
-            uint32_t r0, r1;
-            producer_rows(p, rows_per, n_row, &r0, &r1);
-            const uint32_t a0 = indptr[r0], a1 = indptr[r1];
-            my_off = region_base(a0 - indptr[0], p, n_win) + static_cast<uint64_t>(b) * region_cap(a0, a1, n_win);
+            uint32_t chunk_first;
+            const NonzeroShare share = producer_share(nnz_all, chunk_lo, chunk_nnz, last != 0, producers, p, &chunk_first);
+            my_off = region_base(share.a - chunk_first, p, n_win) + static_cast<uint64_t>(b) * region_cap(share.a, share.b, n_win);
           } else {
             my_off = (static_cast<uint64_t>(p) * n_win + b) * uniform_cap;
           }
@@ -1095,11 +1119,8 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
   const uint32_t shift = bin_window_shift(n_col);
   const uint32_t n_win = div_up(n_col, 1u << shift);
   const unsigned num_cu = static_cast<unsigned>(device_info().num_cu);
-  // two producer workgroups per CU, at least 64 rows each
-  uint32_t producers = 2u * num_cu;
-  if (producers > div_up(n_row, 64)) producers = div_up(n_row, 64);
-  const uint32_t rows_per = div_up(n_row, producers);
-  producers = div_up(n_row, rows_per);
+  // two producer workgroups per CU, each an equal share of the nonzeros
+  const uint32_t producers = 2u * num_cu;
   const uint32_t lds_shift = bin_lds_shift(shift);
   const uint32_t slices = 1u << (shift - lds_shift);
   uint32_t parts = num_cu / (n_win * slices);
@@ -1134,26 +1155,25 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
   fill_zero(stream, y, n_col);
   auto bin_kernel = heter ? (packed ? bin_products_kernel<F, true, true> : bin_products_kernel<F, true, false>)
                           : (packed ? bin_products_kernel<F, false, true> : bin_products_kernel<F, false, false>);
-  // The rows are taken in chunks whose pairs (about kChunkPairBytes) stay in the 256 MB cache in front of the
+  // The nonzeros are taken in chunks whose pairs (about kChunkPairBytes) stay in the 256 MB cache in front of the
   // memory between the kernel that writes them and the kernel that reads them: at 1e8 nonzeros three chunks
   // take 535 us, one 590, six 630 (every chunk is a pair of launches that start and drain on their own, and
   // one more float32 addition per output element).
   uint32_t chunks = div_up(static_cast<uint64_t>(nnz) * bin_pair_bytes<F>(packed), kChunkPairBytes);
   if (chunks > kMaxChunks) chunks = kMaxChunks;
   if (chunks == 0) chunks = 1;
-  const uint32_t chunk_rows = div_up(n_row, chunks);
-  for (uint32_t rb = 0; rb < n_row; rb += chunk_rows) {
-    const uint32_t rows = n_row - rb < chunk_rows ? n_row - rb : chunk_rows;
-    uint32_t prods = 2u * num_cu;
-    if (prods > div_up(rows, 64)) prods = div_up(rows, 64);
-    const uint32_t rper = div_up(rows, prods);
-    prods = div_up(rows, rper);
-    uint32_t pts = parts > prods ? prods : parts;
-    hipLaunchKernelGGL(bin_kernel, dim3(prods), dim3(kBinThreads), 0, stream, data, indices, indptr + rb, vec + rb, y, rows,
-                       rper, n_win, shift, pairs, static_cast<uint64_t>(n_pairs), counts);
-    hipLaunchKernelGGL(add_kernel, dim3(n_win * slices * pts), dim3(kBinThreads), lds, stream, indptr + rb, y, rows, n_col,
-                       rper, n_win, shift, lds_shift, pts, prods, static_cast<const void *>(pairs),
-                       static_cast<uint64_t>(n_pairs), counts, 0u, static_cast<uint32_t *>(nullptr));
+  const uint32_t chunk_nnz = (div_up(nnz, chunks) + 3u) & ~3u;
+  for (uint32_t c = 0; c < chunks; ++c) {
+    const uint64_t lo = static_cast<uint64_t>(c) * chunk_nnz;
+    if (lo >= nnz && c != 0) break;
+    const uint32_t last = (c + 1 == chunks || lo + chunk_nnz >= nnz) ? 1u : 0u;
+    hipLaunchKernelGGL(bin_kernel, dim3(producers), dim3(kBinThreads), 0, stream, data, indices, indptr, vec, y, n_row,
+                       static_cast<uint32_t>(lo), chunk_nnz, last, n_win, shift, pairs, static_cast<uint64_t>(n_pairs), counts);
+    hipLaunchKernelGGL(add_kernel, dim3(n_win * slices * parts), dim3(kBinThreads), lds, stream, indptr, y, n_row, n_col,
+                       static_cast<uint32_t>(lo), chunk_nnz, last, n_win, shift, lds_shift, parts, producers,
+                       static_cast<const void *>(pairs), static_cast<uint64_t>(n_pairs), counts, 0u,
+                       static_cast<uint32_t *>(nullptr));
+    if (last) break;
   }
   return check_launch(target);
 }
@@ -1182,7 +1202,7 @@ bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_o
   if (parts > producers) parts = producers;
   const uint64_t n_pairs = static_cast<uint64_t>(producers) * n_win * cap;
   hipLaunchKernelGGL(add_kernel, dim3(n_win * slices * parts), dim3(kBinThreads), lds, stream,
-                     static_cast<const uint32_t *>(nullptr), y, 0u, n_out, 0u, n_win, shift, lds_shift, parts, producers,
+                     static_cast<const uint32_t *>(nullptr), y, 0u, n_out, 0u, 0u, 0u, n_win, shift, lds_shift, parts, producers,
                      pairs, n_pairs, counts, cap, reset);
   return check_launch(target);
 }

@@ -431,13 +431,17 @@ def test_transposed_csr_matvec_wide_output_sorted_scatter(cuda, oracle_mod, dtyp
   rng = np.random.default_rng(41)
   for n_row, n_col, mean, long_row in ((30_000, 300_000, 50, 0), (50_000, 400_000, 25, 250_000),
                                        (1500, 2_000_000, 1000, 0), (200_000, 140_000, 8, 0),
+                                       # (fewer rows than producer workgroups: these take shares of the nonzeros, not rows)
+                                       (40, 150_000, 50_000, 0), (12, 100_000, 0, 99_000),
                                        # (above 2^21 columns: windows wider than their LDS accumulators, added in slices)
                                        (4000, 5_000_001, 300, 0),
                                        # (above 2^23 columns: positions within a window beyond 16 bits, whole pairs)
                                        (3000, 9_000_000, 400, 0)):
     counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
     if long_row:
-      counts[7] = long_row
+      counts[7 % n_row] = long_row
+      if n_row < 16:
+        counts[:] = long_row
     indices, indptr = synth.counted_csr(counts, n_col, seed=n_row)
     assert indices.shape[0] >= 1 << 20
     data = rng.random(indices.shape[0]).astype(dtype)
