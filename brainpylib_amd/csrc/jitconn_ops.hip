@@ -580,12 +580,20 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
   // Many pairs: bins (also for a narrow output: seeding ahead and the even spread of the streams pay).  The number of pairs is n_in * n_out * p for a
   // dense input; for events it depends on the activity, which the host does not know: bins are sized
   // for one column in eight being active (fuller bins overflow into direct atomics) and used when
-  // one active column in a hundred already means half a million pairs.
+  // one active column in a hundred already means a hundred thousand pairs (10,000 x 10,000 with
+  // conn_prob 0.1: 44, 54 and 61 us at 0.1, 1 and 20 % activity; without bins 40, 44 and 152 us).
   const uint32_t shift = bin_window_shift(n_out);
   const uint32_t n_win = div_up(n_out, 1u << shift);
   const double p_conn = -std::expm1(log_p);
   const double full = static_cast<double>(n_in) * static_cast<double>(n_out) * p_conn;
-  if (n_win <= kBinMaxWindows && full >= (IN == kInDense ? 1048576.0 : 5.0e7)) {
+  const bool bins = n_win <= kBinMaxWindows && full >= (IN == kInDense ? 1048576.0 : 1.0e7);
+  // Event input and fewer pairs: the same list of active columns and the same seeding ahead on the vector unit, but
+  // the walk adds its pairs to `out` with atomics.  (A wave that seeds its own stream spends 2 us of the CU's one
+  // scalar unit on it: with 200,000 active columns of ten synapses each the walk without a list took 1.2 ms.)
+  const bool listed = !bins && IN == kInEvent && n_in >= 2048;
+  if (bins || listed) {
+    const uint32_t n_win = bins ? div_up(n_out, 1u << bin_window_shift(n_out)) : 1u;  // (no bins: every pair overflows)
+    const uint32_t shift = bins ? bin_window_shift(n_out) : 31u;
     uint32_t producers = 2u * static_cast<uint32_t>(device_info().num_cu);
     if (producers > div_up(n_in, kColBinThreads / kWave)) producers = div_up(n_in, kColBinThreads / kWave);
     auto round_up = [](size_t v) { return (v + 255) / 256 * 256; };
@@ -605,6 +613,7 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
       if (IN == kInEvent || group == 1 || pair_bytes <= kColBinBytesMax) break;
       group = (group + 1u) / 2u;
     }
+    if (!bins) cap_d = 0.0, pair_bytes = 0;
     const size_t count_bytes = round_up(static_cast<size_t>(n_win) * producers * sizeof(uint32_t));
     const uint32_t seeded_max = n_in < kSeedChunk ? n_in : kSeedChunk;
     const size_t state_bytes = round_up(static_cast<size_t>(seeded_max) * kMtN * 4);
@@ -654,6 +663,10 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
               in_bins = 0;
             }
           }
+        }
+        if (!bins) {
+          fill_zero(stream, list_count, 1u);  // (the list's counter goes back to zero for the next call)
+          return;
         }
         if (add_uniform_bins<T1>("jitconn column walk", stream, out, n_out, shift, producers, cap, pairs, counts, list_count))
           return;

@@ -109,6 +109,31 @@ def test_index_sets_bit_exact_via_integer_probes(cuda, oracle_mod, shape, p):
       assert np.array_equal(got, want), (shape, p, col_walk)
 
 
+@pytest.mark.parametrize("n_out,n_in,p", [(3000, 1500, 0.05), (5000, 4000, 0.05), (9000, 40_000, 0.02),
+                                          (20_000, 30_000, 0.03)])
+def test_event_column_walk_in_every_regime(cuda, oracle_mod, n_out, n_in, p):
+  # few input columns: every wave lists and seeds its own; from 2,048 columns on: a device list of the active
+  # columns and generators seeded ahead, the pairs added with atomics; from ten million possible pairs on:
+  # through bins.  Unit weight: the outputs are synapse counts, equal to the oracle's bit for bit, at little
+  # and at much activity, twice in a row (the list's counter must be back at zero).
+  lp = oracle_mod.log_p_of(p)
+  rng = np.random.default_rng(n_in)
+  for rate in (0.004, 0.3):
+    ev = rng.random(n_in) < rate
+    want = oracle_mod.jitconn_matvec(ev, log_p=lp, seed=99, n_row=n_out, n_col=n_in, col_walk=True, dense=False,
+                                     per_stream_seed=True)
+    for _ in range(2):
+      got = kernel_call(ev, w_kind="homo", log_p=lp, seed=99, n_row=n_out, n_col=n_in, col_walk=True, dense=False)
+      assert np.array_equal(got, want), (n_out, n_in, p, rate)
+  # uniform weights and float events: sums of a few terms in any order
+  evf = (rng.random(n_in) < 0.05).astype(np.float32)
+  want = oracle_mod.jitconn_matvec(evf, log_p=lp, seed=5, n_row=n_out, n_col=n_in, col_walk=True, dense=False,
+                                   per_stream_seed=True, w_kind="uniform", w_a=-1.0, w_b=2.0)
+  got = kernel_call(evf, w_kind="uniform", w_a=-1.0, w_b=2.0, log_p=lp, seed=5, n_row=n_out, n_col=n_in, col_walk=True,
+                    dense=False)
+  np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
 @pytest.mark.parametrize("n_in", [320_000, 1_500_000, 5_000_000])
 def test_row_walk_with_a_two_level_event_bitmap(cuda, oracle_mod, n_in):
   # more inputs than the 38 KB of LDS the row walk gives to a bitmap cover (311,296): a coarse
