@@ -128,6 +128,11 @@ bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint
                        uint32_t list_cap, void *scratch, size_t scratch_bytes,
                        const uint32_t *active_colbase = nullptr);
 
+// mt19937 states of the generator streams seed + first .. seed + first + count - 1, 624 words each, seeded on
+// the vector unit, 64 streams per wave (jitconn_ops.hip).  A wave that seeds the stream it walks holds its
+// CU's one scalar unit for about 2 us.
+void jitconn_seed_streams(hipStream_t stream, uint32_t seed, uint32_t first, uint32_t count, uint32_t *states);
+
 // Second half of the coarse-sorted scatter for producers other than the CSR one: adds bins laid
 // out uniformly, bin (p, b) = pairs + (p * n_win + b) * cap with counts[b * producers + p]
 // BinPair<F> entries (bins.h; counts above cap mean cap), n_win = ceil(n_out / 2^shift), into the

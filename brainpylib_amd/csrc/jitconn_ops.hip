@@ -768,6 +768,11 @@ __global__ __launch_bounds__(256) void check_log2_kernel(unsigned long long *__r
 }
 
 }  // namespace
+
+void jitconn_seed_streams(hipStream_t stream, uint32_t seed, uint32_t first, uint32_t count, uint32_t *states) {
+  launch_seed_streams(stream, seed, first, count, states);
+}
+
 }  // namespace bpl
 
 using namespace bpl;

@@ -342,6 +342,19 @@ def test_matmat_against_oracle_and_vmapped_matvec(cuda, oracle_mod, m, dtype):
     assert torch.allclose(got_t[i], yi, rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("n", [32_768, 140_000])
+def test_matmat_with_generators_seeded_ahead(cuda, oracle_mod, n):
+  # from 32,768 columns of M on their generators are seeded ahead by a kernel of its own, 131,072 at a time
+  # (140,000: two chunks, the second one short); uniform weights are bit-exact as with any other size
+  m, k, seed, p = 9, 60, 11, 0.1
+  X = np.random.default_rng(n).standard_normal((m, k)).astype(np.float32)
+  lp = oracle_mod.log_p_of(p)
+  want = oracle_mod.jitconn_matmat(X, w_kind="uniform", w_a=-0.5, w_b=1.5, log_p=lp, seed=seed, n=n)
+  for _ in range(2):
+    got = bpl.matmat_prob_conn_uniform_weight(X, w_low=-0.5, w_high=1.5, conn_prob=p, shape=(k, n), seed=seed).cpu().numpy()
+    assert got.shape == (m, n) and np.array_equal(got, want)
+
+
 def test_config_jitconn_matmat_full_size(cuda, oracle_mod):
   # 10,000 x 10,000 implicit matrix, conn_prob 0.1, N(0, 0.01^2) from seed 7, times B[10000, 128]:
   # out = (B^T @ M)^T in the reference's orientation (X = B^T, m = 128).
