@@ -348,6 +348,13 @@ def main():
       bpl.csr_matvec(md["data"], md["indices"], md["indptr"], md["vector"], shape=m["shape"])
     for _ in range(3):
       bpl.cusparse_csr_matvec(md["data"], md["indices"], md["indptr"], md["vector"], shape=m["shape"], transpose=True)
+    # the transposed product whose output fits one float64 window in LDS: 1,000,000 x 16,000, 50 per row
+    ix_n, ip_n = synth.counted_csr(np.full(1_000_000, 50), 16_000, seed=29)
+    rng_n = np.random.default_rng(23)
+    dev_n = [torch.from_numpy(a_).to(dev) for a_ in (rng_n.random(ix_n.shape[0], dtype=np.float32), ix_n, ip_n,
+                                                      rng_n.standard_normal(1_000_000).astype(np.float32))]
+    for _ in range(3):
+      bpl.cusparse_csr_matvec(*dev_n, shape=(1_000_000, 16_000), transpose=True)
     lib = load_kernels()
     cu = torch.cuda.get_device_properties(dev).multi_processor_count
     out = torch.zeros(cu * 2 * 1024, dtype=torch.float32, device=dev)
@@ -668,6 +675,31 @@ def main():
     extra["csr_matvec_2e7_vector_in_lds"] = dict(stats(dur_s), gsop_per_s=ix_s.shape[0] / (dur_s.mean() * 1e-3) / 1e9,
                                                  algorithmic_gb_per_s=8.0 * ix_s.shape[0] / (dur_s.mean() * 1e-3) / 1e9)
     log("csr_matvec 2e7, vector in LDS: %s" % extra["csr_matvec_2e7_vector_in_lds"])
+    # the same matrix transposed: the output (19,000 columns) fits two float64 windows in LDS; and 1,000,000 x 16,000
+    # with 50 per row, whose output fits one (every workgroup walks an equal share of the nonzeros into its window)
+    u_s = rng_s.standard_normal(200_000).astype(np.float32)
+    u_dev = torch.from_numpy(u_s).to(dev)
+    got = bpl.cusparse_csr_matvec(dev_s[0], dev_s[1], dev_s[2], u_dev, shape=(200_000, 19_000), transpose=True).cpu().numpy()
+    check(got, oracle.csr_matvec(d_s, ix_s, ip_s, u_s, shape=(200_000, 19_000), transpose=True),
+          "csr_matvec transposed, two LDS windows",
+          oracle.csr_matvec(d_s, ix_s, ip_s, np.abs(u_s), shape=(200_000, 19_000), transpose=True))
+    ix_n, ip_n = synth.counted_csr(np.full(1_000_000, 50), 16_000, seed=29)
+    d_n = rng_s.random(ix_n.shape[0], dtype=np.float32)
+    u_n = rng_s.standard_normal(1_000_000).astype(np.float32)
+    dev_n = [torch.from_numpy(a_).to(dev) for a_ in (d_n, ix_n, ip_n, u_n)]
+    got = bpl.cusparse_csr_matvec(*dev_n, shape=(1_000_000, 16_000), transpose=True).cpu().numpy()
+    check(got, oracle.csr_matvec(d_n, ix_n, ip_n, u_n, shape=(1_000_000, 16_000), transpose=True),
+          "csr_matvec transposed, one LDS window",
+          oracle.csr_matvec(d_n, ix_n, ip_n, np.abs(u_n), shape=(1_000_000, 16_000), transpose=True))
+    dur_n, _ = time_calls(lambda: bpl.cusparse_csr_matvec(*dev_n, shape=(1_000_000, 16_000), transpose=True),
+                          max(20, args.steps // 4), 5)
+    bytes_n = 8.0 * ix_n.shape[0] + 4.0 * (1_000_001 + 1_000_000 + 16_000)
+    extra["csr_matvec_transposed_5e7_output_in_lds"] = dict(
+      stats(dur_n), gsop_per_s=ix_n.shape[0] / (dur_n.mean() * 1e-3) / 1e9,
+      roofline=dict(bound="hbm", unit="GB/s", achieved=bytes_n / (dur_n.mean() * 1e-3) / 1e9, peak=HBM_PEAK_GBS,
+                    frac=bytes_n / (dur_n.mean() * 1e-3) / 1e9 / HBM_PEAK_GBS))
+    log("csr_matvec transposed 5e7, output in LDS: %s" % extra["csr_matvec_transposed_5e7_output_in_lds"])
+    del dev_n, ix_n, ip_n, d_n, u_n
     del dev_s
     # the same 1,000,000 x 1,000,000 matrix (100 nonzeros per row) driven by events, 1 % and 5 % of
     # the rows active: the shape of a million-neuron network's synaptic update (output far wider than LDS)
