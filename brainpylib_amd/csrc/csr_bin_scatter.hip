@@ -1,21 +1,24 @@
-// Transposed CSR matrix times vector through coarse sorting: y[c] = sum_j v[row(j)] * data[j] over
-// the nonzeros j of column c.  First half of the file: dense vector, every row contributes, output
-// (hundreds of thousands of columns or more) far larger than LDS.  Second half: event vector, only
-// the listed active rows contribute (from 8,192 columns).  One random global atomic per nonzero
-// retires at about 21 G/s on this device; instead the products are first sorted coarsely:
+// Transposed CSR matrix times vector: y[c] = sum_j v[row(j)] * data[j] over the nonzeros j of column c.
+// Three parts: a dense vector and an output far larger than LDS (hundreds of thousands of columns or more):
+// coarse sorting; a dense vector and an output of one or two float64 windows of LDS: a flat walk into the
+// windows, no sorting (flat_window_kernel, in the middle of the file); an event vector, where only the listed
+// active rows contribute (from 8,192 columns): coarse sorting again (last part).  One random global atomic per
+// nonzero retires at about 21 G/s on this device; instead the products are first sorted coarsely:
 //
-//   bin kernel     persistent producer workgroups walk their rows, form (column, product)
-//                  pairs and append each pair to the bin of its output window (a power of two of
-//                  columns, at most 16,384, chosen so that there are about 64 windows),
-//                  in a region of scratch memory private to (producer, window): no global
-//                  atomics, the position comes from a counter in LDS (32-bit integer LDS
-//                  atomics are cheap even when lanes meet).  A pair that does not fit its
-//                  region (a very uneven matrix) is added to y directly instead.
+//   bin kernel     persistent producer workgroups take equal shares of the nonzeros (whatever rows they
+//                  belong to), form (position in window, product) pairs and append each pair to the bin
+//                  of its output window (a power of two of columns, at most 16,384, chosen so that
+//                  there are about 64 windows), in a region of scratch memory private to (producer,
+//                  window): no global atomics, the position comes from a counter in LDS (32-bit integer
+//                  LDS atomics are cheap even when lanes meet).  A pair that does not fit its region (a
+//                  share whose columns crowd into few windows) is added to y directly instead.
 //   window kernel  workgroup (window, part) adds the pairs of its window from a share of the
 //                  producers into a float64 window in LDS (64-bit LDS float adds run at
 //                  several lanes per clock) and adds the window to the zeroed y, contiguous.
 //
-// The arrays are read once, the pairs written and read once: HBM bound instead of atomic bound.
+// The arrays are read once, the pairs (6 bytes each: the product, and the position as 16 bits in an array of
+// its own) written and read once, in chunks that stay in the cache in front of the memory: HBM bound instead
+// of atomic bound.
 #include "bins.h"
 #include "common.h"
 #include "repeated_sum.h"
@@ -29,7 +32,7 @@ constexpr uint32_t kMaxWindows = kBinMaxWindows;
 constexpr uint32_t kRegionSlack = 128;    // pairs a region holds beyond 5/4 of its even share
 constexpr uint32_t kRegionSpacing = kRegionSlack + 8;  // (regions begin and end at multiples of 4 pairs)
 
-// Where producer `p`, whose rows hold nonzeros [a0, a1) counted from the first row of the launch, keeps
+// Where producer `p`, whose share is the nonzeros [a0, a1) counted from the first nonzero of the launch, keeps
 // the pairs of window b: region_base + b * cap, both multiples of 4 pairs (16-byte loads of the products).
 // Both kernels evaluate the same expressions.
 __device__ __forceinline__ uint32_t region_cap(uint32_t a0, uint32_t a1, uint32_t n_win) {
