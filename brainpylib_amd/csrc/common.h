@@ -133,6 +133,20 @@ bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint
 // CU's one scalar unit for about 2 us.
 void jitconn_seed_streams(hipStream_t stream, uint32_t seed, uint32_t first, uint32_t count, uint32_t *states);
 
+// Event input and an output of at most 8,192 columns: the listed active rows' nonzeros are walked flat into
+// one window in LDS per workgroup (csr_bin_scatter.hip).  `counters`: the stream's counters, [0] the number
+// of listed rows (set back to zero by the second kernel), [1] used between the two kernels.  `scratch`:
+// window_event_scatter_bytes() of device memory.  y need not be zeroed.  false (nothing enqueued) if it
+// cannot run.
+template <typename F>
+bool window_event_scatter_usable(uint32_t n_row, uint32_t n_col);
+template <typename F>
+size_t window_event_scatter_bytes(uint32_t n_col);
+template <typename F>
+bool window_event_scatter(hipStream_t stream, const F *data, bool heter, const uint32_t *indices, const uint32_t *indptr,
+                          F *y, uint32_t n_row, uint32_t n_col, uint32_t *counters, const uint2 *active_list,
+                          uint32_t list_cap, void *scratch, size_t scratch_bytes);
+
 // Second half of the coarse-sorted scatter for producers other than the CSR one: adds bins laid
 // out uniformly, bin (p, b) = pairs + (p * n_win + b) * cap with counts[b * producers + p]
 // BinPair<F> entries (bins.h; counts above cap mean cap), n_win = ceil(n_out / 2^shift), into the

@@ -424,23 +424,45 @@ __global__ __launch_bounds__(kBinThreads) void flat_window_kernel(
   for (uint32_t i = tid; i < width; i += kBinThreads) mine[i] = window[i];
 }
 
-// y[c] = the workgroups' windows added in the order of the workgroups, in float64, rounded once
-template <typename F>
-__global__ __launch_bounds__(256) void sum_windows_kernel(const double *__restrict__ partial, F *__restrict__ y,
-                                                          uint32_t n_col, uint32_t groups) {
-  const uint32_t c = blockIdx.x * 256u + threadIdx.x;
-  if (c >= n_col) return;
-  double acc = 0.0;
-  uint32_t g = 0;
-  for (; g + 4 <= groups; g += 4) {  // (four loads in flight; the additions stay in order)
-    const double a0 = partial[static_cast<size_t>(g) * n_col + c];
-    const double a1 = partial[static_cast<size_t>(g + 1) * n_col + c];
-    const double a2 = partial[static_cast<size_t>(g + 2) * n_col + c];
-    const double a3 = partial[static_cast<size_t>(g + 3) * n_col + c];
-    acc = (((acc + a0) + a1) + a2) + a3;
+// y[c] = the sum of the workgroups' windows in a fixed order, in float64, rounded once.  A workgroup takes 32
+// columns; 32 threads per column add every 32nd window, four loads in flight, and their sums are added in
+// LDS (one thread per column through all the windows is a chain of hundreds of round trips).
+constexpr uint32_t kSumCols = 32, kSumSlices = 32;
+template <typename S, typename A>
+__device__ __forceinline__ S sum_windows_of_column(const A *__restrict__ partial, uint32_t n_col, uint32_t groups,
+                                                   bool *mine) {
+  __shared__ S s_part[kSumSlices][kSumCols + 1];
+  const uint32_t lc = threadIdx.x % kSumCols, slice = threadIdx.x / kSumCols;
+  const uint32_t c = blockIdx.x * kSumCols + lc;
+  S acc = S(0);
+  if (c < n_col) {
+    const A *col = partial + c;
+    uint32_t g = slice;
+    for (; g + 3u * kSumSlices < groups; g += 4u * kSumSlices) {
+      const A a0 = col[static_cast<size_t>(g) * n_col], a1 = col[static_cast<size_t>(g + kSumSlices) * n_col];
+      const A a2 = col[static_cast<size_t>(g + 2u * kSumSlices) * n_col], a3 = col[static_cast<size_t>(g + 3u * kSumSlices) * n_col];
+      acc = (((acc + a0) + a1) + a2) + a3;
+    }
+    for (; g < groups; g += kSumSlices) acc += col[static_cast<size_t>(g) * n_col];
   }
-  for (; g < groups; ++g) acc += partial[static_cast<size_t>(g) * n_col + c];
-  y[c] = static_cast<F>(acc);
+  s_part[slice][lc] = acc;
+  __syncthreads();
+  S total = S(0);
+  *mine = slice == 0 && c < n_col;
+  if (*mine) {
+#pragma unroll
+    for (uint32_t k = 0; k < kSumSlices; ++k) total += s_part[k][lc];
+  }
+  return total;
+}
+
+template <typename F>
+__global__ __launch_bounds__(kSumCols * kSumSlices) void sum_windows_kernel(const double *__restrict__ partial,
+                                                                            F *__restrict__ y, uint32_t n_col,
+                                                                            uint32_t groups) {
+  bool mine;
+  const double total = sum_windows_of_column<double, double>(partial, n_col, groups, &mine);
+  if (mine) y[blockIdx.x * kSumCols + threadIdx.x % kSumCols] = static_cast<F>(total);
 }
 
 // grid = n_win * slices * parts; workgroup (b, q, s) adds window b's pairs of producers
@@ -841,6 +863,131 @@ __global__ __launch_bounds__(kBinThreads) __attribute__((amdgpu_num_sgpr(80))) v
   }
 }
 
+// ---- event input, one output window ----------------------------------------------------------------
+// Outputs of at most 8,192 columns and a list of active rows: no sorting, the producers' flat walk over the
+// listed rows' nonzeros adds straight into a window in LDS (float64 for weights; 32-bit synapse counts for a
+// homogeneous weight, whose sum is formed from the count as everywhere), two workgroups per CU, no barrier
+// inside a tile of 1,024 listed rows.  The windows of the workgroups that took part go to scratch memory
+// and a second kernel adds them in a fixed order.  (The window kernel of csr_ops.hip hands whole rows to
+// waves, one after the other: 1,000,000 rows of 100 into 4,000 columns at 5 % events 76 us, this one 38.)
+constexpr uint32_t kWindowEventMaxCols = 8192;
+
+// workgroups that take part: one per kPairsPerProducer active nonzeros (estimated from the mean row length)
+__device__ __forceinline__ uint32_t window_event_producers(uint32_t total, uint32_t nnz, uint32_t n_row, uint32_t launched) {
+  const uint64_t want = (static_cast<uint64_t>(total) * (nnz / n_row + 1u) + kPairsPerProducer - 1u) / kPairsPerProducer;
+  return want < 1u ? 1u : want > launched ? launched : static_cast<uint32_t>(want);
+}
+
+template <typename F, bool HETER>
+__global__ __launch_bounds__(kBinThreads) void active_rows_window_kernel(
+    const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
+    uint32_t n_row, uint32_t n_col, const uint32_t *__restrict__ active_count, const uint2 *__restrict__ active_list,
+    uint32_t list_cap, void *__restrict__ partial, uint32_t *__restrict__ groups_out) {
+  using A = typename std::conditional<HETER, double, uint32_t>::type;  // a window's accumulators
+  extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
+  A *window = reinterpret_cast<A *>(smem_raw);
+  __shared__ uint32_t s_ptr[kTileRows + 1];     // nonzeros of the tile's rows before row k
+  __shared__ uint32_t s_start[kTileRows];       // first nonzero of row k in the matrix
+  __shared__ uint32_t s_hint[kBinThreads + 1];
+  __shared__ uint32_t s_wave[kBinThreads / kWave];
+  constexpr int U = 4;
+  constexpr uint32_t kRound = U * kBinThreads;
+  const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const uint32_t total = active_count[0] < list_cap ? active_count[0] : list_cap;  // (never beyond the list)
+  const uint32_t producers = window_event_producers(total, indptr[n_row], n_row, gridDim.x);
+  const uint32_t p = blockIdx.x;
+  if (p == 0 && tid == 0) groups_out[0] = producers;  // (for the kernel that adds the windows)
+  if (p >= producers) return;
+  for (uint32_t i = tid; i < n_col; i += kBinThreads) window[i] = A(0);
+  const uint32_t lo = static_cast<uint32_t>(static_cast<uint64_t>(p) * total / producers);
+  const uint32_t hi = static_cast<uint32_t>(static_cast<uint64_t>(p + 1) * total / producers);
+
+  auto row_of = [&](uint32_t j, uint32_t a, uint32_t b) {  // largest k in [a, b] with s_ptr[k] <= j
+    while (a < b) {
+      const uint32_t mid = (a + b + 1u) >> 1;
+      if (s_ptr[mid] <= j) a = mid;
+      else b = mid - 1u;
+    }
+    return a;
+  };
+
+  for (uint32_t t0 = lo; t0 < hi; t0 += kTileRows) {
+    const uint32_t rows = (hi - t0 < kTileRows) ? hi - t0 : kTileRows;
+    __syncthreads();  // the previous tile is done with s_ptr / s_start (and the window is cleared)
+    uint2 e = make_uint2(0u, 0u);
+    if (tid < rows) e = active_list[t0 + tid];
+    const uint32_t incl = wave_inclusive_scan_u32(e.y);
+    if (lane == kWave - 1) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t before = 0;
+    for (uint32_t w = 0; w < wave; ++w) before += s_wave[w];
+    if (tid < rows) s_ptr[tid] = before + incl - e.y, s_start[tid] = e.x;
+    if (tid == rows - 1u) s_ptr[rows] = before + incl;
+    __syncthreads();
+    const uint32_t j1 = s_ptr[rows];  // the tile's nonzeros, numbered from 0 (listed rows are never empty)
+    for (uint32_t seg = 0; seg < j1; seg += kSegment) {
+      const uint32_t seg_end = (j1 - seg < kSegment) ? j1 : seg + kSegment;
+      __syncthreads();  // the previous segment is done with s_hint
+      {
+        const uint32_t j = seg + (tid << kHintShift);
+        s_hint[tid] = (j < seg_end) ? row_of(j, 0u, rows - 1u) : rows - 1u;
+        if (tid == 0) s_hint[kBinThreads] = rows - 1u;
+      }
+      __syncthreads();
+      for (uint32_t jb = seg + tid; jb - tid < seg_end; jb += kRound) {
+        // where every nonzero of the lane lies (LDS only), then all the loads together
+        uint32_t at[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t j = jb + u * kBinThreads;
+          const uint32_t jc = j < seg_end ? j : seg_end - 1u;
+          const uint32_t q = (jc - seg) >> kHintShift;
+          const uint32_t k = row_of(jc, s_hint[q], s_hint[q + 1]);
+          at[u] = s_start[k] + (jc - s_ptr[k]);
+        }
+        uint32_t col[U];
+        F val[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          col[u] = indices[at[u]];
+          if (HETER) val[u] = data[at[u]];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (jb + u * kBinThreads < seg_end) {
+            if constexpr (HETER) atomicAdd(&window[col[u]], static_cast<double>(val[u]));
+            else atomicAdd(&window[col[u]], 1u);
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+  A *mine = static_cast<A *>(partial) + static_cast<size_t>(p) * n_col;
+  for (uint32_t i = tid; i < n_col; i += kBinThreads) mine[i] = window[i];
+}
+
+// y[c] = the sum of the windows of the workgroups that took part (their number: counters[1]), in a fixed order
+// (weights: in float64, rounded once; a homogeneous weight: the sum of as many additions of the weight as
+// the windows counted).  Sets the list's counter, counters[0], back to zero for the next call.
+template <typename F, bool HETER>
+__global__ __launch_bounds__(kSumCols * kSumSlices) void sum_active_windows_kernel(const void *__restrict__ partial,
+                                                                                   F *__restrict__ y, uint32_t n_col,
+                                                                                   uint32_t *__restrict__ counters,
+                                                                                   const F *__restrict__ data) {
+  using A = typename std::conditional<HETER, double, uint32_t>::type;
+  using S = typename std::conditional<HETER, double, uint64_t>::type;
+  const uint32_t groups = counters[1];
+  if (blockIdx.x == 0 && threadIdx.x == 0) counters[0] = 0u;
+  bool mine;
+  const S total = sum_windows_of_column<S, A>(static_cast<const A *>(partial), n_col, groups, &mine);
+  if (mine) {
+    const uint32_t c = blockIdx.x * kSumCols + threadIdx.x % kSumCols;
+    if constexpr (HETER) y[c] = static_cast<F>(total);
+    else y[c] = repeated_sum<F>(data[0], total);
+  }
+}
+
 // grid = n_win * slices * parts; workgroup (b, q, s) adds share s of window b's pairs (its 8 runs
 // taken as one sequence) to the zeroed y.  A window wider than the 2^lds_shift float64 accumulators
 // in LDS is cut into `slices` = 2^(shift - lds_shift) slices: the workgroups of slice q read the
@@ -1010,6 +1157,49 @@ inline uint64_t event_run_pairs(uint32_t n_row, uint32_t n_col) {
 }  // namespace
 
 template <typename F>
+bool window_event_scatter_usable(uint32_t n_row, uint32_t n_col) {
+  return n_col != 0 && n_col <= kWindowEventMaxCols && n_row != 0;
+}
+
+// scratch memory behind the list: the windows of two workgroups per CU
+template <typename F>
+size_t window_event_scatter_bytes(uint32_t n_col) {
+  return static_cast<size_t>(2u * static_cast<uint32_t>(device_info().num_cu)) * n_col * sizeof(double);
+}
+
+template <typename F>
+bool window_event_scatter(hipStream_t stream, const F *data, bool heter, const uint32_t *indices, const uint32_t *indptr,
+                          F *y, uint32_t n_row, uint32_t n_col, uint32_t *counters, const uint2 *active_list,
+                          uint32_t list_cap, void *scratch, size_t scratch_bytes) {
+  if (!window_event_scatter_usable<F>(n_row, n_col) || scratch_bytes < window_event_scatter_bytes<F>(n_col)) return false;
+  const unsigned grid = 2u * static_cast<unsigned>(device_info().num_cu);
+  const size_t lds = static_cast<size_t>(n_col) * (heter ? sizeof(double) : sizeof(uint32_t));
+  static thread_local bool attr_set[2] = {false, false};
+  if (!attr_set[heter]) {
+    const void *kernel = heter ? reinterpret_cast<const void *>(active_rows_window_kernel<F, true>)
+                               : reinterpret_cast<const void *>(active_rows_window_kernel<F, false>);
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(kWindowEventMaxCols * sizeof(double))) != hipSuccess) {
+      (void)hipGetLastError();
+      return false;
+    }
+    attr_set[heter] = true;
+  }
+  if (heter) {
+    hipLaunchKernelGGL((active_rows_window_kernel<F, true>), dim3(grid), dim3(kBinThreads), lds, stream, data, indices, indptr,
+                       n_row, n_col, static_cast<const uint32_t *>(counters), active_list, list_cap, scratch, counters + 1);
+    hipLaunchKernelGGL((sum_active_windows_kernel<F, true>), dim3(div_up(n_col, kSumCols)), dim3(kSumCols * kSumSlices), 0, stream,
+                       static_cast<const void *>(scratch), y, n_col, counters, data);
+  } else {
+    hipLaunchKernelGGL((active_rows_window_kernel<F, false>), dim3(grid), dim3(kBinThreads), lds, stream, data, indices, indptr,
+                       n_row, n_col, static_cast<const uint32_t *>(counters), active_list, list_cap, scratch, counters + 1);
+    hipLaunchKernelGGL((sum_active_windows_kernel<F, false>), dim3(div_up(n_col, kSumCols)), dim3(kSumCols * kSumSlices), 0, stream,
+                       static_cast<const void *>(scratch), y, n_col, counters, data);
+  }
+  return true;
+}
+
+template <typename F>
 bool bin_event_scatter_usable(uint32_t n_col) {
   const uint32_t n_win = div_up(n_col, 1u << event_window_shift(n_col));
   return n_win >= 2 && n_win <= kMaxWindows;
@@ -1102,7 +1292,7 @@ bool flat_window_scatter(const char *target, hipStream_t stream, const F *data, 
   }
   hipLaunchKernelGGL(kernel, dim3(shares * slices), dim3(kBinThreads), lds, stream, data, indices, indptr, vec, n_row,
                      n_col, slices, partial);
-  hipLaunchKernelGGL(sum_windows_kernel<F>, dim3(div_up(n_col, 256)), dim3(256), 0, stream,
+  hipLaunchKernelGGL(sum_windows_kernel<F>, dim3(div_up(n_col, kSumCols)), dim3(kSumCols * kSumSlices), 0, stream,
                      static_cast<const double *>(partial), y, n_col, shares);
   return check_launch(target);
 }
@@ -1215,6 +1405,14 @@ template bool add_uniform_bins<float>(const char *, hipStream_t, float *, uint32
 template bool add_uniform_bins<double>(const char *, hipStream_t, double *, uint32_t, uint32_t, uint32_t, uint32_t,
                                        const void *,
                                        const uint32_t *, uint32_t *);
+template bool window_event_scatter_usable<float>(uint32_t, uint32_t);
+template bool window_event_scatter_usable<double>(uint32_t, uint32_t);
+template size_t window_event_scatter_bytes<float>(uint32_t);
+template size_t window_event_scatter_bytes<double>(uint32_t);
+template bool window_event_scatter<float>(hipStream_t, const float *, bool, const uint32_t *, const uint32_t *, float *, uint32_t,
+                                          uint32_t, uint32_t *, const uint2 *, uint32_t, void *, size_t);
+template bool window_event_scatter<double>(hipStream_t, const double *, bool, const uint32_t *, const uint32_t *, double *,
+                                           uint32_t, uint32_t, uint32_t *, const uint2 *, uint32_t, void *, size_t);
 template bool bin_event_scatter_usable<float>(uint32_t);
 template bool bin_event_scatter_usable<double>(uint32_t);
 template size_t bin_event_scatter_bytes<float>(uint32_t, uint32_t);

@@ -1187,6 +1187,28 @@ void launch_scatter(const ScratchSource &src, const F *data, const uint32_t *ind
       bpl_clear_error();  // no scratch memory: the paths below need less or none
     }
   }
+  // Event input, a large matrix (its active rows go to a device list) and an output of one small window: the
+  // flat walk over the listed rows' nonzeros (csr_bin_scatter.hip).  (Not from a fixed arena: the walk below
+  // needs less scratch memory there.)
+  if (MODE == kEvent && !src.fixed() && n_row > 16 * kWinMaxRows && window_event_scatter_usable<F>(n_row, n_col)) {
+    const size_t list_sz = round_up(static_cast<size_t>(n_row) * sizeof(uint2));
+    const size_t need = list_sz + window_event_scatter_bytes<F>(n_col);
+    size_t got = 0;
+    unsigned char *ws = static_cast<unsigned char *>(src.request(need, need, &got));
+    uint32_t *counters = ws ? src.counters() : nullptr;
+    if (ws != nullptr && counters != nullptr) {
+      uint2 *active_list = reinterpret_cast<uint2 *>(ws);
+      launch_collect<F, VT, MODE>(stream, indptr, x, n_row, counters, active_list, static_cast<F *>(nullptr), kAlways,
+                                  static_cast<uint32_t *>(nullptr), 0u, static_cast<F *>(nullptr), 0u);
+      if (window_event_scatter<F>(stream, data, HETER, indices, indptr, y, n_row, n_col, counters, active_list, n_row,
+                                  ws + list_sz, got - list_sz))
+        return;
+      fill_zero(stream, counters, 1u);  // (the walk could not run: the list is not used)
+    } else {
+      if (src.failure_is_final()) return;  // during a capture: the error stands
+      bpl_clear_error();  // no scratch memory: the paths below need less or none
+    }
+  }
   if (n_win <= (MODE == kEvent ? 32u : 4u)) {
     const uint32_t win = div_up(n_col, n_win);
     // about one workgroup per CU in total, at least 64 rows each

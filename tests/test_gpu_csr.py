@@ -461,6 +461,40 @@ def test_transposed_csr_matvec_wide_output_sorted_scatter(cuda, oracle_mod, dtyp
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_event_scatter_into_one_window_from_many_rows(cuda, oracle_mod, dtype):
+  # more than 32,768 rows (the active rows go to a device list) and at most 8,192 columns: the listed rows'
+  # nonzeros are walked flat into one window in LDS per workgroup.  Little and much activity, empty rows, a
+  # row that holds a quarter of the nonzeros, bool and float events, both weight kinds (the homogeneous one
+  # bit for bit), twice in a row (the list's counter must be back at zero).
+  rng = np.random.default_rng(53)
+  for n_row, n_col, mean, hub in ((100_000, 3000, 30, 0), (40_000, 8192, 12, 120_000), (300_000, 700, 3, 0),
+                                  (33_000, 1, 2, 0)):
+    counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
+    counts[rng.integers(0, n_row, size=n_row // 9)] = 0
+    if hub:
+      counts = counts.astype(np.int64)
+      counts[n_row // 5] = min(hub, n_col)
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_row)
+    data = rng.standard_normal(indices.shape[0]).astype(dtype)
+    shape = (n_row, n_col)
+    print("shape", shape, dtype.__name__, flush=True)
+    for rate in (0.0005, 0.05, 0.9):
+      ev = rng.random(n_row) < rate
+      if hub:
+        ev[n_row // 5] = True
+      want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True)
+      mag = oracle_mod.event_csr_matvec(np.abs(data), indices, indptr, ev, shape=shape, transpose=True)
+      for events in (ev, ev.astype(dtype) * 3):
+        for _ in range(2):
+          got = bpl.event_csr_matvec(data, indices, indptr, events, shape=shape, transpose=True).cpu().numpy()
+          assert_close_reordered(got, want, mag, dtype, what="event scatter, one window %s rate %g" % (shape, rate))
+      w = np.array([0.6], dtype=dtype)
+      want = oracle_mod.event_csr_matvec(w, indices, indptr, ev, shape=shape, transpose=True)
+      got = bpl.event_csr_matvec(w, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+      assert np.array_equal(got, want), (shape, rate)  # the reference's repeated additions, bit for bit
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_transposed_csr_matvec_one_output_window_flat_walk(cuda, oracle_mod, dtype):
   # outputs of at most 32,768 columns with at least 2^20 nonzeros: every workgroup walks an equal share of the
   # nonzeros into one float64 window of up to 16,384 columns.  Short rows, empty rows (also first and last), one row that holds a
