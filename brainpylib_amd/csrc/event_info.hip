@@ -193,18 +193,23 @@ void nonzero_entry(const char *target, hipStream_t stream, void **buffers, const
     check_launch(target);
     return;
   }
-  if (d.batch_size > 65535) {
-    set_error("%s: batch_size %u exceeds 65535", target, d.batch_size);
-    return;
-  }
   const uint32_t n_tiles = div_up(d.event_size, kTile);
+  // (a grid holds 65,535 batch rows in its second dimension: more rows are taken that many at a time)
+  constexpr uint32_t kMaxGridY = 65535;
+  const uint32_t rows_at_once = d.batch_size < kMaxGridY ? d.batch_size : kMaxGridY;
   uint32_t *counts = static_cast<uint32_t *>(
-      stream_workspace(stream, static_cast<size_t>(d.batch_size) * n_tiles * sizeof(uint32_t)));
+      stream_workspace(stream, static_cast<size_t>(rows_at_once) * n_tiles * sizeof(uint32_t)));
   if (counts == nullptr) return;
-  const dim3 grid(n_tiles, d.batch_size);
-  hipLaunchKernelGGL(tile_count_kernel<T>, grid, dim3(kThreads), 0, stream, ev, d.event_size, n_tiles, counts);
-  hipLaunchKernelGGL(tile_scan_kernel, dim3(d.batch_size), dim3(kScanThreads), 0, stream, counts, n_tiles, num);
-  hipLaunchKernelGGL(tile_write_kernel<T>, grid, dim3(kThreads), 0, stream, ev, d.event_size, n_tiles, counts, num, ids);
+  for (uint32_t b0 = 0; b0 < d.batch_size; b0 += kMaxGridY) {
+    const uint32_t rows = d.batch_size - b0 < kMaxGridY ? d.batch_size - b0 : kMaxGridY;
+    const T *ev_b = ev + static_cast<size_t>(b0) * d.event_size;
+    int32_t *ids_b = ids + static_cast<size_t>(b0) * d.event_size;
+    const dim3 grid(n_tiles, rows);
+    hipLaunchKernelGGL(tile_count_kernel<T>, grid, dim3(kThreads), 0, stream, ev_b, d.event_size, n_tiles, counts);
+    hipLaunchKernelGGL(tile_scan_kernel, dim3(rows), dim3(kScanThreads), 0, stream, counts, n_tiles, num + b0);
+    hipLaunchKernelGGL(tile_write_kernel<T>, grid, dim3(kThreads), 0, stream, ev_b, d.event_size, n_tiles, counts,
+                       static_cast<const int32_t *>(num + b0), ids_b);
+  }
   check_launch(target);
 }
 

@@ -35,6 +35,23 @@ def test_event_info_edges_and_batch(cuda, oracle_mod):
     assert np.array_equal(ids[b].cpu().numpy(), w_ids) and int(num[b]) == int(w_num[0])
 
 
+def test_event_info_with_more_batch_rows_than_a_grid_dimension(cuda, oracle_mod):
+  # 70,000 rows: more than the 65,535 a grid takes in its second dimension, taken in two passes
+  ev = np.random.default_rng(1).random((70_000, 37)) < 0.3
+  ids, num = bpl.event_info(ev)
+  ids, num = ids.cpu().numpy(), num.cpu().numpy()
+  want_num = ev.sum(axis=1)
+  assert np.array_equal(num.reshape(-1), want_num)
+  for b in (0, 1, 65_534, 65_535, 65_536, 69_999):
+    w_ids, w_num = oracle_mod.event_info(ev[b])
+    assert np.array_equal(ids[b], w_ids) and int(num[b]) == int(w_num[0])
+  # every row: its events in increasing order, then -1
+  order = np.where(ev, np.arange(37), 37 + np.arange(37))
+  want = np.sort(order, axis=1)
+  want = np.where(want < 37, want, -1)
+  assert np.array_equal(ids, want)
+
+
 @pytest.mark.parametrize("dtype", [np.bool_, np.float32])
 def test_event_info_tiles_alignment_and_density(cuda, oracle_mod, dtype):
   # several 4,096-element tiles per row, rows that start at every alignment (one-byte events take a
