@@ -960,6 +960,10 @@ __global__ __launch_bounds__(1024, (MODE == kEvent && BITS == 1) ? 8 : 4) void c
     // (rows of `skip_mean` nonzeros or more on average: the launcher's other kernel has taken this matrix)
     if (skip_mean != 0 && mean >= skip_mean && nnz <= kFlatMaxNnz) return;
   }
+  if constexpr (MODE == kDense && BITS == 2) {
+    // (rows of 4 nonzeros or more but fewer than `skip_mean` on average: the flat walk has taken this matrix)
+    if (skip_mean != 0 && mean >= 4u && mean < skip_mean && nnz <= kFlatMaxNnz) return;
+  }
   if constexpr (MODE == kDense && BITS == 1) {
     // (nothing left to hide but the index and weight streams: the walks of the event gather)
     const VT *xs = reinterpret_cast<const VT *>(s_bits);
@@ -1413,9 +1417,20 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
       bpl_clear_error();
     } else if (n_row >= 16384 && lds_bytes <= 4 * kLdsBitmapCap) {
       // up to four times that: the part that fits is staged (one workgroup per CU), which takes a
-      // quarter or more of the gathers off the L2
+      // quarter or more of the gathers off the L2.  Its walk is row-wise: rows of 4 to 23 nonzeros on average
+      // go to the flat walk over the nonzeros instead (the mean is known on the device only: both are enqueued).
+      constexpr uint32_t kStagedMinMean = 24;
+      bool flat_takes_short_rows = false;
+      if constexpr (std::is_same<F, VT>::value) {
+        const FlatGather flat = csr_flat_gather<F>(target, stream, data, HETER, indices, indptr, x, y, n_row, 4u, kStagedMinMean);
+        if (flat == FlatGather::kFailed) {
+          if (scratch_refused_by_capture()) return;  // (the error stands: a graph must not record a slower path)
+          bpl_clear_error();
+        }
+        flat_takes_short_rows = flat == FlatGather::kEnqueued;
+      }
       if (launch_gather_impl<F, VT, HETER, MODE, 2>(target, stream, data, indices, indptr, x, y, n_row, n_col,
-                                                    kLdsBitmapCap))
+                                                    kLdsBitmapCap, flat_takes_short_rows ? kStagedMinMean : 0u))
         return;
       bpl_clear_error();
     }

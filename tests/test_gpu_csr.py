@@ -742,7 +742,9 @@ def test_csr_matvec_with_16_byte_stream_loads(cuda, oracle_mod, dtype):
   for n_row, n_col, mean, hubs in ((20_000, limit, 30, 0), (16_384, limit + 3, 60, 2), (17_001, 400_000, 100, 3),
                                    (16_400, 300_000, 250, 1), (16_390, 200_000, 500, 0), (16_385, 170_000, 900, 1),
                                    (40_000, 1_000_000, 23, 0), (30_000, 250_000, 24, 40),
-                                   (300_000, 170_000, 3, 0), (280_000, 170_000, 4, 2)):
+                                   (300_000, 170_000, 3, 0), (280_000, 170_000, 4, 2),
+                                   # (a vector of which a part is staged in LDS: that walk from 24 per row on, below it the flat one)
+                                   (40_000, 100_000, 9, 0), (30_000, 90_000, 40, 1), (50_000, 60_000, 23, 0)):
     counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
     counts[rng.integers(0, n_row, 50)] = 0
     counts[rng.integers(0, n_row, 50)] = 1
