@@ -176,6 +176,31 @@ __global__ __launch_bounds__(kThreads) void tile_write_kernel(const T *__restric
   for (uint32_t i = threadIdx.x; i < valid - cnt; i += kThreads) out[tail + i] = -1;
 }
 
+// Rows of at most one tile (4,096 elements): one WAVE per row does all of it, 64 elements a step (flags by
+// ballot, ranks by the count of lower lanes), then the -1 tail and the count.  (A workgroup per row and three
+// kernels, as for long rows, took 4.4 ms for 1,000,000 rows of 100.)
+template <typename T>
+__global__ __launch_bounds__(kThreads) void short_rows_kernel(const T *__restrict__ ev, uint32_t size, uint32_t batch,
+                                                             int32_t *__restrict__ ids, int32_t *__restrict__ event_num) {
+  const uint32_t lane = static_cast<uint32_t>(lane_id());
+  const uint64_t below = (1ull << lane) - 1ull;
+  const uint32_t waves = gridDim.x * (kThreads / kWave);
+  for (uint32_t b = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave; b < batch; b += waves) {
+    const T *row = ev + static_cast<size_t>(b) * size;
+    int32_t *out = ids + static_cast<size_t>(b) * size;
+    uint32_t n = 0;
+    for (uint32_t i0 = 0; i0 < size; i0 += kWave) {
+      const uint32_t i = i0 + lane;
+      const bool on = i < size && row[i] != T(0);
+      const uint64_t m = __ballot(on);
+      if (on) out[n + static_cast<uint32_t>(__popcll(m & below))] = static_cast<int32_t>(i);
+      n += static_cast<uint32_t>(__popcll(m));
+    }
+    for (uint32_t i = n + lane; i < size; i += kWave) out[i] = -1;
+    if (lane == 0) event_num[b] = static_cast<int32_t>(n);
+  }
+}
+
 template <typename T>
 void nonzero_entry(const char *target, hipStream_t stream, void **buffers, const char *opaque, size_t opaque_len) {
   bpl_nonzero_descriptor d;
@@ -190,6 +215,15 @@ void nonzero_entry(const char *target, hipStream_t stream, void **buffers, const
   if (d.batch_size == 0) return;
   if (d.event_size == 0) {
     fill_zero(stream, num, d.batch_size);
+    check_launch(target);
+    return;
+  }
+  if (d.event_size <= kTile && d.batch_size >= 64) {  // many short rows: a wave each
+    const uint32_t rows_per_wg = kThreads / kWave;
+    uint32_t grid = div_up(d.batch_size, rows_per_wg);
+    const uint32_t resident = 8u * static_cast<uint32_t>(device_info().num_cu);
+    if (grid > 8u * resident) grid = 8u * resident;
+    hipLaunchKernelGGL(short_rows_kernel<T>, dim3(grid), dim3(kThreads), 0, stream, ev, d.event_size, d.batch_size, ids, num);
     check_launch(target);
     return;
   }

@@ -36,20 +36,36 @@ def test_event_info_edges_and_batch(cuda, oracle_mod):
 
 
 def test_event_info_with_more_batch_rows_than_a_grid_dimension(cuda, oracle_mod):
-  # 70,000 rows: more than the 65,535 a grid takes in its second dimension, taken in two passes
-  ev = np.random.default_rng(1).random((70_000, 37)) < 0.3
+  # 65,600 rows of two tiles: more than the 65,535 a grid takes in its second dimension, taken in two passes
+  ev = np.random.default_rng(2).random((65_600, 4100)) < 0.01
+  ids, num = bpl.event_info(ev)
+  num = num.cpu().numpy()
+  assert np.array_equal(num.reshape(-1), ev.sum(axis=1))
+  for b in (0, 65_534, 65_535, 65_536, 65_599):
+    w_ids, w_num = oracle_mod.event_info(ev[b])
+    assert np.array_equal(ids[b].cpu().numpy(), w_ids) and int(num[b]) == int(w_num[0])
+  del ids
+
+
+@pytest.mark.parametrize("size", [1, 37, 64, 65, 1000, 4096])
+def test_event_info_of_many_short_rows(cuda, oracle_mod, size):
+  # at least 64 rows of at most one tile: a wave per row
+  ev = np.random.default_rng(size).random((70_000 if size == 37 else 300, size)) < 0.3
   ids, num = bpl.event_info(ev)
   ids, num = ids.cpu().numpy(), num.cpu().numpy()
   want_num = ev.sum(axis=1)
   assert np.array_equal(num.reshape(-1), want_num)
-  for b in (0, 1, 65_534, 65_535, 65_536, 69_999):
+  for b in (0, 1, ev.shape[0] // 2, ev.shape[0] - 1):
     w_ids, w_num = oracle_mod.event_info(ev[b])
     assert np.array_equal(ids[b], w_ids) and int(num[b]) == int(w_num[0])
   # every row: its events in increasing order, then -1
-  order = np.where(ev, np.arange(37), 37 + np.arange(37))
+  order = np.where(ev, np.arange(size), size + np.arange(size))
   want = np.sort(order, axis=1)
-  want = np.where(want < 37, want, -1)
+  want = np.where(want < size, want, -1)
   assert np.array_equal(ids, want)
+  evf = np.where(ev, np.float32(-0.5), np.float32(0))  # float events: nonzero means event
+  ids_f, num_f = bpl.event_info(evf)
+  assert np.array_equal(ids_f.cpu().numpy(), want) and np.array_equal(num_f.cpu().numpy().reshape(-1), want_num)
 
 
 @pytest.mark.parametrize("dtype", [np.bool_, np.float32])
