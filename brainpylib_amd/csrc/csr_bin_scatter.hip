@@ -954,7 +954,7 @@ __global__ __launch_bounds__(kBinThreads) void active_rows_window_kernel(
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-          if (jb + u * kBinThreads < seg_end) {
+          if (jb + u * kBinThreads < seg_end && col[u] < n_col) {  // (a column beyond the output: left out)
             if constexpr (HETER) atomicAdd(&window[col[u]], static_cast<double>(val[u]));
             else atomicAdd(&window[col[u]], 1u);
           }
