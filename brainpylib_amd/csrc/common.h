@@ -95,6 +95,20 @@ template <typename F>
 bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool heter, const uint32_t *indices,
                  const uint32_t *indptr, const F *vec, F *y, uint32_t n_row, uint32_t n_col, uint32_t nnz);
 
+// coo_atomic_sum / coo_event_sum through windows of the result in LDS (coo_window_sum.hip): taken for a long
+// connection list and a result of a few windows.  EVENT: connection i counts if
+// events[pre_ids[i]] and carries values[i]; otherwise it carries values[pre_ids[i]]; HETER false: values[0].
+// 1: enqueued; 0: nothing enqueued, the caller takes another path; -1: nothing enqueued and the call must fail
+// with the error that stands.
+template <typename F, typename I, bool HETER, bool EVENT>
+int coo_window_sum(const char *target, hipStream_t stream, const uint8_t *events, const F *values, const I *post_ids,
+                   const I *pre_ids, F *result, uint32_t conn_size, uint32_t post_size);
+// The same sums with a weight per connection or source into a wider result, through bins (the coarse-sorted
+// scatter); same return values.
+template <typename F, typename I, bool EVENT>
+int coo_bin_sum(const char *target, hipStream_t stream, const uint8_t *events, const F *values, const I *post_ids,
+                const I *pre_ids, F *result, uint32_t conn_size, uint32_t post_size);
+
 // Transposed CSR times dense vector for outputs of at most kFlatWindowMaxSlices windows of kFlatWindowMaxCols
 // columns (a float64 window in LDS per workgroup, the workgroups of a window equal shares of the nonzeros;
 // csr_bin_scatter.hip).  false, having enqueued nothing, if it cannot run (wider output, no scratch memory).

@@ -152,6 +152,14 @@ void coo_event_sum_entry(const char *target, hipStream_t stream, void **buffers,
     return;
   }
   F *result = static_cast<F *>(buffers[4]);
+  if (coo_window_sum<F, I, HETER, true>(target, stream, static_cast<const uint8_t *>(buffers[0]),
+                                        static_cast<const F *>(buffers[3]), static_cast<const I *>(buffers[2]),
+                                        static_cast<const I *>(buffers[1]), result, d.conn_size, d.post_size) != 0)
+    return;  // (enqueued, or failed with its error standing)
+  if (HETER && coo_bin_sum<F, I, true>(target, stream, static_cast<const uint8_t *>(buffers[0]),
+                                       static_cast<const F *>(buffers[3]), static_cast<const I *>(buffers[2]),
+                                       static_cast<const I *>(buffers[1]), result, d.conn_size, d.post_size) != 0)
+    return;
   fill_zero(stream, result, d.post_size);
   if (d.conn_size == 0 || d.post_size == 0) return;
   hipLaunchKernelGGL((coo_event_sum_kernel<F, I, HETER>), dim3(grid_for(d.conn_size, kThreads)), dim3(kThreads), 0,
@@ -171,10 +179,16 @@ void coo_atomic_sum_entry(const char *target, hipStream_t stream, void **buffers
     return;
   }
   F *result = static_cast<F *>(buffers[HETER ? 3 : 2]);
-  fill_zero(stream, result, d.post_size);
-  if (d.conn_size == 0 || d.post_size == 0) return;
   const I *post_ids = static_cast<const I *>(buffers[1]);
   const I *pre_ids = HETER ? static_cast<const I *>(buffers[2]) : post_ids;
+  if (coo_window_sum<F, I, HETER, false>(target, stream, nullptr, static_cast<const F *>(buffers[0]), post_ids, pre_ids,
+                                         result, d.conn_size, d.post_size) != 0)
+    return;  // (enqueued, or failed with its error standing)
+  if (HETER && coo_bin_sum<F, I, false>(target, stream, nullptr, static_cast<const F *>(buffers[0]), post_ids, pre_ids, result,
+                                        d.conn_size, d.post_size) != 0)
+    return;
+  fill_zero(stream, result, d.post_size);
+  if (d.conn_size == 0 || d.post_size == 0) return;
   hipLaunchKernelGGL((coo_atomic_sum_kernel<F, I, HETER>), dim3(grid_for(d.conn_size, kThreads)), dim3(kThreads), 0,
                      stream, static_cast<const F *>(buffers[0]), post_ids, pre_ids, result, d.conn_size);
   check_launch(target);

@@ -65,6 +65,53 @@ def test_coo_event_sum_vs_oracle(cuda, oracle_mod, dtype, itype):
         assert np.array_equal(got, want)  # counts
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("itype", [np.int32, np.int64])
+def test_coo_sums_through_windows_of_the_result(cuda, oracle_mod, dtype, itype):
+  """Long connection lists are added in LDS windows of the result (one window, two slices, a connection count
+  that is no multiple of a lane's four; with one weight up to 32 slices) or, with weights and a wider result,
+  through bins (a fiftieth of the connections crowd into one window and overflow its bins); short lists and a
+  single weight into a very wide result take the atomics."""
+  rng = np.random.default_rng(21)
+  for pre_n, post_n, conn in [(3000, 5000, 600_001), (70000, 16384, 400_003), (500, 20000, 300_002),
+                              (1000, 32768, 262_147), (1000, 32769, 262_147), (40, 1, 140_000),
+                              (2000, 100_000, 1_200_001), (50_000, 3_000_000, 1_100_003), (300, 40_000, 1_048_576)]:
+    pre = rng.integers(0, pre_n, conn).astype(itype)
+    post = rng.integers(0, post_n, conn).astype(itype)
+    # a crowded end of the result (few enough additions per element for the oracle's float32 loop to stay within
+    # the bound used below, enough for that window's bins to overflow)
+    post[: conn // 50] = post_n - 1 - post[: conn // 50] % min(post_n, 7)
+    events = rng.random(pre_n) < 0.3
+    print("case", pre_n, post_n, conn, flush=True)
+    for homo in (False, True):
+      # coo_atomic_sum: a value per source
+      values = np.full(1, 0.1, dtype) if homo else rng.standard_normal(pre_n).astype(dtype)
+      got = bpl.coo_atomic_sum(values, post, post_n, None if homo else pre).cpu().numpy()
+      want = oracle_mod.coo_atomic_sum(values, post, post_n, None if homo else pre)
+      mag = np.bincount(post, weights=np.abs(values[0] if homo else values[pre]) * np.ones(conn), minlength=post_n)
+      if homo:
+        assert np.array_equal(got, want), "coo_atomic_sum of one weight: sums of that many additions"
+      elif post_n == 1:
+        # 140,000 additions to one element: the oracle's own float32 loop drifts by more than the bound below
+        # allows for, so the sum is compared with the one taken in float64
+        exact = np.array([values[pre].astype(np.float64).sum()])
+        assert_close_reordered(got, exact, mag, dtype, what="coo_atomic_sum")
+      else:
+        assert_close_reordered(got, want, mag, dtype, what="coo_atomic_sum")
+      # coo_event_sum: a value per connection
+      values = np.full(1, 0.1, dtype) if homo else rng.standard_normal(conn).astype(dtype)
+      got = bpl.coo_event_sum(events, pre, post, post_n, values).cpu().numpy()
+      want = oracle_mod.coo_event_sum(events, pre, post, post_n, values)
+      mag = oracle_mod.coo_event_sum(events, pre, post, post_n, np.abs(values))
+      if homo:
+        assert np.array_equal(got, want), "coo_event_sum of one weight: sums of that many additions"
+      elif post_n == 1:
+        exact = np.array([(values.astype(np.float64) * events[pre]).sum()])
+        assert_close_reordered(got, exact, mag, dtype, what="coo_event_sum")
+      else:
+        assert_close_reordered(got, want, mag, dtype, what="coo_event_sum")
+
+
 def test_known_answers_and_argument_checks(cuda):
   # brainpylib/_src/compat/tests/test_atomic_sum_cpu.py:16-34
   size = 200
