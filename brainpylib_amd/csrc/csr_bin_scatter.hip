@@ -241,8 +241,22 @@ __global__ __launch_bounds__(kBinThreads) void bin_products_kernel(
           win[t] = j + t < seg_end ? col[t] >> shift : kMaxWindows;  // (kMaxWindows: no pair)
           rel[t] = col[t] & ((1u << shift) - 1u);
         }
+        // (Long rows with their columns in order: all of a wave's nonzeros fall into one window, and as many
+        // atomics on one counter would take their turns.  One lane then reserves the ranks of the whole wave.)
+        bool one_window = true;
+        const uint32_t w_first = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(win[0])));
 #pragma unroll
-        for (int t = 0; t < U; ++t) rank[t] = atomicAdd(&s_cnt[win[t]], 1u);
+        for (int t = 0; t < U; ++t) one_window = one_window && win[t] == w_first;
+        if (__all(one_window)) {
+          uint32_t first_rank = 0;
+          if (tid % kWave == 0) first_rank = atomicAdd(&s_cnt[w_first], static_cast<uint32_t>(U * kWave));
+          first_rank = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(first_rank)));
+#pragma unroll
+          for (int t = 0; t < U; ++t) rank[t] = first_rank + U * (tid % kWave) + t;
+        } else {
+#pragma unroll
+          for (int t = 0; t < U; ++t) rank[t] = atomicAdd(&s_cnt[win[t]], 1u);
+        }
         __syncthreads();
         if (tid < kWave) {  // offsets of the windows within the round: two counters per lane
           const uint32_t c0 = s_cnt[2 * tid], c1 = s_cnt[2 * tid + 1];

@@ -811,8 +811,8 @@ __device__ __forceinline__ void gather_rows_wave(const F *__restrict__ data, con
   for (uint32_t row = blockIdx.x * waves_per_block + threadIdx.x / kWave; row < n_row; row += total_waves) {
     const uint32_t urow = __builtin_amdgcn_readfirstlane(row);
     const uint32_t start = indptr[urow];
-    uint32_t len = indptr[urow + 1] - start;
-    if (len > kHubSteps * U * kWave) len = 0;  // (the whole workgroup takes it: gather_hub_rows())
+    const uint32_t len = indptr[urow + 1] - start;
+    if (len > kHubSteps * U * kWave) continue;  // (a whole workgroup takes it and stores it: gather_hub_rows())
     const uint32_t *ip = indices + start;
     const F *dp = data + (HETER ? start : 0u);
     double acc = 0.0;
@@ -837,6 +837,10 @@ __device__ __forceinline__ void gather_rows_wave(const F *__restrict__ data, con
 // empty, and after its walk every workgroup looks through the bounds of the rows it was dealt again
 // (workgroup b: rows b * gpb + g + k * total_groups, g < gpb) and walks each such row with all its
 // threads: partial sums per lane, a wave sum, one float64 (or integer) LDS atomic per wave.
+// The walk with a wave per row skips such rows without storing anything, and they are dealt one by one
+// (gpb = 1: workgroup b looks at rows b, b + gridDim.x, ...): in a matrix of a few thousand rows that are
+// all this long, sixteen consecutive rows per workgroup would leave most of the device idle (2,000 rows of
+// 50,000: an eighth of the workgroups had rows).
 template <typename F, typename VT, bool HETER, int MODE, int BITS>
 __device__ __forceinline__ void gather_hub_rows(const F *__restrict__ data, const uint32_t *__restrict__ indices,
                                                 const uint32_t *__restrict__ indptr, const VT *__restrict__ x,
@@ -967,27 +971,27 @@ __global__ __launch_bounds__(1024, (MODE == kEvent && BITS == 1) ? 8 : 4) void c
   if constexpr (MODE == kDense && BITS == 1) {
     // (nothing left to hide but the index and weight streams: the walks of the event gather)
     const VT *xs = reinterpret_cast<const VT *>(s_bits);
-    if (mean >= 384) { gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g); gpb = blockDim.x / kWave; hub_len = kHubSteps * 8 * kWave; }
+    if (mean >= 384) { gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g); gpb = 1; hub_len = kHubSteps * 8 * kWave; }
     else if (mean >= 24) { gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 8; hub_len = kHubSteps * 8 * 8; }
     else if (mean >= 12) { gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 4; hub_len = kHubSteps * 8 * 4; }
     else { gather_rows<F, VT, HETER, MODE, BITS, 4, 4>(data, indices, indptr, xs, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 4; hub_len = kHubSteps * 4 * 4; }
   } else if constexpr (MODE == kDense && BITS == 2) {
-    if (mean >= 384) { gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / kWave; hub_len = kHubSteps * 8 * kWave; }
+    if (mean >= 384) { gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = 1; hub_len = kHubSteps * 8 * kWave; }
     else if (mean >= 24) { gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 8; hub_len = kHubSteps * 8 * 8; }
     else { gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 4; hub_len = kHubSteps * 8 * 4; }
   } else if constexpr (MODE == kEvent && (BITS == 2 || BITS == 3)) {
     // An event bitmap above 80 KB leaves room for one workgroup (16 waves) per CU only: every lane
     // then keeps 16 (rows under 48 nonzeros: 8) loads in flight instead of 2 to 8, in groups of
     // 8 or 4 lanes per row, or HBM sees too few requests (1e6 columns, 100 per row: 424 -> 164 us).
-    if (mean >= 384) { gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / kWave; hub_len = kHubSteps * 8 * kWave; }
+    if (mean >= 384) { gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = 1; hub_len = kHubSteps * 8 * kWave; }
     else if (mean >= 48) { gather_rows<F, VT, HETER, MODE, BITS, 8, 16>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 8; hub_len = kHubSteps * 16 * 8; }
     else { gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 4; hub_len = kHubSteps * 8 * 4; }
   } else {
-    if (mean >= 384) { gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / kWave; hub_len = kHubSteps * 8 * kWave; }
+    if (mean >= 384) { gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = 1; hub_len = kHubSteps * 8 * kWave; }
     // (a dense vector is gathered from L2: for rows of 48 .. 191 nonzeros the pipelined 32-lane walk keeps more
     // of those gathers in flight than a wave per row does)
     else if (MODE == kEvent && mean >= 48u) { gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 8; hub_len = kHubSteps * 8 * 8; }
-    else if (MODE == kDense && mean >= 192u) { gather_rows_wave<F, VT, HETER, MODE, BITS, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / kWave; hub_len = kHubSteps * 2 * kWave; }
+    else if (MODE == kDense && mean >= 192u) { gather_rows_wave<F, VT, HETER, MODE, BITS, 2>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = 1; hub_len = kHubSteps * 2 * kWave; }
     else if (mean >= 48) { gather_rows<F, VT, HETER, MODE, BITS, 32, 4>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 32; hub_len = kHubSteps * 4 * 32; }
     else if (MODE == kEvent && mean >= 24) { gather_rows<F, VT, HETER, MODE, BITS, 8, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 8; hub_len = kHubSteps * 8 * 8; }
     else if (MODE == kEvent && mean >= 12) { gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 4; hub_len = kHubSteps * 8 * 4; }
@@ -1319,7 +1323,9 @@ bool launch_gather_impl(const char *target, hipStream_t stream, const F *data, c
   auto kernel = csr_gather_kernel<F, VT, HETER, MODE, BITS>;
   // Small problems: 256-thread workgroups, one wave per row at most.  Large ones: 1024-thread
   // persistent workgroups so that few copies of the event bitmap are built.
-  const int block = (n_row >= 16384) ? 1024 : 256;
+  // (Few rows over many columns, or an LDS image of more than 16 KB per workgroup: the large ones too.)
+  const bool wide = n_col > kHubSteps * 8 * kWave;  // rows can be long enough to go to whole workgroups
+  const int block = (n_row >= 16384 || lds_bytes > 16 * 1024 || (wide && n_row < 2048)) ? 1024 : 256;
   // The occupancy query is the same for every call with the same LDS size: remember the last one.
   struct Cached {
     size_t lds_bytes;
@@ -1345,7 +1351,10 @@ bool launch_gather_impl(const char *target, hipStream_t stream, const F *data, c
   }
   const int per_cu = cached.per_cu;
   const unsigned resident = static_cast<unsigned>(device_info().num_cu) * static_cast<unsigned>(per_cu);
-  const unsigned needed = div_up(n_row, block / kWave);  // one wave per row
+  unsigned needed = div_up(n_row, block / kWave);  // one wave per row
+  // Few rows over many columns may all be long enough to go to whole workgroups, one row each (gather_hub_rows;
+  // the row lengths are known on the device only): then a workgroup per row, or most of the device has no row.
+  if (wide && n_row < 2048) needed = n_row;
   const unsigned grid = needed < resident ? (needed ? needed : 1u) : resident;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), lds_bytes, stream, data, indices, indptr, x, y, n_row,
                      n_col, skip_mean);

@@ -810,6 +810,7 @@ def test_gather_hub_rows(cuda, oracle_mod):
     (100_000, 100_000, 12, {777: 90_000, 778: 5000, 99_999: 2000, 0: 1025}),
     (30_000, 60_000, 30, {5: 50_000, 29_000: 4097}),
     (2000, 50_000, 500, {3: 40_000, 1999: 33_000}),
+    (700, 60_000, 34_000, {0: 33_000, 699: 1}),  # every row but one goes to a whole workgroup, dealt one by one
     (20_000, 2_000_000, 50, {777: 1_000_000}),
   ]
   dev = torch.device("cuda:0")
