@@ -709,8 +709,17 @@ __global__ __launch_bounds__(kBinThreads) __attribute__((amdgpu_num_sgpr(80))) v
   const uint32_t p = blockIdx.x;
   if (p >= producers) return;
   const uint32_t sub = p % kSubRuns;
-  const uint32_t lo = static_cast<uint32_t>(static_cast<uint64_t>(p) * total / producers);
-  const uint32_t hi = static_cast<uint32_t>(static_cast<uint64_t>(p + 1) * total / producers);
+  // Producer p takes an equal share of the listed rows; where there are fewer rows than producers (a few
+  // long rows are active), `parts` producers take a row, each an equal part of its nonzeros.
+  uint32_t lo, hi, part = 0, parts = 1;
+  if (total < producers) {
+    parts = producers / total;
+    lo = p / parts, hi = lo + 1u, part = p % parts;
+    if (lo >= total) return;
+  } else {
+    lo = static_cast<uint32_t>(static_cast<uint64_t>(p) * total / producers);
+    hi = static_cast<uint32_t>(static_cast<uint64_t>(p + 1) * total / producers);
+  }
   if (tid < kMaxWindows) s_cnt[tid] = 0;
   const F w_homo = HETER ? F(0) : data[0];
   // homogeneous weight: a run holds the pairs' columns only, `cap` of them
@@ -730,6 +739,11 @@ __global__ __launch_bounds__(kBinThreads) __attribute__((amdgpu_num_sgpr(80))) v
     __syncthreads();  // the previous tile is done with s_ptr / s_start (and s_cnt is cleared)
     uint2 e = make_uint2(0u, 0u);
     if (tid < rows) e = active_list[t0 + tid];
+    if (parts > 1u) {  // (one row: this producer's part of it, which may be empty)
+      const uint32_t a = static_cast<uint32_t>(static_cast<uint64_t>(e.y) * part / parts);
+      const uint32_t b = static_cast<uint32_t>(static_cast<uint64_t>(e.y) * (part + 1u) / parts);
+      e.x += a, e.y = b - a;
+    }
     const uint32_t incl = wave_inclusive_scan_u32(e.y);
     if (lane == kWave - 1) s_wave[wave] = incl;
     __syncthreads();

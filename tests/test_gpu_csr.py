@@ -495,6 +495,35 @@ def test_event_scatter_into_one_window_from_many_rows(cuda, oracle_mod, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_event_scatter_of_few_long_rows(cuda, oracle_mod, dtype):
+  # fewer active rows than producer workgroups: several producers share a row, each a part of its nonzeros
+  # (5 and about 20 active rows of 34,000; with half of the 700 rows active a producer per row and idle ones),
+  # rows of unequal length, both weight kinds (the homogeneous one bit for bit), twice in a row
+  rng = np.random.default_rng(59)
+  n_row, n_col = 700, 60_000
+  counts = np.full(n_row, 34_000)
+  counts[::7] = 9
+  counts[5] = 60_000
+  indices, indptr = synth.counted_csr(counts, n_col, seed=3)
+  data = rng.standard_normal(indices.shape[0]).astype(dtype)
+  shape = (n_row, n_col)
+  for active in (5, 20, 350):
+    ev = np.zeros(n_row, dtype=bool)
+    ev[rng.choice(n_row, size=active, replace=False)] = True
+    ev[5] = True
+    print("active rows", int(ev.sum()), dtype.__name__, flush=True)
+    want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True)
+    mag = oracle_mod.event_csr_matvec(np.abs(data), indices, indptr, ev, shape=shape, transpose=True)
+    for _ in range(2):
+      got = bpl.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+      assert_close_reordered(got, want, mag, dtype, what="event scatter, %d long rows" % active)
+    w = np.array([0.6], dtype=dtype)
+    want = oracle_mod.event_csr_matvec(w, indices, indptr, ev, shape=shape, transpose=True)
+    got = bpl.event_csr_matvec(w, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+    assert np.array_equal(got, want), active  # the reference's repeated additions, bit for bit
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_transposed_csr_matvec_one_output_window_flat_walk(cuda, oracle_mod, dtype):
   # outputs of at most 32,768 columns with at least 2^20 nonzeros: every workgroup walks an equal share of the
   # nonzeros into one float64 window of up to 16,384 columns.  Short rows, empty rows (also first and last), one row that holds a
