@@ -876,14 +876,18 @@ __device__ __forceinline__ void gather_hub_rows(const F *__restrict__ data, cons
         const uint32_t start = indptr[r], len = indptr[r + 1] - start;
         double acc = 0.0;
         uint32_t hits = 0;
-        constexpr uint32_t U = 4;  // loads in flight per lane
-        for (uint32_t j0 = tid; j0 < len; j0 += U * blockDim.x) {
-          uint32_t col[U];
+        constexpr uint32_t U = 4;  // loads in flight per lane and step; the next step's are requested before this one's are used
+        uint32_t col[U], ncol[U];
+        auto load_cols = [&](uint32_t j0, uint32_t (&c)[U]) {  // (beyond the row: its last index again)
 #pragma unroll
           for (uint32_t u = 0; u < U; ++u) {
             const uint32_t j = j0 + u * blockDim.x;
-            col[u] = indices[start + (j < len ? j : len - 1u)];
+            c[u] = indices[start + (j < len ? j : len - 1u)];
           }
+        };
+        load_cols(tid, col);
+        for (uint32_t j0 = tid; j0 < len; j0 += U * blockDim.x) {
+          load_cols(j0 + U * blockDim.x, ncol);
 #pragma unroll
           for (uint32_t u = 0; u < U; ++u) {
             const uint32_t j = j0 + u * blockDim.x;
@@ -898,6 +902,8 @@ __device__ __forceinline__ void gather_hub_rows(const F *__restrict__ data, cons
               acc += static_cast<double>(static_cast<F>(static_cast<F>(dense_element<VT, BITS>(x, s_bits, coarse_g, col[u])) * d));
             }
           }
+#pragma unroll
+          for (uint32_t u = 0; u < U; ++u) col[u] = ncol[u];
         }
         if (MODE == kEvent && !HETER) {
           hits = wave_sum(hits);
