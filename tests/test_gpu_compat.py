@@ -112,6 +112,27 @@ def test_coo_sums_through_windows_of_the_result(cuda, oracle_mod, dtype, itype):
         assert_close_reordered(got, want, mag, dtype, what="coo_event_sum")
 
 
+def test_coo_sums_of_fifty_million_connections_exact_on_integer_data(cuda):
+  """At a size the CPU loop is not run at: small integers as weights add up exactly in any order, so the result
+  must equal numpy's float64 bincount bit for bit, through the LDS windows (10,000 targets), the slices of a
+  single weight and the bins (100,000 targets)."""
+  rng = np.random.default_rng(33)
+  conn, pre_n = 50_000_000, 100_000
+  pre = rng.integers(0, pre_n, conn, dtype=np.int32)
+  values = rng.integers(-3, 4, pre_n).astype(np.float32)
+  events = rng.random(pre_n) < 0.2
+  per_conn = values[pre]
+  for post_n in (10_000, 100_000):
+    post = rng.integers(0, post_n, conn, dtype=np.int32)
+    print("targets", post_n, flush=True)
+    got = bpl.coo_atomic_sum(values, post, post_n, pre).cpu().numpy()
+    assert np.array_equal(got, np.bincount(post, weights=per_conn, minlength=post_n).astype(np.float32))
+    got = bpl.coo_atomic_sum(np.float32(0.5), post, post_n).cpu().numpy()
+    assert np.array_equal(got, (0.5 * np.bincount(post, minlength=post_n)).astype(np.float32))
+    got = bpl.coo_event_sum(events, pre, post, post_n, per_conn).cpu().numpy()
+    assert np.array_equal(got, np.bincount(post, weights=per_conn * events[pre], minlength=post_n).astype(np.float32))
+
+
 def test_known_answers_and_argument_checks(cuda):
   # brainpylib/_src/compat/tests/test_atomic_sum_cpu.py:16-34
   size = 200
