@@ -876,11 +876,17 @@ __device__ __forceinline__ uint32_t window_event_producers(uint32_t total, uint3
   return want < 1u ? 1u : want > launched ? launched : static_cast<uint32_t>(want);
 }
 
-template <typename F, bool HETER>
+// SELF: no list.  The matrix has at most kSelfListRows rows and every workgroup looks at all events itself
+// (thread t at rows t, t + 1,024, ...: bit b of its mask is row 1,024 b + t; the active rows are numbered thread
+// by thread, then bit by bit, the same in every workgroup), which saves the launch of the kernel that lists
+// them.  Active rows without nonzeros are then among the numbered ones.
+constexpr uint32_t kSelfListRows = 32u * kBinThreads;
+template <typename F, bool HETER, bool SELF>
 __global__ __launch_bounds__(kBinThreads) void active_rows_window_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
     uint32_t n_row, uint32_t n_col, const uint32_t *__restrict__ active_count, const uint2 *__restrict__ active_list,
-    uint32_t list_cap, void *__restrict__ partial, uint32_t *__restrict__ groups_out) {
+    uint32_t list_cap, void *__restrict__ partial, uint32_t *__restrict__ groups_out, const void *__restrict__ events,
+    uint32_t event_width) {
   using A = typename std::conditional<HETER, double, uint32_t>::type;  // a window's accumulators
   extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
   A *window = reinterpret_cast<A *>(smem_raw);
@@ -888,10 +894,42 @@ __global__ __launch_bounds__(kBinThreads) void active_rows_window_kernel(
   __shared__ uint32_t s_start[kTileRows];       // first nonzero of row k in the matrix
   __shared__ uint32_t s_hint[kBinThreads + 1];
   __shared__ uint32_t s_wave[kBinThreads / kWave];
+  __shared__ uint32_t s_mask[SELF ? kBinThreads : 1];        // SELF: the active rows among a thread's 32
+  __shared__ uint32_t s_before[SELF ? kBinThreads + 1 : 1];  // SELF: active rows of the threads before
   constexpr int U = 4;
   constexpr uint32_t kRound = U * kBinThreads;
   const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  const uint32_t total = active_count[0] < list_cap ? active_count[0] : list_cap;  // (never beyond the list)
+  uint32_t total;
+  if constexpr (SELF) {
+    // (every load is issued, beyond the last row for that row again, and none sits in a branch: they are in
+    // flight together)
+    auto scan = [&](const auto *ev) {
+      uint32_t found = 0;
+#pragma unroll
+      for (uint32_t b = 0; b < 32u; ++b) {
+        const uint32_t r = b * kBinThreads + tid;
+        const auto v = ev[r < n_row ? r : n_row - 1u];
+        if (v != 0 && r < n_row) found |= 1u << b;
+      }
+      return found;
+    };
+    const uint32_t m = event_width == 1u   ? scan(static_cast<const uint8_t *>(events))
+                       : event_width == 4u ? scan(static_cast<const float *>(events))
+                                           : scan(static_cast<const double *>(events));
+    s_mask[tid] = m;
+    const uint32_t c = static_cast<uint32_t>(__popc(m));
+    const uint32_t incl = wave_inclusive_scan_u32(c);
+    if (lane == kWave - 1) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t before = 0;
+    for (uint32_t w = 0; w < wave; ++w) before += s_wave[w];
+    s_before[tid] = before + incl - c;
+    if (tid == kBinThreads - 1) s_before[kBinThreads] = before + incl;
+    __syncthreads();
+    total = s_before[kBinThreads];
+  } else {
+    total = active_count[0] < list_cap ? active_count[0] : list_cap;  // (never beyond the list)
+  }
   const uint32_t producers = window_event_producers(total, indptr[n_row], n_row, gridDim.x);
   const uint32_t p = blockIdx.x;
   if (p == 0 && tid == 0) groups_out[0] = producers;  // (for the kernel that adds the windows)
@@ -913,7 +951,24 @@ __global__ __launch_bounds__(kBinThreads) void active_rows_window_kernel(
     const uint32_t rows = (hi - t0 < kTileRows) ? hi - t0 : kTileRows;
     __syncthreads();  // the previous tile is done with s_ptr / s_start (and the window is cleared)
     uint2 e = make_uint2(0u, 0u);
-    if (tid < rows) e = active_list[t0 + tid];
+    if (tid < rows) {
+      if constexpr (SELF) {
+        const uint32_t idx = t0 + tid;
+        uint32_t a = 0, b = kBinThreads - 1u;  // the thread that holds active row idx: the largest a with s_before[a] <= idx
+        while (a < b) {
+          const uint32_t mid = (a + b + 1u) >> 1;
+          if (s_before[mid] <= idx) a = mid;
+          else b = mid - 1u;
+        }
+        uint32_t mask = s_mask[a];
+        for (uint32_t k = idx - s_before[a]; k != 0; --k) mask &= mask - 1u;
+        const uint32_t r = (static_cast<uint32_t>(__ffs(static_cast<int>(mask))) - 1u) * kBinThreads + a;
+        const uint32_t first = indptr[r];
+        e = make_uint2(first, indptr[r + 1] - first);
+      } else {
+        e = active_list[t0 + tid];
+      }
+    }
     const uint32_t incl = wave_inclusive_scan_u32(e.y);
     if (lane == kWave - 1) s_wave[wave] = incl;
     __syncthreads();
@@ -922,7 +977,7 @@ __global__ __launch_bounds__(kBinThreads) void active_rows_window_kernel(
     if (tid < rows) s_ptr[tid] = before + incl - e.y, s_start[tid] = e.x;
     if (tid == rows - 1u) s_ptr[rows] = before + incl;
     __syncthreads();
-    const uint32_t j1 = s_ptr[rows];  // the tile's nonzeros, numbered from 0 (listed rows are never empty)
+    const uint32_t j1 = s_ptr[rows];  // the tile's nonzeros, numbered from 0 (a row without nonzeros is never found by row_of)
     for (uint32_t seg = 0; seg < j1; seg += kSegment) {
       const uint32_t seg_end = (j1 - seg < kSegment) ? j1 : seg + kSegment;
       __syncthreads();  // the previous segment is done with s_hint
@@ -1168,32 +1223,35 @@ size_t window_event_scatter_bytes(uint32_t n_col) {
 template <typename F>
 bool window_event_scatter(hipStream_t stream, const F *data, bool heter, const uint32_t *indices, const uint32_t *indptr,
                           F *y, uint32_t n_row, uint32_t n_col, uint32_t *counters, const uint2 *active_list,
-                          uint32_t list_cap, void *scratch, size_t scratch_bytes) {
+                          uint32_t list_cap, void *scratch, size_t scratch_bytes, const void *events, uint32_t event_width) {
   if (!window_event_scatter_usable<F>(n_row, n_col) || scratch_bytes < window_event_scatter_bytes<F>(n_col)) return false;
+  const bool self = events != nullptr;  // no list: the kernel looks at the events itself
+  if (self && (n_row > kSelfListRows || (event_width != 1u && event_width != 4u && event_width != 8u))) return false;
   const unsigned grid = 2u * static_cast<unsigned>(device_info().num_cu);
   const size_t lds = static_cast<size_t>(n_col) * (heter ? sizeof(double) : sizeof(uint32_t));
-  static thread_local bool attr_set[2] = {false, false};
-  if (!attr_set[heter]) {
-    const void *kernel = heter ? reinterpret_cast<const void *>(active_rows_window_kernel<F, true>)
-                               : reinterpret_cast<const void *>(active_rows_window_kernel<F, false>);
-    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+  // (its 8 KB of masks beside 12.5 KB of row tables: two workgroups must still fit a CU's 160 KB)
+  if (self && lds + 21 * 1024 > 80 * 1024) return false;
+  using Kernel = void (*)(const F *, const uint32_t *, const uint32_t *, uint32_t, uint32_t, const uint32_t *, const uint2 *,
+                          uint32_t, void *, uint32_t *, const void *, uint32_t);
+  const Kernel kernel = heter ? (self ? active_rows_window_kernel<F, true, true> : active_rows_window_kernel<F, true, false>)
+                              : (self ? active_rows_window_kernel<F, false, true> : active_rows_window_kernel<F, false, false>);
+  static thread_local bool attr_set[2][2] = {{false, false}, {false, false}};
+  if (!attr_set[heter][self]) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             static_cast<int>(kWindowEventMaxCols * sizeof(double))) != hipSuccess) {
       (void)hipGetLastError();
       return false;
     }
-    attr_set[heter] = true;
+    attr_set[heter][self] = true;
   }
-  if (heter) {
-    hipLaunchKernelGGL((active_rows_window_kernel<F, true>), dim3(grid), dim3(kBinThreads), lds, stream, data, indices, indptr,
-                       n_row, n_col, static_cast<const uint32_t *>(counters), active_list, list_cap, scratch, counters + 1);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBinThreads), lds, stream, data, indices, indptr, n_row, n_col,
+                     static_cast<const uint32_t *>(counters), active_list, list_cap, scratch, counters + 1, events, event_width);
+  if (heter)
     hipLaunchKernelGGL((sum_active_windows_kernel<F, true>), dim3(div_up(n_col, kSumCols)), dim3(kSumCols * kSumSlices), 0, stream,
                        static_cast<const void *>(scratch), y, n_col, counters, data);
-  } else {
-    hipLaunchKernelGGL((active_rows_window_kernel<F, false>), dim3(grid), dim3(kBinThreads), lds, stream, data, indices, indptr,
-                       n_row, n_col, static_cast<const uint32_t *>(counters), active_list, list_cap, scratch, counters + 1);
+  else
     hipLaunchKernelGGL((sum_active_windows_kernel<F, false>), dim3(div_up(n_col, kSumCols)), dim3(kSumCols * kSumSlices), 0, stream,
                        static_cast<const void *>(scratch), y, n_col, counters, data);
-  }
   return true;
 }
 
@@ -1408,9 +1466,10 @@ template bool window_event_scatter_usable<double>(uint32_t, uint32_t);
 template size_t window_event_scatter_bytes<float>(uint32_t);
 template size_t window_event_scatter_bytes<double>(uint32_t);
 template bool window_event_scatter<float>(hipStream_t, const float *, bool, const uint32_t *, const uint32_t *, float *, uint32_t,
-                                          uint32_t, uint32_t *, const uint2 *, uint32_t, void *, size_t);
+                                          uint32_t, uint32_t *, const uint2 *, uint32_t, void *, size_t, const void *, uint32_t);
 template bool window_event_scatter<double>(hipStream_t, const double *, bool, const uint32_t *, const uint32_t *, double *,
-                                           uint32_t, uint32_t, uint32_t *, const uint2 *, uint32_t, void *, size_t);
+                                           uint32_t, uint32_t, uint32_t *, const uint2 *, uint32_t, void *, size_t, const void *,
+                                           uint32_t);
 template bool bin_event_scatter_usable<float>(uint32_t);
 template bool bin_event_scatter_usable<double>(uint32_t);
 template size_t bin_event_scatter_bytes<float>(uint32_t, uint32_t);

@@ -495,6 +495,38 @@ def test_event_scatter_into_one_window_from_many_rows(cuda, oracle_mod, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_event_scatter_into_one_window_rows_found_by_the_workgroups(cuda, oracle_mod, dtype):
+  # 4,097 to 32,768 rows and at most 8,192 columns: no list, every workgroup numbers the active rows itself
+  # (thread by thread, bit by bit).  The row counts at both ends, empty rows among the active ones, no event,
+  # every row active, bool and float events (also -0.0 and NaN), both weight kinds (the homogeneous one bit
+  # for bit), twice in a row.
+  rng = np.random.default_rng(61)
+  for n_row, n_col, mean in ((4097, 8192, 40), (32_768, 5000, 60), (20_000, 1, 1), (9000, 700, 300), (31_999, 8191, 5)):
+    counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
+    counts[rng.integers(0, n_row, size=n_row // 5)] = 0
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_row)
+    data = rng.standard_normal(indices.shape[0]).astype(dtype)
+    shape = (n_row, n_col)
+    print("shape", shape, dtype.__name__, flush=True)
+    for rate in (0.0, 0.002, 0.1, 1.0):
+      ev = rng.random(n_row) < rate
+      want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True)
+      mag = oracle_mod.event_csr_matvec(np.abs(data), indices, indptr, ev, shape=shape, transpose=True)
+      fev = ev.astype(dtype) * 3
+      fev[~ev] = -0.0
+      if ev.any():
+        fev[np.flatnonzero(ev)[0]] = np.nan
+      for events in (ev, fev):
+        for _ in range(2):
+          got = bpl.event_csr_matvec(data, indices, indptr, events, shape=shape, transpose=True).cpu().numpy()
+          assert_close_reordered(got, want, mag, dtype, what="event scatter, rows found by the workgroups %s rate %g" % (shape, rate))
+      w = np.array([0.6], dtype=dtype)
+      want = oracle_mod.event_csr_matvec(w, indices, indptr, ev, shape=shape, transpose=True)
+      got = bpl.event_csr_matvec(w, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+      assert np.array_equal(got, want), (shape, rate)  # the reference's repeated additions, bit for bit
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_event_scatter_of_few_long_rows(cuda, oracle_mod, dtype):
   # fewer active rows than producer workgroups: several producers share a row, each a part of its nonzeros
   # (5 and about 20 active rows of 34,000; with half of the 700 rows active a producer per row and idle ones),
