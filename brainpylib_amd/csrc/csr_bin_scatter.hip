@@ -886,7 +886,9 @@ __global__ __launch_bounds__(kBinThreads) void active_rows_window_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
     uint32_t n_row, uint32_t n_col, const uint32_t *__restrict__ active_count, const uint2 *__restrict__ active_list,
     uint32_t list_cap, void *__restrict__ partial, uint32_t *__restrict__ groups_out, const void *__restrict__ events,
-    uint32_t event_width) {
+    uint32_t event_width, uint32_t slices, uint32_t slice_cols) {
+  // grid = producers launched * slices: an output wider than one window is taken in `slices` slices of slice_cols
+  // columns by as many sets of workgroups, which all walk the active rows and keep what falls into their slice
   using A = typename std::conditional<HETER, double, uint32_t>::type;  // a window's accumulators
   extern __shared__ __attribute__((aligned(8))) unsigned char smem_raw[];
   A *window = reinterpret_cast<A *>(smem_raw);
@@ -930,11 +932,13 @@ __global__ __launch_bounds__(kBinThreads) void active_rows_window_kernel(
   } else {
     total = active_count[0] < list_cap ? active_count[0] : list_cap;  // (never beyond the list)
   }
-  const uint32_t producers = window_event_producers(total, indptr[n_row], n_row, gridDim.x);
-  const uint32_t p = blockIdx.x;
-  if (p == 0 && tid == 0) groups_out[0] = producers;  // (for the kernel that adds the windows)
+  const uint32_t producers = window_event_producers(total, indptr[n_row], n_row, gridDim.x / slices);
+  const uint32_t p = blockIdx.x / slices, slice = blockIdx.x % slices;
+  if (blockIdx.x == 0 && tid == 0) groups_out[0] = producers;  // (for the kernel that adds the windows)
   if (p >= producers) return;
-  for (uint32_t i = tid; i < n_col; i += kBinThreads) window[i] = A(0);
+  const uint32_t c_lo = slice * slice_cols;
+  const uint32_t width = slices > 1u ? (n_col - c_lo < slice_cols ? n_col - c_lo : slice_cols) : n_col;
+  for (uint32_t i = tid; i < width; i += kBinThreads) window[i] = A(0);
   const uint32_t lo = static_cast<uint32_t>(static_cast<uint64_t>(p) * total / producers);
   const uint32_t hi = static_cast<uint32_t>(static_cast<uint64_t>(p + 1) * total / producers);
 
@@ -1007,17 +1011,18 @@ __global__ __launch_bounds__(kBinThreads) void active_rows_window_kernel(
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-          if (jb + u * kBinThreads < seg_end && col[u] < n_col) {  // (a column beyond the output: left out)
-            if constexpr (HETER) atomicAdd(&window[col[u]], static_cast<double>(val[u]));
-            else atomicAdd(&window[col[u]], 1u);
+          const uint32_t rel = col[u] - c_lo;  // (wraps below the slice; a column beyond the output: left out)
+          if (jb + u * kBinThreads < seg_end && rel < width) {
+            if constexpr (HETER) atomicAdd(&window[rel], static_cast<double>(val[u]));
+            else atomicAdd(&window[rel], 1u);
           }
         }
       }
     }
   }
   __syncthreads();
-  A *mine = static_cast<A *>(partial) + static_cast<size_t>(p) * n_col;
-  for (uint32_t i = tid; i < n_col; i += kBinThreads) mine[i] = window[i];
+  A *mine = static_cast<A *>(partial) + static_cast<size_t>(p) * n_col + c_lo;
+  for (uint32_t i = tid; i < width; i += kBinThreads) mine[i] = window[i];
 }
 
 // y[c] = the sum of the windows of the workgroups that took part (their number: counters[1]), in a fixed order
@@ -1214,25 +1219,42 @@ bool window_event_scatter_usable(uint32_t n_row, uint32_t n_col) {
   return n_col != 0 && n_col <= kWindowEventMaxCols && n_row != 0;
 }
 
-// scratch memory behind the list: the windows of two workgroups per CU
+// Without a list the window shares the LDS with 8 KB of masks: 58 KB of it (7,424 float64 accumulators or
+// 14,848 counts), and an output of up to two such windows of float64 is taken in slices.  (Three and four
+// slices, every slice walking all active nonzeros: 20,000 columns gain 2 us at 5 % events and lose 5 at 20 %
+// against the sorted scatter, 25,000 columns lose at both.)
+constexpr size_t kSelfWindowBytes = 58 * 1024;
+constexpr uint32_t kSelfMaxSlices = 2;
+bool window_event_scatter_self_usable(uint32_t n_row, uint32_t n_col) {
+  return n_col != 0 && n_col <= kSelfMaxSlices * (kSelfWindowBytes / sizeof(double)) && n_row != 0 && n_row <= kSelfListRows;
+}
+
+// scratch memory (behind the list, if there is one): the windows of two workgroups per CU, or, of an output in
+// slices, of as many as take a slice
 template <typename F>
 size_t window_event_scatter_bytes(uint32_t n_col) {
-  return static_cast<size_t>(2u * static_cast<uint32_t>(device_info().num_cu)) * n_col * sizeof(double);
+  const uint32_t resident = 2u * static_cast<uint32_t>(device_info().num_cu);
+  const uint32_t slices = n_col <= kWindowEventMaxCols ? 1u : div_up(n_col, static_cast<uint32_t>(kSelfWindowBytes / sizeof(double)));
+  return static_cast<size_t>(resident / slices) * n_col * sizeof(double);
 }
 
 template <typename F>
 bool window_event_scatter(hipStream_t stream, const F *data, bool heter, const uint32_t *indices, const uint32_t *indptr,
                           F *y, uint32_t n_row, uint32_t n_col, uint32_t *counters, const uint2 *active_list,
                           uint32_t list_cap, void *scratch, size_t scratch_bytes, const void *events, uint32_t event_width) {
-  if (!window_event_scatter_usable<F>(n_row, n_col) || scratch_bytes < window_event_scatter_bytes<F>(n_col)) return false;
   const bool self = events != nullptr;  // no list: the kernel looks at the events itself
-  if (self && (n_row > kSelfListRows || (event_width != 1u && event_width != 4u && event_width != 8u))) return false;
-  const unsigned grid = 2u * static_cast<unsigned>(device_info().num_cu);
-  const size_t lds = static_cast<size_t>(n_col) * (heter ? sizeof(double) : sizeof(uint32_t));
-  // (its 8 KB of masks beside 12.5 KB of row tables: two workgroups must still fit a CU's 160 KB)
-  if (self && lds + 21 * 1024 > 80 * 1024) return false;
+  if (self ? !window_event_scatter_self_usable(n_row, n_col) : !window_event_scatter_usable<F>(n_row, n_col)) return false;
+  if (scratch_bytes < window_event_scatter_bytes<F>(n_col)) return false;
+  if (self && event_width != 1u && event_width != 4u && event_width != 8u) return false;
+  const size_t acc_bytes = heter ? sizeof(double) : sizeof(uint32_t);
+  // (the masks beside 12.5 KB of row tables: two workgroups must still fit a CU's 160 KB)
+  const uint32_t slice_cols = self ? static_cast<uint32_t>(kSelfWindowBytes / acc_bytes) : n_col;
+  const uint32_t slices = self ? div_up(n_col, slice_cols) : 1u;
+  const unsigned launched = 2u * static_cast<unsigned>(device_info().num_cu) / slices;
+  const unsigned grid = launched * slices;
+  const size_t lds = static_cast<size_t>(slices > 1u ? slice_cols : n_col) * acc_bytes;
   using Kernel = void (*)(const F *, const uint32_t *, const uint32_t *, uint32_t, uint32_t, const uint32_t *, const uint2 *,
-                          uint32_t, void *, uint32_t *, const void *, uint32_t);
+                          uint32_t, void *, uint32_t *, const void *, uint32_t, uint32_t, uint32_t);
   const Kernel kernel = heter ? (self ? active_rows_window_kernel<F, true, true> : active_rows_window_kernel<F, true, false>)
                               : (self ? active_rows_window_kernel<F, false, true> : active_rows_window_kernel<F, false, false>);
   static thread_local bool attr_set[2][2] = {{false, false}, {false, false}};
@@ -1245,7 +1267,8 @@ bool window_event_scatter(hipStream_t stream, const F *data, bool heter, const u
     attr_set[heter][self] = true;
   }
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBinThreads), lds, stream, data, indices, indptr, n_row, n_col,
-                     static_cast<const uint32_t *>(counters), active_list, list_cap, scratch, counters + 1, events, event_width);
+                     static_cast<const uint32_t *>(counters), active_list, list_cap, scratch, counters + 1, events, event_width,
+                     slices, slice_cols);
   if (heter)
     hipLaunchKernelGGL((sum_active_windows_kernel<F, true>), dim3(div_up(n_col, kSumCols)), dim3(kSumCols * kSumSlices), 0, stream,
                        static_cast<const void *>(scratch), y, n_col, counters, data);

@@ -1170,6 +1170,28 @@ void launch_scatter(const ScratchSource &src, const F *data, const uint32_t *ind
   const uint32_t n_win = div_up(n_col, win_cap);
   NnzGate direct_gate = kAlways;
   auto round_up = [](size_t v) { return (v + 255) / 256 * 256; };
+  // Event input, 4,097 to 32,768 rows and an output of at most two windows of 7,424 columns: the flat walk over
+  // the active rows' nonzeros into LDS windows (csr_bin_scatter.hip), whose workgroups find the active rows
+  // themselves.  Two launches, where the sorted scatter below needs three and the window kernel further down,
+  // which needs two as well, has 16 workgroups walk their rows one after the other (32,000 x 8,192 with 1,000
+  // per row at 20 % events: 545 us against 31).  (Not from a fixed arena: the walks below need less scratch
+  // memory there.)
+  if constexpr (MODE == kEvent && (sizeof(VT) == 1 || std::is_floating_point<VT>::value)) {
+    if (!src.fixed() && n_row > kSmallRows && window_event_scatter_self_usable(n_row, n_col)) {
+      const size_t need = window_event_scatter_bytes<F>(n_col);
+      size_t got = 0;
+      unsigned char *ws = static_cast<unsigned char *>(src.request(need, need, &got));
+      uint32_t *counters = ws ? src.counters() : nullptr;
+      if (ws != nullptr && counters != nullptr) {
+        if (window_event_scatter<F>(stream, data, HETER, indices, indptr, y, n_row, n_col, counters, nullptr, 0u, ws, got,
+                                    static_cast<const void *>(x), static_cast<uint32_t>(sizeof(VT))))
+          return;
+      } else {
+        if (src.failure_is_final()) return;  // during a capture: the error stands
+        bpl_clear_error();  // no scratch memory: the paths below need less or none
+      }
+    }
+  }
   // Event input and more than 8,192 outputs: the active rows' nonzeros are flattened and sorted
   // coarsely by output window instead (csr_bin_scatter.hip), at a cost that neither grows with the
   // number of windows nor with the number of rows a wave would have to walk in turn.
@@ -1201,29 +1223,7 @@ void launch_scatter(const ScratchSource &src, const F *data, const uint32_t *ind
       bpl_clear_error();  // no scratch memory: the paths below need less or none
     }
   }
-  // Event input and an output of one small window: the flat walk over the active rows' nonzeros
-  // (csr_bin_scatter.hip).  (Not from a fixed arena: the walk below needs less scratch memory there.)
-  // Up to 32,768 rows its workgroups find the active rows themselves: two launches, as the walk below needs,
-  // whose 16 workgroups walk their rows one after the other (32,000 x 8,192 with 1,000 per row at 20 % events:
-  // 545 us against 31; with little activity both take the time of their launches).
-  if constexpr (MODE == kEvent && (sizeof(VT) == 1 || std::is_floating_point<VT>::value)) {
-    if (!src.fixed() && n_row > kSmallRows && n_row <= kWindowEventSelfListRows &&
-        window_event_scatter_usable<F>(n_row, n_col)) {
-      const size_t need = window_event_scatter_bytes<F>(n_col);
-      size_t got = 0;
-      unsigned char *ws = static_cast<unsigned char *>(src.request(need, need, &got));
-      uint32_t *counters = ws ? src.counters() : nullptr;
-      if (ws != nullptr && counters != nullptr) {
-        if (window_event_scatter<F>(stream, data, HETER, indices, indptr, y, n_row, n_col, counters, nullptr, 0u, ws, got,
-                                    static_cast<const void *>(x), static_cast<uint32_t>(sizeof(VT))))
-          return;  // (false: a window of more than 59 KB, which leaves no room for the masks: with the list, below)
-      } else {
-        if (src.failure_is_final()) return;  // during a capture: the error stands
-        bpl_clear_error();  // no scratch memory: the paths below need less or none
-      }
-    }
-  }
-  // A larger matrix (or a window that fills half a CU's LDS): its active rows go to a device list first.
+  // Event input, more rows and an output of one window: the same walk over a device list of the active rows.
   if (MODE == kEvent && !src.fixed() && n_row > kSmallRows && window_event_scatter_usable<F>(n_row, n_col)) {
     const size_t list_sz = round_up(static_cast<size_t>(n_row) * sizeof(uint2));
     const size_t need = list_sz + window_event_scatter_bytes<F>(n_col);

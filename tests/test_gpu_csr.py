@@ -501,7 +501,9 @@ def test_event_scatter_into_one_window_rows_found_by_the_workgroups(cuda, oracle
   # every row active, bool and float events (also -0.0 and NaN), both weight kinds (the homogeneous one bit
   # for bit), twice in a row.
   rng = np.random.default_rng(61)
-  for n_row, n_col, mean in ((4097, 8192, 40), (32_768, 5000, 60), (20_000, 1, 1), (9000, 700, 300), (31_999, 8191, 5)):
+  # Outputs of 7,425 to 14,848 columns are taken in two slices (with one weight in one); wider ones go to the sorted scatter.
+  for n_row, n_col, mean in ((4097, 8192, 40), (32_768, 5000, 60), (20_000, 1, 1), (9000, 700, 300), (31_999, 8191, 5),
+                             (9000, 7425, 30), (10_000, 14_848, 30), (32_768, 14_849, 20)):
     counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
     counts[rng.integers(0, n_row, size=n_row // 5)] = 0
     indices, indptr = synth.counted_csr(counts, n_col, seed=n_row)
