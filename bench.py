@@ -718,6 +718,27 @@ def main():
                                       gsop_per_s=delivered / (dur_w.mean() * 1e-3) / 1e9)
     extra["scatter_1e6x1e6_100_per_row"] = wide
     log("event scatter 1e6 x 1e6: %s" % wide)
+    # a mid-size projection, 32,000 x 8,192 with about 1,000 nonzeros per row: the walk into LDS windows whose
+    # workgroups find the active rows themselves, at three activities
+    counts_m = np.maximum(1, np.random.default_rng(23).poisson(1000, 32_000))
+    ix_m, ip_m = synth.counted_csr(counts_m, 8192, seed=5)
+    d_m = np.random.default_rng(24).random(ix_m.shape[0], dtype=np.float32)
+    dev_m = [torch.from_numpy(a).to(dev) for a in (d_m, ix_m, ip_m)]
+    mid = {}
+    for rate in (0.01, 0.05, 0.2):
+      ev_np = np.random.default_rng(25).random(32_000) < rate
+      ev_m = torch.from_numpy(ev_np).to(dev)
+      want = oracle.event_csr_matvec(d_m, ix_m, ip_m, ev_np, shape=(32_000, 8192), transpose=True)
+      mag = oracle.event_csr_matvec(np.abs(d_m), ix_m, ip_m, ev_np, shape=(32_000, 8192), transpose=True)
+      got = bpl.event_csr_matvec(*dev_m, ev_m, shape=(32_000, 8192), transpose=True)
+      check(got.cpu().numpy(), want, "event_csr_matvec scatter 32,000 x 8,192 at %g" % rate, mag)
+      dur_m, _ = time_calls(lambda: bpl.event_csr_matvec(*dev_m, ev_m, shape=(32_000, 8192), transpose=True), args.steps, 5)
+      delivered = int(np.diff(ip_m)[ev_np].sum())
+      mid["events_%g" % rate] = dict(stats(dur_m), delivered_synapses=delivered,
+                                     gsop_per_s=delivered / (dur_m.mean() * 1e-3) / 1e9)
+    extra["scatter_32000x8192_1000_per_row"] = mid
+    log("event scatter 32,000 x 8,192: %s" % mid)
+    del dev_m
 
   if not args.skip_extra:
     del md
