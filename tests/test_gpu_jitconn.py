@@ -404,6 +404,39 @@ def test_column_walk_through_bins_dense(cuda, oracle_mod, w_kind, a, b, dtype):
   assert abs(y @ Mx - MTy @ x64) <= 1e-9 * max(1.0, abs(y @ Mx))
 
 
+@pytest.mark.parametrize("w_kind,a,b", [("homo", 0.0, 0.0), ("normal", 0.5, 2.0)])
+@pytest.mark.parametrize("n_out,n_in,p", [(4000, 4000, 0.02), (700, 90, 0.3), (5, 3, 0.9), (30_000, 2047, 0.01)])
+def test_column_walk_dense_with_few_pairs(cuda, oracle_mod, w_kind, a, b, n_out, n_in, p):
+  # dense input and fewer than 2^20 possible pairs: every column's generator is seeded ahead and the walk adds
+  # its pairs to the output with atomics (no bins).  Against the oracle's column walk; integer input, so the
+  # homogeneous sums are exact.  And a bound on the time: with every lane seeding its own column's generator
+  # the first shape took 0.5 ms.
+  lp = oracle_mod.log_p_of(p)
+  x = np.random.default_rng(n_in).integers(-3, 4, n_in).astype(np.float32)
+  kw = dict(w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=33, n_row=n_out, n_col=n_in, col_walk=True, dense=True)
+  got = kernel_call(x, **kw)
+  want = oracle_mod.jitconn_matvec(x, **kw)
+  if w_kind == "homo":
+    assert np.array_equal(got, want)
+  else:
+    mag = np.full(n_out, 3.0 * (abs(a) + 5 * abs(b)) * (n_in * p * 2 + 8))
+    assert_close_reordered(got, want, mag, np.float32, what="dense column walk with few pairs")
+  if n_out == 4000 and w_kind == "homo":
+    xd = torch.from_numpy(x).cuda()
+    call = lambda: bpl.matvec_prob_conn_homo_weight(xd, 0.5, conn_prob=p, shape=(n_out, n_in), seed=33, outdim_parallel=False)
+    call()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+      call()
+    e1.record()
+    torch.cuda.synchronize()
+    per_call_us = e0.elapsed_time(e1) * 1e3 / 5
+    print("dense column walk 4,000 x 4,000: %.1f us per call" % per_call_us, flush=True)
+    assert per_call_us < 300.0
+
+
 def test_column_walk_through_bins_sliced_windows(cuda, oracle_mod):
   # more than 2^21 outputs: the bins' windows are wider than their accumulators in LDS and are
   # added in slices
