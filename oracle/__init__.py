@@ -22,7 +22,10 @@ jitconn_matvec (per-stream)     row r == compiled reference with one stream and 
                                 closed form at conn_prob >= 1; geometric-gap statistics;
                                 adjoint identity <y, Mx> == <M^T y, x>; shape-swap identity
 jitconn_matmat                  reference test identity matmat == vmap(matvec(transpose=True));
-                                no reference CPU kernel exists for it
+                                no reference CPU kernel exists for it.  The one-pass form
+                                (each stream generated once) == that definition bit for bit
+                                (tests/test_oracle_jitconn.py); abs sums == float64 numpy on the
+                                explicit matrix
 event_csr_matvec                dense matmul brute force, scipy.sparse, homo == heter(ones*w),
                                 bool == float events, compiled lib/cpu_event_sum.cc (transpose,
                                 bool events)
@@ -154,9 +157,11 @@ def jitconn_stream_weights(seed, w_kind, w_a, w_b, log_p, n, dtype=np.float32, c
 # jitconn operators
 # ---------------------------------------------------------------------------------------------
 def jitconn_matvec(inp, *, w_kind="homo", w_a=0.0, w_b=0.0, log_p, seed, n_row, n_col,
-                   col_walk=False, per_stream_seed=True, out_dtype=None, dense=None):
+                   col_walk=False, per_stream_seed=True, out_dtype=None, dense=None, return_abs=False):
   """Kernel-level jitconn (event) matvec: returns the custom call's result (for ``homo`` that is
   the count / plain sum; the weight is applied by the caller as the reference does).
+  ``return_abs=True`` returns ``(result, abs_sum)``, abs_sum[o] = sum of |addend| over the
+  addends of output o in float64 (what bounds the effect of another order of the additions).
 
   ``inp`` bool -> event input; float with dense=False -> float events (truthiness);
   float with dense=True -> dense vector.  ``n_row`` outputs, ``n_col`` inputs.
@@ -176,25 +181,40 @@ def jitconn_matvec(inp, *, w_kind="homo", w_a=0.0, w_b=0.0, log_p, seed, n_row, 
   assert out_dtype in (np.dtype(np.float32), np.dtype(np.float64))
   out = np.empty(n_row, dtype=out_dtype)
   f32 = out_dtype == np.float32
-  fn = lib().oracle_jitconn_matvec_f32 if f32 else lib().oracle_jitconn_matvec_f64
   ft = ctypes.c_float if f32 else ctypes.c_double
-  fn(_p(buf), ctypes.c_int(in_kind), ctypes.c_int(_W_KINDS[w_kind]), ft(w_a), ft(w_b),
-     ctypes.c_double(log_p), ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_uint32(n_row),
-     ctypes.c_uint32(n_col), ctypes.c_int(int(col_walk)), ctypes.c_int(int(per_stream_seed)), _p(out))
+  args = (_p(buf), ctypes.c_int(in_kind), ctypes.c_int(_W_KINDS[w_kind]), ft(w_a), ft(w_b),
+          ctypes.c_double(log_p), ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_uint32(n_row),
+          ctypes.c_uint32(n_col), ctypes.c_int(int(col_walk)), ctypes.c_int(int(per_stream_seed)), _p(out))
+  if return_abs:
+    abs_sum = np.empty(n_row, dtype=np.float64)
+    (lib().oracle_jitconn_matvec_abs_f32 if f32 else lib().oracle_jitconn_matvec_abs_f64)(*args, _p(abs_sum))
+    return out, abs_sum
+  (lib().oracle_jitconn_matvec_f32 if f32 else lib().oracle_jitconn_matvec_f64)(*args)
   return out
 
 
-def jitconn_matmat(X, *, w_kind="normal", w_a, w_b, log_p, seed, n):
-  """Y[m, n] = X[m, k] @ M[k, n]; column j of M is generator stream seed + j."""
+def jitconn_matmat(X, *, w_kind="normal", w_a, w_b, log_p, seed, n, return_abs=False, by_rows=False):
+  """Y[m, n] = X[m, k] @ M[k, n]; column j of M is generator stream seed + j.
+
+  ``by_rows=True`` is the definition taken literally (one matvec per row of X, the identity of
+  brainpylib/_src/jitconn_ops/tests/matmat_testcase.py:133-138); the default generates every
+  stream once and applies it to all rows, bit for bit the same result.  ``return_abs=True``
+  returns ``(Y, abs_sum)`` with abs_sum[mi, j] = sum of |w * X[mi, i]| over column j's synapses."""
   X = np.ascontiguousarray(X)
   m, k = X.shape
   Y = np.empty((m, n), dtype=X.dtype)
   f32 = X.dtype == np.float32
-  fn = lib().oracle_jitconn_matmat_f32 if f32 else lib().oracle_jitconn_matmat_f64
   ft = ctypes.c_float if f32 else ctypes.c_double
-  fn(_p(X), ctypes.c_int(_W_KINDS[w_kind]), ft(w_a), ft(w_b), ctypes.c_double(log_p),
-     ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_uint32(m), ctypes.c_uint32(k), ctypes.c_uint32(n), _p(Y))
-  return Y
+  args = (_p(X), ctypes.c_int(_W_KINDS[w_kind]), ft(w_a), ft(w_b), ctypes.c_double(log_p),
+          ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_uint32(m), ctypes.c_uint32(k), ctypes.c_uint32(n), _p(Y))
+  if by_rows:
+    assert not return_abs
+    (lib().oracle_jitconn_matmat_by_rows_f32 if f32 else lib().oracle_jitconn_matmat_by_rows_f64)(*args)
+    return Y
+  abs_sum = np.empty((m, n), dtype=np.float64) if return_abs else None
+  (lib().oracle_jitconn_matmat_f32 if f32 else lib().oracle_jitconn_matmat_f64)(
+    *args, _p(abs_sum) if return_abs else ctypes.c_void_p(None))
+  return (Y, abs_sum) if return_abs else Y
 
 
 # ---------------------------------------------------------------------------------------------

@@ -149,10 +149,10 @@ def test_row_walk_with_a_two_level_event_bitmap(cuda, oracle_mod, n_in):
     got = kernel_call(inp, w_kind="homo", log_p=lp, seed=77, n_row=n_out, n_col=n_in, col_walk=False, dense=False)
     assert want.sum() > 0 and np.array_equal(got, want)
   for w_kind, a, b in (("uniform", 0.25, 1.75), ("normal", 0.5, 2.0)):
-    want = oracle_mod.jitconn_matvec(ev, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=77, n_row=n_out, n_col=n_in)
+    want, mag = oracle_mod.jitconn_matvec(ev, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=77, n_row=n_out, n_col=n_in,
+                                          return_abs=True)
     got = kernel_call(ev, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=77, n_row=n_out, n_col=n_in, col_walk=False,
                       dense=False)
-    mag = np.full(n_out, (abs(a) + 5 * abs(b)) * 80)  # about 40 active synapses per row
     assert_close_reordered(got, want, mag, np.float32, what="two-level row walk %s" % w_kind)
 
 
@@ -330,10 +330,9 @@ def test_matmat_against_oracle_and_vmapped_matvec(cuda, oracle_mod, m, dtype):
   got = bpl.matmat_prob_conn_uniform_weight(X, w_low=-0.5, w_high=1.5, conn_prob=p, shape=(k, n), seed=seed).cpu().numpy()
   assert got.shape == (m, n) and np.array_equal(got, want)
   # normal weights: logf/sqrtf of the device vs libm may differ in the last place
-  want = oracle_mod.jitconn_matmat(X, w_kind="normal", w_a=0.0, w_b=0.01, log_p=lp, seed=seed, n=n)
+  want, mag = oracle_mod.jitconn_matmat(X, w_kind="normal", w_a=0.0, w_b=0.01, log_p=lp, seed=seed, n=n, return_abs=True)
   got_t = bpl.matmat_prob_conn_normal_weight(X, w_mu=0.0, w_sigma=0.01, conn_prob=p, shape=(k, n), seed=seed)
   got = got_t.cpu().numpy()
-  mag = oracle_mod.jitconn_matmat(np.abs(X), w_kind="uniform", w_a=0.05, w_b=0.0500001, log_p=lp, seed=seed, n=n)
   assert_close_reordered(got, want, mag, dtype, what="matmat normal")
   # the reference tests' identity: matmat(X) == vmap(matvec(transpose=True))(X)
   for i in range(0, m, max(1, m // 4)):
@@ -362,18 +361,24 @@ def test_config_jitconn_matmat_full_size(cuda, oracle_mod):
   X = np.ascontiguousarray(c["B"].T)
   oracle_mod.set_threads(min(16, len(os.sched_getaffinity(0))))
   lp = oracle_mod.log_p_of(c["conn_prob"])
-  # the oracle on 16 of the 128 rows of X (each regenerates all 10,000 streams: ~1e7 draws per row)
-  rows = np.arange(0, 128, 8)
-  want = oracle_mod.jitconn_matmat(X[rows], w_kind="normal", w_a=c["w_mu"], w_b=c["w_sigma"], log_p=lp, seed=c["seed"],
-                                   n=c["shape"][1])
+  # the oracle on all 128 rows (every stream generated once and applied to every row of X), with
+  # sum(|w x|) per output: the reordering term of the tolerance is computed, not estimated
+  want, mag = oracle_mod.jitconn_matmat(X, w_kind="normal", w_a=c["w_mu"], w_b=c["w_sigma"], log_p=lp, seed=c["seed"],
+                                        n=c["shape"][1], return_abs=True)
+  # the definition itself (one matvec per row of X) on two rows
+  rows = np.array([0, 127])
+  by_rows = oracle_mod.jitconn_matmat(X[rows], w_kind="normal", w_a=c["w_mu"], w_b=c["w_sigma"], log_p=lp,
+                                      seed=c["seed"], n=c["shape"][1], by_rows=True)
   oracle_mod.set_threads(1)
+  assert np.array_equal(by_rows, want[rows])
   got = bpl.matmat_prob_conn_normal_weight(X, w_mu=c["w_mu"], w_sigma=c["w_sigma"], conn_prob=c["conn_prob"],
                                            shape=c["shape"], seed=c["seed"]).cpu().numpy()
   assert got.shape == (128, 10000)
-  # |addends| bound: sum_i |w| |x_i| <= about 0.05 * sum of |x| over the ~1000 connected inputs
-  err = np.abs(got[rows].astype(np.float64) - want)
-  bound = 1e-6 + 1e-5 * np.abs(want) + 4 * np.finfo(np.float32).eps * 0.05 * 1000
-  assert (err <= bound).all(), float(err.max())
+  # the kernel adds in the oracle's order; what differs is the device's logf / sqrtf in the normal
+  # weights (within 4 ulp each): 4 eps sum(|w x|) covers that too
+  outside = assert_close_reordered(got, want, mag, np.float32, what="matmat 10,000 x 10,000 x 128")
+  print("matmat full size: %d of %d outside plain rel 1e-5 / abs 1e-6; max abs err %.3e"
+        % (outside, got.size, float(np.abs(got - want).max())), flush=True)
 
 
 @pytest.mark.parametrize("w_kind,a,b", [("homo", 0.0, 0.0), ("uniform", 0.25, 1.75), ("normal", 0.5, 2.0)])
@@ -388,14 +393,11 @@ def test_column_walk_through_bins_dense(cuda, oracle_mod, w_kind, a, b, dtype):
   x = rng.integers(-3, 4, n_in).astype(dtype)
   got = kernel_call(x, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=21, n_row=n_out, n_col=n_in, col_walk=True,
                     dense=True)
-  want = oracle_mod.jitconn_matvec(x, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=21, n_row=n_out, n_col=n_in,
-                                   col_walk=True, dense=True)
+  want, mag = oracle_mod.jitconn_matvec(x, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=21, n_row=n_out, n_col=n_in,
+                                        col_walk=True, dense=True, return_abs=True)
   if w_kind == "homo":
     assert np.array_equal(got, want)
   else:
-    # bound on the sum of |addends| per output: |x| <= 3, |w| <= |a| + 5 |b| (5 sigma / the uniform range),
-    # about n_in * p addends, doubled
-    mag = np.full(n_out, 3.0 * (abs(a) + 5 * abs(b)) * n_in * 0.05 * 2)
     assert_close_reordered(got, want, mag, dtype, what="binned column walk %s" % w_kind)
   y = rng.integers(-3, 4, n_out).astype(np.float64)
   x64 = x.astype(np.float64)
@@ -415,11 +417,10 @@ def test_column_walk_dense_with_few_pairs(cuda, oracle_mod, w_kind, a, b, n_out,
   x = np.random.default_rng(n_in).integers(-3, 4, n_in).astype(np.float32)
   kw = dict(w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=33, n_row=n_out, n_col=n_in, col_walk=True, dense=True)
   got = kernel_call(x, **kw)
-  want = oracle_mod.jitconn_matvec(x, **kw)
+  want, mag = oracle_mod.jitconn_matvec(x, return_abs=True, **kw)
   if w_kind == "homo":
     assert np.array_equal(got, want)
   else:
-    mag = np.full(n_out, 3.0 * (abs(a) + 5 * abs(b)) * (n_in * p * 2 + 8))
     assert_close_reordered(got, want, mag, np.float32, what="dense column walk with few pairs")
   if n_out == 4000 and w_kind == "homo":
     xd = torch.from_numpy(x).cuda()
@@ -446,12 +447,11 @@ def test_column_walk_through_bins_sliced_windows(cuda, oracle_mod):
   x = rng.integers(-3, 4, n_in).astype(np.float32)
   for w_kind, a, b in (("homo", 0.0, 0.0), ("uniform", 0.25, 1.75)):
     got = kernel_call(x, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=5, n_row=n_out, n_col=n_in, col_walk=True, dense=True)
-    want = oracle_mod.jitconn_matvec(x, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=5, n_row=n_out, n_col=n_in,
-                                     col_walk=True, dense=True)
+    want, mag = oracle_mod.jitconn_matvec(x, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=5, n_row=n_out, n_col=n_in,
+                                          col_walk=True, dense=True, return_abs=True)
     if w_kind == "homo":
       assert np.array_equal(got, want)
     else:
-      mag = np.full(n_out, 3.0 * (abs(a) + abs(b)) * 16)
       assert_close_reordered(got, want, mag, np.float32, what="sliced binned column walk")
 
 
@@ -495,14 +495,14 @@ def test_random_shapes_walks_weights_and_inputs_against_oracle(cuda, oracle_mod,
       inp, dense = rng.integers(-3, 4, n_in).astype(dtype), True
     stream_seed = int(rng.integers(0, 2 ** 31))
     print("case", case, n_out, n_in, col_walk, "%.2e" % p, w_kind, kind, dtype.__name__, flush=True)
-    want = oracle_mod.jitconn_matvec(inp, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=stream_seed, n_row=n_out,
-                                     n_col=n_in, col_walk=col_walk, dense=(None if kind == "bool" else dense))
+    want, mag = oracle_mod.jitconn_matvec(inp, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=stream_seed, n_row=n_out,
+                                          n_col=n_in, col_walk=col_walk, dense=(None if kind == "bool" else dense),
+                                          return_abs=True)
     got = kernel_call(inp, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=stream_seed, n_row=n_out, n_col=n_in,
                       col_walk=col_walk, dense=dense)
     if w_kind == "homo":
       assert np.array_equal(got, want)  # counts / sums of small integers
     else:
-      mag = np.full(n_out, 3.0 * (abs(a) + 5 * abs(b)) * (syn * 3 + 20))
       assert_close_reordered(got, want, mag, np.float32 if kind == "bool" else dtype, what="case %d" % case)
 
 
@@ -589,10 +589,8 @@ def test_row_walk_with_generators_seeded_inside_the_kernel(cuda, oracle_mod, n_o
       assert want.any() and np.array_equal(got.astype(np.float64), want.astype(np.float64)), (inp.dtype, dense)
   for w_kind, a, b in (("uniform", 0.25, 1.75), ("normal", 0.5, 2.0)):
     for inp, dense, dt in ((ev, False, np.float32), (vec.astype(np.float32), True, np.float32), (vec, True, np.float64)):
-      want = oracle_mod.jitconn_matvec(inp, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=5, n_row=n_out, n_col=n_in,
-                                       dense=dense, per_stream_seed=True)
+      want, mag = oracle_mod.jitconn_matvec(inp, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=5, n_row=n_out, n_col=n_in,
+                                            dense=dense, per_stream_seed=True, return_abs=True)
       got = kernel_call(inp, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=5, n_row=n_out, n_col=n_in, col_walk=False,
                         dense=dense)
-      # about 200 synapses per row (20 of them active for events), inputs up to 3 in magnitude
-      mag = np.full(n_out, (abs(a) + 5 * abs(b)) * (3 * 260 if dense else 60))
       assert_close_reordered(got, want, mag, dt, what="fused row walk %s" % w_kind)

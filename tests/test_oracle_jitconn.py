@@ -173,3 +173,48 @@ def test_matmat_is_vmapped_transposed_matvec(oracle_mod):
     yi = oracle_mod.jitconn_matvec(X[i], w_kind="normal", w_a=0.0, w_b=0.01, log_p=lp, seed=7, n_row=n, n_col=k,
                                    dense=True, per_stream_seed=True)
     assert np.array_equal(Y[i], yi)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("w_kind,a,b", [("homo", 0.0, 0.0), ("uniform", -0.5, 1.5), ("normal", 0.0, 0.01)])
+def test_matmat_one_pass_equals_the_definition_and_its_abs_sums(oracle_mod, dtype, w_kind, a, b):
+  # the one-pass form (each stream generated once, applied to all rows of X) against the
+  # definition taken literally, bit for bit; its abs sums against |M| @ |X| of the explicit matrix
+  m, k, n, seed = 7, 90, 50, 13
+  X = np.random.default_rng(4).standard_normal((m, k)).astype(dtype)
+  lp = oracle_mod.log_p_of(0.15)
+  kw = dict(w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=seed, n=n)
+  oracle_mod.set_threads(3)
+  Y, mag = oracle_mod.jitconn_matmat(X, return_abs=True, **kw)
+  oracle_mod.set_threads(1)
+  assert np.array_equal(Y, oracle_mod.jitconn_matmat(X, by_rows=True, **kw))
+  assert np.array_equal(Y, oracle_mod.jitconn_matmat(X, **kw))
+  M = np.zeros((k, n))
+  for j in range(n):
+    idx, w = oracle_mod.jitconn_stream_weights(seed + j, w_kind, a, b, lp, k, dtype=dtype)
+    M[idx, j] = w
+  assert_close(mag, np.abs(X).astype(np.float64) @ np.abs(M), rtol=1e-6, atol=1e-12)
+  assert_close(Y, X.astype(np.float64) @ M, rtol=1e-4, atol=1e-4 * float(mag.max()))
+
+
+@pytest.mark.parametrize("col_walk", [False, True])
+@pytest.mark.parametrize("kind", ["bool", "dense"])
+def test_matvec_abs_sums(oracle_mod, col_walk, kind):
+  # abs_sum[o] = sum |addend| == the same walk over |weights| and |input|; the result is unchanged
+  n_out, n_in, seed = 35, 80, 3
+  lp = oracle_mod.log_p_of(0.2)
+  rng = np.random.default_rng(9)
+  inp = (rng.random(n_in) < 0.4) if kind == "bool" else rng.standard_normal(n_in)
+  kw = dict(w_kind="normal", w_a=0.0, w_b=1.0, log_p=lp, seed=seed, n_row=n_out, n_col=n_in, col_walk=col_walk,
+            dense=(None if kind == "bool" else True), out_dtype=np.float64)
+  out, mag = oracle_mod.jitconn_matvec(inp, return_abs=True, **kw)
+  assert np.array_equal(out, oracle_mod.jitconn_matvec(inp, **kw))
+  M = np.zeros((n_out, n_in))
+  for s in range(n_in if col_walk else n_out):
+    idx, w = oracle_mod.jitconn_stream_weights(seed + s, "normal", 0.0, 1.0, lp, n_out if col_walk else n_in,
+                                               dtype=np.float64)
+    if col_walk:
+      M[idx, s] = w
+    else:
+      M[s, idx] = w
+  assert_close(mag, np.abs(M) @ np.abs(inp.astype(np.float64)), rtol=1e-12, atol=1e-12)
