@@ -56,6 +56,13 @@ def load_kernels():
   lib.bench_gather_fma4.restype = i
   lib.bench_stream.argtypes = [vp, vp, vp, u64, i, i]
   lib.bench_stream.restype = i
+  u32 = ctypes.c_uint32
+  lib.bench_lds_atomic.argtypes = [vp, vp, i, i, i]
+  lib.bench_lds_atomic.restype = i
+  lib.bench_global_atomic.argtypes = [vp, vp, u32, i, i, i]
+  lib.bench_global_atomic.restype = i
+  lib.bench_l2_read.argtypes = [vp, vp, vp, u32, i, i]
+  lib.bench_l2_read.restype = i
   return lib
 
 
@@ -80,13 +87,27 @@ def recorded_counters(key, kernel_us, tolerance=0.05, **must_match):
   return entry
 
 
-def time_calls(fn, steps, warmup):
+# The device raises its clocks only under sustained load: for the first 50-100 ms after an idle spell (a host-side
+# oracle computation, say) kernels that are bound by instruction issue run 15-20 % slower (jitconn matmat: 285 us
+# against 240 us from the hundredth call on).  Every timed region is therefore preceded by at least this much
+# untimed work of the same kind, beyond the W warm-up calls asked for.
+CLOCK_WARM_S = 0.15
+
+
+def time_calls(fn, steps, warmup, warm_s=None):
   """Per-call GPU durations (HIP events on the stream the kernels are enqueued on) and the
-  wall time of the K back-to-back calls."""
+  wall time of the K back-to-back calls.  Untimed before them: `warmup` calls, then further calls
+  until `warm_s` seconds (default CLOCK_WARM_S) have passed since the first one."""
   import torch
+  warm_s = CLOCK_WARM_S if warm_s is None else warm_s
+  tw = time.perf_counter()
   for _ in range(warmup):
     fn()
   torch.cuda.synchronize()
+  while time.perf_counter() - tw < warm_s:
+    for _ in range(4):
+      fn()
+    torch.cuda.synchronize()
   starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
   ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
   t0 = time.perf_counter()
@@ -229,6 +250,63 @@ def check(got, want, what, mag=None):
   return outside_plain
 
 
+def parity_record(got, outside_plain, bound):
+  """What a leg says about its parity gate: how many elements were compared, how many of them lay outside the
+  plain rel 1e-5 / abs 1e-6 bound (and passed through the reordering term only), violations (always 0: a
+  violation ends the run), and which bound applied."""
+  return dict(elements=int(np.asarray(got).size), outside_plain=int(outside_plain), violations=0, bound=bound)
+
+
+def roofline_record(bound, achieved, peak, unit, **more):
+  return dict(bound=bound, achieved=float(achieved), peak=float(peak), unit=unit, frac=float(achieved) / float(peak), **more)
+
+
+def device_rates(lib, dev):
+  """Rates of the device's building blocks that the kernels' designs are argued from, measured in this run:
+  LDS read-modify-writes by type, atomic adds in device memory (random addresses; one address), and the rate at
+  which the L2s deliver lines of a buffer that stays resident in them.  A few milliseconds in all."""
+  import ctypes
+  import torch
+  stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+  cu = torch.cuda.get_device_properties(dev).multi_processor_count
+  rates = {}
+
+  def timed(fn, reps=5):
+    if fn() != 0:
+      raise SystemExit("a device-rate kernel failed to launch")
+    d, _ = time_calls(fn, reps, 2, warm_s=0.05)
+    return float(np.median(d)) * 1e-3  # seconds
+
+  blocks, iters = 2 * cu, 2048
+  out = torch.zeros(blocks, dtype=torch.float32, device=dev)
+  ops = blocks * 1024 * iters
+  base = timed(lambda: lib.bench_lds_atomic(stream, out.data_ptr(), blocks, iters, 4))
+  for mode, name in ((0, "lds_add_f32"), (1, "lds_add_u32"), (2, "lds_add_f64"), (3, "lds_write_b32")):
+    t = timed(lambda: lib.bench_lds_atomic(stream, out.data_ptr(), blocks, iters, mode))
+    rates[name + "_g_per_s"] = ops / t / 1e9
+    rates[name + "_g_per_s_less_address_arithmetic"] = ops / max(t - base, 1e-9) / 1e9
+  rates["lds_workload"] = "%d workgroups of 1,024 threads, %d random operations per thread in a 64 KB window" % (blocks, iters)
+  for n in (100_000, 1_000_000, 16_000_000):
+    y = torch.zeros(n, dtype=torch.float32, device=dev)
+    gb, gi = 4096, 64
+    t = timed(lambda: lib.bench_global_atomic(stream, y.data_ptr(), n, gb, gi, 0))
+    rates["global_atomic_add_f32_random_%d_g_per_s" % n] = gb * 256 * gi / t / 1e9
+    del y
+  cnt = torch.zeros(64, dtype=torch.int32, device=dev)
+  sb, si = 512, 256
+  t = timed(lambda: lib.bench_global_atomic(stream, cnt.data_ptr(), 1, sb, si, 1))
+  rates["global_atomic_same_address_ns_each"] = t / (sb * si) * 1e9
+  # 2 MB: well inside each 4 MB L2
+  n16 = (2 << 20) // 16
+  buf = torch.empty(n16 * 4, dtype=torch.int32, device=dev).random_()
+  for per_cu in (1, 2):
+    lb, reps = cu * per_cu, 16
+    o2 = torch.zeros(lb * 1024, dtype=torch.int32, device=dev)
+    t = timed(lambda: lib.bench_l2_read(stream, buf.data_ptr(), o2.data_ptr(), n16, reps, lb))
+    rates["l2_read_2MB_%d_workgroups_per_cu_tb_per_s" % per_cu] = lb * reps * n16 * 16.0 / t / 1e12
+  return rates
+
+
 def reference_shapes(bpl, synth, torch, dev):
   """The reference's benchmark scripts time 100 jitted calls including dispatch on an unstated GPU; their
   docstring figures (seconds per 100 calls) are quoted as ms per call.  Ours: mean HIP-event time per call."""
@@ -286,6 +364,9 @@ def main():
                        "of jitconn event matvec (1e6 x 1e6, p=0.001) in both walks.  jitconn-normal: three "
                        "row walks of the same matrix with normal weights.  jitconn-dense: three row walks over a "
                        "dense vector.  matmat: three calls of jitconn matmat 10,000 x 10,000 x 128.  Nothing else runs.")
+  ap.add_argument("--rates", action="store_true",
+                  help="only the device's building-block rates (LDS atomics by type, atomics in device memory, L2 line "
+                       "delivery): one JSON line {\"device_rates\": ...}")
   ap.add_argument("--reference-shapes", action="store_true",
                   help="instead of the headline run: the shapes of the reference's own benchmark scripts "
                        "(event_matvec_jitconn_performance.py, csr_matvec_VS_cusparse_csr_matvec.py), with the "
@@ -307,6 +388,10 @@ def main():
 
   if args.reference_shapes:
     reference_shapes(bpl, synth, torch, dev)
+    return
+
+  if args.rates:
+    print(json.dumps({"device_rates": device_rates(load_kernels(), dev)}), flush=True)
     return
 
   if args.pmc == "jitconn":
@@ -398,12 +483,12 @@ def main():
   cold_gather_us = (time.perf_counter() - t1) * 1e6  # this process's first call of the operator
   got_g = got_dev.cpu().numpy()
   del got_dev
-  check(got_g, want_g, "event_csr_matvec gather 1e8 nnz")
+  outside_g = check(got_g, want_g, "event_csr_matvec gather 1e8 nnz")
   want_s = oracle.event_csr_matvec(c["data"], c["indices"], c["indptr"], c["events"], shape=c["shape"], transpose=True)
   mag_s = oracle.event_csr_matvec(np.abs(c["data"]), c["indices"], c["indptr"], c["events"], shape=c["shape"],
                                   transpose=True)
   got_s = bpl.event_csr_matvec(data, indices, indptr, events, shape=c["shape"], transpose=True).cpu().numpy()
-  check(got_s, want_s, "event_csr_matvec scatter 1e8 nnz", mag_s)
+  outside_s = check(got_s, want_s, "event_csr_matvec scatter 1e8 nnz", mag_s)
 
   if args.pmc == "scatter":
     for _ in range(3):
@@ -452,13 +537,17 @@ def main():
   log("gather: %.1f us/call (events) %.1f us/step (wall)  %.1f GSOP/s  %.0f GB/s algorithmic" % (
     kernel_ms * 1e3, ms_per_step * 1e3, value, achieved))
 
-  extra = {"gather_call_us": stats(dur), "nnz": nnz, "hits": hits, "active_rows": active}
+  extra = {"gather_call_us": stats(dur), "nnz": nnz, "hits": hits, "active_rows": active,
+           "gather_parity": parity_record(got_g, outside_g, "rel 1e-5 / abs 1e-6 (the row sums are formed in the "
+                                                            "oracle's order in float64 and rounded once)")}
   one = single_call_us(gather)
   copy_rate = copy_bandwidth_gb_per_s(dev)
   extra["hbm_copy_gb_per_s"] = copy_rate  # 1 GiB device-to-device copy, read + write
   log("device-to-device copy of 1 GiB: %.0f GB/s (read + write)" % copy_rate)
   # what plain 16-byte loads over the same number of bytes reach at this kernel's occupancy
   bench_lib = load_kernels()
+  extra["device_rates"] = device_rates(bench_lib, dev)
+  log("device rates: %s" % extra["device_rates"])
   rec = recorded_counters("event_csr_gather_1e8", kernel_ms * 1e3, nnz=nnz)
   traffic = float(rec["hbm_bytes_per_launch"]) if rec else None
   streams = stream_ceiling(bench_lib, dev, int(traffic) if traffic else bytes_gather, 20)
@@ -497,7 +586,11 @@ def main():
     extra["scatter_1e8"] = dict(stats(dur_s), delivered_synapses=delivered,
                                 gsop_per_s=delivered / (dur_s.mean() * 1e-3) / 1e9,
                                 algorithmic_gb_per_s=bytes_scatter / (dur_s.mean() * 1e-3) / 1e9,
-                                wall_us_per_call=wall_s / args.steps * 1e6)
+                                wall_us_per_call=wall_s / args.steps * 1e6,
+                                roofline=roofline_record("hbm", bytes_scatter / (dur_s.mean() * 1e-3) / 1e9, HBM_PEAK_GBS,
+                                                         "GB/s", algorithmic_bytes_per_call=bytes_scatter,
+                                                         launches_per_call=2),
+                                parity=parity_record(got_s, outside_s, "rel 1e-5 / abs 1e-6 + 4 eps sum|addends|"))
     if not args.skip_cpu:
       t1 = time.perf_counter()
       for _ in range(20):
@@ -520,8 +613,16 @@ def main():
     dur_h, _ = time_calls(lambda: bpl.event_csr_matvec(w, indices, indptr, events, shape=c["shape"]), args.steps,
                           args.warmup)
     bytes_h = 4 * (n_row + 1) + 4 * nnz + n_col + 4 * n_row
+    got_h = bpl.event_csr_matvec(w, indices, indptr, events, shape=c["shape"]).cpu().numpy()
+    want_h = oracle.event_csr_matvec(np.array([0.6], np.float32), c["indices"], c["indptr"], c["events"], shape=c["shape"])
+    if not np.array_equal(got_h, want_h):
+      raise SystemExit("parity gate failed for the homogeneous gather (bit for bit)")
     extra["gather_homo_1e8"] = dict(stats(dur_h), gsop_per_s=nnz / (dur_h.mean() * 1e-3) / 1e9,
-                                    algorithmic_gb_per_s=bytes_h / (dur_h.mean() * 1e-3) / 1e9)
+                                    algorithmic_gb_per_s=bytes_h / (dur_h.mean() * 1e-3) / 1e9,
+                                    roofline=roofline_record("hbm", bytes_h / (dur_h.mean() * 1e-3) / 1e9, HBM_PEAK_GBS,
+                                                             "GB/s", algorithmic_bytes_per_call=bytes_h),
+                                    parity=dict(elements=int(got_h.size), outside_plain=0, violations=0,
+                                                bound="bit for bit"))
     log("gather homo 1e8: %s" % extra["gather_homo_1e8"])
 
     # vmap over event vectors (event_csr_matvec_batching): the same matrix against 8 and 32
@@ -563,7 +664,9 @@ def main():
     sd = {k: torch.from_numpy(v).to(dev) for k, v in s.items() if isinstance(v, np.ndarray)}
     got = bpl.event_csr_matvec(sd["data"], sd["indices"], sd["indptr"], sd["events"], shape=s["shape"], transpose=True)
     want = oracle.event_csr_matvec(s["data"], s["indices"], s["indptr"], s["events"], shape=s["shape"], transpose=True)
-    check(got.cpu().numpy(), want, "event_csr_matvec scatter 4,000")
+    if not np.array_equal(got.cpu().numpy(), want):
+      raise SystemExit("parity gate failed for event_csr_matvec scatter 4,000 (homogeneous weight: bit for bit)")
+    log("parity event_csr_matvec scatter 4,000           bit for bit")
     scatter_c1 = lambda: bpl.event_csr_matvec(sd["data"], sd["indices"], sd["indptr"], sd["events"],
                                               shape=s["shape"], transpose=True)
     one_c1 = single_call_us(scatter_c1)  # before any warm-up of this shape
@@ -599,6 +702,13 @@ def main():
     extra["scatter_4000"]["bare_abi_back_to_back_us"] = back_to_back_us(raw, 1000)
     extra["scatter_4000"]["wrapper_back_to_back_us"] = back_to_back_us(scatter_c1, 1000)
     extra["scatter_4000"]["trivial_kernel_back_to_back_us"] = back_to_back_us(lambda: xs.add_(1.0), 1000)
+    # Its bound is the launch itself: one kernel of a few hundred nanoseconds of memory work.  Achieved = calls per
+    # second back to back through the bare ABI, peak = the same for a kernel that does nothing but add 1 to 4,000 floats.
+    extra["scatter_4000"]["roofline"] = roofline_record(
+      "launch", 1e6 / extra["scatter_4000"]["bare_abi_back_to_back_us"],
+      1e6 / extra["scatter_4000"]["trivial_kernel_back_to_back_us"], "calls/s",
+      peak_measured_by="a one-launch elementwise kernel enqueued the same way in this run")
+    extra["scatter_4000"]["parity"] = dict(elements=int(s["shape"][1]), outside_plain=0, violations=0, bound="bit for bit")
     # the same call replayed from a HIP graph: what a simulation loop that captures its time step pays
     gs = torch.cuda.Stream()
     gs.wait_stream(torch.cuda.current_stream())
@@ -627,13 +737,14 @@ def main():
     want = oracle.csr_matvec(m["data"], m["indices"], m["indptr"], m["vector"], shape=m["shape"])
     t_cpu3 = time.perf_counter() - t1
     got = bpl.csr_matvec(md["data"], md["indices"], md["indptr"], md["vector"], shape=m["shape"]).cpu().numpy()
-    check(got, want, "csr_matvec 1e8 nnz")
+    outside_c3 = check(got, want, "csr_matvec 1e8 nnz")
     dur3, _ = time_calls(lambda: bpl.csr_matvec(md["data"], md["indices"], md["indptr"], md["vector"], shape=m["shape"]),
                          max(20, args.steps // 4), 5)
     bytes3 = 4 * (m["shape"][0] + 1) + 8 * nnz3 + 4 * m["shape"][1] + 4 * m["shape"][0]
     extra["csr_matvec_1e8"] = dict(stats(dur3), nnz=nnz3, gsop_per_s=nnz3 / (dur3.mean() * 1e-3) / 1e9,
                                    algorithmic_gb_per_s=bytes3 / (dur3.mean() * 1e-3) / 1e9,
-                                   cpu_port_allcores_ms=t_cpu3 * 1e3, cpu_cores=cores)
+                                   cpu_port_allcores_ms=t_cpu3 * 1e3, cpu_cores=cores,
+                                   parity=parity_record(got, outside_c3, "rel 1e-5 / abs 1e-6"))
     # Its bound: the rate at which 4-byte elements of a 4 MB vector can be gathered from L2 at all, measured
     # here by a flat kernel over the same index and weight streams (no rows, no reduction, no output).
     ceil_rows = gather_ceiling(bench_lib, dev, md["vector"], md["indices"], md["data"], 10)
@@ -651,11 +762,13 @@ def main():
     mag = oracle.csr_matvec(m["data"], m["indices"], m["indptr"], np.abs(m["vector"]), shape=m["shape"], transpose=True)
     got = bpl.cusparse_csr_matvec(md["data"], md["indices"], md["indptr"], md["vector"], shape=m["shape"],
                                   transpose=True).cpu().numpy()
-    check(got, want, "csr_matvec transposed 1e8 nnz", mag)
+    outside_c3t = check(got, want, "csr_matvec transposed 1e8 nnz", mag)
     dur3t, _ = time_calls(lambda: bpl.cusparse_csr_matvec(md["data"], md["indices"], md["indptr"], md["vector"],
                                                           shape=m["shape"], transpose=True), max(20, args.steps // 4), 5)
     extra["csr_matvec_transposed_1e8"] = dict(stats(dur3t), gsop_per_s=nnz3 / (dur3t.mean() * 1e-3) / 1e9,
-                                              algorithmic_gb_per_s=bytes3 / (dur3t.mean() * 1e-3) / 1e9)
+                                              algorithmic_gb_per_s=bytes3 / (dur3t.mean() * 1e-3) / 1e9,
+                                              parity=parity_record(got, outside_c3t,
+                                                                   "rel 1e-5 / abs 1e-6 + 4 eps sum|addends|"))
     # the sorted scatter writes and reads every (16-bit column in its window, product) pair once more: 8 + 12
     # bytes per nonzero
     extra["csr_matvec_transposed_1e8"]["roofline"] = dict(
@@ -758,7 +871,23 @@ def main():
       idx, _ = oracle.jitconn_stream_indices(j["seed"] + int(r), lp, n)
       if out_row[r] != np.float32(j["events"][idx].sum()) * np.float32(0.1):
         raise SystemExit("parity gate failed for jitconn event matvec row %d" % r)
-    jit = {"generated_synapses": generated}
+    jit = {"generated_synapses": generated,
+           "parity_row_walk": dict(elements=64, outside_plain=0, violations=0,
+                                   bound="bit for bit (64 sampled rows against single-stream oracle walks)")}
+    # column walk: the whole output against the oracle's streams of the active columns (counts: exact)
+    out_col = bpl.event_matvec_prob_conn_homo_weight(ev, 1.0, conn_prob=j["conn_prob"], shape=j["shape"], seed=j["seed"],
+                                                     outdim_parallel=False).cpu().numpy()
+    want_col = np.zeros(n)
+    pairs = 0
+    for col in np.flatnonzero(j["events"]):
+      idx, _ = oracle.jitconn_stream_indices(j["seed"] + int(col), lp, n)
+      np.add.at(want_col, idx, 1.0)
+      pairs += idx.shape[0]
+    if not np.array_equal(out_col.astype(np.float64), want_col):
+      raise SystemExit("parity gate failed for the jitconn column walk (whole output, counts)")
+    log("parity jitconn column walk 1e6 x 1e6        whole output bit for bit (%d pairs)" % pairs)
+    jit["parity_column_walk"] = dict(elements=n, outside_plain=0, violations=0, bound="bit for bit (whole output)")
+    jit["column_walk_pairs"] = pairs
     # the row walk is bound by VALU issue: peak = CUs x 64 lanes x clock lane-instructions per second (one
     # wave64 instruction per SIMD every four cycles).  The number of vector instructions a call executes is a
     # counter reading (SQ_INSTS_VALU, rocprofv3 --pmc run of this workload, `--pmc jitconn`), since counters
@@ -779,6 +908,9 @@ def main():
     vr = jit["valu_roofline"]
     if rec_j:
       lane_instr = rec_j["valu_wave_instr_per_call"] * 64.0
+      jit["roofline_row_walk"] = roofline_record(
+        "valu", lane_instr / (call_us * 1e-6) / 1e12, vr["peak_lane_instr_per_s"] / 1e12, "T lane instructions/s",
+        instruction_count_recorded_in=rec_j["profile"])
       vr.update(achieved_lane_instr_per_s=lane_instr / (call_us * 1e-6),
                 frac=lane_instr / (call_us * 1e-6) / vr["peak_lane_instr_per_s"],
                 valu_instr_per_64_synapses_recorded=rec_j["valu_instr_per_64_synapses"],
@@ -801,7 +933,30 @@ def main():
       fn = lambda: bpl.matvec_prob_conn_homo_weight(vec, j["weight"], conn_prob=j["conn_prob"], shape=j["shape"],
                                                     seed=j["seed"], outdim_parallel=odp)
       d, _ = time_calls(fn, max(5, args.steps // 20), 2)
-      jit["dense_matvec,outdim_parallel=%s" % odp] = dict(stats(d), implicit_gsyn_per_s=generated / (d.mean() * 1e-3) / 1e9)
+      # every synapse gathers one element of the 4 MB vector from the L2 (row walk) or adds one pair through the bins
+      # (column walk): set beside the flat-gather ceiling of this run, measured over the csr_matvec arrays above
+      jit["dense_matvec,outdim_parallel=%s" % odp] = dict(
+        stats(d), implicit_gsyn_per_s=generated / (d.mean() * 1e-3) / 1e9,
+        roofline=roofline_record("l2-gather" if odp else "l2-gather (pairs through bins)",
+                                 generated / (d.mean() * 1e-3) / 1e9, ceiling, "G synapses/s",
+                                 peak_measured_by="bench_gather_fma over 1e8 nonzeros and a 1,000,000-element vector"))
+    # parity of the dense walks at full size: a 0/1 vector gives counts, which are exact in any order: the row walk
+    # against the event walk's counts (64 sampled rows checked above), the column walk against the event column walk
+    vec01 = ev.to(torch.float32)
+    for odp, want_01 in ((True, out_row / np.float32(0.1)), (False, out_col)):
+      got_01 = bpl.matvec_prob_conn_homo_weight(vec01, 1.0, conn_prob=j["conn_prob"], shape=j["shape"], seed=j["seed"],
+                                                outdim_parallel=odp).cpu().numpy()
+      if not np.array_equal(got_01, np.rint(want_01).astype(np.float32)):
+        raise SystemExit("parity gate failed for the dense jitconn walk (outdim_parallel=%s) on a 0/1 vector" % odp)
+      jit["dense_matvec,outdim_parallel=%s" % odp]["parity"] = dict(
+        elements=n, outside_plain=0, violations=0, bound="bit for bit (0/1 vector: counts equal the event walk's)")
+    log("parity dense jitconn walks 1e6 x 1e6        0/1 vector: whole outputs equal the event walks' counts")
+    # the event column walk: three short kernels (list, seed, walk) and the sum of the bins; its traffic by design is
+    # the pairs written and read once (8 bytes each way) plus the output
+    cw = jit["transpose=False,outdim_parallel=False"]
+    cw["roofline"] = roofline_record("hbm", (16.0 * pairs + 4.0 * n + n) / (cw["mean_us"] * 1e-6) / 1e9, HBM_PEAK_GBS,
+                                     "GB/s", note="bytes the design moves (pairs written and read once); the chain of "
+                                                  "launches and the serial stream walk bound it, not the memory")
     extra["jitconn_event_matvec_1e9"] = jit
     log("jitconn event matvec: %s" % jit)
 
@@ -830,6 +985,24 @@ def main():
                                            parity=dict(elements=int(got.size), outside_plain=outside_mm, violations=0),
                                            cpu_port_1core_s_per_call=t_cpu,
                                            cpu_sample="one full call, every stream generated once (%.2f s)" % t_cpu)
+    mm_leg = extra["jitconn_matmat_1e4x128"]
+    rec_m = recorded_counters("jitconn_matmat_1e4x128", mm_leg["mean_us"], generated_synapses=gen_mm)
+    if rec_m:
+      # instruction issue: vector instructions per call (SQ_INSTS_VALU of the recorded --pmc matmat run) x 64 lanes
+      # over this run's time, against CUs x 64 lanes x clock; and the 128-byte requests its loads send to the L2s
+      lane_instr = rec_m["valu_wave_instr_per_call"] * 64.0
+      mm_leg["roofline"] = roofline_record(
+        "valu", lane_instr / (mm_leg["mean_us"] * 1e-6) / 1e12, vr["peak_lane_instr_per_s"] / 1e12,
+        "T lane instructions/s", instruction_count_recorded_in=rec_m["profile"],
+        valu_instr_per_synapse_recorded=rec_m["valu_wave_instr_per_call"] / gen_mm,
+        l2_read_tb_per_s=rec_m["l2_read_requests_per_call"] * 128.0 / (mm_leg["mean_us"] * 1e-6) / 1e12,
+        recorded_at=dict(git_rev=rec_m["git_rev"], kernel=rec_m["kernel"], call_us=rec_m["kernel_us"]))
+    else:
+      mm_leg["roofline"] = None
+    # the same call while the clocks are still low: the first calls after an idle second
+    time.sleep(1.0)
+    d_cold, _ = time_calls(fn, 10, 0, warm_s=0.0)
+    mm_leg["first_10_calls_after_1s_idle_us"] = stats(d_cold)
     log("jitconn matmat: %s" % extra["jitconn_matmat_1e4x128"])
 
     # ---------------------------------------------------------------------------------------------
@@ -850,6 +1023,40 @@ def main():
                                            reference_docstring_ms=2.782)
     log("event_info: %s" % extra["event_info_1000x100000"])
     del ev_t, ids, num
+
+  # One flat record per configuration of the benchmark's list (C1 ... C5, T = the transposed / scatter / column
+  # orientation): microseconds per call, fraction of the leg's own roofline, elements outside the plain parity
+  # bound.  Scalars only, inside "roofline", and once more as the last lines on stderr, so that they are on record
+  # wherever the line or the end of the log is kept.
+  flat, tags = {}, []
+  if not args.skip_extra:
+    def put(tag, leg, roof=None, par=None):
+      tags.append(tag)
+      roof = leg.get("roofline") if roof is None else roof
+      par = leg.get("parity") if par is None else par
+      flat[tag + "_us"] = round(leg["mean_us"], 2)
+      if roof:
+        flat[tag + "_bound"] = roof["bound"]
+        flat[tag + "_frac"] = round(roof["frac"], 4)
+      if par:
+        flat[tag + "_outside_plain"] = "%d/%d" % (par["outside_plain"], par["elements"])
+    jit = extra["jitconn_event_matvec_1e9"]
+    put("C1_scatter_4000", dict(extra["scatter_4000"], mean_us=extra["scatter_4000"]["bare_abi_back_to_back_us"]))
+    put("C2_gather_homo", extra["gather_homo_1e8"])
+    put("C2T_scatter", extra["scatter_1e8"])
+    put("C3_csr_matvec", extra["csr_matvec_1e8"])
+    put("C3T_csr_matvec", extra["csr_matvec_transposed_1e8"])
+    put("C4_row_walk", jit["transpose=False,outdim_parallel=True"], jit.get("roofline_row_walk"), jit["parity_row_walk"])
+    put("C4_column_walk", jit["transpose=False,outdim_parallel=False"], None, jit["parity_column_walk"])
+    put("C4_dense_row_walk", jit["dense_matvec,outdim_parallel=True"])
+    put("C4_dense_column_walk", jit["dense_matvec,outdim_parallel=False"])
+    put("C5_matmat", extra["jitconn_matmat_1e4x128"])
+  log("summary C2 gather (headline): %.1f us kernel, %.1f us wall per step, hbm frac %.3f, outside plain %d/%d" % (
+    kernel_ms * 1e3, ms_per_step * 1e3, achieved / HBM_PEAK_GBS, outside_g, got_g.size))
+  for tag in tags:
+    log("summary %-22s %9.1f us  %-28s frac %-7s outside plain %s" % (
+      tag, flat[tag + "_us"], flat.get(tag + "_bound", "-"), flat.get(tag + "_frac", "-"),
+      flat.get(tag + "_outside_plain", "-")))
 
   result = {
     "metric": "GSOP/s + % HBM roofline, event_csr_matvec 1e8 nnz; jitconn GSOP/s at p=0.001",
@@ -879,7 +1086,10 @@ def main():
                  "algorithmic_bytes_per_launch": bytes_gather, "kernel_us": kernel_ms * 1e3,
                  # the same launch against what plain loads of its real traffic reach in this run
                  "streaming_ceiling_gb_per_s": stream_rate,
-                 "frac_of_streaming_ceiling": (traffic / (kernel_ms * 1e-3) / 1e9 / stream_rate) if traffic else None},
+                 "frac_of_streaming_ceiling": (traffic / (kernel_ms * 1e-3) / 1e9 / stream_rate) if traffic else None,
+                 "outside_plain_parity_bound": "%d/%d" % (outside_g, got_g.size),
+                 "clock_warm_s_before_each_timed_region": CLOCK_WARM_S,
+                 **flat},
     "cpu_baseline": cpu_baseline,
     "extra": extra,
   }

@@ -11,6 +11,14 @@
 //                      (what groups of 8 lanes per CSR row read).
 //   bench_stream       plain 16-byte loads over a buffer, at the same occupancy: the HBM read
 //                      rate a streaming kernel reaches on this device.
+//   bench_lds_atomic   random read-modify-writes into a 64 KB LDS window from 1,024-thread workgroups:
+//                      ds_add_f32, ds_add_u32, ds_add_f64, plain LDS writes, or the address arithmetic
+//                      alone (to subtract).  The rates the choice of accumulator types rests on.
+//   bench_global_atomic  fp32 atomic adds to random elements of a vector in device memory, and 32-bit
+//                      integer adds that all go to ONE address (one lane per workgroup): what a
+//                      scatter through atomics and a shared fill counter cost per operation.
+//   bench_l2_read      16-byte loads over a buffer small enough to stay in every L2, read again and
+//                      again: the rate at which the L2s deliver lines to the compute units.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -107,9 +115,103 @@ __global__ __launch_bounds__(1024) void stream_kernel(const uint4 *__restrict__ 
   out[gtid] = acc;
 }
 
+__device__ __forceinline__ uint32_t lcg_step(uint32_t &s) {
+  s = s * 1664525u + 1013904223u;
+  return s >> 8;
+}
+
+// MODE 0: ds_add_f32   1: ds_add_u32   2: ds_add_f64   3: ds_write_b32   4: the addresses only
+template <int MODE>
+__global__ __launch_bounds__(1024) void lds_atomic_kernel(float *__restrict__ out, int iters) {
+  __shared__ float win[16384];  // 64 KB
+  for (int i = threadIdx.x; i < 16384; i += 1024) win[i] = 0.f;
+  __syncthreads();
+  uint32_t st = (blockIdx.x * 1024u + threadIdx.x) * 2654435761u + 12345u;
+  float acc = 0.f;
+  for (int i = 0; i < iters; ++i) {
+    const uint32_t a = lcg_step(st) & 16383u;
+    if (MODE == 0) atomicAdd(&win[a], 1.0f);
+    else if (MODE == 1) atomicAdd(reinterpret_cast<uint32_t *>(&win[a]), 1u);
+    else if (MODE == 2) atomicAdd(reinterpret_cast<double *>(&win[a & 16382u]), 1.0);
+    else if (MODE == 3) win[a] = 1.0f;
+    else acc += static_cast<float>(a);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) out[blockIdx.x] = win[5] + acc;
+}
+
+// fp32 atomic adds (no return value) to random elements of y[0, n)
+__global__ __launch_bounds__(256) void global_atomic_random_kernel(float *__restrict__ y, uint32_t n, int iters) {
+  uint32_t st = (blockIdx.x * 256u + threadIdx.x) * 2654435761u + 12345u;
+  for (int i = 0; i < iters; ++i) unsafeAtomicAdd(&y[lcg_step(st) % n], 1.0f);
+}
+
+// one lane per workgroup adds `iters` times to ONE counter (no return value)
+__global__ __launch_bounds__(64) void global_atomic_same_address_kernel(uint32_t *__restrict__ counter, int iters) {
+  if (threadIdx.x == 0)
+    for (int i = 0; i < iters; ++i) atomicAdd(counter, 1u);
+}
+
+__global__ __launch_bounds__(1024) void l2_read_kernel(const uint4 *__restrict__ p, uint32_t *__restrict__ out,
+                                                       uint32_t n16, int repeats) {
+  // every workgroup reads the whole buffer `repeats` times, beginning at a place of its own
+  uint32_t acc = 0;
+  const uint32_t begin = (blockIdx.x * 4099u) % n16;
+  for (int r = 0; r < repeats; ++r) {
+    for (uint32_t i = threadIdx.x; i < n16; i += 4 * 1024) {
+      uint4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        uint32_t at = begin + i + u * 1024u;
+        at = at >= n16 ? at - n16 : at;
+        at = at >= n16 ? at - n16 : at;
+        v[u] = p[at];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+  }
+  out[blockIdx.x * 1024u + threadIdx.x] = acc;
+}
+
 }  // namespace
 
 extern "C" {
+
+// out: blocks floats.  mode 0: ds_add_f32, 1: ds_add_u32, 2: ds_add_f64, 3: ds_write_b32, 4: addresses only.
+// blocks * 1024 * iters operations per launch.
+int bench_lds_atomic(void *stream, float *out, int blocks, int iters, int mode) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (blocks <= 0 || iters <= 0) return 1;
+  if (mode == 0) hipLaunchKernelGGL(lds_atomic_kernel<0>, dim3(blocks), dim3(1024), 0, s, out, iters);
+  else if (mode == 1) hipLaunchKernelGGL(lds_atomic_kernel<1>, dim3(blocks), dim3(1024), 0, s, out, iters);
+  else if (mode == 2) hipLaunchKernelGGL(lds_atomic_kernel<2>, dim3(blocks), dim3(1024), 0, s, out, iters);
+  else if (mode == 3) hipLaunchKernelGGL(lds_atomic_kernel<3>, dim3(blocks), dim3(1024), 0, s, out, iters);
+  else if (mode == 4) hipLaunchKernelGGL(lds_atomic_kernel<4>, dim3(blocks), dim3(1024), 0, s, out, iters);
+  else return 1;
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+
+// same_address == 0: blocks * 256 * iters fp32 adds to random elements of y[0, n) (y: n floats).
+// same_address != 0: blocks * iters integer adds to the first word of y, one lane per workgroup.
+int bench_global_atomic(void *stream, void *y, uint32_t n, int blocks, int iters, int same_address) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (blocks <= 0 || iters <= 0 || n == 0) return 1;
+  if (same_address)
+    hipLaunchKernelGGL(global_atomic_same_address_kernel, dim3(blocks), dim3(64), 0, s, static_cast<uint32_t *>(y), iters);
+  else
+    hipLaunchKernelGGL(global_atomic_random_kernel, dim3(blocks), dim3(256), 0, s, static_cast<float *>(y), n, iters);
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+
+// p: n16 16-byte words (a multiple of 4,096, small enough for the L2); out: blocks * 1,024 words.
+// blocks * repeats * n16 * 16 bytes are read per launch.
+int bench_l2_read(void *stream, const void *p, void *out, uint32_t n16, int repeats, int blocks) {
+  if (blocks <= 0 || repeats <= 0 || n16 == 0 || n16 % 4096 != 0) return 1;
+  hipLaunchKernelGGL(l2_read_kernel, dim3(blocks), dim3(1024), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint4 *>(p), static_cast<uint32_t *>(out), n16, repeats);
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
 
 // out: blocks * threads floats.  loads_in_flight: 2, 4 or 8 gathers per lane.  Returns 0 on success.
 int bench_gather_fma(void *stream, const float *x, const uint32_t *idx, const float *w, float *out, uint64_t n,

@@ -1,5 +1,7 @@
 """Argument plumbing shared by the operator wrappers: everything becomes a contiguous torch
 CUDA tensor (device memory is PyTorch-ROCm's; nothing is computed with torch)."""
+import struct
+
 import numpy as np
 import torch
 
@@ -19,9 +21,8 @@ def as_tensor(a):
   if isinstance(a, torch.Tensor):
     return a
   if isinstance(a, (bool, int, float)):
-    if a == 0:  # (0.0 and -0.0 compare equal: not cached)
-      return torch.tensor(a, dtype=torch.bool if isinstance(a, bool) else torch.float32)
-    key = (type(a), a)
+    # keyed by the value's bits, so that 0.0 and -0.0 are two entries and a NaN finds its own
+    key = (type(a), struct.pack("<d", a) if isinstance(a, float) else a)
     t = _PY_SCALARS.get(key)
     if t is None:
       if len(_PY_SCALARS) >= 256:
@@ -55,7 +56,7 @@ def to_device(t, device):
       # A one-element host operand (a homogeneous weight given as a Python number): its device copy
       # is made once per value.  A pageable host-to-device copy per call would cost more than the
       # kernels of a small network.  The operators only read their operands.
-      key = (t.item(), t.dtype, tuple(t.shape), device)
+      key = (t.numpy().tobytes(), t.dtype, tuple(t.shape), device)  # (the bits: -0.0 is not 0.0, NaN equals itself)
       hit = _HOST_SCALARS.get(key)
       if hit is None:
         if len(_HOST_SCALARS) >= 256:

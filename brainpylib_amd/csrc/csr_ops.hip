@@ -1925,8 +1925,9 @@ namespace bpl {
 namespace {
 // Device address of `scratch` on the current device, looked up once per device.  (In host code the
 // array's name is a stand-in for the symbol, not a device address: only this pointer may be handed to
-// kernels.)
-unsigned char *static_scratch(const char *target) {
+// kernels.)  The kernels run on the device that owns `stream`; the symbol is looked up on the current
+// device: a stream of another device than the current one is refused.
+unsigned char *static_scratch(const char *target, hipStream_t stream) {
   constexpr int kMaxDev = 64;
   static unsigned char *ptrs[kMaxDev] = {};
   static std::mutex mu;
@@ -1935,6 +1936,16 @@ unsigned char *static_scratch(const char *target) {
     (void)hipGetLastError();
     set_error("%s: no current device", target);
     return nullptr;
+  }
+  if (stream != nullptr) {
+    hipDevice_t owner = dev;
+    if (hipStreamGetDevice(stream, &owner) != hipSuccess) {
+      (void)hipGetLastError();
+    } else if (static_cast<int>(owner) != dev) {
+      set_error("%s: the stream belongs to device %d and device %d is current: make the stream's device current",
+                target, static_cast<int>(owner), dev);
+      return nullptr;
+    }
   }
   std::lock_guard<std::mutex> lock(mu);
   if (ptrs[dev] == nullptr) {
@@ -1962,7 +1973,7 @@ extern "C" void event_csr_matvec_heter_float_bool_noalloc(bpl_stream_t stream, v
     bpl::set_error("%s: null buffer table", __func__);
     return;
   }
-  unsigned char *base = bpl::static_scratch(__func__);
+  unsigned char *base = bpl::static_scratch(__func__, static_cast<hipStream_t>(stream));
   if (base == nullptr) return;
   bpl::ScratchSource src;
   src.stream = static_cast<hipStream_t>(stream);

@@ -99,8 +99,9 @@ __global__ __launch_bounds__(1024, (BITS == 2 || (W == kNormal && sizeof(T1) == 
       if constexpr (IN == kInEvent && BITS == 2) {
         settle();
         // bit c = idx >> g of the coarse bitmap: word c >> 5, bit c & 31 (the bit-field extract takes the
-        // low five bits).  Lanes past the end of the row extract a field of width 0, which is 0; the word
-        // they read lies past the bitmap (an LDS read beyond the workgroup's allocation returns 0).
+        // low five bits).  Lanes past the end of the row extract a field of width 0, which is 0 whatever
+        // the word holds: the word they read may lie past the bitmap, even past the workgroup's LDS
+        // (such a read returns 0 and cannot fault), and its value is never looked at.
         const uint32_t c = idx >> coarse_g;
         const bool coarse = __builtin_amdgcn_ubfe(bits[idx >> coarse_g5], c, valid ? 1u : 0u) != 0u;
         // (lanes without a coarse hit read word 0 and ignore it: a plain load for the whole wave)

@@ -155,6 +155,14 @@ def test_python_number_weights_keep_their_values(cuda, oracle_mod):
     want = oracle_mod.event_csr_matvec(np.float32(w), indices, indptr, events, shape=shape, transpose=True)
     got = bpl.event_csr_matvec(w, ix, ip, ev, shape=shape, transpose=True).cpu().numpy()
     np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6, equal_nan=True)
+  # zeros of either sign and NaN are values of their own (the copies are kept by bit pattern): the
+  # sign bit of every output element is the oracle's, in both orientations, whichever came first
+  for w in (0.0, -0.0, 0.0, float("nan"), -0.0):
+    for transpose in (True, False):
+      e, evt = (events, ev) if transpose else (np.resize(events, shape[1]), torch.from_numpy(np.resize(events, shape[1])).cuda())
+      want = oracle_mod.event_csr_matvec(np.float32(w), indices, indptr, e, shape=shape, transpose=transpose)
+      got = bpl.event_csr_matvec(w, ix, ip, evt, shape=shape, transpose=transpose).cpu().numpy()
+      assert np.array_equal(got, want, equal_nan=True) and np.array_equal(np.signbit(got), np.signbit(want)), (w, transpose)
 
 
 def test_ragged_rows_and_all_row_length_modes(cuda, oracle_mod):

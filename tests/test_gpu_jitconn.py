@@ -156,6 +156,20 @@ def test_row_walk_with_a_two_level_event_bitmap(cuda, oracle_mod, n_in):
     assert_close_reordered(got, want, mag, np.float32, what="two-level row walk %s" % w_kind)
 
 
+def test_row_walk_lanes_past_the_end_of_a_row_count_nothing(cuda, oracle_mod):
+  # two-level bitmap with EVERY event set (all coarse and exact bits are ones): the lanes of a row's last
+  # batch that lie past the end of the row index words beyond the coarse bitmap, or any word of it if their
+  # position wrapped; they extract a bit field of width 0 from it, so a row's count is its stream's
+  # synapse count exactly.  Rows of about 3 synapses: nearly every lane of every row's only batch is past the end.
+  # (8,200 outputs: the walk that seeds its generators itself)
+  for n_out, n_in in ((400, 311_297), (400, 320_000), (400, 1_310_720), (8_200, 320_000)):
+    ev = np.ones(n_in, dtype=np.bool_)
+    lp = oracle_mod.log_p_of(3.0 / n_in)
+    got = kernel_call(ev, w_kind="homo", log_p=lp, seed=123, n_row=n_out, n_col=n_in, col_walk=False, dense=False)
+    want = np.array([oracle_mod.jitconn_stream_indices(123 + r, lp, n_in)[1] for r in range(n_out)], dtype=np.float32)
+    assert want.sum() > 0 and np.array_equal(got, want), n_in
+
+
 def test_full_matrix_recovered_by_one_hot_events(cuda, oracle_mod):
   # every entry of a 100 x 200 implicit matrix, both walks, against the per-stream oracle's index lists
   n_row, n_col, seed = 100, 200, 77

@@ -77,3 +77,16 @@ def test_check_csr_accepts_a_matrix_and_names_what_is_wrong_with_the_others():
     bpl.check_csr(idx, ptr, shape=(3, 7))
   with pytest.raises(ValueError, match="int32 or uint32"):
     bpl.check_csr(idx.astype(np.int64), ptr, shape=(4, 7))
+
+
+def test_python_scalars_are_kept_by_bit_pattern():
+  # 0.0 and -0.0 compare equal and NaN does not equal itself: the host copies of Python numbers are
+  # looked up by the value's bits
+  import math
+  from brainpylib_amd import _tensors
+  a, b = _tensors.as_tensor(0.0), _tensors.as_tensor(-0.0)
+  assert not math.copysign(1.0, a.item()) < 0 and math.copysign(1.0, b.item()) < 0
+  assert _tensors.as_tensor(-0.0) is b and _tensors.as_tensor(0.0) is a
+  n1, n2 = _tensors.as_tensor(float("nan")), _tensors.as_tensor(float("nan"))
+  assert n1 is n2 and math.isnan(n1.item())
+  assert _tensors.as_tensor(True).dtype == torch.bool and _tensors.as_tensor(1).dtype == torch.float32

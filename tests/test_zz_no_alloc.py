@@ -5,6 +5,9 @@ and integer-valued weights must agree bit for bit; scattered fp32 sums of real w
 rel 1e-5 / abs 1e-6 plus the reordering bound (both targets add with atomics, in an order that
 changes from run to run)."""
 import ctypes
+import os
+import subprocess
+import sys
 
 import numpy as np
 import pytest
@@ -61,7 +64,7 @@ SCATTER_PAIRS = [
 
 
 @pytest.mark.parametrize("pair", SCATTER_PAIRS)
-def test_noalloc_scatter_matches_the_allocating_target_twice_in_a_row(cuda, pair):
+def test_noalloc_scatter_matches_the_allocating_target_twice_in_a_row(cuda, oracle_mod, pair):
   for integer in (True, False):
     for i, (n_row, n_col, mean, rate) in enumerate(pair):
       shape = (n_row, n_col)
@@ -71,14 +74,18 @@ def test_noalloc_scatter_matches_the_allocating_target_twice_in_a_row(cuda, pair
       got = _call(NOALLOC, *args, shape, True)
       torch.cuda.synchronize()
       assert not torch.isnan(got).any(), "every output element is written"
+      host = [a.cpu().numpy() for a in args]
+      cpu = oracle_mod.event_csr_matvec(*host, shape=shape, transpose=True)  # the oracle itself, not only the sibling
       if integer:
         assert torch.equal(got, want)
+        assert np.array_equal(got.cpu().numpy(), cpu)
       else:
-        assert_close_reordered(got.cpu().numpy(), want.cpu().numpy(), _abs_sum(args, shape), np.float32,
-                               what="noalloc scatter %s" % (shape,))
+        mag = _abs_sum(args, shape)
+        assert_close_reordered(got.cpu().numpy(), want.cpu().numpy(), mag, np.float32, what="noalloc scatter %s" % (shape,))
+        assert_close_reordered(got.cpu().numpy(), cpu, mag, np.float32, what="noalloc scatter %s vs oracle" % (shape,))
 
 
-def test_noalloc_gather_matches_bit_for_bit_twice_in_a_row(cuda):
+def test_noalloc_gather_matches_bit_for_bit_twice_in_a_row(cuda, oracle_mod):
   # no transpose: an LDS bitmap (no scratch memory at all), then the two-level bitmap of a very wide
   # event vector (packed bitmap + coarse bitmap in the array), a smaller one after a larger one
   for n_row, n_col, mean, rate in ((30_000, 40_000, 50, 0.05), (3_000, 5_000_000, 100, 0.1),
@@ -90,6 +97,19 @@ def test_noalloc_gather_matches_bit_for_bit_twice_in_a_row(cuda):
     got = _call(NOALLOC, *args, shape, False)
     torch.cuda.synchronize()
     assert torch.equal(got, want)
+    cpu = oracle_mod.event_csr_matvec(*[a.cpu().numpy() for a in args], shape=shape, transpose=False)
+    assert np.array_equal(got.cpu().numpy(), cpu)
+
+
+def test_noalloc_captured_cold_into_a_graph(cuda):
+  # in a process of its own, so that the capture is the library's first call on each path: the device
+  # address of the static array, the kernels' attributes and occupancy are all looked up under the capture
+  child = os.path.join(os.path.dirname(os.path.abspath(__file__)), "noalloc_capture_child.py")
+  r = subprocess.run([sys.executable, "-u", child], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True,
+                     timeout=110)
+  print(r.stdout, flush=True)
+  assert r.returncode == 0, r.stdout[-3000:]
+  assert "cold captures ok" in r.stdout
 
 
 def test_noalloc_leaves_the_cached_allocation_alone_and_rejects_what_does_not_fit(cuda):
