@@ -18,8 +18,13 @@ void set_error(const char *fmt, ...);
 
 // Checks `opaque_len == sizeof(T)` and copies the descriptor out of the opaque bytes
 // (the pointer is not assumed to be aligned).  Returns false and records an error otherwise.
+// Every entry point calls this first (through unpack): what an earlier call on this thread left in
+// the capture-refusal flag says nothing about this one.
+void begin_call();
+
 template <typename T>
 inline bool unpack(const char *target, const char *opaque, size_t opaque_len, T *out) {
+  begin_call();
   if (opaque == nullptr || opaque_len != sizeof(T)) {
     set_error("%s: invalid opaque object size %zu (expected %zu)", target, opaque_len, sizeof(T));
     return false;
@@ -60,6 +65,8 @@ constexpr size_t kStreamCounterBytes = 256;
 // that needs less scratch memory must then give up with the error standing: a graph that
 // silently records the slow path would replay it for good.
 bool scratch_refused_by_capture();
+// A call that gives up must leave an error: records "<target>: <why>" unless one already stands.
+void ensure_error(const char *target, const char *why);
 
 // Where the launchers of one call take their scratch memory from: the cached allocation of the
 // call's stream (above), or a fixed arena that the entry point owns and that is never grown (the

@@ -1144,6 +1144,7 @@ template <typename F, typename VT, bool HETER, int MODE>
 void launch_scatter(const ScratchSource &src, const F *data, const uint32_t *indices, const uint32_t *indptr,
                     const VT *x, F *y, uint32_t n_row, uint32_t n_col) {
   hipStream_t stream = src.stream;
+  const char *target = MODE == kEvent ? "event scatter" : "transposed csr_matvec";
   if (n_col == 0) return;
   if (n_row == 0) {
     fill_zero(stream, y, n_col);
@@ -1187,7 +1188,7 @@ void launch_scatter(const ScratchSource &src, const F *data, const uint32_t *ind
                                     static_cast<const void *>(x), static_cast<uint32_t>(sizeof(VT))))
           return;
       } else {
-        if (src.failure_is_final()) return;  // during a capture: the error stands
+        if (src.failure_is_final()) return ensure_error(target, "nothing was enqueued: the path that the scratch memory at hand allows could not be launched");  // during a capture: the error stands
         bpl_clear_error();  // no scratch memory: the paths below need less or none
       }
     }
@@ -1219,7 +1220,7 @@ void launch_scatter(const ScratchSource &src, const F *data, const uint32_t *ind
         return;
       fill_zero(stream, counters, 1u);  // (the sort could not run: the list is not used)
     } else {
-      if (src.failure_is_final()) return;  // beyond a fixed arena, or during a capture: the error stands
+      if (src.failure_is_final()) return ensure_error(target, "nothing was enqueued: the path that the scratch memory at hand allows could not be launched");  // beyond a fixed arena, or during a capture: the error stands
       bpl_clear_error();  // no scratch memory: the paths below need less or none
     }
   }
@@ -1239,7 +1240,7 @@ void launch_scatter(const ScratchSource &src, const F *data, const uint32_t *ind
         return;
       fill_zero(stream, counters, 1u);  // (the walk could not run: the list is not used)
     } else {
-      if (src.failure_is_final()) return;  // during a capture: the error stands
+      if (src.failure_is_final()) return ensure_error(target, "nothing was enqueued: the path that the scratch memory at hand allows could not be launched");  // during a capture: the error stands
       bpl_clear_error();  // no scratch memory: the paths below need less or none
     }
   }
@@ -1297,7 +1298,7 @@ void launch_scatter(const ScratchSource &src, const F *data, const uint32_t *ind
       if (ws != nullptr && got < ws_bytes) want_partial = false;  // (a fixed arena too small for the partial outputs)
       uint32_t *counters = (use_list && (ws != nullptr || ws_bytes == 0)) ? src.counters() : nullptr;
       if (ws_bytes != 0 && (ws == nullptr || (use_list && counters == nullptr))) {
-        if (src.failure_is_final()) return;  // beyond a fixed arena, or during a capture: the error stands
+        if (src.failure_is_final()) return ensure_error(target, "nothing was enqueued: the path that the scratch memory at hand allows could not be launched");  // beyond a fixed arena, or during a capture: the error stands
         // no scratch memory: the direct kernel needs none
         bpl_clear_error();
         fill_zero(stream, y, n_col);
@@ -1409,7 +1410,7 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
                                                               n_col, static_cast<size_t>(c_words) * 4))
           return;
       }
-      if (src.failure_is_final()) return;  // beyond a fixed arena, or during a capture: the error stands
+      if (src.failure_is_final()) return ensure_error(target, "nothing was enqueued: the path that the scratch memory at hand allows could not be launched");  // beyond a fixed arena, or during a capture: the error stands
       bpl_clear_error();
     }
   }
@@ -1424,7 +1425,7 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
                                                 reinterpret_cast<const PackedBits *>(bits), y, n_row, n_col);
       return;
     }
-    if (src.failure_is_final()) return;  // beyond a fixed arena, or during a capture: the error stands
+    if (src.failure_is_final()) return ensure_error(target, "nothing was enqueued: the path that the scratch memory at hand allows could not be launched");  // beyond a fixed arena, or during a capture: the error stands
     bpl_clear_error();
   }
   if (MODE == kEvent) {
@@ -1459,7 +1460,7 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
       if constexpr (std::is_same<F, VT>::value) {
         const FlatGather flat = csr_flat_gather<F>(target, stream, data, HETER, indices, indptr, x, y, n_row, 4u, kStagedMinMean);
         if (flat == FlatGather::kFailed) {
-          if (scratch_refused_by_capture()) return;  // (the error stands: a graph must not record a slower path)
+          if (scratch_refused_by_capture()) return ensure_error(target, "nothing was enqueued: the path that the scratch memory at hand allows could not be launched");  // (the error stands: a graph must not record a slower path)
           bpl_clear_error();
         }
         flat_takes_short_rows = flat == FlatGather::kEnqueued;
@@ -1487,7 +1488,7 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
           return;
         }
         if (flat == FlatGather::kFailed) {
-          if (scratch_refused_by_capture()) return;  // (the error stands: a graph must not record a slower path)
+          if (scratch_refused_by_capture()) return ensure_error(target, "nothing was enqueued: the path that the scratch memory at hand allows could not be launched");  // (the error stands: a graph must not record a slower path)
           bpl_clear_error();
         }
       }
@@ -1525,6 +1526,7 @@ void csr_matvec_entry(const char *target, hipStream_t stream, void **buffers, co
                       size_t opaque_len, int vector_slot) {
   bpl_double_size_descriptor d;
   uint32_t nnz = 0;  // known only to the transposed targets' longer descriptor
+  begin_call();
   if (TRANSPOSE && opaque != nullptr && opaque_len == sizeof(bpl_csr_transpose_descriptor)) {
     bpl_csr_transpose_descriptor t;
     std::memcpy(&t, opaque, sizeof(t));
@@ -1548,14 +1550,14 @@ void csr_matvec_entry(const char *target, hipStream_t stream, void **buffers, co
     const uint32_t plain_windows = div_up(d.n_col, static_cast<uint32_t>((128u * 1024u) / sizeof(double)));
     if (plain_windows > kFlatWindowMaxSlices && d.n_row > 0 && bin_scatter_usable<F>(d.n_col, nnz)) {
       if (bin_scatter<F>(target, stream, data, HETER, indices, indptr, vec, out, d.n_row, d.n_col, nnz)) return;
-      if (scratch_refused_by_capture()) return;  // (the error stands)
+      if (scratch_refused_by_capture()) return ensure_error(target, "nothing was enqueued: the path that the scratch memory at hand allows could not be launched");  // (the error stands)
     }
     // One or two windows and a matrix worth a chip full of workgroups: the flat walk over the nonzeros, once per
     // window (167 and 330 us at 1e8 nonzeros; the sort takes 420).  (Smaller ones, and callers whose descriptor
     // does not say how many nonzeros there are, keep the walk that hands rows to waves.)
     if (plain_windows <= kFlatWindowMaxSlices && nnz >= (1u << 20)) {
       if (flat_window_scatter<F>(target, stream, data, HETER, indices, indptr, vec, out, d.n_row, d.n_col)) return;
-      if (scratch_refused_by_capture()) return;  // (the error stands)
+      if (scratch_refused_by_capture()) return ensure_error(target, "nothing was enqueued: the path that the scratch memory at hand allows could not be launched");  // (the error stands)
     }
     launch_scatter<F, F, HETER, kDense>(ScratchSource{stream}, data, indices, indptr, vec, out, d.n_row, d.n_col);
     check_launch(target);
@@ -1861,7 +1863,7 @@ void event_csr_batching_entry(const char *target, hipStream_t stream, void **buf
         check_launch(target);
         return;
       }
-      if (scratch_refused_by_capture()) return;
+      if (scratch_refused_by_capture()) return ensure_error(target, "nothing was enqueued: the path that the scratch memory at hand allows could not be launched");
       bpl_clear_error();
     }
   }

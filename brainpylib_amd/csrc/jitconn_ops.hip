@@ -618,7 +618,8 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
       if (IN == kInEvent || group == 1 || pair_bytes <= kColBinBytesMax) break;
       group = (group + 1u) / 2u;
     }
-    if (!bins) cap_d = 0.0, pair_bytes = 0;
+    // no bins (every pair goes to `out` with an atomic): nothing to size and nothing to empty between the chunks
+    if (!bins) cap_d = 0.0, pair_bytes = 0, group = chunks;
     const size_t count_bytes = round_up(static_cast<size_t>(n_win) * producers * sizeof(uint32_t));
     const uint32_t seeded_max = n_in < kSeedChunk ? n_in : kSeedChunk;
     const size_t state_bytes = round_up(static_cast<size_t>(seeded_max) * kMtN * 4);
@@ -679,7 +680,7 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
         if (list_count != nullptr) fill_zero(stream, list_count, 1u);
         out_cleared = false;
       } else {
-        if (scratch_refused_by_capture()) return;
+        if (scratch_refused_by_capture()) return ensure_error("jitconn column walk", "nothing was enqueued: the path that the scratch memory at hand allows could not be launched");
         bpl_clear_error();
       }
     }

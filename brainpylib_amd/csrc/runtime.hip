@@ -91,6 +91,10 @@ bool capturing(hipStream_t stream) {
 }  // namespace
 
 bool scratch_refused_by_capture() { return t_refused_by_capture; }
+void begin_call() { t_refused_by_capture = false; }
+void ensure_error(const char *target, const char *why) {
+  if (t_error.empty()) set_error("%s: %s", target, why);
+}
 
 void *stream_workspace(hipStream_t stream, size_t bytes) {
   t_refused_by_capture = false;
@@ -176,6 +180,12 @@ void *ScratchSource::request(size_t want, size_t need, size_t *got) const {
   if (!fixed()) {
     void *p = stream_workspace(stream, want);
     *got = p ? want : 0;
+    if (p == nullptr && need < want && !t_refused_by_capture) {
+      // the larger size could not be allocated: the least the caller can work with
+      t_error.clear();
+      p = stream_workspace(stream, need);
+      *got = p ? need : 0;
+    }
     return p;
   }
   if (need > arena_bytes) {

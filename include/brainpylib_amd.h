@@ -196,6 +196,9 @@ const char *bpl_version(void);
  * never freed (earlier work and HIP graphs captured earlier may still use it).  While a stream is
  * being captured into a HIP graph nothing can be allocated: a call that would have to fails with
  * an error and enqueues nothing, so run every shape once on the stream before capturing it.
+ * All graphs captured on one stream use that stream's buffer: their replays must be ordered with
+ * each other and with eager calls on the capture stream (replaying two of them at once on
+ * different streams, or one of them beside eager work on the capture stream, races on the buffer).
  * This query reports the current buffer of `stream` on the current device (its address and size)
  * and the bytes of retired buffers; it returns 0 if the stream has no buffer yet.  Any of the
  * three pointers may be NULL. */
@@ -251,7 +254,11 @@ BPL_TARGET(event_csr_matvec_homo_double_double);
  *   columns: 8 bytes per row.  no transpose: nothing up to 1,302,528 columns, n_col / 8 bytes +
  *   160 KiB beyond.
  *   All calls on one GPU share the array: calls that overlap on one GPU (different streams)
- *   race; calls on one stream, or ordered by events, are safe. */
+ *   race; calls on one stream, or ordered by events, are safe.
+ *   May be captured cold: the first call of a process on a stream the library has never seen may
+ *   be the captured one (the array's device address, kernel attributes and occupancy are looked
+ *   up under the capture; none of these allocates).  The stream must belong to the current
+ *   device. */
 BPL_TARGET(event_csr_matvec_heter_float_bool_noalloc);
 
 /* ------------------------------------------------------------------------------------------

@@ -421,7 +421,8 @@ def test_column_walk_through_bins_dense(cuda, oracle_mod, w_kind, a, b, dtype):
 
 
 @pytest.mark.parametrize("w_kind,a,b", [("homo", 0.0, 0.0), ("normal", 0.5, 2.0)])
-@pytest.mark.parametrize("n_out,n_in,p", [(4000, 4000, 0.02), (700, 90, 0.3), (5, 3, 0.9), (30_000, 2047, 0.01)])
+@pytest.mark.parametrize("n_out,n_in,p", [(4000, 4000, 0.02), (700, 90, 0.3), (5, 3, 0.9), (30_000, 2047, 0.01),
+                                          (2 ** 24 + 5, 7, 2e-6), (2 ** 24 + 5, 140_000, 4e-7)])
 def test_column_walk_dense_with_few_pairs(cuda, oracle_mod, w_kind, a, b, n_out, n_in, p):
   # dense input and fewer than 2^20 possible pairs: every column's generator is seeded ahead and the walk adds
   # its pairs to the output with atomics (no bins).  Against the oracle's column walk; integer input, so the
@@ -441,15 +442,19 @@ def test_column_walk_dense_with_few_pairs(cuda, oracle_mod, w_kind, a, b, n_out,
     call = lambda: bpl.matvec_prob_conn_homo_weight(xd, 0.5, conn_prob=p, shape=(n_out, n_in), seed=33, outdim_parallel=False)
     call()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
+    # best of five groups of five calls (a shared box or low clocks slow single groups down): about 70 us when the
+    # generators are seeded ahead, 500 us when every lane seeds its own
+    best = float("inf")
     for _ in range(5):
-      call()
-    e1.record()
-    torch.cuda.synchronize()
-    per_call_us = e0.elapsed_time(e1) * 1e3 / 5
-    print("dense column walk 4,000 x 4,000: %.1f us per call" % per_call_us, flush=True)
-    assert per_call_us < 300.0
+      e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+      e0.record()
+      for _ in range(5):
+        call()
+      e1.record()
+      torch.cuda.synchronize()
+      best = min(best, e0.elapsed_time(e1) * 1e3 / 5)
+    print("dense column walk 4,000 x 4,000: %.1f us per call (best of 5 groups)" % best, flush=True)
+    assert best < 300.0
 
 
 def test_column_walk_through_bins_sliced_windows(cuda, oracle_mod):

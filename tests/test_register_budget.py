@@ -71,11 +71,14 @@ def test_kernels_meant_to_share_a_cu_fit_twice(kernels):
 
 
 def test_no_kernel_spills_vector_registers_unexpectedly(kernels):
-  # scratch-memory spills are tolerated only where the eight-wave budget was chosen knowingly
-  # (double normal weights behind the two-level bitmap: 6-7 registers; float normal weights with the
-  # generators seeded inside the kernel: 2-4 registers, and still 13 % faster than seeding ahead)
-  allowed = (r"jitconn_rowwalk_kernel<double, bpl::PackedBits, 0, 2, 2, (true|false)>",
-             r"jitconn_rowwalk_kernel<float, [\w: ]+, \d, 2, \d, true>")
-  spilled = [k.split("(")[0] for k, (_, _, spill) in kernels.items()
-             if spill and not any(re.search(a, k) for a in allowed)]
+  # scratch-memory spills are tolerated only where the eight-wave budget was chosen knowingly, by exact
+  # instantiation and with a cap on the count: double normal weights behind the two-level bitmap
+  # (2 registers; 4 with the generators seeded inside the kernel)
+  allowed = {"jitconn_rowwalk_kernel<double, bpl::PackedBits, 0, 2, 2, false>": 4,
+             "jitconn_rowwalk_kernel<double, bpl::PackedBits, 0, 2, 2, true>": 8}
+  spilled = []
+  for k, (_, _, spill) in kernels.items():
+    name = k.split("(")[0].replace("void ", "").replace("bpl::jitconn", "jitconn").strip()
+    if spill and spill > allowed.get(name, 0):
+      spilled.append("%s: %d" % (name, spill))
   assert not spilled, spilled
