@@ -60,8 +60,9 @@ __device__ __forceinline__ F scattered_sum(F w, uint64_t n) {
   return repeated_sum<F>(w, n);
 }
 __device__ __forceinline__ float gathered_sum(float w, uint32_t n) {
-  // up to 2^29 additions of a 24-bit weight are exact in float64: the product, rounded once
-  return static_cast<float>(static_cast<double>(w) * static_cast<double>(n));
+  // up to 2^29 additions of a 24-bit weight are exact in float64: the product, rounded once.  The sum starts
+  // from +0: a weight of -0 (or no synapse at all) leaves +0, as 0 + (-0) does
+  return static_cast<float>(0.0 + static_cast<double>(w) * static_cast<double>(n));
 }
 __device__ __forceinline__ double gathered_sum(double w, uint32_t n) { return repeated_sum<double>(w, n); }
 
