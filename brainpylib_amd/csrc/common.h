@@ -143,11 +143,18 @@ template <typename F>
 size_t bin_event_scatter_bytes(uint32_t n_row, uint32_t n_col);
 template <typename F>
 size_t bin_event_scatter_min_bytes(uint32_t n_col);
-template <typename F>
-bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint32_t *indices, const uint32_t *indptr,
+// I: the type of the column indices and row offsets (uint32_t, or uint64_t for the older csr_event_sum; the
+// listed (first nonzero, length) entries are 32-bit either way).
+template <typename F, typename I>
+bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const I *indices, const I *indptr,
                        F *y, uint32_t n_row, uint32_t n_col, uint32_t *active_count, const uint2 *active_list,
                        uint32_t list_cap, void *scratch, size_t scratch_bytes,
                        const uint32_t *active_colbase = nullptr);
+// csr_event_sum with 64-bit index arrays through the sorted event scatter (csr_ops.hip).  1: enqueued (a matrix of
+// 2^32 nonzeros or more leaves the zeroed result untouched); 0: nothing enqueued, take another path; -1: failed.
+template <typename F, bool HETER>
+int csr_event_sum_wide(const char *target, hipStream_t stream, const uint8_t *events, const uint64_t *indices,
+                        const uint64_t *indptr, const F *values, F *result, uint32_t pre_size, uint32_t post_size);
 
 // mt19937 states of the generator streams seed + first .. seed + first + count - 1, 624 words each, seeded on
 // the vector unit, 64 streams per wave (jitconn_ops.hip).  A wave that seeds the stream it walks holds its

@@ -678,9 +678,9 @@ constexpr uint32_t kDirectWord = 1;           // (fill counters sit at multiples
 // (At most 80 scalar registers: measured on this device, a 1,024-thread workgroup whose waves hold
 // 81..96 of them is alone on its CU, as it would be with more than 64 vector registers; the
 // float producer crossed that line by one register and took 37 instead of 27 us.)
-template <typename F, bool HETER>
+template <typename F, bool HETER, typename I>
 __global__ __launch_bounds__(kBinThreads) __attribute__((amdgpu_num_sgpr(80))) void bin_active_rows_kernel(
-    const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
+    const F *__restrict__ data, const I *__restrict__ indices, const I *__restrict__ indptr,
     uint32_t n_row, const uint32_t *__restrict__ active_count, const uint2 *__restrict__ active_list,
     uint32_t list_cap, const uint32_t *__restrict__ active_colbase, F *__restrict__ y, uint32_t shift, uint32_t cap,
     BinPair<F> *__restrict__ pairs, uint32_t *__restrict__ fill) {
@@ -698,7 +698,7 @@ __global__ __launch_bounds__(kBinThreads) __attribute__((amdgpu_num_sgpr(80))) v
   __shared__ uint8_t s_window[kRound];
   const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const uint32_t total = active_count[0] < list_cap ? active_count[0] : list_cap;  // (never beyond the list)
-  const uint32_t nnz = indptr[n_row];
+  const uint32_t nnz = static_cast<uint32_t>(indptr[n_row]);  // (64-bit offsets: listed only below 2^32 nonzeros)
   // with little activity a few producers finish sooner than a chip full of them
   const uint64_t want = (static_cast<uint64_t>(total) * (nnz / n_row + 1u) + kPairsPerProducer - 1u) / kPairsPerProducer;
   const uint32_t producers = want < 1u ? 1u : want > gridDim.x ? gridDim.x : static_cast<uint32_t>(want);
@@ -782,7 +782,7 @@ __global__ __launch_bounds__(kBinThreads) __attribute__((amdgpu_num_sgpr(80))) v
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-          col[u] = indices[at[u]];
+          col[u] = static_cast<uint32_t>(indices[at[u]]);
           val[u] = HETER ? data[at[u]] : w_homo;
         }
 #pragma unroll
@@ -1058,14 +1058,14 @@ __global__ __launch_bounds__(kSumCols * kSumSlices) void sum_active_windows_kern
 // of its own for the sums: 100,000 x 100,000, 1e8 nnz, 0.1 % events 20 against 23 us, 5 % 52 against
 // 48 us.  With little activity the rows are added to y as sums of the weight itself, which is exact
 // too: additions of one value give the same bits in any order.)
-template <typename F, bool HETER>
+template <typename F, bool HETER, typename I>
 __global__ __launch_bounds__(kBinThreads) void add_window_runs_kernel(F *__restrict__ y, uint32_t n_col, uint32_t shift,
                                                                       uint32_t lds_shift, uint32_t parts, uint32_t cap,
                                                                       const BinPair<F> *__restrict__ pairs,
                                                                       const uint32_t *__restrict__ fill,
                                                                       uint32_t *__restrict__ reset,
                                                                       const F *__restrict__ data,
-                                                                      const uint32_t *__restrict__ indices,
+                                                                      const I *__restrict__ indices,
                                                                       const uint2 *__restrict__ active_list,
                                                                       const uint32_t *__restrict__ active_colbase) {
   constexpr bool heter = HETER;
@@ -1299,8 +1299,8 @@ size_t bin_event_scatter_min_bytes(uint32_t n_col) {
   return kBinEventFillBytes + static_cast<size_t>(kMinRunPairs) * n_win * kSubRuns * sizeof(BinPair<F>);
 }
 
-template <typename F>
-bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint32_t *indices, const uint32_t *indptr,
+template <typename F, typename I>
+bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const I *indices, const I *indptr,
                        F *y, uint32_t n_row, uint32_t n_col, uint32_t *active_count, const uint2 *active_list,
                        uint32_t list_cap, void *scratch, size_t scratch_bytes, const uint32_t *active_colbase) {
   const uint32_t shift = event_window_shift(n_col);
@@ -1316,12 +1316,12 @@ bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint
   const unsigned num_cu = static_cast<unsigned>(device_info().num_cu);
   uint32_t parts = num_cu / n_win;
   if (parts == 0) parts = 1;
-  auto add_kernel = heter ? add_window_runs_kernel<F, true> : add_window_runs_kernel<F, false>;
+  auto add_kernel = heter ? add_window_runs_kernel<F, true, I> : add_window_runs_kernel<F, false, I>;
   const uint32_t lds_shift = bin_lds_shift(shift);
   const uint32_t slices = 1u << (shift - lds_shift);
   if (slices > 1) parts = 1;
   const size_t lds = sizeof(double) << lds_shift;
-  static thread_local bool attr_set[2] = {false, false};
+  static thread_local bool attr_set[2] = {false, false};  // (per instantiation: one pair for every index type)
   if (!attr_set[heter] && lds > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(add_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             static_cast<int>(lds)) != hipSuccess) {
@@ -1332,10 +1332,10 @@ bool bin_event_scatter(hipStream_t stream, const F *data, bool heter, const uint
   }
   const uint32_t producers = 2u * num_cu;
   if (heter)
-    hipLaunchKernelGGL((bin_active_rows_kernel<F, true>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
+    hipLaunchKernelGGL((bin_active_rows_kernel<F, true, I>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
                        indptr, n_row, active_count, active_list, list_cap, active_colbase, y, shift, cap, pairs, fill);
   else
-    hipLaunchKernelGGL((bin_active_rows_kernel<F, false>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
+    hipLaunchKernelGGL((bin_active_rows_kernel<F, false, I>), dim3(producers), dim3(kBinThreads), 0, stream, data, indices,
                        indptr, n_row, active_count, active_list, list_cap, active_colbase, y, shift, cap, pairs, fill);
   hipLaunchKernelGGL(add_kernel, dim3(n_win * slices * parts), dim3(kBinThreads), lds, stream, y, n_col, shift,
                      lds_shift, parts, cap, pairs, fill, active_count, data, indices, active_list, active_colbase);
@@ -1499,11 +1499,18 @@ template size_t bin_event_scatter_bytes<float>(uint32_t, uint32_t);
 template size_t bin_event_scatter_bytes<double>(uint32_t, uint32_t);
 template size_t bin_event_scatter_min_bytes<float>(uint32_t);
 template size_t bin_event_scatter_min_bytes<double>(uint32_t);
-template bool bin_event_scatter<float>(hipStream_t, const float *, bool, const uint32_t *, const uint32_t *, float *, uint32_t,
-                                       uint32_t, uint32_t *, const uint2 *, uint32_t, void *, size_t, const uint32_t *);
-template bool bin_event_scatter<double>(hipStream_t, const double *, bool, const uint32_t *, const uint32_t *, double *,
-                                        uint32_t, uint32_t, uint32_t *, const uint2 *, uint32_t, void *, size_t,
-                                        const uint32_t *);
+template bool bin_event_scatter<float, uint32_t>(hipStream_t, const float *, bool, const uint32_t *, const uint32_t *, float *,
+                                                 uint32_t, uint32_t, uint32_t *, const uint2 *, uint32_t, void *, size_t,
+                                                 const uint32_t *);
+template bool bin_event_scatter<double, uint32_t>(hipStream_t, const double *, bool, const uint32_t *, const uint32_t *,
+                                                  double *, uint32_t, uint32_t, uint32_t *, const uint2 *, uint32_t, void *,
+                                                  size_t, const uint32_t *);
+template bool bin_event_scatter<float, uint64_t>(hipStream_t, const float *, bool, const uint64_t *, const uint64_t *, float *,
+                                                 uint32_t, uint32_t, uint32_t *, const uint2 *, uint32_t, void *, size_t,
+                                                 const uint32_t *);
+template bool bin_event_scatter<double, uint64_t>(hipStream_t, const double *, bool, const uint64_t *, const uint64_t *,
+                                                  double *, uint32_t, uint32_t, uint32_t *, const uint2 *, uint32_t, void *,
+                                                  size_t, const uint32_t *);
 template bool flat_window_scatter<float>(const char *, hipStream_t, const float *, bool, const uint32_t *, const uint32_t *,
                                          const float *, float *, uint32_t, uint32_t);
 template bool flat_window_scatter<double>(const char *, hipStream_t, const double *, bool, const uint32_t *,

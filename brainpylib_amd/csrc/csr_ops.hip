@@ -198,19 +198,27 @@ constexpr int kWinMaxRows = 2048;  // rows per workgroup = capacity of the activ
 // kCollectPerThread and reserves its list positions with one atomic (atomics on one address
 // retire at about 15 ns each, whoever issues them: one per 1,024 rows cost 14 us for a million rows).
 // Optional chores for the kernels that follow: `clear[0 .. n_clear)` and `zero[0 .. n_zero)` are set to zero.
-template <typename F, typename VT, int MODE, int kCollectPerThread>
+// I: the type of the row offsets.  64-bit offsets (the older csr_event_sum) are listed as 32-bit (first
+// nonzero, length) too; a matrix of 2^32 nonzeros or more is not listed at all (the chores are still done
+// and the list stays empty: the caller has a kernel for such matrices that runs in that case only).
+template <typename F, typename VT, int MODE, int kCollectPerThread, typename I = uint32_t>
 __global__ __launch_bounds__(kWinThreads) void collect_active_rows_kernel(
-    const uint32_t *__restrict__ indptr, const VT *__restrict__ x, uint32_t n_row, uint32_t *__restrict__ counter,
+    const I *__restrict__ indptr, const VT *__restrict__ x, uint32_t n_row, uint32_t *__restrict__ counter,
     uint2 *__restrict__ list, F *__restrict__ scales, NnzGate gate, uint32_t *__restrict__ clear, uint32_t n_clear,
     F *__restrict__ zero, uint32_t n_zero) {
   // (The list holds n_row entries.  The counter is zero when a call starts, so positions stay below
   // n_row; should an earlier call have failed half way and left it set, nothing is written beyond.)
-  if (!gate.open(indptr, n_row)) return;
+  if constexpr (sizeof(I) == 4) {
+    if (!gate.open(reinterpret_cast<const uint32_t *>(indptr), n_row)) return;
+  }
   __shared__ uint32_t s_count, s_base;
   const uint32_t tid = threadIdx.x, lane = tid % kWave;
   if (tid == 0) s_count = 0;
   for (uint32_t i = blockIdx.x * kWinThreads + tid; i < n_clear; i += gridDim.x * kWinThreads) clear[i] = 0u;
   for (uint32_t i = blockIdx.x * kWinThreads + tid; i < n_zero; i += gridDim.x * kWinThreads) zero[i] = F(0);
+  if constexpr (sizeof(I) == 8) {
+    if ((static_cast<uint64_t>(indptr[n_row]) >> 32) != 0) return;
+  }
   __syncthreads();
   const uint32_t r0 = blockIdx.x * (kWinThreads * kCollectPerThread) + tid;
   bool on[kCollectPerThread];
@@ -235,8 +243,8 @@ __global__ __launch_bounds__(kWinThreads) void collect_active_rows_kernel(
     start[e] = len[e] = at[e] = 0;
     if (on[e]) {
       const uint32_t r = r0 + e * kWinThreads;
-      start[e] = indptr[r];
-      len[e] = indptr[r + 1] - start[e];
+      start[e] = static_cast<uint32_t>(indptr[r]);
+      len[e] = static_cast<uint32_t>(indptr[r + 1]) - start[e];
       on[e] = len[e] != 0;
     }
   }
@@ -265,15 +273,15 @@ template <typename F, typename VT, int MODE>
 unsigned collect_workgroups(uint32_t n_row) {
   return n_row > 262144u ? div_up(n_row, 4 * kWinThreads) : div_up(n_row, kWinThreads);
 }
-template <typename F, typename VT, int MODE>
-void launch_collect(hipStream_t stream, const uint32_t *indptr, const VT *x, uint32_t n_row, uint32_t *counter,
+template <typename F, typename VT, int MODE, typename I = uint32_t>
+void launch_collect(hipStream_t stream, const I *indptr, const VT *x, uint32_t n_row, uint32_t *counter,
                     uint2 *list, F *scales, NnzGate gate, uint32_t *clear, uint32_t n_clear, F *zero, uint32_t n_zero) {
   const unsigned wgs = collect_workgroups<F, VT, MODE>(n_row);
   if (n_row > 262144u)
-    hipLaunchKernelGGL((collect_active_rows_kernel<F, VT, MODE, 4>), dim3(wgs), dim3(kWinThreads), 0, stream, indptr, x,
+    hipLaunchKernelGGL((collect_active_rows_kernel<F, VT, MODE, 4, I>), dim3(wgs), dim3(kWinThreads), 0, stream, indptr, x,
                        n_row, counter, list, scales, gate, clear, n_clear, zero, n_zero);
   else
-    hipLaunchKernelGGL((collect_active_rows_kernel<F, VT, MODE, 1>), dim3(wgs), dim3(kWinThreads), 0, stream, indptr, x,
+    hipLaunchKernelGGL((collect_active_rows_kernel<F, VT, MODE, 1, I>), dim3(wgs), dim3(kWinThreads), 0, stream, indptr, x,
                        n_row, counter, list, scales, gate, clear, n_clear, zero, n_zero);
 }
 
@@ -1903,6 +1911,55 @@ void csr_event_sum_i32_entry(const char *target, hipStream_t stream, void **buff
 }
 
 }  // namespace
+
+// csr_event_sum with 64-bit index arrays (the older operator family, compat_ops.hip) through the sorted event
+// scatter: the kernels read the 64-bit offsets and columns where they lie (no narrowed copy: that would move
+// twelve bytes per nonzero of the whole matrix, the scatter only touches the active rows).  For results of
+// more than 8,192 elements; `result` need not be zeroed.  A matrix of 2^32 nonzeros or more leaves the result
+// at zero (the caller follows with its atomic kernel, which runs in that case only).  1: enqueued; 0: nothing
+// enqueued, the caller takes its own path; -1: nothing enqueued and the call must fail with the error that stands.
+template <typename F, bool HETER>
+int csr_event_sum_wide(const char *target, hipStream_t stream, const uint8_t *events, const uint64_t *indices,
+                        const uint64_t *indptr, const F *values, F *result, uint32_t pre_size, uint32_t post_size) {
+  if (post_size <= 8192 || !bin_event_scatter_usable<F>(post_size)) return 0;
+  auto round_up = [](size_t v) { return (v + 255) / 256 * 256; };
+  const size_t list_sz = round_up(static_cast<size_t>(pre_size) * sizeof(uint2));
+  const ScratchSource src{stream};
+  size_t got = 0;
+  unsigned char *ws = static_cast<unsigned char *>(src.request(list_sz + bin_event_scatter_bytes<F>(pre_size, post_size),
+                                                               list_sz + bin_event_scatter_min_bytes<F>(post_size), &got));
+  uint32_t *counters = ws ? src.counters() : nullptr;
+  if (ws == nullptr || counters == nullptr) {
+    if (src.failure_is_final()) {
+      ensure_error(target, "nothing was enqueued: no scratch memory while the stream is being captured");
+      return -1;  // (the error stands: the caller must not record a slower path into the graph)
+    }
+    bpl_clear_error();
+    return 0;
+  }
+  uint2 *active_list = reinterpret_cast<uint2 *>(ws);
+  const unsigned collectors = collect_workgroups<F, uint8_t, kEvent>(pre_size);
+  const bool fold_zero = post_size <= 32ull * collectors * kWinThreads;
+  if (!fold_zero) fill_zero(stream, result, post_size);
+  launch_collect<F, uint8_t, kEvent, uint64_t>(stream, indptr, events, pre_size, counters, active_list,
+                                               static_cast<F *>(nullptr), kAlways, reinterpret_cast<uint32_t *>(ws + list_sz),
+                                               static_cast<uint32_t>(kBinEventFillBytes / sizeof(uint32_t)), result,
+                                               fold_zero ? post_size : 0u);
+  if (bin_event_scatter<F>(stream, values, HETER, indices, indptr, result, pre_size, post_size, counters, active_list,
+                           pre_size, ws + list_sz, got - list_sz))
+    return check_launch(target) ? 1 : -1;
+  // (the sort could not run: the list is not used; the result is zero, as the caller's own kernel expects it)
+  fill_zero(stream, counters, 1u);
+  return 0;
+}
+template int csr_event_sum_wide<float, false>(const char *, hipStream_t, const uint8_t *, const uint64_t *, const uint64_t *,
+                                               const float *, float *, uint32_t, uint32_t);
+template int csr_event_sum_wide<float, true>(const char *, hipStream_t, const uint8_t *, const uint64_t *, const uint64_t *,
+                                              const float *, float *, uint32_t, uint32_t);
+template int csr_event_sum_wide<double, false>(const char *, hipStream_t, const uint8_t *, const uint64_t *, const uint64_t *,
+                                                const double *, double *, uint32_t, uint32_t);
+template int csr_event_sum_wide<double, true>(const char *, hipStream_t, const uint8_t *, const uint64_t *, const uint64_t *,
+                                               const double *, double *, uint32_t, uint32_t);
 }  // namespace bpl
 
 // ------------------------------------------------------------------------------------------------

@@ -24,10 +24,14 @@ namespace {
 
 constexpr int kTile = 32;
 
-// XT[c][r] = X[r][c] for r < m (rows of XT have m_pad entries, the padding is zeroed)
+// XT[r / pass_rows][c][r % pass_rows] = X[r][c] for r < m: the transposed operand in slices of pass_rows rows of
+// X (a multiple of 32), every slice contiguous, its rows pass_rows entries long; rows m .. m_pad - 1 are zero.
+// (In one array of rows of m_pad entries the pieces that a pass reads lie m_pad entries apart and share a
+// fraction of the L2's sets.)
 template <typename T>
 __global__ __launch_bounds__(kTile * 8) void transpose_pad_kernel(const T *__restrict__ X, T *__restrict__ XT,
-                                                                  uint32_t m, uint32_t k, uint32_t m_pad) {
+                                                                  uint32_t m, uint32_t k, uint32_t m_pad,
+                                                                  uint32_t pass_rows) {
   __shared__ T tile[kTile][kTile + 1];
   const uint32_t c0 = blockIdx.x * kTile, r0 = blockIdx.y * kTile;
   const uint32_t tx = threadIdx.x % kTile, ty = threadIdx.x / kTile;  // 32 x 8
@@ -38,7 +42,8 @@ __global__ __launch_bounds__(kTile * 8) void transpose_pad_kernel(const T *__res
   __syncthreads();
   for (uint32_t i = ty; i < kTile; i += 8) {
     const uint32_t c = c0 + i, r = r0 + tx;
-    if (c < k && r < m_pad) XT[static_cast<size_t>(c) * m_pad + r] = tile[tx][i];
+    if (c < k && r < m_pad)
+      XT[(static_cast<size_t>(r / pass_rows) * k + c) * pass_rows + r % pass_rows] = tile[tx][i];
   }
 }
 
@@ -54,13 +59,16 @@ struct __attribute__((aligned(2 * sizeof(T1)))) Synapse {
   T1 w;
 };
 
-// MT = 64-row tiles of Y one wave accumulates (m_pad / 64 per pass of blockIdx.y)
+// MT = 64-row tiles of Y one wave accumulates; a launch is one pass over MT * 64 rows of X (pass number `pass`).
+// (The passes are launches of their own, one after the other: as the second dimension of one grid the
+// workgroups of two passes run side by side nearly all the time, two slices of XT compete for the L2s, and
+// eight passes of 256 rows took 5.7 ms instead of 3.8.)
 template <typename T1, int W, int MT>
 __global__ __launch_bounds__(256) void jitconn_matmat_kernel(const T1 *__restrict__ XT, T1 *__restrict__ Y,
                                                              uint32_t m, uint32_t k, uint32_t n, uint32_t m_pad,
                                                              uint32_t seed, double log_p, T1 wa, T1 wb,
                                                              uint32_t first, uint32_t count,
-                                                             const uint32_t *__restrict__ states) {
+                                                             const uint32_t *__restrict__ states, uint32_t pass) {
   constexpr int kWaves = 4;
   constexpr int kWords = StreamLds<T1, W>::words;
   __shared__ __attribute__((aligned(8))) uint32_t s_state[kWaves * kWords];
@@ -69,11 +77,12 @@ __global__ __launch_bounds__(256) void jitconn_matmat_kernel(const T1 *__restric
   const uint32_t wave = threadIdx.x / kWave;
   uint32_t *st = s_state + wave * kWords;
   Synapse<T1> *syn = s_syn + wave * kWave;
-  const uint32_t row_base = blockIdx.y * (MT * kWave);  // first row of Y of this pass
-  // byte offsets into XT fit 32 bits (checked by the host): one add per synapse instead of a 64-bit product
-  const uint32_t row_bytes = m_pad * static_cast<uint32_t>(sizeof(T1));
+  const uint32_t row_base = pass * (MT * kWave);  // first row of Y of this pass
+  // byte offsets into the pass's slice of XT fit 32 bits (checked by the host): one add per synapse instead of a
+  // 64-bit product
+  constexpr uint32_t row_bytes = MT * kWave * static_cast<uint32_t>(sizeof(T1));
   // (a wave-uniform base and a 32-bit offset per lane: one address add per synapse and the base in scalar registers)
-  const char *xt_base = reinterpret_cast<const char *>(XT + row_base);
+  const char *xt_base = reinterpret_cast<const char *>(XT + static_cast<size_t>(pass) * k * (MT * kWave));
   const uint32_t lane_bytes = static_cast<uint32_t>(lane) * static_cast<uint32_t>(sizeof(T1));
 
   // columns first .. first + count - 1 of M, their generators seeded ahead: states[c] for column first + c
@@ -98,7 +107,7 @@ __global__ __launch_bounds__(256) void jitconn_matmat_kernel(const T1 *__restric
         syn[slot].w = w;
       }
       __builtin_amdgcn_wave_barrier();
-      constexpr int U = (MT >= 4) ? 4 : 8;
+      constexpr int U = 8;
       uint32_t i = 0;
       for (; i + U <= count; i += U) {
         T1 ws[U];
@@ -148,16 +157,20 @@ void matmat_entry(const char *target, hipStream_t stream, void **buffers, const 
   T1 *Y = static_cast<T1 *>(buffers[1]);
   const uint32_t m = d.m, k = d.k, n = d.n;
   if (m == 0 || n == 0) return;
-  // rows of XT are padded to what one pass of the kernel reads: 64, 128 or a multiple of 256
+  // rows of X are padded to what the passes of the kernel read: one pass of 64 or 128 rows, or several of 128.
+  // (A pass regenerates the matrix, but its slice of XT, 5 MB for 10,000 inputs, stays in the L2s: 2,048 rows of X
+  // against a 10,000 x 10,000 matrix take 3.2 ms with uniform and 3.7 ms with normal weights in 16 passes of 128,
+  // 3.7 and 3.8 ms in 8 passes of 256, whose slices do not.)
   uint32_t m_pad = (m + kWave - 1) / kWave * kWave;
-  if (m_pad > 2 * kWave) m_pad = (m + 4 * kWave - 1) / (4 * kWave) * (4 * kWave);
+  const uint32_t pass_rows = m_pad > 2 * kWave ? 2 * kWave : m_pad;
+  m_pad = (m + pass_rows - 1) / pass_rows * pass_rows;
   if (k == 0) {
     fill_zero(stream, Y, m * n);  // m * n fits 32 bits whenever Y is addressable by the kernels below
     check_launch(target);
     return;
   }
-  if (static_cast<uint64_t>(k) * m_pad * sizeof(T1) > 0xffffffffull) {
-    set_error("%s: the transposed operand (%u x %u) exceeds 4 GiB", target, k, m_pad);
+  if (static_cast<uint64_t>(k) * pass_rows * sizeof(T1) > 0xffffffffull) {
+    set_error("%s: a slice of the transposed operand (%u x %u) exceeds 4 GiB", target, k, pass_rows);
     return;
   }
   // scratch memory: [XT][the generator states of a chunk of columns, seeded ahead on the vector unit]
@@ -172,23 +185,22 @@ void matmat_entry(const char *target, hipStream_t stream, void **buffers, const 
   T1 *XT = reinterpret_cast<T1 *>(ws);
   uint32_t *states = reinterpret_cast<uint32_t *>(ws + xt_bytes);
   hipLaunchKernelGGL(transpose_pad_kernel<T1>, dim3(div_up(k, kTile), div_up(m_pad, kTile)), dim3(kTile * 8), 0,
-                     stream, X, XT, m, k, m_pad);
+                     stream, X, XT, m, k, m_pad, pass_rows);
   const T1 wa = static_cast<T1>(d.w_a), wb = static_cast<T1>(d.w_b);
-  const uint32_t tiles = m_pad / kWave;
+  const uint32_t tiles = pass_rows / kWave, passes = m_pad / pass_rows;
   for (uint32_t first = 0; first < n; first += chunk) {
     const uint32_t count = n - first < chunk ? n - first : chunk;
     if (ahead) jitconn_seed_streams(stream, d.seed, first, count, states);
     const unsigned grid_x = div_up(count, 4);
     const uint32_t *pre = ahead ? states : nullptr;
-    if (tiles == 1) {
-      hipLaunchKernelGGL((jitconn_matmat_kernel<T1, W, 1>), dim3(grid_x, 1), dim3(256), 0, stream, XT, Y, m, k, n, m_pad,
-                         d.seed, d.log_p, wa, wb, first, count, pre);
-    } else if (tiles == 2) {
-      hipLaunchKernelGGL((jitconn_matmat_kernel<T1, W, 2>), dim3(grid_x, 1), dim3(256), 0, stream, XT, Y, m, k, n, m_pad,
-                         d.seed, d.log_p, wa, wb, first, count, pre);
-    } else {
-      hipLaunchKernelGGL((jitconn_matmat_kernel<T1, W, 4>), dim3(grid_x, div_up(tiles, 4)), dim3(256), 0, stream, XT, Y,
-                         m, k, n, m_pad, d.seed, d.log_p, wa, wb, first, count, pre);
+    for (uint32_t pass = 0; pass < passes; ++pass) {
+      if (tiles == 1) {
+        hipLaunchKernelGGL((jitconn_matmat_kernel<T1, W, 1>), dim3(grid_x), dim3(256), 0, stream, XT, Y, m, k, n, m_pad,
+                           d.seed, d.log_p, wa, wb, first, count, pre, pass);
+      } else {
+        hipLaunchKernelGGL((jitconn_matmat_kernel<T1, W, 2>), dim3(grid_x), dim3(256), 0, stream, XT, Y, m, k, n, m_pad,
+                           d.seed, d.log_p, wa, wb, first, count, pre, pass);
+      }
     }
   }
   check_launch(target);

@@ -48,6 +48,30 @@ def test_csr_event_sum_wide_golden(cuda):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_csr_event_sum_64_bit_ids_through_the_sorted_scatter(cuda, oracle_mod, dtype):
+  # 64-bit index arrays and a result of more than 8,192 elements: the sorted event scatter reads the 64-bit
+  # columns and offsets as they are.  Against the oracle (lib/cpu_event_sum.cc's loop): one weight bit for bit,
+  # weights per connection within the reordered-sum bound; activity on both sides of the direct-atomics
+  # threshold, empty rows, a result narrower and wider than the matrix has rows.
+  for (pre, post, mean, rate) in ((30_000, 20_000, 40, 0.1), (30_000, 20_000, 40, 0.001), (5_000, 300_000, 300, 0.3),
+                                  (200_000, 9_000, 10, 0.5)):
+    rng = np.random.default_rng(pre + post)
+    counts = np.minimum(rng.poisson(mean, size=pre), post)
+    indices, indptr = synth.counted_csr(counts, post, seed=pre)
+    events = rng.random(pre) < rate
+    wide = (indices.astype(np.int64), indptr.astype(np.int64))
+    print("case", pre, post, mean, rate, dtype.__name__, flush=True)
+    for values in (np.array([0.6], dtype=dtype), rng.standard_normal(indices.shape[0]).astype(dtype)):
+      want = oracle_mod.csr_event_sum(events, (indices, indptr), post, values)
+      got = bpl.csr_event_sum(events, wide, post, values).cpu().numpy()
+      if values.shape[0] == 1:
+        assert np.array_equal(got, want)
+      else:
+        mag = oracle_mod.csr_event_sum(events, (indices, indptr), post, np.abs(values))
+        assert_close_reordered(got, want, mag, dtype, what="csr_event_sum i64, sorted scatter")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("itype", [np.int32, np.uint32, np.int64])
 def test_coo_event_sum_vs_oracle(cuda, oracle_mod, dtype, itype):
   rng = np.random.default_rng(9)

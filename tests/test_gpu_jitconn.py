@@ -331,10 +331,11 @@ def test_config_jitconn_event_full_size(cuda, oracle_mod):
   assert float(got_row.astype(np.float64) @ y) == float(MTy.astype(np.float64) @ ev)
 
 
-@pytest.mark.parametrize("m", [1, 5, 8, 15, 33, 64, 70, 130, 300])
+@pytest.mark.parametrize("m", [1, 5, 8, 15, 33, 64, 70, 128, 130, 300, 600, 2048])
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_matmat_against_oracle_and_vmapped_matvec(cuda, oracle_mod, m, dtype):
-  # m values of the reference test (matmat_testcase.py:39-44) plus tile boundaries of the kernel
+  # m values of the reference test (matmat_testcase.py:39-44) plus tile boundaries of the kernel and row counts
+  # that take several passes of 128 rows (the last one partly filled)
   k, n, seed, p = 230, 150, 7, 0.2
   X = np.random.default_rng(m).standard_normal((m, k)).astype(dtype)
   lp = oracle_mod.log_p_of(p)
