@@ -318,7 +318,7 @@ __global__ __launch_bounds__(1024) void collect_active_columns_kernel(const VT *
 // [0, n_list) of a list: column list_col[k] with value list_val[k] (event input: the active
 // columns), or, without a list, column first + k with value in[first + k] (dense input).  Waves
 // take entries round robin over the whole grid, so every wave walks the same number of streams.
-// The generators of the first n_seeded entries were seeded ahead on the vector unit (`states`);
+// Not FUSED: the generators of the first n_seeded entries were seeded ahead on the vector unit (`states`);
 // a wave seeding its own generator does it on the CU's one scalar unit, about 2 us each, and a
 // CU's waves queue up for it.  A pair for output window b (2^shift outputs) of workgroup p goes to
 // pairs[(p * n_win + b) * cap + position]; the positions continue from `counts` (zero before the
@@ -327,28 +327,41 @@ __global__ __launch_bounds__(1024) void collect_active_columns_kernel(const VT *
 constexpr int kColBinThreads = 1024;  // 16 waves share one set of bins: 4 times fewer, 4 times larger bins
 constexpr size_t kColBinBytesMax = static_cast<size_t>(3) << 30;  // bins of the dense column walk (scratch memory)
 
-template <typename T1, typename VT, int IN, int W>
+//
+// FUSED: the generators are seeded inside this kernel instead, as in the row walk: workgroup p takes the
+// entries p, p + G, p + 2 G, ... (G workgroups), 64 of them are a batch, its waves take (batch, entry) tasks
+// from a counter in LDS, and the wave that takes the first entry of batch j first seeds batch j + 1 on the
+// vector unit (lane per stream) into slot (j + 1) % 3 of the workgroup's ring of seeded states in device
+// memory (`states`, kFuseRingBytes per workgroup), which the other waves read back from the L2.  Only the
+// first batch of a workgroup is waited for; n_seeded is not used.
+template <typename T1, typename VT, int IN, int W, bool FUSED>
 __global__ __launch_bounds__(kColBinThreads, sizeof(T1) == 4 ? 8 : 4) void jitconn_colwalk_bins_kernel(
     const VT *__restrict__ in, T1 *__restrict__ out, uint32_t n_out, uint32_t seed, double log_p, T1 wa, T1 wb,
     uint32_t first, uint32_t n_list_host, const uint32_t *__restrict__ n_list_dev,
-    const uint32_t *__restrict__ list_col, const T1 *__restrict__ list_val, const uint32_t *__restrict__ states,
+    const uint32_t *__restrict__ list_col, const T1 *__restrict__ list_val, uint32_t *states,
     uint32_t n_seeded, uint32_t n_win, uint32_t shift, uint32_t cap, BinPair<T1> *__restrict__ pairs,
     uint32_t *__restrict__ counts) {
   constexpr int kWaves = kColBinThreads / kWave;
   constexpr int kWords = StreamLds<T1, W>::words;
   __shared__ __attribute__((aligned(8))) uint32_t s_state[kWaves * kWords];
   __shared__ uint32_t s_cnt[kBinMaxWindows];
+  __shared__ uint32_t s_task, s_ready[kFuseSlots], s_loaded[kFuseSlots];
 
   const int lane = lane_id();
   const uint32_t wave = threadIdx.x / kWave;
   const uint32_t p = blockIdx.x;
   if (threadIdx.x < n_win) s_cnt[threadIdx.x] = counts[static_cast<size_t>(threadIdx.x) * gridDim.x + p];
+  if (threadIdx.x == 0) {
+    s_task = 0;
+    for (uint32_t k = 0; k < kFuseSlots; ++k) s_ready[k] = 0, s_loaded[k] = 0;
+  }
   __syncthreads();
   BinPair<T1> *region = pairs + static_cast<uint64_t>(p) * n_win * cap;
   uint32_t *st = s_state + wave * kWords;
   const uint32_t n_list = n_list_dev ? *n_list_dev : n_list_host;
 
-  for (uint32_t k = wave * gridDim.x + p; k < n_list; k += gridDim.x * kWaves) {
+  // list entry k: its stream, seeded at `pre` (or nullptr: the wave seeds it itself)
+  auto walk_entry = [&](uint32_t k, const uint32_t *pre, auto &&loaded) {
     uint32_t col;
     T1 val;
     if (list_col != nullptr) {
@@ -357,9 +370,11 @@ __global__ __launch_bounds__(kColBinThreads, sizeof(T1) == 4 ? 8 : 4) void jitco
     } else {
       col = first + k;
       val = static_cast<T1>(in[col]);
-      if (!is_event(val)) continue;  // a zero input adds nothing (wave uniform)
+      if (!is_event(val)) {  // a zero input adds nothing (wave uniform)
+        loaded();
+        return;
+      }
     }
-    const uint32_t *pre = (k < n_seeded) ? states + static_cast<size_t>(k) * kMtN : nullptr;
     walk_stream<T1, W>(st, lane, seed + col, pre, n_out, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
       if (valid) {
         T1 add;
@@ -376,7 +391,64 @@ __global__ __launch_bounds__(kColBinThreads, sizeof(T1) == 4 ? 8 : 4) void jitco
           atomic_add(&out[idx], add);
         }
       }
-    });
+    }, loaded);
+  };
+
+  if constexpr (!FUSED) {
+    for (uint32_t k = wave * gridDim.x + p; k < n_list; k += gridDim.x * kWaves)
+      walk_entry(k, (k < n_seeded) ? states + static_cast<size_t>(k) * kMtN : nullptr, NoLoadHook());
+  } else {
+    // this workgroup's entries: p + i * G for i < mine
+    const uint32_t mine = n_list > p ? (n_list - p + gridDim.x - 1u) / gridDim.x : 0u;
+    const uint32_t batches = (mine + kFuseBatch - 1u) / kFuseBatch;
+    uint32_t *ring = states + static_cast<size_t>(p) * kFuseSlots * kFuseBatch * kMtN;
+    auto seed_batch = [&](uint32_t j) {
+      const uint32_t slot = j % kFuseSlots;
+      const uint32_t i = j * kFuseBatch + static_cast<uint32_t>(lane);
+      uint32_t col = 0;
+      if (i < mine) {
+        const uint32_t k = p + i * gridDim.x;
+        col = list_col != nullptr ? list_col[k] : first + k;
+      }
+      const uint32_t left = mine - j * kFuseBatch;
+      mt_seed_batch(st, lane, seed + col, ring + static_cast<size_t>(slot) * kFuseBatch * kMtN,
+                    left < kFuseBatch ? left : kFuseBatch);
+      __hip_atomic_store(&s_ready[slot], j + 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
+    if (wave == 0 && batches != 0) seed_batch(0);
+    for (;;) {
+      // (every lane adds one: the counter advances by 64 per task, any lane's old value / 64 is the task)
+      const uint32_t t = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(
+                             static_cast<int>(atomicAdd(&s_task, 1u)))) / kWave;
+      const uint32_t j = t / kFuseBatch, r = t % kFuseBatch;
+      if (j >= batches) break;
+      if (r == 0 && j + 1 < batches) {
+        // slot (j + 1) % 3 last held batch j - 2: (j + 1) / 3 batches have used it, 64 loads each
+        const uint32_t slot = (j + 1u) % kFuseSlots, need = ((j + 1u) / kFuseSlots) * kFuseBatch;
+        bool free_ = false;
+        for (uint32_t spin = 0; spin < kFuseSpin && !free_; ++spin) {
+          free_ = __hip_atomic_load(&s_loaded[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) >= need;
+          if (!free_) __builtin_amdgcn_s_sleep(2);
+        }
+        if (free_) seed_batch(j + 1u);
+        else __hip_atomic_store(&s_ready[slot], kFuseNotSeeded | (j + 2u), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+      const uint32_t slot = j % kFuseSlots;
+      uint32_t flag = 0;
+      for (uint32_t spin = 0; spin < kFuseSpin; ++spin) {
+        flag = __hip_atomic_load(&s_ready[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if ((flag & ~kFuseNotSeeded) >= j + 1u) break;
+        flag = kFuseNotSeeded;
+        __builtin_amdgcn_s_sleep(2);
+      }
+      const uint32_t *pre = (flag & kFuseNotSeeded) ? nullptr : ring + (static_cast<size_t>(slot) * kFuseBatch + r) * kMtN;
+      auto loaded = [&]() {
+        if (lane == 0) __hip_atomic_fetch_add(&s_loaded[slot], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      };
+      const uint32_t i = j * kFuseBatch + r;
+      if (i < mine) walk_entry(p + i * gridDim.x, pre, loaded);
+      else loaded();
+    }
   }
   __syncthreads();
   if (threadIdx.x < n_win) counts[static_cast<size_t>(threadIdx.x) * gridDim.x + p] = s_cnt[threadIdx.x];
@@ -578,7 +650,7 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
     return;
   }
   bool out_cleared = false;  // (with event input and bins, the kernel that lists the active columns clears it)
-  // Many pairs: bins (also for a narrow output: seeding ahead and the even spread of the streams pay).  The number of pairs is n_in * n_out * p for a
+  // Many pairs: bins (also for a narrow output: seeding on the vector unit and the even spread of the streams pay).  The number of pairs is n_in * n_out * p for a
   // dense input; for events it depends on the activity, which the host does not know: bins are sized
   // for one column in eight being active (fuller bins overflow into direct atomics) and used when
   // one active column in a hundred already means a hundred thousand pairs (10,000 x 10,000 with
@@ -588,10 +660,10 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
   const double p_conn = -std::expm1(log_p);
   const double full = static_cast<double>(n_in) * static_cast<double>(n_out) * p_conn;
   const bool bins = n_win <= kBinMaxWindows && full >= (IN == kInDense ? 1048576.0 : 1.0e7);
-  // Event input and fewer pairs: the same list of active columns and the same seeding ahead on the vector unit, but
+  // Event input and fewer pairs: the same list of active columns and the same seeding on the vector unit, but
   // the walk adds its pairs to `out` with atomics.  (A wave that seeds its own stream spends 2 us of the CU's one
   // scalar unit on it: with 200,000 active columns of ten synapses each the walk without a list took 1.2 ms.)
-  // A dense input with fewer pairs takes the same walk over all its columns, seeded ahead chunk by chunk (4,000 x
+  // A dense input with fewer pairs takes the same walk over all its columns, chunk by chunk (4,000 x
   // 4,000 with conn_prob 0.02: 0.5 ms where every lane seeded the generator of its own column).
   // (Event input with fewer than 2,048 columns stays with the walk below: at 1 % activity its one launch takes 26 us
   // against the 35 us of list, seeds and walk, though 125 against 47 us at 20 %.)
@@ -621,8 +693,8 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
     // no bins (every pair goes to `out` with an atomic): nothing to size and nothing to empty between the chunks
     if (!bins) cap_d = 0.0, pair_bytes = 0, group = chunks;
     const size_t count_bytes = round_up(static_cast<size_t>(n_win) * producers * sizeof(uint32_t));
-    const uint32_t seeded_max = n_in < kSeedChunk ? n_in : kSeedChunk;
-    const size_t state_bytes = round_up(static_cast<size_t>(seeded_max) * kMtN * 4);
+    // the workgroups' rings of generator states, seeded inside the walk
+    const size_t state_bytes = round_up(static_cast<size_t>(producers) * kFuseRingBytes);
     const size_t list_bytes = (IN == kInEvent) ? round_up(static_cast<size_t>(n_in) * 4) : 0;
     const size_t val_bytes = (IN == kInEvent) ? round_up(static_cast<size_t>(n_in) * sizeof(T1)) : 0;
     uint32_t *list_count = (IN == kInEvent) ? stream_counters(stream) : nullptr;
@@ -636,31 +708,26 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
         uint32_t *states = reinterpret_cast<uint32_t *>(ws + pair_bytes + count_bytes);
         uint32_t *list_col = list_bytes ? reinterpret_cast<uint32_t *>(ws + pair_bytes + count_bytes + state_bytes) : nullptr;
         T1 *list_val = val_bytes ? reinterpret_cast<T1 *>(ws + pair_bytes + count_bytes + state_bytes + list_bytes) : nullptr;
-        auto walk = jitconn_colwalk_bins_kernel<T1, VT, IN, W>;
+        auto walk = jitconn_colwalk_bins_kernel<T1, VT, IN, W, true>;
         out_cleared = true;
         if (IN == kInEvent) {
-          // the active columns, their generators seeded ahead (those beyond kSeedChunk seed themselves), one walk
+          // the active columns, then one walk that seeds their generators as it goes
           hipLaunchKernelGGL((collect_active_columns_kernel<T1, VT>), dim3(div_up(n_in, kCollectCols)), dim3(1024), 0, stream,
                              in, n_in, list_count, list_col, list_val, counts, n_win * producers, out, n_out);
-          hipLaunchKernelGGL(mt_seed_streams_kernel, dim3(div_up(seeded_max, kSeedThreads)), dim3(kSeedThreads), 0,
-                             stream, seed, 0u, seeded_max, states, static_cast<const uint32_t *>(list_col),
-                             static_cast<const uint32_t *>(list_count));
           hipLaunchKernelGGL(walk, dim3(producers), dim3(kColBinThreads), 0, stream, in, out, n_out, seed, log_p, wa, wb,
                              0u, 0u, static_cast<const uint32_t *>(list_count), static_cast<const uint32_t *>(list_col),
-                             static_cast<const T1 *>(list_val), static_cast<const uint32_t *>(states), seeded_max,
-                             n_win, shift, cap, pairs, counts);
+                             static_cast<const T1 *>(list_val), states, 0u, n_win, shift, cap, pairs, counts);
         } else {
-          // every column, a chunk of seeded generators at a time; the bins are emptied after every `group` chunks
+          // every column, a chunk at a time; the bins are emptied after every `group` chunks
           fill_zero(stream, out, n_out);
           fill_zero(stream, counts, n_win * producers);
           uint32_t in_bins = 0;
           for (uint32_t first = 0; first < n_in; first += kSeedChunk) {
             const uint32_t count = (n_in - first < kSeedChunk) ? n_in - first : kSeedChunk;
-            launch_seed_streams(stream, seed, first, count, states);
             hipLaunchKernelGGL(walk, dim3(producers), dim3(kColBinThreads), 0, stream, in, out, n_out, seed, log_p, wa,
                                wb, first, count, static_cast<const uint32_t *>(nullptr),
-                               static_cast<const uint32_t *>(nullptr), static_cast<const T1 *>(nullptr),
-                               static_cast<const uint32_t *>(states), count, n_win, shift, cap, pairs, counts);
+                               static_cast<const uint32_t *>(nullptr), static_cast<const T1 *>(nullptr), states, 0u,
+                               n_win, shift, cap, pairs, counts);
             if (++in_bins == group && first + kSeedChunk < n_in) {
               if (!add_uniform_bins<T1>("jitconn column walk", stream, out, n_out, shift, producers, cap, pairs, counts,
                                         static_cast<uint32_t *>(nullptr)))
