@@ -929,6 +929,207 @@ __device__ __forceinline__ void gather_hub_rows(const F *__restrict__ data, cons
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// event gather, walked flat (bitmaps of more than 80 KB, rows of 16 to 383 nonzeros on average)
+// ------------------------------------------------------------------------------------------------
+// The row-wise walks pad every row to whole steps of its lane group: with 100 nonzeros per row and 8 lanes
+// x 16 loads per row a quarter of the index requests lie beyond their row.  Here every wave owns a contiguous
+// range of the nonzeros that begins and ends at row boundaries (the rows whose first nonzero lies in its
+// equal share of the nonzeros: no row is shared by two waves, so nothing is left for a second kernel) and
+// takes it in steps of 1,024: four 16-byte nontemporal loads of indices per lane (the next step's are
+// requested before this step's are used), sixteen probes of the event bitmap in LDS per lane.  Rows are
+// looked up for the HITS only: the lanes leave the positions of their hits (some 5 % of the nonzeros) in a
+// queue in LDS, compacted by a prefix sum over the wave, and every lane then takes one hit: its weight, a
+// six-step search of a window of 65 row offsets in LDS for its row, one atomic addition to that row's
+// accumulator (float64; a homogeneous weight: a 32-bit count).  Rows that end inside the step are stored.
+constexpr uint32_t kFlatEvRows = 64;     // rows of a window (one per lane)
+constexpr uint32_t kFlatEvQueue = 256;   // hits queued at a time (more in a step: further rounds)
+constexpr uint32_t kFlatEvMinMean = 16, kFlatEvMaxMean = 384;
+constexpr uint32_t kFlatEvWaves = 16;
+// static LDS of the walk: windows, accumulators and queues of 16 waves
+constexpr size_t kFlatEvLdsBytes = kFlatEvWaves * ((kFlatEvRows + 2) * 4 + kFlatEvRows * 8 + kFlatEvQueue * 2) + 256;
+// the largest event bitmap that is kept whole in LDS (beside that; wider event vectors get a two-level bitmap)
+constexpr size_t kLdsEventBitmapCap = (kLdsBitmapCap - kFlatEvLdsBytes) / 256 * 256;
+
+// the first row r in [0, n_row] with indptr[r] >= pos, for pos <= indptr[n_row]: the wave searches together,
+// 64 probes a round
+__device__ __forceinline__ uint32_t first_row_from(const uint32_t *__restrict__ indptr, uint32_t n_row, uint32_t pos,
+                                                   uint32_t lane) {
+  uint32_t lo = 0, hi = n_row;  // the answer lies in [lo, hi]: indptr[r] < pos for r < lo, indptr[hi] >= pos
+  while (lo < hi) {
+    const uint32_t span = hi - lo;
+    const uint32_t stride = span / kWave + (span % kWave ? 1u : 0u);
+    const uint64_t probe = static_cast<uint64_t>(lo) + static_cast<uint64_t>(lane) * stride;
+    const bool below = probe < hi && indptr[probe] < pos;  // (the lanes for which this holds form a prefix)
+    const uint32_t cnt = static_cast<uint32_t>(__popcll(__ballot(below)));
+    if (cnt == 0) return lo;  // indptr[lo] >= pos
+    // indptr[lo + (cnt - 1) stride] < pos, and the probe after it (if it lies below hi) is not below pos
+    const uint64_t next = static_cast<uint64_t>(lo) + static_cast<uint64_t>(cnt) * stride;
+    if (next < hi) hi = static_cast<uint32_t>(next);
+    lo += (cnt - 1u) * stride + 1u;
+  }
+  return lo;
+}
+
+template <typename F, bool HETER>
+__device__ __forceinline__ void gather_rows_flat_event(const F *__restrict__ data, const uint32_t *__restrict__ indices,
+                                                       const uint32_t *__restrict__ indptr, F *__restrict__ y,
+                                                       uint32_t n_row, uint32_t nnz, const uint32_t *s_bits) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  using A = typename std::conditional<HETER, double, uint32_t>::type;
+  constexpr int U = 4;
+  constexpr uint32_t kStep = 4u * U * kWave;  // nonzeros per step
+  __shared__ uint32_t s_ptr_all[kFlatEvWaves][kFlatEvRows + 2];
+  __shared__ A s_sum_all[kFlatEvWaves][kFlatEvRows];
+  __shared__ uint16_t s_queue_all[kFlatEvWaves][kFlatEvQueue];
+  const uint32_t lane = static_cast<uint32_t>(lane_id()), wv = threadIdx.x / kWave;
+  uint32_t *s_ptr = s_ptr_all[wv];
+  A *s_sum = s_sum_all[wv];
+  uint16_t *s_queue = s_queue_all[wv];
+  const uint32_t waves = gridDim.x * (blockDim.x / kWave), w = blockIdx.x * (blockDim.x / kWave) + wv;
+  const F w_homo = HETER ? F(0) : data[0];
+  // equal shares of the nonzeros, in whole steps; the wave's rows are those that begin in its share
+  const uint64_t share = ((static_cast<uint64_t>(nnz) + waves - 1u) / waves + kStep - 1u) / kStep * kStep;
+  const uint64_t pos0 = static_cast<uint64_t>(w) * share, pos1 = pos0 + share;
+  if (pos0 >= nnz && w != 0) return;
+  uint32_t r = (w == 0) ? 0u : first_row_from(indptr, n_row, static_cast<uint32_t>(pos0), lane);
+  const uint32_t r_end = (pos1 >= nnz) ? n_row : first_row_from(indptr, n_row, static_cast<uint32_t>(pos1), lane);
+  if (r >= r_end) return;
+  const uint32_t begin = indptr[r], end = indptr[r_end];
+  if (begin == end) {  // rows without nonzeros only
+    for (uint32_t i = r + lane; i < r_end; i += kWave) y[i] = F(0);
+    return;
+  }
+  s_sum[lane] = A(0);
+  if (lane == 0) s_ptr[kFlatEvRows + 1] = 0xffffffffu;
+
+  auto load_indices = [&](uint32_t s0, u32x4 (&ci)[U]) {  // lane l: quads s0 / 4 + l, + 64, ...
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t q = s0 / 4u + static_cast<uint32_t>(u) * kWave + lane;
+      ci[u] = u32x4{0u, 0u, 0u, 0u};
+      if (s0 < end && 4u * q < end) {
+        if (4u * q + 4u <= nnz) {
+          ci[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(indices) + q);
+        } else {  // (the array's last, partial quad)
+          if (4u * q + 0u < nnz) ci[u].x = indices[4u * q + 0u];
+          if (4u * q + 1u < nnz) ci[u].y = indices[4u * q + 1u];
+          if (4u * q + 2u < nnz) ci[u].z = indices[4u * q + 2u];
+        }
+      }
+    }
+  };
+  // The indices of the next two steps are under way while a step is worked on (with one step ahead the walk
+  // streamed at 3.4 TB/s).  The second one is requested at the END of a step, behind the gathers of the hits'
+  // weights: waiting for a load means waiting for every load issued before it, and the step before's request
+  // has arrived by then.
+  u32x4 ci[U], ci1[U], ci2[U];
+  const uint32_t first_step = begin / 4u * 4u;  // (steps begin at whole quads; what lies before `begin` is masked)
+  load_indices(first_step, ci);
+  load_indices(first_step + kStep, ci1);
+  load_indices(first_step + 2u * kStep, ci2);  // (a step at or beyond the end of the range loads nothing)
+  for (uint32_t s0 = first_step; s0 < end; s0 += kStep) {
+    const uint32_t s1 = (end - s0 > kStep) ? s0 + kStep : end;
+    uint32_t ptr_lane, ptr_last;
+    auto load_window = [&]() {
+      const uint64_t k = static_cast<uint64_t>(r) + lane;
+      ptr_lane = k <= n_row ? indptr[k] : 0xffffffffu;
+      ptr_last = static_cast<uint64_t>(r) + kFlatEvRows <= n_row ? indptr[r + kFlatEvRows] : 0xffffffffu;
+    };
+    load_window();
+    // the sixteen probes: bit 4 u + t of `hits` = nonzero 4 (s0 / 4 + 64 u + lane) + t is in the range and its
+    // column has an event
+    uint32_t hits = 0;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t c[4] = {ci[u].x, ci[u].y, ci[u].z, ci[u].w};
+#pragma unroll
+      for (int t = 0; t < 4; ++t)  // (the bit-field extract takes the low five bits of its offset)
+        hits |= __builtin_amdgcn_ubfe(s_bits[c[t] >> 5], c[t], 1u) << (4 * u + t);
+    }
+    if (s0 < begin || s1 - s0 < kStep) {  // (the first and the last step of the range only: what lies outside is column 0)
+      uint32_t inside = 0;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t p0 = 4u * (s0 / 4u + static_cast<uint32_t>(u) * kWave + lane);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const uint32_t p = p0 + static_cast<uint32_t>(t);
+          inside |= ((p >= begin && p < s1) ? 1u : 0u) << (4 * u + t);
+        }
+      }
+      hits &= inside;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) ci[u] = ci1[u];
+    // where the lane's hits go in the step's sequence of hits
+    const uint32_t mine = static_cast<uint32_t>(__popc(hits));
+    const uint32_t incl = wave_inclusive_scan_u32(mine);
+    const uint32_t total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(incl), kWave - 1));
+    auto fill_queue = [&](uint32_t base) {  // hits number base .. base + 255 of the step: (u, lane, t) each
+      uint32_t m = hits, at = incl - mine;
+      while (m != 0u) {
+        const uint32_t b = static_cast<uint32_t>(__ffs(static_cast<int>(m))) - 1u;
+        m &= m - 1u;
+        if (at - base < kFlatEvQueue) s_queue[at - base] = static_cast<uint16_t>(((b >> 2) << 8) | (lane << 2) | (b & 3u));
+        ++at;
+      }
+    };
+    if (total != 0u && total <= kFlatEvQueue) fill_queue(0u);
+    // windows of 64 rows from r on, until one reaches beyond the step
+    for (;;) {
+      s_ptr[lane] = ptr_lane;
+      if (lane == 0) s_ptr[kFlatEvRows] = ptr_last;
+      __builtin_amdgcn_wave_barrier();
+      const uint32_t lo = s_ptr[0], hi = ptr_last;
+      const uint32_t top = hi < s1 ? hi : s1;  // the window takes the hits at nonzeros [lo, top)
+      for (uint32_t base = 0; base < total; base += kFlatEvQueue) {
+        if (total > kFlatEvQueue) {
+          __builtin_amdgcn_wave_barrier();
+          fill_queue(base);
+          __builtin_amdgcn_wave_barrier();
+        }
+        const uint32_t n = total - base < kFlatEvQueue ? total - base : kFlatEvQueue;
+        for (uint32_t i = lane; i < n; i += kWave) {
+          const uint32_t e = s_queue[i];
+          const uint32_t p = 4u * (s0 / 4u + (e >> 8) * kWave + ((e >> 2) & 63u)) + (e & 3u);
+          if (p >= lo && p < top) {
+            uint32_t k = 0;  // the last k < 64 with s_ptr[k] <= p
+#pragma unroll
+            for (uint32_t step = kFlatEvRows / 2; step != 0; step >>= 1)
+              if (s_ptr[k + step] <= p) k += step;
+            if constexpr (HETER) atomicAdd(&s_sum[k], static_cast<double>(data[p]));
+            else atomicAdd(&s_sum[k], 1u);
+          }
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+      // rows of the window that end inside the step (a prefix of the window) are stored
+      const uint64_t row = static_cast<uint64_t>(r) + lane;
+      const bool ended = row < r_end && s_ptr[lane + 1u] <= s1;
+      const uint32_t n_ended = static_cast<uint32_t>(__popcll(__ballot(ended)));
+      if (ended) {
+        if constexpr (HETER) y[row] = static_cast<F>(s_sum[lane]);
+        else y[row] = gathered_sum(w_homo, s_sum[lane]);
+      }
+      const A open = n_ended < kFlatEvRows ? s_sum[n_ended] : A(0);  // (wave uniform address: a broadcast)
+      __builtin_amdgcn_wave_barrier();
+      s_sum[lane] = A(0);
+      r += n_ended;
+      if (n_ended < kFlatEvRows || r >= r_end) {
+        if (lane == 0) s_sum[0] = open;
+        break;
+      }
+      load_window();
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int u = 0; u < U; ++u) ci1[u] = ci2[u];
+    load_indices(s0 + 3u * kStep, ci2);
+  }
+}
+
 // (Event input with the bitmap in LDS is meant to run two workgroups per CU: eight waves per SIMD, asked
 // for here because the homogeneous-weight walks sit at exactly 64 registers and the hub-row pass behind
 // them would otherwise raise the kernel's allocation to 66.)
@@ -998,6 +1199,14 @@ __global__ __launch_bounds__(1024, (MODE == kEvent && BITS == 1) ? 8 : 4) void c
     // An event bitmap above 80 KB leaves room for one workgroup (16 waves) per CU only: every lane
     // then keeps 16 (rows under 48 nonzeros: 8) loads in flight instead of 2 to 8, in groups of
     // 8 or 4 lanes per row, or HBM sees too few requests (1e6 columns, 100 per row: 424 -> 164 us).
+    if constexpr (BITS == 2) {
+      // rows of 16 to 383 nonzeros on average: the flat walk over the nonzeros, which leaves no row to the pass below
+      if (mean >= kFlatEvMinMean && mean < kFlatEvMaxMean && nnz <= kFlatMaxNnz && blockDim.x == kFlatEvWaves * kWave &&
+          (reinterpret_cast<uintptr_t>(indices) & 15u) == 0) {
+        gather_rows_flat_event<F, HETER>(data, indices, indptr, y, n_row, nnz, s_bits);
+        return;
+      }
+    }
     if (mean >= 384) { gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = 1; hub_len = kHubSteps * 8 * kWave; }
     else if (mean >= 48) { gather_rows<F, VT, HETER, MODE, BITS, 8, 16>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 8; hub_len = kHubSteps * 16 * 8; }
     else { gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 4; hub_len = kHubSteps * 8 * 4; }
@@ -1405,7 +1614,7 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
   if constexpr (MODE == kEvent && !std::is_same<VT, PackedBits>::value) {
     // A bitmap that does not fit LDS (more than 1.3 million columns): two levels, the exact one in
     // global memory and a coarse one (one bit per 2^g columns) for LDS, both built here.
-    if ((static_cast<size_t>(n_col) + 31) / 32 * 4 > kLdsBitmapCap) {
+    if ((static_cast<size_t>(n_col) + 31) / 32 * 4 > kLdsEventBitmapCap) {
       const uint32_t g = coarse_shift(n_col);
       const uint32_t n_words = (n_col + 31u) / 32u, off = coarse_offset_words(n_col);
       const uint32_t c_words = (coarse_bits(n_col, g) + 31u) / 32u;
@@ -1423,23 +1632,30 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
       bpl_clear_error();
     }
   }
-  if constexpr (MODE == kEvent && sizeof(VT) > 1 && !std::is_same<VT, PackedBits>::value) {
+  if constexpr (MODE == kEvent && !std::is_same<VT, PackedBits>::value) {
     // Wide event types: every persistent workgroup would read the whole vector (4 or 8 bytes per
-    // element) to build its bitmap; pack it once instead and hand the words to the kernels.
+    // element) to build its bitmap; pack it once instead and hand the words to the kernels.  Byte events
+    // likewise from 655,360 columns on (a bitmap of more than 80 KB, one workgroup per CU: 256 workgroups that
+    // each read a megabyte of events take longer than one small kernel and 125 KB per workgroup).
     const size_t words = (static_cast<size_t>(n_col) + 31) / 32;
-    uint32_t *bits = static_cast<uint32_t *>(src.request((words + 1) * sizeof(uint32_t)));
-    if (bits != nullptr) {
+    uint32_t *bits = (sizeof(VT) > 1 || words * 4 > 80 * 1024 - 512)
+                         ? static_cast<uint32_t *>(src.request((words + 1) * sizeof(uint32_t)))
+                         : nullptr;
+    if (sizeof(VT) == 1 && words * 4 <= 80 * 1024 - 512) {
+      // (byte events and a bitmap that leaves room for two workgroups per CU: they pack it themselves)
+    } else if (bits != nullptr) {
       pack_event_bitmap<VT>(stream, x, n_col, bits);
       launch_gather<F, PackedBits, HETER, MODE>(target, src, data, indices, indptr,
                                                 reinterpret_cast<const PackedBits *>(bits), y, n_row, n_col);
       return;
+    } else {
+      if (src.failure_is_final()) return ensure_error(target, "nothing was enqueued: the path that the scratch memory at hand allows could not be launched");  // beyond a fixed arena, or during a capture: the error stands
+      bpl_clear_error();
     }
-    if (src.failure_is_final()) return ensure_error(target, "nothing was enqueued: the path that the scratch memory at hand allows could not be launched");  // beyond a fixed arena, or during a capture: the error stands
-    bpl_clear_error();
   }
   if (MODE == kEvent) {
     const size_t lds_bytes = (static_cast<size_t>(n_col) + 31) / 32 * 4;
-    const size_t lds_cap = kLdsBitmapCap;
+    const size_t lds_cap = kLdsEventBitmapCap;
     if (lds_bytes <= lds_cap) {
       const bool ok = lds_bytes > 80 * 1024 - 512  // (two workgroups per CU below: 80 KB each, less their static LDS)
                           ? launch_gather_impl<F, VT, HETER, MODE, 2>(target, stream, data, indices, indptr, x, y, n_row,

@@ -238,6 +238,50 @@ def test_gather_row_length_modes_with_a_bitmap_that_fills_lds(cuda, oracle_mod):
     assert_close(got, want)
 
 
+@pytest.mark.parametrize("kind", ["ragged", "even", "step", "hub", "few", "dense_events", "offset"])
+def test_gather_flat_walk_over_the_nonzeros_of_short_rows(cuda, oracle_mod, kind):
+  # more than 655,360 columns and rows of 16 to 383 nonzeros on average: every wave walks a contiguous range of the
+  # nonzeros that begins and ends at row boundaries and looks rows up for the hits only.  Integer weights: the sums
+  # are exact, so every output is compared bit for bit (weights per nonzero, one weight, float events, float64).
+  rng = np.random.default_rng(sum(map(ord, kind)))
+  n_col, rate = 900_000, 0.05
+  if kind == "ragged":      # empty rows, rows of one nonzero, rows of a thousand
+    counts = rng.choice([0, 1, 3, 40, 150, 1000], size=60_000, p=[0.2, 0.1, 0.2, 0.3, 0.15, 0.05])
+  elif kind == "even":      # every row 100 nonzeros: ten rows and a bit per step of 1,024
+    counts = np.full(200_000, 100)
+  elif kind == "step":      # rows of exactly one step and of exactly one quad
+    counts = np.where(np.arange(30_000) % 3 == 0, 1024, 4)
+  elif kind == "hub":       # one row longer than a wave's whole share, between rows of 30
+    counts = np.full(40_000, 30)
+    counts[17_777] = 700_000
+  elif kind == "few":       # fewer rows than waves
+    counts = rng.integers(16, 200, size=1_500)
+  elif kind == "dense_events":  # most nonzeros hit: the queue of hits is filled in several rounds per step
+    counts, rate = rng.poisson(60, size=50_000), 0.9
+  else:                     # many empty rows in a row, the matrix's last nonzeros in a partial quad
+    counts = np.where((np.arange(90_001) // 500) % 2 == 0, 0, 70)
+    counts[-1] = 3
+  indices, indptr = synth.counted_csr(np.minimum(counts, n_col), n_col, seed=len(counts))
+  nnz, n_row = indices.shape[0], len(counts)
+  mean = nnz // n_row
+  assert 16 <= mean < 384, mean
+  shape = (n_row, n_col)
+  ev = rng.random(n_col) < rate
+  print("kind", kind, shape, "nnz", nnz, "mean", mean, flush=True)
+  for dtype in (np.float32, np.float64):
+    data = rng.integers(-3, 4, size=nnz).astype(dtype)
+    want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape)
+    got = bpl.event_csr_matvec(data, indices, indptr, ev, shape=shape).cpu().numpy()
+    assert np.array_equal(got, want), (kind, dtype, int((got != want).sum()), np.flatnonzero(got != want)[:5])
+    w = np.array([0.37], dtype=dtype)
+    want = oracle_mod.event_csr_matvec(w, indices, indptr, ev, shape=shape)
+    got = bpl.event_csr_matvec(w, indices, indptr, ev, shape=shape).cpu().numpy()
+    assert np.array_equal(got, want), (kind, dtype, "one weight")
+  evf = (ev * rng.uniform(0.5, 2.0, n_col)).astype(np.float64)
+  got = bpl.event_csr_matvec(data, indices, indptr, evf, shape=shape).cpu().numpy()
+  assert np.array_equal(got, oracle_mod.event_csr_matvec(data, indices, indptr, evf, shape=shape)), (kind, "float events")
+
+
 def test_gather_with_a_two_level_event_bitmap(cuda, oracle_mod):
   # more columns than a bitmap in LDS can cover (1.3 million): a coarse bitmap (one bit per 2^g
   # columns) in LDS and the exact one in global memory; g = 2, 4 and 6 (both ways the coarse
