@@ -280,11 +280,10 @@ def device_rates(lib, dev):
   blocks, iters = 2 * cu, 2048
   out = torch.zeros(blocks, dtype=torch.float32, device=dev)
   ops = blocks * 1024 * iters
-  base = timed(lambda: lib.bench_lds_atomic(stream, out.data_ptr(), blocks, iters, 4))
-  for mode, name in ((0, "lds_add_f32"), (1, "lds_add_u32"), (2, "lds_add_f64"), (3, "lds_write_b32")):
+  for mode, name in ((0, "lds_add_f32"), (1, "lds_add_u32"), (2, "lds_add_f64"), (3, "lds_write_b32"),
+                     (4, "lds_address_arithmetic_only")):
     t = timed(lambda: lib.bench_lds_atomic(stream, out.data_ptr(), blocks, iters, mode))
     rates[name + "_g_per_s"] = ops / t / 1e9
-    rates[name + "_g_per_s_less_address_arithmetic"] = ops / max(t - base, 1e-9) / 1e9
   rates["lds_workload"] = "%d workgroups of 1,024 threads, %d random operations per thread in a 64 KB window" % (blocks, iters)
   for n in (100_000, 1_000_000, 16_000_000):
     y = torch.zeros(n, dtype=torch.float32, device=dev)
