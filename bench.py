@@ -353,7 +353,7 @@ def main():
   ap.add_argument("--warmup", type=int, default=20)
   ap.add_argument("--skip-extra", action="store_true", help="only the headline workload")
   ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU baseline")
-  ap.add_argument("--pmc", choices=["gather", "scatter", "csr", "jitconn", "jitconn-normal", "jitconn-dense", "matmat"],
+  ap.add_argument("--pmc", choices=["gather", "scatter", "csr", "jitconn", "jitconn-normal", "jitconn-dense", "jitconn-dense-column", "matmat"],
                   default=None,
                   help="counter-collection mode for rocprofv3 --pmc.  gather: three plain copies of 400 MB "
                        "(the calibration kernel), three calls of the headline kernel and three plain streams over "
@@ -404,12 +404,12 @@ def main():
     log("pmc mode done")
     return
 
-  if args.pmc == "jitconn-dense":
+  if args.pmc in ("jitconn-dense", "jitconn-dense-column"):
     j = synth.config_jitconn_event()
     vec = torch.randn(j["shape"][0], dtype=torch.float32, device=dev)
     for _ in range(3):
       bpl.matvec_prob_conn_homo_weight(vec, j["weight"], conn_prob=j["conn_prob"], shape=j["shape"], seed=j["seed"],
-                                       outdim_parallel=True)
+                                       outdim_parallel=args.pmc == "jitconn-dense")
     torch.cuda.synchronize()
     log("pmc mode done")
     return

@@ -181,12 +181,14 @@ bool window_event_scatter(hipStream_t stream, const F *data, bool heter, const u
 bool window_event_scatter_self_usable(uint32_t n_row, uint32_t n_col);
 
 // Second half of the coarse-sorted scatter for producers other than the CSR one: adds bins laid
-// out uniformly, bin (p, b) = pairs + (p * n_win + b) * cap with counts[b * producers + p]
-// BinPair<F> entries (bins.h; counts above cap mean cap), n_win = ceil(n_out / 2^shift), into the
-// zeroed y.  `reset` (optional): a device counter of the producer's that the kernel sets to zero.
+// out uniformly, bin (p, b) = the places from (p * n_win + b) * cap with counts[b * producers + p]
+// entries (counts above cap mean cap), n_win = ceil(n_out / 2^shift), into the zeroed y.  The places are
+// BinPair<F> entries (bins.h), or, `packed` (windows of at most 2^16 outputs, cap a multiple of 4): an
+// array of producers * n_win * cap values with the 16-bit positions within the window in an array behind
+// it.  `reset` (optional): a device counter of the producer's that the kernel sets to zero.
 template <typename F>
 bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_out, uint32_t shift, uint32_t producers,
-                      uint32_t cap, const void *pairs, const uint32_t *counts, uint32_t *reset);
+                      uint32_t cap, const void *pairs, bool packed, const uint32_t *counts, uint32_t *reset);
 
 inline unsigned div_up(unsigned long long a, unsigned long long b) {
   return static_cast<unsigned>((a + b - 1) / b);

@@ -337,7 +337,7 @@ int coo_bin_sum(const char *target, hipStream_t stream, const uint8_t *events, c
     const uint32_t hi = lo + chunk_conn < conn_size ? static_cast<uint32_t>(lo + chunk_conn) : conn_size;
     hipLaunchKernelGGL((bin_connections_kernel<F, I, EVENT>), dim3(producers), dim3(kCooThreads), 0, stream, events, values,
                        post_ids, pre_ids, static_cast<uint32_t>(lo), hi, post_size, result, n_win, shift, cap, pairs, counts);
-    if (!add_uniform_bins<F>(target, stream, result, post_size, shift, producers, cap, pairs, counts, nullptr)) return -1;
+    if (!add_uniform_bins<F>(target, stream, result, post_size, shift, producers, cap, pairs, false, counts, nullptr)) return -1;
   }
   return check_launch(target) ? 1 : -1;
 }

@@ -1454,20 +1454,20 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
 // the zeroed y of n_out elements: bin (p, b) = pairs + (p * n_win + b) * cap with counts[b * producers + p] pairs.
 template <typename F>
 bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_out, uint32_t shift, uint32_t producers,
-                      uint32_t cap, const void *pairs, const uint32_t *counts, uint32_t *reset) {
+                      uint32_t cap, const void *pairs, bool packed, const uint32_t *counts, uint32_t *reset) {
   const uint32_t n_win = div_up(n_out, 1u << shift);
-  auto add_kernel = add_bins_kernel<F, false>;
+  auto add_kernel = packed ? add_bins_kernel<F, true> : add_bins_kernel<F, false>;
   const uint32_t lds_shift = bin_lds_shift(shift);
   const uint32_t slices = 1u << (shift - lds_shift);
   const size_t lds = sizeof(double) << lds_shift;
-  static thread_local bool attr_set = false;
-  if (!attr_set && lds > 64 * 1024) {
+  static thread_local bool attr_set[2] = {false, false};
+  if (!attr_set[packed] && lds > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(add_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             static_cast<int>(lds)) != hipSuccess) {
       (void)hipGetLastError();
       return false;
     }
-    attr_set = true;
+    attr_set[packed] = true;
   }
   uint32_t parts = static_cast<uint32_t>(device_info().num_cu) / (n_win * slices);
   if (parts == 0) parts = 1;
@@ -1480,10 +1480,9 @@ bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_o
 }
 
 template bool add_uniform_bins<float>(const char *, hipStream_t, float *, uint32_t, uint32_t, uint32_t, uint32_t, const void *,
-                                      const uint32_t *, uint32_t *);
+                                      bool, const uint32_t *, uint32_t *);
 template bool add_uniform_bins<double>(const char *, hipStream_t, double *, uint32_t, uint32_t, uint32_t, uint32_t,
-                                       const void *,
-                                       const uint32_t *, uint32_t *);
+                                       const void *, bool, const uint32_t *, uint32_t *);
 template bool window_event_scatter_usable<float>(uint32_t, uint32_t);
 template bool window_event_scatter_usable<double>(uint32_t, uint32_t);
 template size_t window_event_scatter_bytes<float>(uint32_t);

@@ -321,9 +321,12 @@ __global__ __launch_bounds__(1024) void collect_active_columns_kernel(const VT *
 // Not FUSED: the generators of the first n_seeded entries were seeded ahead on the vector unit (`states`);
 // a wave seeding its own generator does it on the CU's one scalar unit, about 2 us each, and a
 // CU's waves queue up for it.  A pair for output window b (2^shift outputs) of workgroup p goes to
-// pairs[(p * n_win + b) * cap + position]; the positions continue from `counts` (zero before the
-// first launch of a call), so that a call may be split into several launches; a pair that finds
+// place (p * n_win + b) * cap + position of the bins; the positions continue from `counts` (zero before
+// the first launch of a call), so that a call may be split into several launches; a pair that finds
 // its bin full is added to `out` directly.  add_uniform_bins() then adds the bins window by window.
+// The bins hold n_pairs places: `packed` (windows of at most 2^16 outputs) as an array of values with an
+// array of 16-bit positions within the window behind it, 6 bytes a pair instead of 8 (10 instead of 16):
+// the pairs are written once and read once, and that traffic is what a walk over a dense vector costs.
 constexpr int kColBinThreads = 1024;  // 16 waves share one set of bins: 4 times fewer, 4 times larger bins
 constexpr size_t kColBinBytesMax = static_cast<size_t>(3) << 30;  // bins of the dense column walk (scratch memory)
 
@@ -339,8 +342,8 @@ __global__ __launch_bounds__(kColBinThreads, sizeof(T1) == 4 ? 8 : 4) void jitco
     const VT *__restrict__ in, T1 *__restrict__ out, uint32_t n_out, uint32_t seed, double log_p, T1 wa, T1 wb,
     uint32_t first, uint32_t n_list_host, const uint32_t *__restrict__ n_list_dev,
     const uint32_t *__restrict__ list_col, const T1 *__restrict__ list_val, uint32_t *states,
-    uint32_t n_seeded, uint32_t n_win, uint32_t shift, uint32_t cap, BinPair<T1> *__restrict__ pairs,
-    uint32_t *__restrict__ counts) {
+    uint32_t n_seeded, uint32_t n_win, uint32_t shift, uint32_t cap, void *__restrict__ pairs, uint64_t n_pairs,
+    uint32_t packed, uint32_t *__restrict__ counts) {
   constexpr int kWaves = kColBinThreads / kWave;
   constexpr int kWords = StreamLds<T1, W>::words;
   __shared__ __attribute__((aligned(8))) uint32_t s_state[kWaves * kWords];
@@ -356,7 +359,9 @@ __global__ __launch_bounds__(kColBinThreads, sizeof(T1) == 4 ? 8 : 4) void jitco
     for (uint32_t k = 0; k < kFuseSlots; ++k) s_ready[k] = 0, s_loaded[k] = 0;
   }
   __syncthreads();
-  BinPair<T1> *region = pairs + static_cast<uint64_t>(p) * n_win * cap;
+  const uint64_t region = static_cast<uint64_t>(p) * n_win * cap;  // first place of this workgroup's bins
+  T1 *const packed_val = static_cast<T1 *>(pairs);
+  uint16_t *const packed_rel = reinterpret_cast<uint16_t *>(packed_val + n_pairs);
   uint32_t *st = s_state + wave * kWords;
   const uint32_t n_list = n_list_dev ? *n_list_dev : n_list_host;
 
@@ -383,10 +388,17 @@ __global__ __launch_bounds__(kColBinThreads, sizeof(T1) == 4 ? 8 : 4) void jitco
         const uint32_t b = idx >> shift;
         const uint32_t slot = atomicAdd(&s_cnt[b], 1u);
         if (slot < cap) {
-          BinPair<T1> e;
-          e.rel = idx & ((1u << shift) - 1u);
-          e.val = add;
-          region[static_cast<uint64_t>(b) * cap + slot] = e;
+          const uint64_t at = region + static_cast<uint64_t>(b) * cap + slot;
+          const uint32_t rel = idx & ((1u << shift) - 1u);
+          if (packed) {
+            packed_val[at] = add;
+            packed_rel[at] = static_cast<uint16_t>(rel);
+          } else {
+            BinPair<T1> e;
+            e.rel = rel;
+            e.val = add;
+            static_cast<BinPair<T1> *>(pairs)[at] = e;
+          }
         } else {
           atomic_add(&out[idx], add);
         }
@@ -677,6 +689,8 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
     // Dense input: the bins are emptied (added to `out`) after every `group` chunks of kSeedChunk columns,
     // the largest number of chunks whose pairs fit kColBinBytesMax of scratch memory (every column of a
     // 1,000,000 x 1,000,000 matrix with conn_prob 0.001 at once would take 10.7 GB).
+    const bool packed = shift <= 16;
+    const size_t pair_size = packed ? sizeof(T1) + 2 : sizeof(BinPair<T1>);
     const uint32_t chunks = div_up(n_in, kSeedChunk);
     uint32_t group = chunks;
     double cap_d = 0.0;
@@ -686,7 +700,8 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
       const double per_bin = full * share / (static_cast<double>(producers) * n_win);  // every column active
       cap_d = 1.25 * per_bin + 6.0 * std::sqrt(per_bin) + 128.0;
       if (IN == kInEvent) cap_d = cap_d / 8.0 < 512.0 ? 512.0 : cap_d / 8.0;
-      pair_bytes = round_up(static_cast<size_t>(producers) * n_win * static_cast<size_t>(cap_d) * sizeof(BinPair<T1>));
+      cap_d = std::floor(cap_d / 4.0) * 4.0;  // (packed bins begin at multiples of four places)
+      pair_bytes = round_up(static_cast<size_t>(producers) * n_win * static_cast<size_t>(cap_d) * pair_size);
       if (IN == kInEvent || group == 1 || pair_bytes <= kColBinBytesMax) break;
       group = (group + 1u) / 2u;
     }
@@ -703,7 +718,8 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
       unsigned char *ws = static_cast<unsigned char *>(
         stream_workspace(stream, pair_bytes + count_bytes + state_bytes + list_bytes + val_bytes));
       if (ws != nullptr) {
-        BinPair<T1> *pairs = reinterpret_cast<BinPair<T1> *>(ws);
+        void *pairs = ws;
+        const uint64_t n_pairs = static_cast<uint64_t>(producers) * n_win * cap;
         uint32_t *counts = reinterpret_cast<uint32_t *>(ws + pair_bytes);
         uint32_t *states = reinterpret_cast<uint32_t *>(ws + pair_bytes + count_bytes);
         uint32_t *list_col = list_bytes ? reinterpret_cast<uint32_t *>(ws + pair_bytes + count_bytes + state_bytes) : nullptr;
@@ -716,7 +732,7 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
                              in, n_in, list_count, list_col, list_val, counts, n_win * producers, out, n_out);
           hipLaunchKernelGGL(walk, dim3(producers), dim3(kColBinThreads), 0, stream, in, out, n_out, seed, log_p, wa, wb,
                              0u, 0u, static_cast<const uint32_t *>(list_count), static_cast<const uint32_t *>(list_col),
-                             static_cast<const T1 *>(list_val), states, 0u, n_win, shift, cap, pairs, counts);
+                             static_cast<const T1 *>(list_val), states, 0u, n_win, shift, cap, pairs, n_pairs, packed ? 1u : 0u, counts);
         } else {
           // every column, a chunk at a time; the bins are emptied after every `group` chunks
           fill_zero(stream, out, n_out);
@@ -727,9 +743,9 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
             hipLaunchKernelGGL(walk, dim3(producers), dim3(kColBinThreads), 0, stream, in, out, n_out, seed, log_p, wa,
                                wb, first, count, static_cast<const uint32_t *>(nullptr),
                                static_cast<const uint32_t *>(nullptr), static_cast<const T1 *>(nullptr), states, 0u,
-                               n_win, shift, cap, pairs, counts);
+                               n_win, shift, cap, pairs, n_pairs, packed ? 1u : 0u, counts);
             if (++in_bins == group && first + kSeedChunk < n_in) {
-              if (!add_uniform_bins<T1>("jitconn column walk", stream, out, n_out, shift, producers, cap, pairs, counts,
+              if (!add_uniform_bins<T1>("jitconn column walk", stream, out, n_out, shift, producers, cap, pairs, packed, counts,
                                         static_cast<uint32_t *>(nullptr)))
                 return;  // (the error stands: part of the pairs is in `out` already)
               fill_zero(stream, counts, n_win * producers);
@@ -741,7 +757,7 @@ void launch_colwalk(hipStream_t stream, const VT *in, T1 *out, uint32_t n_out, u
           if (list_count != nullptr) fill_zero(stream, list_count, 1u);  // (the list's counter goes back to zero for the next call)
           return;
         }
-        if (add_uniform_bins<T1>("jitconn column walk", stream, out, n_out, shift, producers, cap, pairs, counts, list_count))
+        if (add_uniform_bins<T1>("jitconn column walk", stream, out, n_out, shift, producers, cap, pairs, packed, counts, list_count))
           return;
         // (the bins could not be added: nothing reached `out` yet except overflow pairs; start over)
         if (list_count != nullptr) fill_zero(stream, list_count, 1u);

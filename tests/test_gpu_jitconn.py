@@ -421,6 +421,28 @@ def test_column_walk_through_bins_dense(cuda, oracle_mod, w_kind, a, b, dtype):
   assert abs(y @ Mx - MTy @ x64) <= 1e-9 * max(1.0, abs(y @ Mx))
 
 
+@pytest.mark.parametrize("w_kind,a,b", [("homo", 0.0, 0.0), ("uniform", 0.25, 1.75)])
+@pytest.mark.parametrize("n_out,n_in,p,dtype", [(3_000_000, 300, 0.0015, np.float32), (3_000_000, 300, 0.0015, np.float64),
+                                                (9_000_000, 100, 0.0015, np.float32)])
+def test_column_walk_through_bins_wide_windows(cuda, oracle_mod, w_kind, a, b, n_out, n_in, p, dtype):
+  # outputs of more than two million elements: the windows grow beyond the 16,384 accumulators a workgroup
+  # holds at once (3,000,000: windows of 32,768 outputs added in two slices, pairs still packed with 16-bit
+  # positions; 9,000,000: windows of 131,072 outputs in eight slices, whole pairs).  Integer input: the
+  # homogeneous sums are exact.
+  lp = oracle_mod.log_p_of(p)
+  rng = np.random.default_rng(n_out % 1000)
+  x = rng.integers(-3, 4, n_in).astype(dtype)
+  x[x == 0] = 1
+  got = kernel_call(x, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=5, n_row=n_out, n_col=n_in, col_walk=True, dense=True)
+  want, mag = oracle_mod.jitconn_matvec(x, w_kind=w_kind, w_a=a, w_b=b, log_p=lp, seed=5, n_row=n_out, n_col=n_in,
+                                        col_walk=True, dense=True, return_abs=True)
+  assert mag.sum() > 1_048_576  # (enough pairs for the bins)
+  if w_kind == "homo":
+    assert np.array_equal(got, want)
+  else:
+    assert_close_reordered(got, want, mag, dtype, what="binned column walk, wide windows")
+
+
 @pytest.mark.parametrize("w_kind,a,b", [("homo", 0.0, 0.0), ("normal", 0.5, 2.0)])
 @pytest.mark.parametrize("n_out,n_in,p", [(4000, 4000, 0.02), (700, 90, 0.3), (5, 3, 0.9), (30_000, 2047, 0.01),
                                           (2 ** 24 + 5, 7, 2e-6), (2 ** 24 + 5, 140_000, 4e-7)])
