@@ -381,12 +381,36 @@ __global__ __launch_bounds__(kColBinThreads, sizeof(T1) == 4 ? 8 : 4) void jitco
       }
     }
     walk_stream<T1, W>(st, lane, seed + col, pre, n_out, log_p, wa, wb, [&](uint32_t idx, T1 w, bool valid) {
+      const uint32_t b = idx >> shift;
+      uint32_t slot = 0;
+      if constexpr (W != kNormal) {
+        // The positions rise from lane to lane and the lanes that hold a synapse are the first ones of the
+        // wave, so the lanes of a batch that meet in one window are neighbours (sixteen of them with
+        // 16,384-output windows and conn_prob 0.001, all 64 with a dense matrix).  A returning addition
+        // of several lanes to ONE counter occupies the CU's LDS for 64 cycles (measured; 7 when every lane
+        // has a counter of its own), so the first lane of every run of equal windows reserves the places
+        // of the whole run and the others fetch its answer (12 cycles with the shuffle): 3 to 6 % of the
+        // walk, whose larger cost is the scattered stores of the pairs.  Lanes 0 and 32 begin runs of their
+        // own, which keeps the masks at 32 bits.
+        const uint32_t n_valid = static_cast<uint32_t>(__popcll(__ballot(valid)));
+        const uint64_t heads = __ballot(b != wave_shift_up1(b)) | 0x100000001ull;
+        const uint32_t half = lane < 32 ? static_cast<uint32_t>(heads) : static_cast<uint32_t>(heads >> 32);
+        const uint32_t up = 31u - (static_cast<uint32_t>(lane) & 31u);  // lanes above this one in its half
+        const uint32_t rank = static_cast<uint32_t>(__builtin_clz(half << up));  // lanes from the run's first to this one
+        // the next run begins `run` lanes above this one (a run ends with its half at the latest)
+        const uint32_t above = ((half >> 1) >> (31u - up)) | (0x80000000u >> (31u - up));
+        uint32_t run = static_cast<uint32_t>(__builtin_ctz(above)) + 1u;
+        if (run > n_valid - static_cast<uint32_t>(lane)) run = n_valid - static_cast<uint32_t>(lane);
+        uint32_t first_slot = 0;
+        if (valid && rank == 0u) first_slot = atomicAdd(&s_cnt[b], run);
+        slot = static_cast<uint32_t>(__shfl(static_cast<int>(first_slot), lane - static_cast<int>(rank))) + rank;
+      } else if (valid) {
+        slot = atomicAdd(&s_cnt[b], 1u);  // (normal weights: the lanes that hold a synapse are not neighbours)
+      }
       if (valid) {
         T1 add;
         if (IN == kInDense) add = (W == kHomo) ? val : static_cast<T1>(w * val);
         else add = w;  // homo: w == 1
-        const uint32_t b = idx >> shift;
-        const uint32_t slot = atomicAdd(&s_cnt[b], 1u);
         if (slot < cap) {
           const uint64_t at = region + static_cast<uint64_t>(b) * cap + slot;
           const uint32_t rel = idx & ((1u << shift) - 1u);
