@@ -54,7 +54,7 @@ def load_kernels():
   lib.bench_gather_fma.restype = i
   lib.bench_gather_fma4.argtypes = [vp, vp, vp, vp, vp, u64, i, i, i, i, i]
   lib.bench_gather_fma4.restype = i
-  lib.bench_stream.argtypes = [vp, vp, vp, u64, i, i]
+  lib.bench_stream.argtypes = [vp, vp, vp, u64, i, i, i]
   lib.bench_stream.restype = i
   u32 = ctypes.c_uint32
   lib.bench_lds_atomic.argtypes = [vp, vp, i, i, i]
@@ -188,8 +188,8 @@ def gather_ceiling(lib, dev, x, idx, w, steps):
 
 
 def stream_ceiling(lib, dev, n_bytes, steps):
-  """GB/s of plain 16-byte loads over `n_bytes` of HBM at a persistent kernel's occupancies: the read rate a
-  streaming kernel reaches on this device (the published peak is not reachable by any kernel)."""
+  """GB/s of 16-byte loads, plain and nontemporal, over `n_bytes` of HBM at a persistent kernel's occupancies:
+  the read rate a streaming kernel reaches on this device (the published peak is not reachable by any kernel)."""
   import ctypes
   import torch
   n16 = n_bytes // 16
@@ -197,15 +197,16 @@ def stream_ceiling(lib, dev, n_bytes, steps):
   cu = torch.cuda.get_device_properties(dev).multi_processor_count
   stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
   rows = []
-  for per_cu, threads in ((2, 1024), (1, 1024), (4, 512), (8, 256)):
-    blocks = cu * per_cu
-    out = torch.zeros(blocks * threads, dtype=torch.int32, device=dev)
-    fn = lambda: lib.bench_stream(stream, buf.data_ptr(), out.data_ptr(), n16, blocks, threads)
-    if fn() != 0:
-      raise SystemExit("bench_stream failed to launch")
-    d, _ = time_calls(fn, steps, 2)
-    rows.append(dict(workgroups_per_cu=per_cu, threads=threads, us=float(d.mean() * 1e3),
-                     gb_per_s=n16 * 16 / (d.mean() * 1e-3) / 1e9))
+  for nt in (0, 1):
+    for per_cu, threads in ((2, 1024), (1, 1024), (4, 512), (8, 256)):
+      blocks = cu * per_cu
+      out = torch.zeros(blocks * threads, dtype=torch.int32, device=dev)
+      fn = lambda: lib.bench_stream(stream, buf.data_ptr(), out.data_ptr(), n16, blocks, threads, nt)
+      if fn() != 0:
+        raise SystemExit("bench_stream failed to launch")
+      d, _ = time_calls(fn, steps, 2)
+      rows.append(dict(workgroups_per_cu=per_cu, threads=threads, nontemporal=bool(nt), us=float(d.mean() * 1e3),
+                       gb_per_s=n16 * 16 / (d.mean() * 1e-3) / 1e9))
   return rows
 
 
@@ -284,6 +285,10 @@ def device_rates(lib, dev):
                      (4, "lds_address_arithmetic_only")):
     t = timed(lambda: lib.bench_lds_atomic(stream, out.data_ptr(), blocks, iters, mode))
     rates[name + "_g_per_s"] = ops / t / 1e9
+  # returning additions with 1, 4 and 16 neighbouring lanes per counter: time of a CU's LDS per wave instruction (2.4 cycles per ns)
+  for mode, lanes in ((101, 1), (104, 4), (116, 16)):
+    t = timed(lambda: lib.bench_lds_atomic(stream, out.data_ptr(), blocks, iters, mode))
+    rates["lds_returning_add_%d_lanes_per_counter_ns_per_wave_instruction_and_cu" % lanes] = t / (blocks / cu * 16 * iters) * 1e9
   rates["lds_workload"] = "%d workgroups of 1,024 threads, %d random operations per thread in a 64 KB window" % (blocks, iters)
   for n in (100_000, 1_000_000, 16_000_000):
     y = torch.zeros(n, dtype=torch.float32, device=dev)
@@ -513,7 +518,7 @@ def main():
     out = torch.zeros(cu * 2 * 1024, dtype=torch.int32, device=dev)
     for _ in range(3):
       lib.bench_stream(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), buf.data_ptr(), out.data_ptr(),
-                       740_000_000 // 16, cu * 2, 1024)
+                       740_000_000 // 16, cu * 2, 1024, 0)
     torch.cuda.synchronize()
     log("pmc mode done")
     return
@@ -552,7 +557,7 @@ def main():
   streams = stream_ceiling(bench_lib, dev, int(traffic) if traffic else bytes_gather, 20)
   stream_rate = max(r["gb_per_s"] for r in streams)
   extra["hbm_stream_read"] = dict(best_gb_per_s=stream_rate, runs=streams)
-  log("plain 16-byte loads: %s" % streams)
+  log("16-byte loads, plain and nontemporal: %s" % streams)
   if traffic:
     extra["gather_hbm_traffic_gb_per_s"] = traffic / (kernel_ms * 1e-3) / 1e9
     extra["gather_traffic_over_copy_rate"] = extra["gather_hbm_traffic_gb_per_s"] / copy_rate

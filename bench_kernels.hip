@@ -94,7 +94,14 @@ __global__ __launch_bounds__(1024) void gather_fma4_kernel(const float *__restri
   out[static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x] = static_cast<float>(acc);
 }
 
-__global__ __launch_bounds__(1024) void stream_kernel(const uint4 *__restrict__ p, uint32_t *__restrict__ out,
+typedef uint32_t stream_u32x4 __attribute__((ext_vector_type(4)));
+template <bool NT>
+__device__ __forceinline__ stream_u32x4 stream_word(const stream_u32x4 *p) {
+  return NT ? __builtin_nontemporal_load(p) : *p;
+}
+// NT: the loads are marked nontemporal, as the kernels mark the arrays they read once.
+template <bool NT>
+__global__ __launch_bounds__(1024) void stream_kernel(const stream_u32x4 *__restrict__ p, uint32_t *__restrict__ out,
                                                       uint64_t n16) {
   constexpr int U = 4;
   const uint64_t total = static_cast<uint64_t>(gridDim.x) * blockDim.x;
@@ -102,14 +109,14 @@ __global__ __launch_bounds__(1024) void stream_kernel(const uint4 *__restrict__ 
   uint32_t acc = 0;
   uint64_t base = gtid;
   for (; base + (U - 1) * total < n16; base += U * total) {
-    uint4 v[U];
+    stream_u32x4 v[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) v[u] = p[base + u * total];
+    for (int u = 0; u < U; ++u) v[u] = stream_word<NT>(p + base + u * total);
 #pragma unroll
     for (int u = 0; u < U; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
   }
   for (; base < n16; base += total) {
-    const uint4 v = p[base];
+    const stream_u32x4 v = stream_word<NT>(p + base);
     acc ^= v.x ^ v.y ^ v.z ^ v.w;
   }
   out[gtid] = acc;
@@ -138,6 +145,19 @@ __global__ __launch_bounds__(1024) void lds_atomic_kernel(float *__restrict__ ou
   }
   __syncthreads();
   if (threadIdx.x == 0) out[blockIdx.x] = win[5] + acc;
+}
+
+// Returning 32-bit additions in LDS where G neighbouring lanes share a counter (a wave's counters differ from
+// the other waves'); every addition depends on the answer of the one before it.
+template <int G>
+__global__ __launch_bounds__(1024) void lds_shared_counter_kernel(float *__restrict__ out, int iters) {
+  __shared__ uint32_t cnt[4096];
+  for (int i = threadIdx.x; i < 4096; i += 1024) cnt[i] = 0u;
+  __syncthreads();
+  const uint32_t lane = threadIdx.x % 64u, wave = threadIdx.x / 64u;
+  uint32_t acc = 0;
+  for (int i = 0; i < iters; ++i) acc += atomicAdd(&cnt[(wave * 64u + lane / G + (acc & 1u)) & 4095u], 1u);
+  out[blockIdx.x] = static_cast<float>(__builtin_amdgcn_readfirstlane(static_cast<int>(acc)) & 1);
 }
 
 // fp32 atomic adds (no return value) to random elements of y[0, n)
@@ -178,7 +198,8 @@ __global__ __launch_bounds__(1024) void l2_read_kernel(const uint4 *__restrict__
 
 extern "C" {
 
-// out: blocks floats.  mode 0: ds_add_f32, 1: ds_add_u32, 2: ds_add_f64, 3: ds_write_b32, 4: addresses only.
+// out: blocks floats.  mode 0: ds_add_f32, 1: ds_add_u32, 2: ds_add_f64, 3: ds_write_b32, 4: addresses only;
+// 101, 104, 116: returning 32-bit additions with 1, 4, 16 neighbouring lanes per counter.
 // blocks * 1024 * iters operations per launch.
 int bench_lds_atomic(void *stream, float *out, int blocks, int iters, int mode) {
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -188,6 +209,9 @@ int bench_lds_atomic(void *stream, float *out, int blocks, int iters, int mode) 
   else if (mode == 2) hipLaunchKernelGGL(lds_atomic_kernel<2>, dim3(blocks), dim3(1024), 0, s, out, iters);
   else if (mode == 3) hipLaunchKernelGGL(lds_atomic_kernel<3>, dim3(blocks), dim3(1024), 0, s, out, iters);
   else if (mode == 4) hipLaunchKernelGGL(lds_atomic_kernel<4>, dim3(blocks), dim3(1024), 0, s, out, iters);
+  else if (mode == 101) hipLaunchKernelGGL(lds_shared_counter_kernel<1>, dim3(blocks), dim3(1024), 0, s, out, iters);
+  else if (mode == 104) hipLaunchKernelGGL(lds_shared_counter_kernel<4>, dim3(blocks), dim3(1024), 0, s, out, iters);
+  else if (mode == 116) hipLaunchKernelGGL(lds_shared_counter_kernel<16>, dim3(blocks), dim3(1024), 0, s, out, iters);
   else return 1;
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
@@ -253,10 +277,11 @@ int bench_gather_fma4(void *stream, const float *x, const uint32_t *idx, const f
 }
 
 // p: n16 16-byte words; out: blocks * threads words.
-int bench_stream(void *stream, const void *p, void *out, uint64_t n16, int blocks, int threads) {
+int bench_stream(void *stream, const void *p, void *out, uint64_t n16, int blocks, int threads, int nontemporal) {
   if (blocks <= 0 || threads <= 0 || threads > 1024) return 1;
-  hipLaunchKernelGGL(stream_kernel, dim3(blocks), dim3(threads), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const uint4 *>(p), static_cast<uint32_t *>(out), n16);
+  auto kernel = nontemporal ? stream_kernel<true> : stream_kernel<false>;
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(threads), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const stream_u32x4 *>(p), static_cast<uint32_t *>(out), n16);
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
