@@ -58,6 +58,16 @@ __device__ __forceinline__ void load_quad(const double *p, double (&v)[4]) {
   const bin_f64x2 a = *reinterpret_cast<const bin_f64x2 *>(p), b = *reinterpret_cast<const bin_f64x2 *>(p + 2);
   v[0] = a.x, v[1] = a.y, v[2] = b.x, v[3] = b.y;
 }
+typedef uint32_t bin_u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void load_quad_once(const float *p, float (&v)[4]) {  // (nontemporal)
+  const bin_f32x4 t = __builtin_nontemporal_load(reinterpret_cast<const bin_f32x4 *>(p));
+  v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+}
+__device__ __forceinline__ void load_quad_once(const double *p, double (&v)[4]) {
+  const bin_f64x2 a = __builtin_nontemporal_load(reinterpret_cast<const bin_f64x2 *>(p));
+  const bin_f64x2 b = __builtin_nontemporal_load(reinterpret_cast<const bin_f64x2 *>(p + 2));
+  v[0] = a.x, v[1] = a.y, v[2] = b.x, v[3] = b.y;
+}
 // U consecutive columns or weights for a lane, from an address that is a multiple of the element's size only.
 // Nontemporal: the arrays pass through once, and lines of pairs that are written a piece per round must stay in
 // the L2 until they are whole (120 -> 99 us per 33 million nonzeros; nontemporal STORES of the pairs: 190 us)
@@ -454,7 +464,10 @@ __global__ __launch_bounds__(kSumCols * kSumSlices) void sum_windows_kernel(cons
 // wider than the 2^lds_shift accumulators in LDS is added slice by slice, every slice reading the pairs).
 // Bin of (producer p, window b): derived from the producers' shares of the nonzeros as in bin_products_kernel,
 // or, with indptr == nullptr, the uniform layout pairs + (p * n_win + b) * uniform_cap.
-template <typename F, bool PACKED>
+// ONCE: the pairs are read with nontemporal loads (bins of a jitconn column walk: gigabytes that passed
+// through memory; 1e8 pairs: 524 -> 484 us with the walk).  The CSR product's chunks come back from the
+// cache in front of the memory, where the hint costs (454 -> 510 us).
+template <typename F, bool PACKED, bool ONCE>
 __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *__restrict__ indptr,
                                                                F *__restrict__ y, uint32_t n_row, uint32_t n_col,
                                                                uint32_t chunk_lo, uint32_t chunk_nnz, uint32_t last,
@@ -578,9 +591,15 @@ __global__ __launch_bounds__(kBinThreads) void add_bins_kernel(const uint32_t *_
       const uint32_t i = i0 + 4u * (static_cast<uint32_t>(u) * kWave + lane);
       e.valid[u] = i < n ? n - i : 0u;
       const uint64_t at = bin_off + (i < n ? i : 0u);
-      const uint2 r = *reinterpret_cast<const uint2 *>(packed.rel + at);
-      e.r[u][0] = r.x, e.r[u][1] = r.y;
-      load_quad(packed.val + at, e.v[u]);
+      if constexpr (ONCE) {
+        const bin_u32x2 r = __builtin_nontemporal_load(reinterpret_cast<const bin_u32x2 *>(packed.rel + at));
+        e.r[u][0] = r.x, e.r[u][1] = r.y;
+        load_quad_once(packed.val + at, e.v[u]);
+      } else {
+        const uint2 r = *reinterpret_cast<const uint2 *>(packed.rel + at);
+        e.r[u][0] = r.x, e.r[u][1] = r.y;
+        load_quad(packed.val + at, e.v[u]);
+      }
     }
   };
   auto add_packed = [&](const PackedStep &e) {
@@ -1413,7 +1432,7 @@ bool bin_scatter(const char *target, hipStream_t stream, const F *data, bool het
   void *pairs = ws;
   uint32_t *counts = reinterpret_cast<uint32_t *>(ws + pair_bytes);
 
-  auto add_kernel = packed ? add_bins_kernel<F, true> : add_bins_kernel<F, false>;
+  auto add_kernel = packed ? add_bins_kernel<F, true, false> : add_bins_kernel<F, false, false>;
   const size_t lds = sizeof(double) << lds_shift;
   static thread_local bool attr_set[2] = {false, false};
   if (!attr_set[packed] && lds > 64 * 1024) {
@@ -1456,7 +1475,7 @@ template <typename F>
 bool add_uniform_bins(const char *target, hipStream_t stream, F *y, uint32_t n_out, uint32_t shift, uint32_t producers,
                       uint32_t cap, const void *pairs, bool packed, const uint32_t *counts, uint32_t *reset) {
   const uint32_t n_win = div_up(n_out, 1u << shift);
-  auto add_kernel = packed ? add_bins_kernel<F, true> : add_bins_kernel<F, false>;
+  auto add_kernel = packed ? add_bins_kernel<F, true, true> : add_bins_kernel<F, false, false>;
   const uint32_t lds_shift = bin_lds_shift(shift);
   const uint32_t slices = 1u << (shift - lds_shift);
   const size_t lds = sizeof(double) << lds_shift;
