@@ -833,9 +833,14 @@ __device__ __forceinline__ void gather_rows_wave(const F *__restrict__ data, con
     const F *dp = data + (HETER ? start : 0u);
     double acc = 0.0;
     uint32_t hits = 0;
-    uint32_t b = 0;
-    for (; b + U * kWave <= len; b += U * kWave) step(ip, dp, b, len, false, acc, hits);
-    if (b < len) step(ip, dp, b, len, true, acc, hits);
+    // Rows that lie a multiple of 4 KB apart (1,024 nonzeros each, say) would have every wave of the device at the
+    // same offset within 4 KB at the same time, and with it on the same memory channels (1,024 per row: 16 % slower
+    // per nonzero than 1,000 per row).  So the rows begin at different full steps, by their number, and wrap.
+    const uint32_t full = len / (U * kWave);  // steps without a guard
+    const uint32_t first = urow & (full >= 4u ? 3u : full >= 2u ? 1u : 0u);
+    for (uint32_t i = first; i < full; ++i) step(ip, dp, i * (U * kWave), len, false, acc, hits);
+    for (uint32_t i = 0; i < first; ++i) step(ip, dp, i * (U * kWave), len, false, acc, hits);
+    if (full * (U * kWave) < len) step(ip, dp, full * (U * kWave), len, true, acc, hits);
     if (MODE == kEvent && !HETER) {
       hits = wave_sum(hits);
       // n additions of the same fp32 value into a float64 accumulator are exact: n * w
