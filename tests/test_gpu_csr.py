@@ -193,6 +193,33 @@ def test_ragged_rows_and_all_row_length_modes(cuda, oracle_mod):
     assert_close_reordered(got, want, mag, what="event scatter mean %d" % mean)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_gather_long_rows_that_begin_at_different_steps(cuda, oracle_mod, dtype):
+  # rows of 384 nonzeros or more take a wave each, in steps of 512 (float64: the same walk), and begin at a full
+  # step chosen by the row's number: rows of exactly 1, 2, 3, 4 and 9 full steps, with and without a partial
+  # last step, every row number modulo 4 among them.  Integer weights: the sums are exact whatever the order.
+  rng = np.random.default_rng(21)
+  n_col = 40_000
+  lengths = [512, 1024, 1536, 2048, 4608, 513, 1023, 1025, 2049, 2047, 4096 + 5, 700, 385]
+  counts = np.array([lengths[(i * 5 + i // 13) % len(lengths)] for i in range(416)])
+  indices, indptr = synth.counted_csr(counts, n_col, seed=4)
+  data = rng.integers(-8, 9, indices.shape[0]).astype(dtype)
+  shape = (counts.shape[0], n_col)
+  for rate in (0.05, 0.6):
+    ev = rng.random(n_col) < rate
+    want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape)
+    got = bpl.event_csr_matvec(data, indices, indptr, ev, shape=shape).cpu().numpy()
+    assert np.array_equal(got, want), "heterogeneous, events %g" % rate
+    w = np.array([3.0], dtype)
+    want = oracle_mod.event_csr_matvec(w, indices, indptr, ev, shape=shape)
+    got = bpl.event_csr_matvec(w, indices, indptr, ev, shape=shape).cpu().numpy()
+    assert np.array_equal(got, want), "one weight, events %g" % rate
+  v = rng.integers(-4, 5, n_col).astype(dtype)
+  want = oracle_mod.csr_matvec(data, indices, indptr, v, shape=shape)
+  got = bpl.csr_matvec(data, indices, indptr, v, shape=shape).cpu().numpy()
+  assert np.array_equal(got, want), "dense vector"
+
+
 def test_unaligned_event_vector_and_large_bitmap(cuda, oracle_mod):
   # an event vector that does not start on a 16-byte boundary, and one whose bitmap needs more
   # than 64 KiB of LDS (n_col > 524288)
