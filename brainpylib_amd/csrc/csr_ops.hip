@@ -661,6 +661,8 @@ __device__ __forceinline__ VT dense_element(const VT *__restrict__ x, const uint
   return x[col];
 }
 
+typedef uint32_t row_u32x4 __attribute__((ext_vector_type(4), aligned(4)));  // (a row begins at any nonzero)
+typedef float row_f32x4 __attribute__((ext_vector_type(4), aligned(4)));
 template <typename F, typename VT, bool HETER, int MODE, int BITS, int G, int U>
 __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const uint32_t *__restrict__ indices,
                                             const uint32_t *__restrict__ indptr, const VT *__restrict__ x,
@@ -670,6 +672,14 @@ __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const ui
   const uint32_t gl = threadIdx.x % G;
   const uint32_t total_groups = gridDim.x * groups_per_block;
   const F w_homo = HETER ? F(0) : data[0];
+  // A lane takes its U nonzeros of a step as U / Q runs of Q consecutive ones, each with ONE load of Q indices
+  // (and weights): slot u of lane gl is nonzero Q * ((u / Q) * G + gl) + u % Q of the step.  With a nonzero per
+  // load a group's G lanes asked for G * 4 bytes of a line per instruction and for the same line again with the
+  // next one, U times over.
+  // (not with the dense vector staged in LDS, float: that walk has no registers to spare for two workgroups per CU)
+  constexpr int Q = ((U == 4 || U == 8) && !(MODE == kDense && BITS == 1)) ? 4 : 1;
+  auto slot = [&](int u) { return static_cast<uint32_t>(Q * ((u / Q) * G) + u % Q) + static_cast<uint32_t>(Q) * gl; };
+  const uint32_t nnz = Q > 1 ? indptr[n_row] : 0u;  // (a run of Q is loaded whole only where the arrays hold all of it)
   // A row of more than kHubSteps steps looks empty here: gather_hub_rows() gives it to the whole workgroup.
   constexpr uint32_t hub_len = kHubSteps * U * G;
   auto bounds = [&](uint32_t r, uint32_t &s, uint32_t &e) {
@@ -686,10 +696,38 @@ __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const ui
 
   auto load_cols = [&](uint32_t b, uint32_t e, uint32_t (&c)[U]) {
     const uint32_t safe = e ? e - 1 : 0u;  // any valid element (the matrix has at least one)
+    if constexpr (Q > 1) {
+      if (static_cast<uint64_t>(b) + U * G <= nnz) {
+        // (what lies beyond the row's end are the next rows' indices: valid columns, left out by their number)
+#pragma unroll
+        for (int q = 0; q < U / Q; ++q) {
+          const row_u32x4 v = *reinterpret_cast<const row_u32x4 *>(indices + b + slot(Q * q));
+          c[Q * q] = v.x, c[Q * q + 1] = v.y, c[Q * q + 2] = v.z, c[Q * q + 3] = v.w;
+        }
+        return;
+      }
+    }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const uint32_t j = b + u * G + gl;
+      const uint32_t j = b + slot(u);
       c[u] = indices[j < e ? j : safe];
+    }
+  };
+  auto load_weights = [&](uint32_t b, uint32_t e, auto &d) {  // (dense vector: every weight of the step)
+    if constexpr (Q > 1 && sizeof(F) == 4) {
+      if (static_cast<uint64_t>(b) + U * G <= nnz) {
+#pragma unroll
+        for (int q = 0; q < U / Q; ++q) {
+          const row_f32x4 v = *reinterpret_cast<const row_f32x4 *>(data + b + slot(Q * q));
+          d[Q * q] = v.x, d[Q * q + 1] = v.y, d[Q * q + 2] = v.z, d[Q * q + 3] = v.w;
+        }
+        return;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t j = b + slot(u);
+      d[u] = data[j < e ? j : (e ? e - 1 : 0u)];
     }
   };
 
@@ -709,10 +747,14 @@ __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const ui
     F val[U];
     bool use[U];
     bool hits_u[U];
+    // (sixteen weights in registers beside sixteen columns are more than two workgroups per CU leave room for)
+    constexpr bool kWeightRuns = MODE == kDense && HETER && Q > 1;
+    F wgt[kWeightRuns ? U : 1];
+    if constexpr (kWeightRuns) load_weights(base, end, wgt);
     if constexpr (MODE == kEvent && BITS == 3) event_hits<BITS, U>(s_bits, x, col, coarse_g, hits_u);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const uint32_t j = base + u * G + gl;
+      const uint32_t j = base + slot(u);
       const bool ok = j < end;
       if (MODE == kEvent) {
         bool hit;
@@ -724,7 +766,9 @@ __device__ __forceinline__ void gather_rows(const F *__restrict__ data, const ui
         if (HETER && hit) val[u] = data[j];
       } else {
         use[u] = ok;
-        const F d = HETER ? data[ok ? j : (end ? end - 1 : 0u)] : w_homo;
+        F d = w_homo;
+        if constexpr (kWeightRuns) d = wgt[u];
+        else if constexpr (HETER) d = data[ok ? j : (end ? end - 1 : 0u)];
         // product formed in F, then widened (the reference multiplies two F values)
         val[u] = static_cast<F>(static_cast<F>(dense_element<VT, BITS>(x, s_bits, coarse_g, col[u])) * d);
       }
