@@ -593,7 +593,7 @@ def main():
                                 wall_us_per_call=wall_s / args.steps * 1e6,
                                 roofline=roofline_record("hbm", bytes_scatter / (dur_s.mean() * 1e-3) / 1e9, HBM_PEAK_GBS,
                                                          "GB/s", algorithmic_bytes_per_call=bytes_scatter,
-                                                         launches_per_call=2),
+                                                         launches_per_call=3),
                                 parity=parity_record(got_s, outside_s, "rel 1e-5 / abs 1e-6 + 4 eps sum|addends|"))
     if not args.skip_cpu:
       t1 = time.perf_counter()
