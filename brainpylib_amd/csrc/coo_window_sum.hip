@@ -210,8 +210,13 @@ __global__ __launch_bounds__(kCooThreads) void bin_connections_kernel(
       win[t] = on ? static_cast<uint32_t>(post[t]) >> shift : kNone;
       rel[t] = static_cast<uint32_t>(post[t]) & ((1u << shift) - 1u);
     }
+    // (only the lanes that hold a pair: with an event vector most hold none, and additions of many lanes to the
+    // one spare counter would be taken one after the other, 64 cycles of the CU's LDS per instruction)
 #pragma unroll
-    for (int t = 0; t < U; ++t) rank[t] = atomicAdd(&s_cnt[win[t]], 1u);
+    for (int t = 0; t < U; ++t) {
+      rank[t] = 0;
+      if (win[t] != kNone) rank[t] = atomicAdd(&s_cnt[win[t]], 1u);
+    }
     __syncthreads();
     if (tid < kWave) {  // offsets of the windows within the round: two counters per lane
       const uint32_t c0 = s_cnt[2 * tid], c1 = s_cnt[2 * tid + 1];
