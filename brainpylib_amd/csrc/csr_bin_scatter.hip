@@ -91,6 +91,11 @@ __device__ __forceinline__ void load_consecutive(const double *p, double (&v)[2]
   const bin_f64x2_unaligned t = __builtin_nontemporal_load(reinterpret_cast<const bin_f64x2_unaligned *>(p));
   v[0] = t.x, v[1] = t.y;
 }
+__device__ __forceinline__ void load_consecutive(const double *p, double (&v)[4]) {
+  const bin_f64x2_unaligned a = __builtin_nontemporal_load(reinterpret_cast<const bin_f64x2_unaligned *>(p));
+  const bin_f64x2_unaligned b = __builtin_nontemporal_load(reinterpret_cast<const bin_f64x2_unaligned *>(p + 2));
+  v[0] = a.x, v[1] = a.y, v[2] = b.x, v[3] = b.y;
+}
 template <typename F>
 struct PackedBins {
   F *val;
@@ -900,6 +905,7 @@ __device__ __forceinline__ uint32_t window_event_producers(uint32_t total, uint3
 // by thread, then bit by bit, the same in every workgroup), which saves the launch of the kernel that lists
 // them.  Active rows without nonzeros are then among the numbered ones.
 constexpr uint32_t kSelfListRows = 32u * kBinThreads;
+typedef uint32_t row4_u32 __attribute__((ext_vector_type(4), aligned(4)));
 template <typename F, bool HETER, bool SELF>
 __global__ __launch_bounds__(kBinThreads) void active_rows_window_kernel(
     const F *__restrict__ data, const uint32_t *__restrict__ indices, const uint32_t *__restrict__ indptr,
@@ -1010,28 +1016,52 @@ __global__ __launch_bounds__(kBinThreads) void active_rows_window_kernel(
         if (tid == 0) s_hint[kBinThreads] = rows - 1u;
       }
       __syncthreads();
-      for (uint32_t jb = seg + tid; jb - tid < seg_end; jb += kRound) {
-        // where every nonzero of the lane lies (LDS only), then all the loads together
+      for (uint32_t jb = seg; jb < seg_end; jb += kRound) {
+        // A lane takes U consecutive nonzeros of the round: one search for the row of the first (LDS only), a
+        // walk from there for the others, and where they lie in one listed row (all but the few that cross
+        // into the next) one request for their columns and one for their weights.
+        const uint32_t j0 = jb + U * tid;
         uint32_t at[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const uint32_t j = jb + u * kBinThreads;
-          const uint32_t jc = j < seg_end ? j : seg_end - 1u;
+        {
+          const uint32_t jc = j0 < seg_end ? j0 : seg_end - 1u;
           const uint32_t q = (jc - seg) >> kHintShift;
-          const uint32_t k = row_of(jc, s_hint[q], s_hint[q + 1]);
-          at[u] = s_start[k] + (jc - s_ptr[k]);
+          uint32_t k = row_of(jc, s_hint[q], s_hint[q + 1]);
+          uint32_t e = s_ptr[k + 1u];
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+            const uint32_t ju = j0 + u < seg_end ? j0 + u : seg_end - 1u;
+            while (e <= ju) e = s_ptr[++k + 1u];  // (ends: ju < seg_end <= s_ptr[rows])
+            at[u] = s_start[k] + (ju - s_ptr[k]);
+          }
         }
         uint32_t col[U];
         F val[U];
+        bool together = j0 + U <= seg_end;  // (the listed rows are in no order: every one of the U is compared)
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          col[u] = indices[at[u]];
-          if (HETER) val[u] = data[at[u]];
+        for (int u = 1; u < U; ++u) together = together && at[u] == at[0] + static_cast<uint32_t>(u);
+        if (together) {
+          if (slices == 1u) {  // (the arrays pass through once; with slices the other slices' workgroups want the lines too)
+            load_consecutive(indices + at[0], col);
+            if (HETER) load_consecutive(data + at[0], val);
+          } else {
+            const row4_u32 c4 = *reinterpret_cast<const row4_u32 *>(indices + at[0]);
+            col[0] = c4.x, col[1] = c4.y, col[2] = c4.z, col[3] = c4.w;
+            if (HETER) {
+#pragma unroll
+              for (int u = 0; u < U; ++u) val[u] = data[at[0] + u];
+            }
+          }
+        } else {
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+            col[u] = indices[at[u]];
+            if (HETER) val[u] = data[at[u]];
+          }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const uint32_t rel = col[u] - c_lo;  // (wraps below the slice; a column beyond the output: left out)
-          if (jb + u * kBinThreads < seg_end && rel < width) {
+          if (j0 + u < seg_end && rel < width) {
             if constexpr (HETER) atomicAdd(&window[rel], static_cast<double>(val[u]));
             else atomicAdd(&window[rel], 1u);
           }
