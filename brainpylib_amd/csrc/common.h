@@ -161,13 +161,13 @@ int csr_event_sum_wide(const char *target, hipStream_t stream, const uint8_t *ev
 // CU's one scalar unit for about 2 us.
 void jitconn_seed_streams(hipStream_t stream, uint32_t seed, uint32_t first, uint32_t count, uint32_t *states);
 
-// Event input and an output of at most 8,192 columns: the listed active rows' nonzeros are walked flat into
-// one window in LDS per workgroup (csr_bin_scatter.hip).  `counters`: the stream's counters, [0] the number
+// Event input and an output of at most 8,192 columns (a homogeneous weight: of a few slices of 14,848): the listed
+// active rows' nonzeros are walked flat into one window in LDS per workgroup (csr_bin_scatter.hip).  `counters`: the stream's counters, [0] the number
 // of listed rows (set back to zero by the second kernel), [1] used between the two kernels.  `scratch`:
 // window_event_scatter_bytes() of device memory.  y need not be zeroed.  false (nothing enqueued) if it
 // cannot run.
 template <typename F>
-bool window_event_scatter_usable(uint32_t n_row, uint32_t n_col);
+bool window_event_scatter_usable(uint32_t n_row, uint32_t n_col, bool heter);
 template <typename F>
 size_t window_event_scatter_bytes(uint32_t n_col);
 template <typename F>

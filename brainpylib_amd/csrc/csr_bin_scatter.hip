@@ -1263,11 +1263,6 @@ inline uint64_t event_run_pairs(uint32_t n_row, uint32_t n_col) {
 
 }  // namespace
 
-template <typename F>
-bool window_event_scatter_usable(uint32_t n_row, uint32_t n_col) {
-  return n_col != 0 && n_col <= kWindowEventMaxCols && n_row != 0;
-}
-
 // Without a list the window shares the LDS with 8 KB of masks: 58 KB of it (7,424 float64 accumulators or
 // 14,848 counts), and an output of up to two such windows of float64 is taken in slices.  (Three and four
 // slices, every slice walking all active nonzeros: 20,000 columns gain 2 us at 5 % events and lose 5 at 20 %
@@ -1278,12 +1273,34 @@ bool window_event_scatter_self_usable(uint32_t n_row, uint32_t n_col) {
   return n_col != 0 && n_col <= kSelfMaxSlices * (kSelfWindowBytes / sizeof(double)) && n_row != 0 && n_row <= kSelfListRows;
 }
 
+// A homogeneous weight counts synapses in 32-bit integers, 14,848 to a window of 58 KB, and an output of up to four
+// such windows is taken in slices by as many sets of workgroups, which all walk the active rows (their indices
+// come from the L2s after the first set's read): no pairs written and read back.  50,000 x 50,000 with 5,000 per
+// row: 33 / 81 / 267 us through the sorted scatter at 1 / 5 / 20 % events, 30 / 54 / 139 us so; 50,000 x 20,000
+// with 1,000 per row: 22 / 36 / 73 / 185 us at 1 / 5 / 20 / 60 % against 21 / 26 / 34 / 57 us.  Every workgroup
+// that takes part leaves a window of the output's width behind, whatever the activity, which matrices of many
+// short rows do not earn back at the 1 % of a quiet network (1,000,000 x 59,000 with 100 per row: 26 -> 34 us,
+// and 175 -> 117 us at 30 %; the host knows the rows, not their lengths): up to 65,536 rows.  Weights per synapse
+// (float64 accumulators, half as many to a window) gain only from 20 % activity on and stay with the sorted scatter.
+constexpr uint32_t kListedHomoMaxSlices = 4;
+constexpr uint32_t kListedHomoMaxRows = 65536;
+template <typename F>
+bool window_event_scatter_usable(uint32_t n_row, uint32_t n_col, bool heter) {
+  if (n_col == 0 || n_row == 0) return false;
+  if (n_col <= kWindowEventMaxCols) return true;
+  return !heter && n_row <= kListedHomoMaxRows &&
+         n_col <= kListedHomoMaxSlices * static_cast<uint32_t>(kSelfWindowBytes / sizeof(uint32_t));
+}
+
+
 // scratch memory (behind the list, if there is one): the windows of two workgroups per CU, or, of an output in
 // slices, of as many as take a slice
 template <typename F>
 size_t window_event_scatter_bytes(uint32_t n_col) {
   const uint32_t resident = 2u * static_cast<uint32_t>(device_info().num_cu);
-  const uint32_t slices = n_col <= kWindowEventMaxCols ? 1u : div_up(n_col, static_cast<uint32_t>(kSelfWindowBytes / sizeof(double)));
+  // (the fewest slices an output of this width is taken in, those of 32-bit counts, and float64 accumulators:
+  // enough for either kind of weight)
+  const uint32_t slices = n_col <= kWindowEventMaxCols ? 1u : div_up(n_col, static_cast<uint32_t>(kSelfWindowBytes / sizeof(uint32_t)));
   return static_cast<size_t>(resident / slices) * n_col * sizeof(double);
 }
 
@@ -1292,13 +1309,14 @@ bool window_event_scatter(hipStream_t stream, const F *data, bool heter, const u
                           F *y, uint32_t n_row, uint32_t n_col, uint32_t *counters, const uint2 *active_list,
                           uint32_t list_cap, void *scratch, size_t scratch_bytes, const void *events, uint32_t event_width) {
   const bool self = events != nullptr;  // no list: the kernel looks at the events itself
-  if (self ? !window_event_scatter_self_usable(n_row, n_col) : !window_event_scatter_usable<F>(n_row, n_col)) return false;
+  if (self ? !window_event_scatter_self_usable(n_row, n_col) : !window_event_scatter_usable<F>(n_row, n_col, heter)) return false;
   if (scratch_bytes < window_event_scatter_bytes<F>(n_col)) return false;
   if (self && event_width != 1u && event_width != 4u && event_width != 8u) return false;
   const size_t acc_bytes = heter ? sizeof(double) : sizeof(uint32_t);
   // (the masks beside 12.5 KB of row tables: two workgroups must still fit a CU's 160 KB)
-  const uint32_t slice_cols = self ? static_cast<uint32_t>(kSelfWindowBytes / acc_bytes) : n_col;
-  const uint32_t slices = self ? div_up(n_col, slice_cols) : 1u;
+  const bool sliced = self || n_col > kWindowEventMaxCols;
+  const uint32_t slice_cols = sliced ? static_cast<uint32_t>(kSelfWindowBytes / acc_bytes) : n_col;
+  const uint32_t slices = sliced ? div_up(n_col, slice_cols) : 1u;
   const unsigned launched = 2u * static_cast<unsigned>(device_info().num_cu) / slices;
   const unsigned grid = launched * slices;
   const size_t lds = static_cast<size_t>(slices > 1u ? slice_cols : n_col) * acc_bytes;
@@ -1532,8 +1550,8 @@ template bool add_uniform_bins<float>(const char *, hipStream_t, float *, uint32
                                       bool, const uint32_t *, uint32_t *);
 template bool add_uniform_bins<double>(const char *, hipStream_t, double *, uint32_t, uint32_t, uint32_t, uint32_t,
                                        const void *, bool, const uint32_t *, uint32_t *);
-template bool window_event_scatter_usable<float>(uint32_t, uint32_t);
-template bool window_event_scatter_usable<double>(uint32_t, uint32_t);
+template bool window_event_scatter_usable<float>(uint32_t, uint32_t, bool);
+template bool window_event_scatter_usable<double>(uint32_t, uint32_t, bool);
 template size_t window_event_scatter_bytes<float>(uint32_t);
 template size_t window_event_scatter_bytes<double>(uint32_t);
 template bool window_event_scatter<float>(hipStream_t, const float *, bool, const uint32_t *, const uint32_t *, float *, uint32_t,

@@ -1470,7 +1470,8 @@ void launch_scatter(const ScratchSource &src, const F *data, const uint32_t *ind
   // Event input and more than 8,192 outputs: the active rows' nonzeros are flattened and sorted
   // coarsely by output window instead (csr_bin_scatter.hip), at a cost that neither grows with the
   // number of windows nor with the number of rows a wave would have to walk in turn.
-  if (MODE == kEvent && n_col > 8192 && bin_event_scatter_usable<F>(n_col)) {
+  const bool listed_windows = MODE == kEvent && !src.fixed() && n_row > kSmallRows && window_event_scatter_usable<F>(n_row, n_col, HETER);
+  if (MODE == kEvent && n_col > 8192 && bin_event_scatter_usable<F>(n_col) && !listed_windows) {
     const size_t list_sz = round_up(static_cast<size_t>(n_row) * sizeof(uint2));
     size_t got = 0;
     unsigned char *ws = static_cast<unsigned char *>(src.request(list_sz + bin_event_scatter_bytes<F>(n_row, n_col),
@@ -1499,7 +1500,7 @@ void launch_scatter(const ScratchSource &src, const F *data, const uint32_t *ind
     }
   }
   // Event input, more rows and an output of one window: the same walk over a device list of the active rows.
-  if (MODE == kEvent && !src.fixed() && n_row > kSmallRows && window_event_scatter_usable<F>(n_row, n_col)) {
+  if (listed_windows) {
     const size_t list_sz = round_up(static_cast<size_t>(n_row) * sizeof(uint2));
     const size_t need = list_sz + window_event_scatter_bytes<F>(n_col);
     size_t got = 0;

@@ -574,6 +574,41 @@ def test_event_scatter_into_one_window_from_many_rows(cuda, oracle_mod, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_event_scatter_of_one_weight_into_slices_of_the_output(cuda, oracle_mod, dtype):
+  # a homogeneous weight, 32,769 to 65,536 rows and an output of up to four windows of 14,848 counts: the listed
+  # rows are walked once per slice of the output into integer windows in LDS.  Widths at both ends of one, two
+  # and four slices, the widths and row counts just beyond (the sorted scatter), little and much activity, empty
+  # rows and a row that holds a large share of the nonzeros; bit for bit, twice in a row.  Weights per synapse
+  # of the same matrices take the sorted scatter.
+  rng = np.random.default_rng(61)
+  for n_row, n_col, mean, hub in ((40_000, 14_849, 20, 0), (65_536, 29_696, 9, 50_000), (33_000, 59_392, 25, 0),
+                                  (50_000, 59_393, 10, 0), (65_537, 20_000, 12, 0), (45_000, 44_544, 40, 0)):
+    counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
+    counts[rng.integers(0, n_row, size=n_row // 9)] = 0
+    if hub:
+      counts = counts.astype(np.int64)
+      counts[n_row // 3] = min(hub, n_col)
+    indices, indptr = synth.counted_csr(counts, n_col, seed=n_col)
+    shape = (n_row, n_col)
+    print("shape", shape, dtype.__name__, flush=True)
+    w = np.array([0.6], dtype=dtype)
+    data = rng.standard_normal(indices.shape[0]).astype(dtype)
+    for rate in (0.0005, 0.05, 0.9):
+      ev = rng.random(n_row) < rate
+      if hub:
+        ev[n_row // 3] = True
+      want = oracle_mod.event_csr_matvec(w, indices, indptr, ev, shape=shape, transpose=True)
+      for events in (ev, ev.astype(dtype) * 3):
+        for _ in range(2):
+          got = bpl.event_csr_matvec(w, indices, indptr, events, shape=shape, transpose=True).cpu().numpy()
+          assert np.array_equal(got, want), (shape, rate)  # the reference's repeated additions, bit for bit
+      want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True)
+      mag = oracle_mod.event_csr_matvec(np.abs(data), indices, indptr, ev, shape=shape, transpose=True)
+      got = bpl.event_csr_matvec(data, indices, indptr, ev, shape=shape, transpose=True).cpu().numpy()
+      assert_close_reordered(got, want, mag, dtype, what="event scatter beside the sliced windows %s rate %g" % (shape, rate))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_event_scatter_into_one_window_rows_found_by_the_workgroups(cuda, oracle_mod, dtype):
   # 4,097 to 32,768 rows and at most 8,192 columns: no list, every workgroup numbers the active rows itself
   # (thread by thread, bit by bit).  The row counts at both ends, empty rows among the active ones, no event,
