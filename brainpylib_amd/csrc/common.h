@@ -177,8 +177,9 @@ bool window_event_scatter(hipStream_t stream, const F *data, bool heter, const u
                           uint32_t event_width = 0);
 // With `events` (the events themselves, elements of event_width = 1, 4 or 8 bytes: bytes, float or double, nonzero =
 // event) the kernel finds the active rows itself: no list (active_list may be nullptr, list_cap is not used), one
-// launch fewer.  For at most 32,768 rows; the output may then have up to 14,848 columns (taken in two slices).
-bool window_event_scatter_self_usable(uint32_t n_row, uint32_t n_col);
+// launch fewer.  For at most 32,768 rows; the output may then have up to 14,848 columns (taken in two slices;
+// with a homogeneous weight up to 59,392 in four).
+bool window_event_scatter_self_usable(uint32_t n_row, uint32_t n_col, bool heter);
 
 // Second half of the coarse-sorted scatter for producers other than the CSR one: adds bins laid
 // out uniformly, bin (p, b) = the places from (p * n_win + b) * cap with counts[b * producers + p]

@@ -1269,8 +1269,11 @@ inline uint64_t event_run_pairs(uint32_t n_row, uint32_t n_col) {
 // against the sorted scatter, 25,000 columns lose at both.)
 constexpr size_t kSelfWindowBytes = 58 * 1024;
 constexpr uint32_t kSelfMaxSlices = 2;
-bool window_event_scatter_self_usable(uint32_t n_row, uint32_t n_col) {
-  return n_col != 0 && n_col <= kSelfMaxSlices * (kSelfWindowBytes / sizeof(double)) && n_row != 0 && n_row <= kSelfListRows;
+bool window_event_scatter_self_usable(uint32_t n_row, uint32_t n_col, bool heter) {
+  // (a homogeneous weight: up to four slices of 14,848 integer counts, as with a list of the active rows below)
+  const uint32_t widest = heter ? kSelfMaxSlices * static_cast<uint32_t>(kSelfWindowBytes / sizeof(double))
+                                : 4u * static_cast<uint32_t>(kSelfWindowBytes / sizeof(uint32_t));
+  return n_col != 0 && n_col <= widest && n_row != 0 && n_row <= kSelfListRows;
 }
 
 // A homogeneous weight counts synapses in 32-bit integers, 14,848 to a window of 58 KB, and an output of up to four
@@ -1309,7 +1312,7 @@ bool window_event_scatter(hipStream_t stream, const F *data, bool heter, const u
                           F *y, uint32_t n_row, uint32_t n_col, uint32_t *counters, const uint2 *active_list,
                           uint32_t list_cap, void *scratch, size_t scratch_bytes, const void *events, uint32_t event_width) {
   const bool self = events != nullptr;  // no list: the kernel looks at the events itself
-  if (self ? !window_event_scatter_self_usable(n_row, n_col) : !window_event_scatter_usable<F>(n_row, n_col, heter)) return false;
+  if (self ? !window_event_scatter_self_usable(n_row, n_col, heter) : !window_event_scatter_usable<F>(n_row, n_col, heter)) return false;
   if (scratch_bytes < window_event_scatter_bytes<F>(n_col)) return false;
   if (self && event_width != 1u && event_width != 4u && event_width != 8u) return false;
   const size_t acc_bytes = heter ? sizeof(double) : sizeof(uint32_t);

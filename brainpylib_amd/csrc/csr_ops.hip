@@ -1452,7 +1452,7 @@ void launch_scatter(const ScratchSource &src, const F *data, const uint32_t *ind
   // per row at 20 % events: 545 us against 31).  (Not from a fixed arena: the walks below need less scratch
   // memory there.)
   if constexpr (MODE == kEvent && (sizeof(VT) == 1 || std::is_floating_point<VT>::value)) {
-    if (!src.fixed() && n_row > kSmallRows && window_event_scatter_self_usable(n_row, n_col)) {
+    if (!src.fixed() && n_row > kSmallRows && window_event_scatter_self_usable(n_row, n_col, HETER)) {
       const size_t need = window_event_scatter_bytes<F>(n_col);
       size_t got = 0;
       unsigned char *ws = static_cast<unsigned char *>(src.request(need, need, &got));

@@ -581,8 +581,10 @@ def test_event_scatter_of_one_weight_into_slices_of_the_output(cuda, oracle_mod,
   # rows and a row that holds a large share of the nonzeros; bit for bit, twice in a row.  Weights per synapse
   # of the same matrices take the sorted scatter.
   rng = np.random.default_rng(61)
+  # (up to 32,768 rows the workgroups find the active rows themselves: the same slices without the list)
   for n_row, n_col, mean, hub in ((40_000, 14_849, 20, 0), (65_536, 29_696, 9, 50_000), (33_000, 59_392, 25, 0),
-                                  (50_000, 59_393, 10, 0), (65_537, 20_000, 12, 0), (45_000, 44_544, 40, 0)):
+                                  (50_000, 59_393, 10, 0), (65_537, 20_000, 12, 0), (45_000, 44_544, 40, 0),
+                                  (20_000, 59_392, 30, 0), (32_768, 30_000, 15, 25_000), (5_000, 59_393, 50, 0)):
     counts = np.minimum(rng.poisson(mean, size=n_row), n_col)
     counts[rng.integers(0, n_row, size=n_row // 9)] = 0
     if hub:
