@@ -1727,8 +1727,10 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
     // A dense vector that fits LDS beside nothing else (up to 40,704 floats), under persistent
     // workgroups (few copies): staged there.  Gathers from L2 cap the product at about 140 G nonzeros
     // per second whatever the vector's size; from LDS the index and weight streams are the limit.
+    // (From 2,048 rows: 10,000 x 10,000 with 1,000 per row 28 -> 19 us, 8,000 x 30,000 with 300 per row 15 -> 12 us;
+    // a matrix of few nonzeros pays up to a microsecond for the copies, 12,000 x 38,000 with 50 per row 8.8 -> 9.3 us.)
     const size_t lds_bytes = static_cast<size_t>(n_col) * sizeof(VT);
-    if (n_row >= 16384 && n_col > 0 && lds_bytes <= kLdsBitmapCap) {
+    if (n_row >= 2048 && n_col > 0 && lds_bytes <= kLdsBitmapCap) {
       if (launch_gather_impl<F, VT, HETER, MODE, 1>(target, stream, data, indices, indptr, x, y, n_row, n_col,
                                                     lds_bytes))
         return;
