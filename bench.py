@@ -835,6 +835,37 @@ def main():
                                       gsop_per_s=delivered / (dur_w.mean() * 1e-3) / 1e9)
     extra["scatter_1e6x1e6_100_per_row"] = wide
     log("event scatter 1e6 x 1e6: %s" % wide)
+    # the gather over the same matrix (5 % of the columns have an event), and over 500,000 x 500,000 with 100 per
+    # row: short rows behind a bitmap of 125 KB (one workgroup per CU) and of 62.5 KB (two): the walks over
+    # the nonzeros that look rows up for the hits only
+    short = {}
+    for tag, sm, smd in (("1e6x1e6", m, md), ("5e5x5e5", None, None)):
+      if sm is None:
+        r_s = np.random.default_rng(31)
+        sm = dict(shape=(500_000, 500_000), indices=r_s.integers(0, 500_000, size=50_000_000, dtype=np.int32),
+                  indptr=(np.arange(500_001, dtype=np.int64) * 100).astype(np.int32),
+                  data=r_s.random(50_000_000, dtype=np.float32))
+        smd = {k: torch.from_numpy(v).to(dev) for k, v in sm.items() if isinstance(v, np.ndarray)}
+      ev_np = np.random.default_rng(18).random(sm["shape"][1]) < 0.05
+      ev_s = torch.from_numpy(ev_np).to(dev)
+      nnz_s = int(sm["indices"].shape[0])
+      for name, w_np, w_dev in (("heter", sm["data"], smd["data"]),
+                                ("homo", sm["data"][:1], smd["data"][:1].contiguous())):
+        want = oracle.event_csr_matvec(w_np, sm["indices"], sm["indptr"], ev_np, shape=sm["shape"])
+        mag = oracle.event_csr_matvec(np.abs(w_np), sm["indices"], sm["indptr"], ev_np, shape=sm["shape"])
+        got = bpl.event_csr_matvec(w_dev, smd["indices"], smd["indptr"], ev_s, shape=sm["shape"])
+        check(got.cpu().numpy(), want, "event_csr_matvec gather %s %s" % (tag, name), mag)
+        dur_s, _ = time_calls(lambda: bpl.event_csr_matvec(w_dev, smd["indices"], smd["indptr"], ev_s, shape=sm["shape"]),
+                              args.steps, 5)
+        bytes_s = nnz_s * (8 if name == "heter" else 4) + 8 * sm["shape"][0]
+        short["%s_%s" % (tag, name)] = dict(
+          stats(dur_s), nnz=nnz_s,
+          roofline=dict(bound="hbm", unit="GB/s", achieved=bytes_s / (dur_s.mean() * 1e-3) / 1e9, peak=HBM_PEAK_GBS,
+                        frac=bytes_s / (dur_s.mean() * 1e-3) / 1e9 / HBM_PEAK_GBS))
+      if tag != "1e6x1e6":
+        del sm, smd
+    extra["gather_100_per_row"] = short
+    log("event gather, 100 per row: %s" % short)
     # a mid-size projection, 32,000 x 8,192 with about 1,000 nonzeros per row: the walk into LDS windows whose
     # workgroups find the active rows themselves, at three activities
     counts_m = np.maximum(1, np.random.default_rng(23).poisson(1000, 32_000))

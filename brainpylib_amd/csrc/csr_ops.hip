@@ -987,70 +987,109 @@ __device__ __forceinline__ void gather_hub_rows(const F *__restrict__ data, cons
 
 
 // ------------------------------------------------------------------------------------------------
-// event gather, walked flat (bitmaps of more than 80 KB, rows of 16 to 383 nonzeros on average)
+// event gather, walked flat (rows of 16 to 383 nonzeros on average)
 // ------------------------------------------------------------------------------------------------
 // The row-wise walks pad every row to whole steps of its lane group: with 100 nonzeros per row and 8 lanes
 // x 16 loads per row a quarter of the index requests lie beyond their row.  Here every wave owns a contiguous
 // range of the nonzeros that begins and ends at row boundaries (the rows whose first nonzero lies in its
 // equal share of the nonzeros: no row is shared by two waves, so nothing is left for a second kernel) and
-// takes it in steps of 1,024: four 16-byte nontemporal loads of indices per lane (the next step's are
-// requested before this step's are used), sixteen probes of the event bitmap in LDS per lane.  Rows are
-// looked up for the HITS only: the lanes leave the positions of their hits (some 5 % of the nonzeros) in a
-// queue in LDS, compacted by a prefix sum over the wave, and every lane then takes one hit: its weight, a
-// six-step search of a window of 65 row offsets in LDS for its row, one atomic addition to that row's
-// accumulator (float64; a homogeneous weight: a 32-bit count).  Rows that end inside the step are stored.
+// takes it in steps of 768 or 1,024: three or four 16-byte nontemporal loads of indices per lane (the next
+// steps' are under way while a step is worked on), twelve or sixteen probes of the event bitmap in LDS per
+// lane.  Rows are looked up for the HITS only: the lanes leave the positions of their hits (some 5 % of the
+// nonzeros) in a queue in LDS, compacted by a prefix sum over the wave, and every lane then takes one hit: its
+// weight, a six-step search of a window of 65 row offsets in LDS for its row, one atomic addition to that
+// row's accumulator (float64; a homogeneous weight: a 32-bit count).  Rows that end inside the step are stored.
 constexpr uint32_t kFlatEvRows = 64;     // rows of a window (one per lane)
-constexpr uint32_t kFlatEvQueue = 256;   // hits queued at a time (more in a step: further rounds)
 constexpr uint32_t kFlatEvMinMean = 16, kFlatEvMaxMean = 384;
+constexpr uint32_t kFlatEvSharedMaxMean = 256, kFlatEvSharedMinNnz = 45000000;  // (in the kernel that shares its CU)
 constexpr uint32_t kFlatEvWaves = 16;
-// static LDS of the walk: windows, accumulators and queues of 16 waves
-constexpr size_t kFlatEvLdsBytes = kFlatEvWaves * ((kFlatEvRows + 2) * 4 + kFlatEvRows * 8 + kFlatEvQueue * 2) + 256;
+#ifndef FLAT_U
+#define FLAT_U 3
+#define FLAT_DEPTH 2
+#endif
+// Loads of four indices per lane and step, and steps under way.  One workgroup per CU (a bitmap of more than 80
+// KB): 4 and 3, 48 registers of indices.  Two workgroups per CU must keep to 64 registers: 3 and 2.
+constexpr int kFlatEvQuadsAlone = 4, kFlatEvDepthAlone = 3, kFlatEvQuadsShared = FLAT_U, kFlatEvDepthShared = FLAT_DEPTH;
+// hits queued at a time (more in a step: further rounds)
+constexpr uint32_t kFlatEvQueueAlone = 256, kFlatEvQueueShared = 128;
+// LDS of the walk behind the bitmap: accumulators, windows of row offsets and queues of 16 waves
+constexpr size_t flat_event_wave_bytes(uint32_t queue) { return kFlatEvRows * 8 + (kFlatEvRows + 4) * 4 + queue * 2; }
+constexpr size_t flat_event_lds_bytes(uint32_t queue) { return kFlatEvWaves * flat_event_wave_bytes(queue); }
 // the largest event bitmap that is kept whole in LDS (beside that; wider event vectors get a two-level bitmap)
-constexpr size_t kLdsEventBitmapCap = (kLdsBitmapCap - kFlatEvLdsBytes) / 256 * 256;
-
-// the first row r in [0, n_row] with indptr[r] >= pos, for pos <= indptr[n_row]: the wave searches together,
-// 64 probes a round
-__device__ __forceinline__ uint32_t first_row_from(const uint32_t *__restrict__ indptr, uint32_t n_row, uint32_t pos,
-                                                   uint32_t lane) {
-  uint32_t lo = 0, hi = n_row;  // the answer lies in [lo, hi]: indptr[r] < pos for r < lo, indptr[hi] >= pos
-  while (lo < hi) {
-    const uint32_t span = hi - lo;
-    const uint32_t stride = span / kWave + (span % kWave ? 1u : 0u);
-    const uint64_t probe = static_cast<uint64_t>(lo) + static_cast<uint64_t>(lane) * stride;
-    const bool below = probe < hi && indptr[probe] < pos;  // (the lanes for which this holds form a prefix)
-    const uint32_t cnt = static_cast<uint32_t>(__popcll(__ballot(below)));
-    if (cnt == 0) return lo;  // indptr[lo] >= pos
-    // indptr[lo + (cnt - 1) stride] < pos, and the probe after it (if it lies below hi) is not below pos
-    const uint64_t next = static_cast<uint64_t>(lo) + static_cast<uint64_t>(cnt) * stride;
-    if (next < hi) hi = static_cast<uint32_t>(next);
-    lo += (cnt - 1u) * stride + 1u;
-  }
-  return lo;
+constexpr size_t kLdsEventBitmapCap = (kLdsBitmapCap - flat_event_lds_bytes(kFlatEvQueueAlone)) / 256 * 256;
+// the largest bitmap that leaves room for two workgroups per CU (80 KB each, less the kernel's static LDS)
+constexpr size_t kLdsSharedBitmapCap = 80 * 1024 - 512;
+// where the walk's memory begins behind a bitmap of n_col bits (in 32-bit words)
+__host__ __device__ inline uint32_t flat_event_lds_offset(uint32_t n_col) { return ((n_col + 31u) / 32u + 3u) & ~3u; }
+// Whether a workgroup of the kernel that shares its CU is given the walk's memory behind its bitmap (the
+// launcher and the kernel decide alike)
+__host__ __device__ inline bool flat_event_shared_fits(uint32_t n_row, uint32_t n_col) {
+  return n_row >= 16384u &&
+         static_cast<size_t>(flat_event_lds_offset(n_col)) * 4 + flat_event_lds_bytes(kFlatEvQueueShared) <= kLdsSharedBitmapCap;
 }
 
-template <typename F, bool HETER>
+// For each of two positions pos <= indptr[n_row]: the first row r in [0, n_row] with indptr[r] >= pos.  The wave
+// searches together, 64 probes a round, and both searches go round by round side by side (their probes are
+// under way together: half the dependent round trips of one search after the other).
+__device__ __forceinline__ void first_rows_from(const uint32_t *__restrict__ indptr, uint32_t n_row, uint32_t pos_a,
+                                                uint32_t pos_b, uint32_t lane, uint32_t &row_a, uint32_t &row_b) {
+  // an answer lies in [lo, hi]: indptr[r] < pos for r < lo, indptr[hi] >= pos
+  uint32_t lo_a = 0, hi_a = n_row, lo_b = 0, hi_b = n_row;
+  while (lo_a < hi_a || lo_b < hi_b) {
+    const uint32_t span_a = hi_a - lo_a, span_b = hi_b - lo_b;
+    const uint32_t stride_a = span_a / kWave + (span_a % kWave ? 1u : 0u);
+    const uint32_t stride_b = span_b / kWave + (span_b % kWave ? 1u : 0u);
+    const uint64_t probe_a = static_cast<uint64_t>(lo_a) + static_cast<uint64_t>(lane) * stride_a;
+    const uint64_t probe_b = static_cast<uint64_t>(lo_b) + static_cast<uint64_t>(lane) * stride_b;
+    const uint32_t at_a = probe_a < hi_a ? indptr[probe_a] : 0xffffffffu;
+    const uint32_t at_b = probe_b < hi_b ? indptr[probe_b] : 0xffffffffu;
+    // (the lanes whose probe lies below the position form a prefix)
+    const uint32_t cnt_a = static_cast<uint32_t>(__popcll(__ballot(probe_a < hi_a && at_a < pos_a)));
+    const uint32_t cnt_b = static_cast<uint32_t>(__popcll(__ballot(probe_b < hi_b && at_b < pos_b)));
+    if (cnt_a == 0) {
+      hi_a = lo_a;  // indptr[lo] >= pos
+    } else {
+      // indptr[lo + (cnt - 1) stride] < pos, and the probe after it (if it lies below hi) is not below pos
+      const uint64_t next = static_cast<uint64_t>(lo_a) + static_cast<uint64_t>(cnt_a) * stride_a;
+      if (next < hi_a) hi_a = static_cast<uint32_t>(next);
+      lo_a += (cnt_a - 1u) * stride_a + 1u;
+    }
+    if (cnt_b == 0) {
+      hi_b = lo_b;
+    } else {
+      const uint64_t next = static_cast<uint64_t>(lo_b) + static_cast<uint64_t>(cnt_b) * stride_b;
+      if (next < hi_b) hi_b = static_cast<uint32_t>(next);
+      lo_b += (cnt_b - 1u) * stride_b + 1u;
+    }
+  }
+  row_a = lo_a;
+  row_b = lo_b;
+}
+
+template <typename F, bool HETER, int U, int DEPTH, uint32_t QUEUE>
 __device__ __forceinline__ void gather_rows_flat_event(const F *__restrict__ data, const uint32_t *__restrict__ indices,
                                                        const uint32_t *__restrict__ indptr, F *__restrict__ y,
-                                                       uint32_t n_row, uint32_t nnz, const uint32_t *s_bits) {
+                                                       uint32_t n_row, uint32_t nnz, const uint32_t *s_bits,
+                                                       uint32_t *s_work) {
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   using A = typename std::conditional<HETER, double, uint32_t>::type;
-  constexpr int U = 4;
+  static_assert(DEPTH == 2 || DEPTH == 3, "two or three sets of index registers");
   constexpr uint32_t kStep = 4u * U * kWave;  // nonzeros per step
-  __shared__ uint32_t s_ptr_all[kFlatEvWaves][kFlatEvRows + 2];
-  __shared__ A s_sum_all[kFlatEvWaves][kFlatEvRows];
-  __shared__ uint16_t s_queue_all[kFlatEvWaves][kFlatEvQueue];
   const uint32_t lane = static_cast<uint32_t>(lane_id()), wv = threadIdx.x / kWave;
-  uint32_t *s_ptr = s_ptr_all[wv];
-  A *s_sum = s_sum_all[wv];
-  uint16_t *s_queue = s_queue_all[wv];
+  // the wave's part of `s_work` (16-byte aligned): 64 accumulators, 66 row offsets, the queue
+  uint32_t *mine_lds = s_work + wv * (flat_event_wave_bytes(QUEUE) / 4);
+  A *s_sum = reinterpret_cast<A *>(mine_lds);
+  uint32_t *s_ptr = mine_lds + kFlatEvRows * 2;
+  uint16_t *s_queue = reinterpret_cast<uint16_t *>(s_ptr + kFlatEvRows + 4);
   const uint32_t waves = gridDim.x * (blockDim.x / kWave), w = blockIdx.x * (blockDim.x / kWave) + wv;
   const F w_homo = HETER ? F(0) : data[0];
   // equal shares of the nonzeros, in whole steps; the wave's rows are those that begin in its share
   const uint64_t share = ((static_cast<uint64_t>(nnz) + waves - 1u) / waves + kStep - 1u) / kStep * kStep;
   const uint64_t pos0 = static_cast<uint64_t>(w) * share, pos1 = pos0 + share;
-  if (pos0 >= nnz && w != 0) return;
-  uint32_t r = (w == 0) ? 0u : first_row_from(indptr, n_row, static_cast<uint32_t>(pos0), lane);
-  const uint32_t r_end = (pos1 >= nnz) ? n_row : first_row_from(indptr, n_row, static_cast<uint32_t>(pos1), lane);
+  if (pos0 >= nnz) return;  // (nnz > 0, so wave 0 goes on)
+  uint32_t r, r_last;
+  first_rows_from(indptr, n_row, static_cast<uint32_t>(pos0), pos1 >= nnz ? nnz : static_cast<uint32_t>(pos1), lane, r, r_last);
+  const uint32_t r_end = (pos1 >= nnz) ? n_row : r_last;  // (the last wave also takes the rows without nonzeros at the end)
   if (r >= r_end) return;
   const uint32_t begin = indptr[r], end = indptr[r_end];
   if (begin == end) {  // rows without nonzeros only
@@ -1060,42 +1099,48 @@ __device__ __forceinline__ void gather_rows_flat_event(const F *__restrict__ dat
   s_sum[lane] = A(0);
   if (lane == 0) s_ptr[kFlatEvRows + 1] = 0xffffffffu;
 
-  auto load_indices = [&](uint32_t s0, u32x4 (&ci)[U]) {  // lane l: quads s0 / 4 + l, + 64, ...
+  // the step that begins at nonzero s0: lane l takes the quads s0 / 4 + l, + 64, ...
+  // Every lane loads, without a condition: a quad beyond the array's last whole one is replaced by that one (its
+  // hits are masked below, in the last step of a range, and the array's last, partial quad is probed there).
+  const uint32_t q_last = nnz / 4u - 1u;
+  auto load_indices = [&](uint32_t s0, u32x4 (&ci)[U]) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t q = s0 / 4u + static_cast<uint32_t>(u) * kWave + lane;
-      ci[u] = u32x4{0u, 0u, 0u, 0u};
-      if (s0 < end && 4u * q < end) {
-        if (4u * q + 4u <= nnz) {
-          ci[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(indices) + q);
-        } else {  // (the array's last, partial quad)
-          if (4u * q + 0u < nnz) ci[u].x = indices[4u * q + 0u];
-          if (4u * q + 1u < nnz) ci[u].y = indices[4u * q + 1u];
-          if (4u * q + 2u < nnz) ci[u].z = indices[4u * q + 2u];
-        }
-      }
+      ci[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(indices) + (q < q_last ? q : q_last));
     }
   };
-  // The indices of the next two steps are under way while a step is worked on (with one step ahead the walk
-  // streamed at 3.4 TB/s).  The second one is requested at the END of a step, behind the gathers of the hits'
-  // weights: waiting for a load means waiting for every load issued before it, and the step before's request
-  // has arrived by then.
-  u32x4 ci[U], ci1[U], ci2[U];
+  // the window of row offsets from row r on
+  uint32_t ptr_lane, ptr_last;
+  auto load_window = [&]() {
+    const uint64_t k = static_cast<uint64_t>(r) + lane;
+    ptr_lane = k <= n_row ? indptr[k] : 0xffffffffu;
+    ptr_last = static_cast<uint64_t>(r) + kFlatEvRows <= n_row ? indptr[r + kFlatEvRows] : 0xffffffffu;
+  };
+  auto store_window = [&]() {
+    s_ptr[lane] = ptr_lane;
+    if (lane == 0) s_ptr[kFlatEvRows] = ptr_last;
+  };
+  // The indices of the next DEPTH - 1 steps are under way while a step is worked on (with one step ahead and 16
+  // waves per CU the walk streamed at 3.4 TB/s).  Every step works from a set of registers of its own and, at its
+  // END, requests the step DEPTH ahead into the same set (copying between sets would wait for the request just
+  // made); the request comes behind the gathers of the hits' weights, because waiting for a load means waiting
+  // for every load issued before it.  The window of row offsets of the next step is requested just before.
+  // (The first requests are made in the order in which the steps make them, and kept in that order: how many
+  // later requests a wait may leave under way is fixed at compile time from BOTH ways into the loop.)
+  u32x4 ci0[U], ci1[U], ci2[DEPTH == 3 ? U : 1];
   const uint32_t first_step = begin / 4u * 4u;  // (steps begin at whole quads; what lies before `begin` is masked)
-  load_indices(first_step, ci);
+  load_window();
+  __builtin_amdgcn_sched_barrier(0);
+  load_indices(first_step, ci0);
+  __builtin_amdgcn_sched_barrier(0);
   load_indices(first_step + kStep, ci1);
-  load_indices(first_step + 2u * kStep, ci2);  // (a step at or beyond the end of the range loads nothing)
-  for (uint32_t s0 = first_step; s0 < end; s0 += kStep) {
+  __builtin_amdgcn_sched_barrier(0);
+  if constexpr (DEPTH == 3) load_indices(first_step + 2u * kStep, ci2);
+  __builtin_amdgcn_sched_barrier(0);
+  auto step = [&](const uint32_t s0, u32x4 (&ci)[U]) {
     const uint32_t s1 = (end - s0 > kStep) ? s0 + kStep : end;
-    uint32_t ptr_lane, ptr_last;
-    auto load_window = [&]() {
-      const uint64_t k = static_cast<uint64_t>(r) + lane;
-      ptr_lane = k <= n_row ? indptr[k] : 0xffffffffu;
-      ptr_last = static_cast<uint64_t>(r) + kFlatEvRows <= n_row ? indptr[r + kFlatEvRows] : 0xffffffffu;
-    };
-    load_window();
-    // the sixteen probes: bit 4 u + t of `hits` = nonzero 4 (s0 / 4 + 64 u + lane) + t is in the range and its
-    // column has an event
+    // the probes: bit 4 u + t of `hits` = nonzero s0 + 256 u + 4 lane + t is in the range and its column has an event
     uint32_t hits = 0;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -1104,57 +1149,64 @@ __device__ __forceinline__ void gather_rows_flat_event(const F *__restrict__ dat
       for (int t = 0; t < 4; ++t)  // (the bit-field extract takes the low five bits of its offset)
         hits |= __builtin_amdgcn_ubfe(s_bits[c[t] >> 5], c[t], 1u) << (4 * u + t);
     }
-    if (s0 < begin || s1 - s0 < kStep) {  // (the first and the last step of the range only: what lies outside is column 0)
+    if (s0 < begin || s1 - s0 < kStep) {  // (the first and the last step of the range only)
+      // of the lane's quad u, the nonzeros number [from, to) lie in [begin, s1)
       uint32_t inside = 0;
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const uint32_t p0 = 4u * (s0 / 4u + static_cast<uint32_t>(u) * kWave + lane);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const uint32_t p = p0 + static_cast<uint32_t>(t);
-          inside |= ((p >= begin && p < s1) ? 1u : 0u) << (4 * u + t);
-        }
+        const uint32_t p0 = s0 + static_cast<uint32_t>(u) * 4u * kWave + 4u * lane;
+        const uint32_t from = begin > p0 ? (begin - p0 < 4u ? begin - p0 : 4u) : 0u;
+        const uint32_t to = s1 > p0 ? (s1 - p0 < 4u ? s1 - p0 : 4u) : 0u;
+        inside |= ((0xfu << from) & ~(0xfu << to) & 0xfu) << (4 * u);
       }
       hits &= inside;
+      // the array's last, partial quad was not loaded: the lane whose quad it is probes its one to three columns
+      const uint32_t tail = nnz & ~3u;
+      if (tail != nnz && s1 == nnz && tail >= s0 && ((tail - s0) / 4u) % kWave == lane) {
+        const uint32_t shift = (tail - s0) / (4u * kWave) * 4u;
+        hits &= ~(0xfu << shift);
+        for (uint32_t p = tail > begin ? tail : begin; p < nnz; ++p) {
+          const uint32_t c = indices[p];
+          hits |= __builtin_amdgcn_ubfe(s_bits[c >> 5], c, 1u) << (shift + (p - tail));
+        }
+      }
     }
-#pragma unroll
-    for (int u = 0; u < U; ++u) ci[u] = ci1[u];
     // where the lane's hits go in the step's sequence of hits
     const uint32_t mine = static_cast<uint32_t>(__popc(hits));
     const uint32_t incl = wave_inclusive_scan_u32(mine);
     const uint32_t total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(incl), kWave - 1));
-    auto fill_queue = [&](uint32_t base) {  // hits number base .. base + 255 of the step: (u, lane, t) each
+    // hits number base .. base + QUEUE - 1 of the step: the distance of each from s0 (256 u + 4 lane + t)
+    auto fill_queue = [&](uint32_t base) {
       uint32_t m = hits, at = incl - mine;
       while (m != 0u) {
         const uint32_t b = static_cast<uint32_t>(__ffs(static_cast<int>(m))) - 1u;
         m &= m - 1u;
-        if (at - base < kFlatEvQueue) s_queue[at - base] = static_cast<uint16_t>(((b >> 2) << 8) | (lane << 2) | (b & 3u));
+        if (at - base < QUEUE) s_queue[at - base] = static_cast<uint16_t>(((b >> 2) << 8) | (lane << 2) | (b & 3u));
         ++at;
       }
     };
-    if (total != 0u && total <= kFlatEvQueue) fill_queue(0u);
-    // windows of 64 rows from r on, until one reaches beyond the step
+    if (total != 0u && total <= QUEUE) fill_queue(0u);
+    // windows of 64 rows from r on, until one reaches beyond the step (the first one was requested a step ago;
+    // the loop reads it from LDS only, so that the wait for a further window's request stays on that path)
+    store_window();
     for (;;) {
-      s_ptr[lane] = ptr_lane;
-      if (lane == 0) s_ptr[kFlatEvRows] = ptr_last;
       __builtin_amdgcn_wave_barrier();
-      const uint32_t lo = s_ptr[0], hi = ptr_last;
+      const uint32_t lo = s_ptr[0], hi = s_ptr[kFlatEvRows];
       const uint32_t top = hi < s1 ? hi : s1;  // the window takes the hits at nonzeros [lo, top)
-      for (uint32_t base = 0; base < total; base += kFlatEvQueue) {
-        if (total > kFlatEvQueue) {
+      for (uint32_t base = 0; base < total; base += QUEUE) {
+        if (total > QUEUE) {
           __builtin_amdgcn_wave_barrier();
           fill_queue(base);
           __builtin_amdgcn_wave_barrier();
         }
-        const uint32_t n = total - base < kFlatEvQueue ? total - base : kFlatEvQueue;
+        const uint32_t n = total - base < QUEUE ? total - base : QUEUE;
         for (uint32_t i = lane; i < n; i += kWave) {
-          const uint32_t e = s_queue[i];
-          const uint32_t p = 4u * (s0 / 4u + (e >> 8) * kWave + ((e >> 2) & 63u)) + (e & 3u);
+          const uint32_t p = s0 + s_queue[i];
           if (p >= lo && p < top) {
             uint32_t k = 0;  // the last k < 64 with s_ptr[k] <= p
 #pragma unroll
-            for (uint32_t step = kFlatEvRows / 2; step != 0; step >>= 1)
-              if (s_ptr[k + step] <= p) k += step;
+            for (uint32_t half = kFlatEvRows / 2; half != 0; half >>= 1)
+              if (s_ptr[k + half] <= p) k += half;
             if constexpr (HETER) atomicAdd(&s_sum[k], static_cast<double>(data[p]));
             else atomicAdd(&s_sum[k], 1u);
           }
@@ -1178,11 +1230,21 @@ __device__ __forceinline__ void gather_rows_flat_event(const F *__restrict__ dat
         break;
       }
       load_window();
+      store_window();
     }
     __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int u = 0; u < U; ++u) ci1[u] = ci2[u];
-    load_indices(s0 + 3u * kStep, ci2);
+    load_window();
+    load_indices(s0 + static_cast<uint32_t>(DEPTH) * kStep, ci);
+  };
+  for (uint32_t s0 = first_step;;) {
+    step(s0, ci0);
+    if ((s0 += kStep) >= end) break;
+    step(s0, ci1);
+    if ((s0 += kStep) >= end) break;
+    if constexpr (DEPTH == 3) {
+      step(s0, ci2);
+      if ((s0 += kStep) >= end) break;
+    }
   }
 }
 
@@ -1259,7 +1321,8 @@ __global__ __launch_bounds__(1024, (MODE == kEvent && BITS == 1) ? 8 : 4) void c
       // rows of 16 to 383 nonzeros on average: the flat walk over the nonzeros, which leaves no row to the pass below
       if (mean >= kFlatEvMinMean && mean < kFlatEvMaxMean && nnz <= kFlatMaxNnz && blockDim.x == kFlatEvWaves * kWave &&
           (reinterpret_cast<uintptr_t>(indices) & 15u) == 0) {
-        gather_rows_flat_event<F, HETER>(data, indices, indptr, y, n_row, nnz, s_bits);
+        gather_rows_flat_event<F, HETER, kFlatEvQuadsAlone, kFlatEvDepthAlone, kFlatEvQueueAlone>(
+          data, indices, indptr, y, n_row, nnz, s_bits, s_bits + flat_event_lds_offset(n_col));
         return;
       }
     }
@@ -1267,6 +1330,20 @@ __global__ __launch_bounds__(1024, (MODE == kEvent && BITS == 1) ? 8 : 4) void c
     else if (mean >= 48) { gather_rows<F, VT, HETER, MODE, BITS, 8, 16>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 8; hub_len = kHubSteps * 16 * 8; }
     else { gather_rows<F, VT, HETER, MODE, BITS, 4, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = blockDim.x / 4; hub_len = kHubSteps * 8 * 4; }
   } else {
+    if constexpr (MODE == kEvent && BITS == 1 && HETER) {
+      // The same walk within 64 registers, where the launcher left room for it behind the bitmap.  A wave's steps
+      // form one chain of dependent round trips (row offsets, probes, search, the hits' weights), so the walk pays
+      // from some 6,000 nonzeros per wave on: 500,000 x 500,000 with 100 per row 88 -> 76 us, 2,000,000 x 500,000
+      // with 30 per row 116 -> 85 us, but 350,000 x 350,000 with 100 per row 56 -> 60 us.  With one weight the
+      // row-wise walk has no weights to wait for and stays ahead (46 against 57 us for the first of these).
+      if (mean >= kFlatEvMinMean && mean < kFlatEvSharedMaxMean && nnz >= kFlatEvSharedMinNnz && nnz <= kFlatMaxNnz &&
+          blockDim.x == kFlatEvWaves * kWave && (reinterpret_cast<uintptr_t>(indices) & 15u) == 0 &&
+          flat_event_shared_fits(n_row, n_col)) {
+        gather_rows_flat_event<F, HETER, kFlatEvQuadsShared, kFlatEvDepthShared, kFlatEvQueueShared>(
+          data, indices, indptr, y, n_row, nnz, s_bits, s_bits + flat_event_lds_offset(n_col));
+        return;
+      }
+    }
     if (mean >= 384) { gather_rows_wave<F, VT, HETER, MODE, BITS, 8>(data, indices, indptr, x, y, n_row, s_bits, coarse_g); gpb = 1; hub_len = kHubSteps * 8 * kWave; }
     // (a dense vector is gathered from L2: for rows of 48 .. 191 nonzeros the pipelined 32-lane walk keeps more
     // of those gathers in flight than a wave per row does)
@@ -1695,10 +1772,10 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
     // likewise from 655,360 columns on (a bitmap of more than 80 KB, one workgroup per CU: 256 workgroups that
     // each read a megabyte of events take longer than one small kernel and 125 KB per workgroup).
     const size_t words = (static_cast<size_t>(n_col) + 31) / 32;
-    uint32_t *bits = (sizeof(VT) > 1 || words * 4 > 80 * 1024 - 512)
+    uint32_t *bits = (sizeof(VT) > 1 || words * 4 > kLdsSharedBitmapCap)
                          ? static_cast<uint32_t *>(src.request((words + 1) * sizeof(uint32_t)))
                          : nullptr;
-    if (sizeof(VT) == 1 && words * 4 <= 80 * 1024 - 512) {
+    if (sizeof(VT) == 1 && words * 4 <= kLdsSharedBitmapCap) {
       // (byte events and a bitmap that leaves room for two workgroups per CU: they pack it themselves)
     } else if (bits != nullptr) {
       pack_event_bitmap<VT>(stream, x, n_col, bits);
@@ -1714,11 +1791,15 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
     const size_t lds_bytes = (static_cast<size_t>(n_col) + 31) / 32 * 4;
     const size_t lds_cap = kLdsEventBitmapCap;
     if (lds_bytes <= lds_cap) {
-      const bool ok = lds_bytes > 80 * 1024 - 512  // (two workgroups per CU below: 80 KB each, less their static LDS)
+      // (behind the bitmap: the memory of the flat walk over short rows, where it fits)
+      const size_t walk_at = static_cast<size_t>(flat_event_lds_offset(n_col)) * 4;
+      const size_t shared_bytes =
+        flat_event_shared_fits(n_row, n_col) ? walk_at + flat_event_lds_bytes(kFlatEvQueueShared) : lds_bytes;
+      const bool ok = lds_bytes > kLdsSharedBitmapCap  // (two workgroups per CU below)
                           ? launch_gather_impl<F, VT, HETER, MODE, 2>(target, stream, data, indices, indptr, x, y, n_row,
-                                                                      n_col, lds_bytes)
+                                                                      n_col, walk_at + flat_event_lds_bytes(kFlatEvQueueAlone))
                           : launch_gather_impl<F, VT, HETER, MODE, 1>(target, stream, data, indices, indptr, x, y, n_row,
-                                                                      n_col, lds_bytes);
+                                                                      n_col, shared_bytes);
       if (ok) return;
       bpl_clear_error();
     }

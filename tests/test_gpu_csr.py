@@ -309,6 +309,45 @@ def test_gather_flat_walk_over_the_nonzeros_of_short_rows(cuda, oracle_mod, kind
   assert np.array_equal(got, oracle_mod.event_csr_matvec(data, indices, indptr, evf, shape=shape)), (kind, "float events")
 
 
+@pytest.mark.parametrize("kind", ["ragged", "even", "dense_events"])
+def test_gather_flat_walk_in_the_kernel_that_shares_its_cu(cuda, oracle_mod, kind):
+  # A bitmap of at most 64 KB, weights per nonzero, rows of 16 to 255 nonzeros on average and 45 million nonzeros
+  # or more: the same walk with three loads per lane and step, in the kernel that runs two workgroups per CU.
+  # Integer weights: every output is compared bit for bit.  (Columns may repeat within a row: the sums do not care.)
+  rng = np.random.default_rng(sum(map(ord, kind)) + 1)
+  n_col, rate = 400_000, 0.05
+  if kind == "ragged":      # empty rows, rows of one nonzero, rows of a thousand, one row longer than a wave's share
+    counts = rng.choice([0, 1, 3, 40, 150, 1000], size=560_000, p=[0.2, 0.1, 0.2, 0.3, 0.15, 0.05])
+    counts[333_333] = 300_000
+  elif kind == "even":      # the widest bitmap that fits; runs of empty rows, also at the end; the last quad is partial
+    n_col = 518_144
+    counts = np.full(480_000, 100)
+    counts[100_000:105_000] = 0
+    counts[-3_000:] = 0
+    counts[-3_001] = 3
+  else:                     # most nonzeros hit: the queue of hits is filled in several rounds per step
+    counts, rate = rng.poisson(60, size=800_000), 0.9
+  counts = np.asarray(counts, dtype=np.int64)
+  n_row = len(counts)
+  indptr = np.zeros(n_row + 1, dtype=np.int32)
+  indptr[1:] = np.cumsum(counts)
+  nnz = int(indptr[-1])
+  indices = rng.integers(0, n_col, size=nnz, dtype=np.int32)
+  mean = nnz // n_row
+  assert 16 <= mean < 256 and nnz >= 45_000_000, (mean, nnz)
+  shape = (n_row, n_col)
+  ev = rng.random(n_col) < rate
+  print("kind", kind, shape, "nnz", nnz, "mean", mean, flush=True)
+  for dtype in (np.float32, np.float64):
+    data = rng.integers(-3, 4, size=nnz).astype(dtype)
+    want = oracle_mod.event_csr_matvec(data, indices, indptr, ev, shape=shape)
+    got = bpl.event_csr_matvec(data, indices, indptr, ev, shape=shape).cpu().numpy()
+    assert np.array_equal(got, want), (kind, dtype, int((got != want).sum()), np.flatnonzero(got != want)[:5])
+  evf = (ev * rng.uniform(0.5, 2.0, n_col)).astype(np.float64)  # (events of the weights' type)
+  got = bpl.event_csr_matvec(data, indices, indptr, evf, shape=shape).cpu().numpy()
+  assert np.array_equal(got, oracle_mod.event_csr_matvec(data, indices, indptr, evf, shape=shape)), (kind, "float events")
+
+
 def test_gather_with_a_two_level_event_bitmap(cuda, oracle_mod):
   # more columns than a bitmap in LDS can cover (1.3 million): a coarse bitmap (one bit per 2^g
   # columns) in LDS and the exact one in global memory; g = 2, 4 and 6 (both ways the coarse
