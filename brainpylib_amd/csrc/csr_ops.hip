@@ -1003,13 +1003,9 @@ constexpr uint32_t kFlatEvRows = 64;     // rows of a window (one per lane)
 constexpr uint32_t kFlatEvMinMean = 16, kFlatEvMaxMean = 384;
 constexpr uint32_t kFlatEvSharedMaxMean = 256, kFlatEvSharedMinNnz = 45000000;  // (in the kernel that shares its CU)
 constexpr uint32_t kFlatEvWaves = 16;
-#ifndef FLAT_U
-#define FLAT_U 3
-#define FLAT_DEPTH 2
-#endif
 // Loads of four indices per lane and step, and steps under way.  One workgroup per CU (a bitmap of more than 80
 // KB): 4 and 3, 48 registers of indices.  Two workgroups per CU must keep to 64 registers: 3 and 2.
-constexpr int kFlatEvQuadsAlone = 4, kFlatEvDepthAlone = 3, kFlatEvQuadsShared = FLAT_U, kFlatEvDepthShared = FLAT_DEPTH;
+constexpr int kFlatEvQuadsAlone = 4, kFlatEvDepthAlone = 3, kFlatEvQuadsShared = 3, kFlatEvDepthShared = 2;
 // hits queued at a time (more in a step: further rounds)
 constexpr uint32_t kFlatEvQueueAlone = 256, kFlatEvQueueShared = 128;
 // LDS of the walk behind the bitmap: accumulators, windows of row offsets and queues of 16 waves
@@ -1791,10 +1787,10 @@ void launch_gather(const char *target, const ScratchSource &src, const F *data, 
     const size_t lds_bytes = (static_cast<size_t>(n_col) + 31) / 32 * 4;
     const size_t lds_cap = kLdsEventBitmapCap;
     if (lds_bytes <= lds_cap) {
-      // (behind the bitmap: the memory of the flat walk over short rows, where it fits)
+      // (behind the bitmap: the memory of the flat walk over short rows, where it fits and is used)
       const size_t walk_at = static_cast<size_t>(flat_event_lds_offset(n_col)) * 4;
       const size_t shared_bytes =
-        flat_event_shared_fits(n_row, n_col) ? walk_at + flat_event_lds_bytes(kFlatEvQueueShared) : lds_bytes;
+        HETER && flat_event_shared_fits(n_row, n_col) ? walk_at + flat_event_lds_bytes(kFlatEvQueueShared) : lds_bytes;
       const bool ok = lds_bytes > kLdsSharedBitmapCap  // (two workgroups per CU below)
                           ? launch_gather_impl<F, VT, HETER, MODE, 2>(target, stream, data, indices, indptr, x, y, n_row,
                                                                       n_col, walk_at + flat_event_lds_bytes(kFlatEvQueueAlone))
