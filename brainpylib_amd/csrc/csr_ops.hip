@@ -993,8 +993,8 @@ __device__ __forceinline__ void gather_hub_rows(const F *__restrict__ data, cons
 // x 16 loads per row a quarter of the index requests lie beyond their row.  Here every wave owns a contiguous
 // range of the nonzeros that begins and ends at row boundaries (the rows whose first nonzero lies in its
 // equal share of the nonzeros: no row is shared by two waves, so nothing is left for a second kernel) and
-// takes it in steps of 768 or 1,024: three or four 16-byte nontemporal loads of indices per lane (the next
-// steps' are under way while a step is worked on), twelve or sixteen probes of the event bitmap in LDS per
+// takes it in steps of 768 or 1,280: three or five 16-byte nontemporal loads of indices per lane (the next
+// step's are under way while a step is worked on), twelve or twenty probes of the event bitmap in LDS per
 // lane.  Rows are looked up for the HITS only: the lanes leave the positions of their hits (some 5 % of the
 // nonzeros) in a queue in LDS, compacted by a prefix sum over the wave, and every lane then takes one hit: its
 // weight, a six-step search of a window of 65 row offsets in LDS for its row, one atomic addition to that
@@ -1003,9 +1003,12 @@ constexpr uint32_t kFlatEvRows = 64;     // rows of a window (one per lane)
 constexpr uint32_t kFlatEvMinMean = 16, kFlatEvMaxMean = 384;
 constexpr uint32_t kFlatEvSharedMaxMean = 256, kFlatEvSharedMinNnz = 45000000;  // (in the kernel that shares its CU)
 constexpr uint32_t kFlatEvWaves = 16;
-// Loads of four indices per lane and step, and steps under way.  One workgroup per CU (a bitmap of more than 80
-// KB): 4 and 3, 48 registers of indices.  Two workgroups per CU must keep to 64 registers: 3 and 2.
-constexpr int kFlatEvQuadsAlone = 4, kFlatEvDepthAlone = 3, kFlatEvQuadsShared = 3, kFlatEvDepthShared = 2;
+// Loads of four indices per lane and step, and sets of index registers (steps under way).  One workgroup per CU (a
+// bitmap of more than 80 KB): 5 and 2 (steps of 1,280 nonzeros; measured against 3..8 loads and 2 or 3 sets: 4 and 3
+// took 146 / 94 us for 1,000,000 x 1,000,000 with 100 per row, weights per nonzero / one weight, 5 and 2 141 / 86; steps
+// that are a power of two in bytes were the slowest of their neighbours every time).  Two workgroups per CU must keep to
+// 64 registers: 3 and 2.
+constexpr int kFlatEvQuadsAlone = 5, kFlatEvDepthAlone = 2, kFlatEvQuadsShared = 3, kFlatEvDepthShared = 2;
 // hits queued at a time (more in a step: further rounds)
 constexpr uint32_t kFlatEvQueueAlone = 256, kFlatEvQueueShared = 128;
 // LDS of the walk behind the bitmap: accumulators, windows of row offsets and queues of 16 waves

@@ -274,10 +274,10 @@ def test_gather_flat_walk_over_the_nonzeros_of_short_rows(cuda, oracle_mod, kind
   n_col, rate = 900_000, 0.05
   if kind == "ragged":      # empty rows, rows of one nonzero, rows of a thousand
     counts = rng.choice([0, 1, 3, 40, 150, 1000], size=60_000, p=[0.2, 0.1, 0.2, 0.3, 0.15, 0.05])
-  elif kind == "even":      # every row 100 nonzeros: ten rows and a bit per step of 1,024
+  elif kind == "even":      # every row 100 nonzeros: twelve rows and a bit per step of 1,280
     counts = np.full(200_000, 100)
   elif kind == "step":      # rows of exactly one step and of exactly one quad
-    counts = np.where(np.arange(30_000) % 3 == 0, 1024, 4)
+    counts = np.where(np.arange(40_000) % 4 == 0, 1280, 4)
   elif kind == "hub":       # one row longer than a wave's whole share, between rows of 30
     counts = np.full(40_000, 30)
     counts[17_777] = 700_000
