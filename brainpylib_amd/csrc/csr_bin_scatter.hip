@@ -894,9 +894,18 @@ __global__ __launch_bounds__(kBinThreads) __attribute__((amdgpu_num_sgpr(80))) v
 // waves, one after the other: 1,000,000 rows of 100 into 4,000 columns at 5 % events 76 us, this one 38.)
 constexpr uint32_t kWindowEventMaxCols = 8192;
 
-// workgroups that take part: one per kPairsPerProducer active nonzeros (estimated from the mean row length)
-__device__ __forceinline__ uint32_t window_event_producers(uint32_t total, uint32_t nnz, uint32_t n_row, uint32_t launched) {
-  const uint64_t want = (static_cast<uint64_t>(total) * (nnz / n_row + 1u) + kPairsPerProducer - 1u) / kPairsPerProducer;
+// Workgroups that take part.  P of them walk pairs / P active nonzeros each (estimated from the mean row length) and
+// then each writes its window of `window_bytes` for the kernel that adds the windows to read: the two costs are
+// equal where a workgroup takes sqrt(pairs * window_bytes / c) nonzeros, c = the cost of a byte of window over the
+// cost of a nonzero: measured 300 with one weight, 600 with weights per nonzero (a float64 atomic per nonzero).
+// (4,096 per workgroup whatever the window: 50,000 x 50,000 with 200 per row, one weight, at 1 / 5 % events 20 / 31 us
+// instead of 17 / 23; 32,000 x 8,192 with 1,000 per row at 5 % 24 instead of 19.5, with weights 21 instead of 19.)
+__device__ __forceinline__ uint32_t window_event_producers(uint32_t total, uint32_t nnz, uint32_t n_row, uint32_t launched,
+                                                           uint32_t window_bytes, bool heter) {
+  const uint64_t pairs = static_cast<uint64_t>(total) * (nnz / n_row + 1u);
+  float each = __builtin_sqrtf(static_cast<float>(pairs) * static_cast<float>(window_bytes) * (heter ? 1.f / 600.f : 1.f / 300.f));
+  each = each < 2048.f ? 2048.f : each > 65536.f ? 65536.f : each;
+  const uint64_t want = (pairs + static_cast<uint32_t>(each) - 1u) / static_cast<uint32_t>(each);
   return want < 1u ? 1u : want > launched ? launched : static_cast<uint32_t>(want);
 }
 
@@ -957,7 +966,8 @@ __global__ __launch_bounds__(kBinThreads) void active_rows_window_kernel(
   } else {
     total = active_count[0] < list_cap ? active_count[0] : list_cap;  // (never beyond the list)
   }
-  const uint32_t producers = window_event_producers(total, indptr[n_row], n_row, gridDim.x / slices);
+  const uint32_t producers = window_event_producers(total, indptr[n_row], n_row, gridDim.x / slices,
+                                                    n_col * static_cast<uint32_t>(sizeof(A)), HETER);
   const uint32_t p = blockIdx.x / slices, slice = blockIdx.x % slices;
   if (blockIdx.x == 0 && tid == 0) groups_out[0] = producers;  // (for the kernel that adds the windows)
   if (p >= producers) return;
